@@ -1,0 +1,319 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused mHC layer path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--mode graph|eager]
+
+A step is one forward + backward pass of the layer over one batch of synthetic, seeded input
+that is already resident in HBM, issued through the C ABI (libmhc_hip.so).  Prints ONE JSON
+line.  `value` is microseconds per step over K back-to-back steps (wall clock, synchronised on
+both sides); `roofline` prices the same step's device time (HIP events on the launch stream)
+against the algorithmic HBM bytes of the configuration; `cpu_baseline` is the naive PyTorch
+restatement of the layer (the oracle) timed on this machine's host cores.
+
+Configurations (BASELINE.json order): c1 static fp32 forward; c2..c5 dynamic bf16 fwd+bwd.
+View "L" (default): the layer computes f = RMSNorm(x_agg) * w itself, as MHCLayer does.
+View "K": f [B, C] is an input and df an output (kernel-level view of the configurations).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "mhc.cu_amd"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+CONFIGS = {
+    "c1": dict(kind="static", B=320, n=4, C=1280, dtype="f32", bwd=False),
+    "c2": dict(kind="dynamic", B=320, n=4, C=1280, dtype="bf16", bwd=True),
+    "c3": dict(kind="dynamic", B=1280, n=4, C=2560, dtype="bf16", bwd=True),
+    "c4": dict(kind="dynamic", B=256, n=8, C=1280, dtype="bf16", bwd=True),
+    "c5": dict(kind="dynamic", B=128, n=32, C=1280, dtype="bf16", bwd=True),
+}
+T_ITERS, EPS = 20, 1e-6
+
+
+def algorithmic_bytes(cfg, view):
+    """Compulsory HBM traffic of one step: (forward, backward) bytes.
+
+    forward : read x [+ f], read phi (dynamic), write y
+    backward: read dy, x [+ f], read phi, write dx [+ df], write dphi (fp32)
+    """
+    B, n, C = cfg["B"], cfg["n"], cfg["C"]
+    s = 4 if cfg["dtype"] == "f32" else 2
+    BnC, BC, nC, D = B * n * C, B * C, n * C, n * n + 2 * n
+    fvec = BC if view == "K" else 0
+    phi = 2 * nC * D if cfg["kind"] == "dynamic" else 0
+    fwd = s * (BnC + fvec) + phi + s * BnC
+    bwd = 0
+    if cfg["bwd"]:
+        bwd = s * (2 * BnC + fvec) + phi + s * (BnC + fvec) + 2 * phi  # dphi fp32 = 2x bf16 phi bytes
+    return fwd, bwd
+
+
+class Step:
+    """Pre-allocated tensors and the two C-ABI calls of one configuration."""
+
+    def __init__(self, cfg, view, torch):
+        from mhc import _lib
+        from oracle import naive_mhc as nm
+
+        self.torch, self.lib, self._lib = torch, _lib.lib, _lib
+        self.cfg, self.view = cfg, view
+        B, n, C = cfg["B"], cfg["n"], cfg["C"]
+        dev = torch.device("cuda:0")
+        act = torch.float32 if cfg["dtype"] == "f32" else torch.bfloat16
+        bf = cfg["dtype"] == "bf16"
+        self.dynamic = cfg["kind"] == "dynamic"
+        if self.dynamic:
+            x, dy, f, p = nm.make_dynamic_inputs(B, n, C, bf16_round=bf, with_f=(view == "K"))
+        else:
+            x, dy, f, p = nm.make_static_inputs(B, n, C, with_f=(view == "K"))
+        self.host = dict(x=x, dy=dy, f=f, p=p)
+        to = lambda t, dt: t.to(dt).to(dev).contiguous()
+        self.x, self.dy = to(x, act), to(dy, act)
+        self.f = None if f is None else to(f, act)
+        self.w = to(p["w"], torch.bfloat16 if bf else torch.float32)
+        D = n * n + 2 * n
+        f32 = dict(dtype=torch.float32, device=dev)
+        self.y = torch.empty((B, n, C), dtype=act, device=dev)
+        self.dx = torch.empty_like(self.x)
+        self.df = None if f is None else torch.empty_like(self.f)
+        self.dw = torch.empty(C, **f32)
+        self.q = torch.empty(B, **f32)
+        if self.dynamic:
+            phi = torch.cat([p["phi_pre"], p["phi_post"], p["phi_res"]], 0)
+            self.phi = to(phi, torch.bfloat16 if bf else torch.float32)
+            self.bias = to(torch.cat([p["b_pre"], p["b_post"], p["b_res"].reshape(-1)]), torch.float32)
+            self.alpha = to(torch.stack([p["alpha_pre"], p["alpha_post"], p["alpha_res"]]), torch.float32)
+            self.Hp, self.Ho = torch.empty((B, n), **f32), torch.empty((B, n), **f32)
+            self.M, self.P = torch.empty((B, n, n), **f32), torch.empty((B, D), **f32)
+            self.r = torch.empty(B, **f32)
+            self.dphi = torch.empty((D, n * C), **f32)
+            self.dbias, self.dalpha = torch.empty(D, **f32), torch.empty(3, **f32)
+            nbytes = self.lib.mhc_layer_dynamic_workspace_bytes(B, n, C)
+        else:
+            self.Hl = [to(p[k], torch.float32) for k in ("H_pre", "H_post", "H_res")]
+            self.Hp, self.Ho = torch.empty(n, **f32), torch.empty(n, **f32)
+            self.M = torch.empty((n, n), **f32)
+            self.dH = [torch.empty(n, **f32), torch.empty(n, **f32), torch.empty((n, n), **f32)]
+            nbytes = self.lib.mhc_layer_static_workspace_bytes(B, n, C)
+        self.ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+
+    def _stream(self):
+        return ctypes.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+
+    def forward(self):
+        L, c, p, dc = self.lib, self.cfg, self._lib.ptr, self._lib.dtype_code
+        B, n, C = c["B"], c["n"], c["C"]
+        if self.dynamic:
+            st = L.mhc_layer_fwd_dynamic(p(self.x), dc(self.x), p(self.w), dc(self.w), p(self.phi), dc(self.phi),
+                                         p(self.bias), p(self.alpha), p(self.f), p(self.y), dc(self.y),
+                                         p(self.Hp), p(self.Ho), p(self.M), p(self.P), p(self.r), p(self.q),
+                                         B, n, C, T_ITERS, EPS, p(self.ws), self.ws.numel(), self._stream())
+        else:
+            st = L.mhc_layer_fwd(p(self.x), dc(self.x), p(self.w), dc(self.w), p(self.Hl[0]), p(self.Hl[1]),
+                                 p(self.Hl[2]), p(self.f), p(self.y), dc(self.y), p(self.Hp), p(self.Ho),
+                                 p(self.M), p(self.q), B, n, C, T_ITERS, EPS, p(self.ws), self.ws.numel(),
+                                 self._stream())
+        self._lib.check("forward", st)
+
+    def backward(self):
+        L, c, p, dc = self.lib, self.cfg, self._lib.ptr, self._lib.dtype_code
+        B, n, C = c["B"], c["n"], c["C"]
+        if self.dynamic:
+            st = L.mhc_layer_bwd_dynamic(p(self.dy), dc(self.dy), p(self.x), dc(self.x), p(self.w), dc(self.w),
+                                         p(self.phi), dc(self.phi), p(self.bias), p(self.alpha), p(self.f),
+                                         p(self.Hp), p(self.Ho), p(self.M), p(self.P), p(self.r), p(self.q),
+                                         p(self.dx), p(self.df), p(self.dw), p(self.dphi), p(self.dbias),
+                                         p(self.dalpha), B, n, C, T_ITERS, EPS, p(self.ws), self.ws.numel(),
+                                         self._stream())
+        else:
+            st = L.mhc_layer_bwd(p(self.dy), dc(self.dy), p(self.x), dc(self.x), p(self.w), dc(self.w),
+                                 p(self.Hl[0]), p(self.Hl[1]), p(self.Hl[2]), p(self.f), p(self.Hp), p(self.Ho),
+                                 p(self.M), p(self.q), p(self.dx), p(self.df), p(self.dw), p(self.dH[0]),
+                                 p(self.dH[1]), p(self.dH[2]), B, n, C, T_ITERS, EPS, p(self.ws),
+                                 self.ws.numel(), self._stream())
+        self._lib.check("backward", st)
+
+    def step(self):
+        self.forward()
+        if self.cfg["bwd"]:
+            self.backward()
+
+
+def trimmed_mean(v):
+    v = sorted(v)
+    k = len(v) // 10
+    v = v[k:len(v) - k] if len(v) > 2 * k else v
+    return sum(v) / len(v)
+
+
+def event_times(torch, fn, reps, flush=None):
+    """Device time of fn() in microseconds, one HIP-event pair per call on the current stream."""
+    out = []
+    for _ in range(reps):
+        if flush is not None:
+            flush.fill_(1.0)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        out.append(e0.elapsed_time(e1) * 1e3)
+    return out
+
+
+def cpu_baseline(step, torch, budget_s=20.0):
+    """The oracle (naive PyTorch layer) on the host cores: same seeded inputs, fp32."""
+    from oracle import naive_mhc as nm
+
+    cfg, h = step.cfg, step.host
+    cores = torch.get_num_threads()
+    f = h["f"]
+
+    def run():
+        if cfg["kind"] == "dynamic":
+            if cfg["bwd"]:
+                nm.mhc_dynamic_fwd_bwd(h["x"], h["p"], h["dy"], T_ITERS, EPS, f_inject=f)
+            else:
+                with torch.no_grad():
+                    p = h["p"]
+                    nm.mhc_dynamic_forward(h["x"], p["w"], p["phi_pre"], p["phi_post"], p["phi_res"],
+                                           p["alpha_pre"], p["alpha_post"], p["alpha_res"], p["b_pre"],
+                                           p["b_post"], p["b_res"], T_ITERS, EPS, f_inject=f)
+        else:
+            if cfg["bwd"]:
+                nm.mhc_static_fwd_bwd(h["x"], h["p"], h["dy"], T_ITERS, EPS, f_inject=f)
+            else:
+                with torch.no_grad():
+                    p = h["p"]
+                    nm.mhc_static_forward(h["x"], p["w"], p["H_pre"], p["H_post"], p["H_res"], T_ITERS,
+                                          EPS, f_inject=f)
+
+    for _ in range(3):
+        run()
+    times, t_start = [], time.perf_counter()
+    while len(times) < 10 or (time.perf_counter() - t_start < budget_s and len(times) < 200):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_start > 3 * budget_s:
+            break
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": med * 1e6, "unit": "us/layer", "cores": cores, "kind": "port",
+            "sample": f"{len(times)} runs of the full {cfg['kind']} "
+                      f"{'fwd+bwd' if cfg['bwd'] else 'fwd'} step at B={cfg['B']} n={cfg['n']} C={cfg['C']}, "
+                      f"fp32 naive PyTorch layer, median"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--view", default="L", choices=["L", "K"])
+    ap.add_argument("--mode", default="graph", choices=["graph", "eager"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1 "
+              "(every sample is independent, see DESIGN.md for how the path would shard)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    cfg = CONFIGS[a.config]
+    step = Step(cfg, a.view, torch)
+
+    # ---- warm-up, optional graph capture ---------------------------------------------------
+    for _ in range(max(a.warmup, 1)):
+        step.step()
+    torch.cuda.synchronize()
+    mode, graph = a.mode, None
+    if mode == "graph":
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step.step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step.step()
+            graph.replay()
+            torch.cuda.synchronize()
+        except Exception as exc:  # capture is an optimisation of the launch path only
+            print(f"bench.py: graph capture failed ({exc}); using eager launches", file=sys.stderr)
+            mode, graph = "eager", None
+    run = graph.replay if graph is not None else step.step
+
+    # ---- timed region: exactly K steps -------------------------------------------------------
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    us_per_step = wall / a.steps * 1e6
+
+    # ---- device time with HIP events on the launch stream (warm and cold caches) -------------
+    reps = min(max(a.steps, 20), 200)
+    dev_step = trimmed_mean(event_times(torch, run, reps))
+    dev_fwd = trimmed_mean(event_times(torch, step.forward, reps))
+    dev_bwd = trimmed_mean(event_times(torch, step.backward, reps)) if cfg["bwd"] else 0.0
+    flush = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda")
+    cold_step = trimmed_mean(event_times(torch, run, min(reps, 50), flush=flush))
+    del flush
+
+    fwd_b, bwd_b = algorithmic_bytes(cfg, a.view)
+    alg = fwd_b + bwd_b
+    achieved = alg / (dev_step * 1e-6) / 1e9
+    out = {
+        "metric": "mHC fwd+bwd us/layer" if cfg["bwd"] else "mHC fwd us/layer",
+        "value": us_per_step,
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": us_per_step / 1e3,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": cfg["dtype"],
+        "data": "synthetic",
+        "config": {"workload": f"{a.config}: {cfg['kind']}-H mHC layer "
+                               f"{'fwd+bwd' if cfg['bwd'] else 'fwd'} B={cfg['B']} C={cfg['C']} n={cfg['n']} "
+                               f"{cfg['dtype']} T={T_ITERS} eps={EPS}",
+                   "view": a.view, "launch": mode, "cache": "warm (back-to-back steps)"},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "whole step (all launches of one forward+backward)",
+                     "algorithmic_bytes": alg, "device_us": dev_step,
+                     "fwd": {"algorithmic_bytes": fwd_b, "device_us": dev_fwd,
+                             "achieved": fwd_b / (dev_fwd * 1e-6) / 1e9},
+                     "bwd": ({"algorithmic_bytes": bwd_b, "device_us": dev_bwd,
+                              "achieved": bwd_b / (dev_bwd * 1e-6) / 1e9} if cfg["bwd"] else None),
+                     "cold_cache": {"device_us": cold_step, "achieved": alg / (cold_step * 1e-6) / 1e9,
+                                    "flush": "512 MiB fill before every step"}},
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(step, torch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

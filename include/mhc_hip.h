@@ -1,0 +1,158 @@
+/*
+ * mhc_hip.h - C ABI of the MI355X (gfx950) mHC layer library, libmhc_hip.so.
+ *
+ * Plain pointers and sizes only.  Every pointer is a DEVICE pointer unless stated otherwise;
+ * every call only enqueues work on `stream` (a hipStream_t passed as void*, NULL = the
+ * default stream) and returns a status immediately.  The library keeps no global mutable
+ * state, never allocates, never synchronises, never prints and never exits: the caller owns
+ * all memory, including the scratch `workspace` (size from the *_workspace_bytes queries,
+ * 256-byte aligned).  Calls are re-entrant across streams as long as each in-flight call has
+ * its own workspace.
+ *
+ * Each entry point names the interface of the reference (AndreSlavescu/mHC.cu) that it
+ * replaces; paths are relative to the reference tree.
+ *
+ * Tensor layouts (row-major, contiguous):
+ *   x, y, dy, dx      [B, n, C]     activations, dtype MHC_F32 or MHC_BF16
+ *   f, df             [B, C]        same dtype as x
+ *   w (rmsnorm)       [C]           MHC_F32 or MHC_BF16
+ *   phi, dphi         [D, nC]       D = n*n + 2n, rows [pre(n) | post(n) | res(n*n, i*n+j)];
+ *                                   phi MHC_F32 or MHC_BF16, dphi always fp32
+ *   bias, dbias       [D]   fp32    same row order (b_pre | b_post | b_res)
+ *   alpha, dalpha     [3]   fp32    (alpha_pre, alpha_post, alpha_res), read on the device
+ *   H_pre, H_post     [B, n] fp32   activated coefficients (static H: [n])
+ *   M                 [B, n, n] fp32 Sinkhorn-normalised mixing matrix (static H: [n, n])
+ *   P                 [B, D] fp32   rows of RMSNorm(x_flat) @ phi^T (before alpha and bias)
+ *   r, q              [B]   fp32    r = rms of x_flat, q = rms of the aggregated stream
+ */
+#ifndef MHC_HIP_H
+#define MHC_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define MHC_API __attribute__((visibility("default")))
+#else
+#define MHC_API
+#endif
+
+#define MHC_ABI_VERSION 1
+#define MHC_MAX_N 32
+
+enum mhc_dtype { MHC_F32 = 0, MHC_BF16 = 1 };
+
+enum mhc_status {
+    MHC_OK = 0,
+    MHC_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
+    MHC_ERR_BAD_N = 2,          /* expansion rate outside 1..MHC_MAX_N */
+    MHC_ERR_BAD_SHAPE = 3,      /* B, C or iters not positive / too large */
+    MHC_ERR_BAD_DTYPE = 4,      /* unknown or unsupported dtype combination */
+    MHC_ERR_MISALIGNED = 5,     /* a tensor base pointer is not 16-byte aligned */
+    MHC_ERR_WORKSPACE = 6,      /* workspace NULL, misaligned or too small */
+    MHC_ERR_LAUNCH = 7          /* the HIP runtime refused a kernel launch */
+};
+
+/* Version of this header the library was built from (== MHC_ABI_VERSION). */
+MHC_API int mhc_abi_version(void);
+
+/* Static, NUL-terminated description of a status code (host pointer). */
+MHC_API const char *mhc_status_string(int status);
+
+/* ------------------------------------------------------------------------------------------
+ * Dynamic-H layer.  Replaces mhc_cuda.mhc_layer_fwd_dynamic / mhc_layer_bwd_dynamic
+ * (src/python/bindings.cu:405-481, :483-542) together with the part of the backward that the
+ * reference runs as torch code (src/python/mhc/ops.py:276-361).
+ * ---------------------------------------------------------------------------------------- */
+
+/* Scratch bytes needed by one dynamic forward or backward call of this shape. */
+MHC_API size_t mhc_layer_dynamic_workspace_bytes(int B, int n, int C);
+
+/*
+ * y = M_b x_b + H_post_b (x) f_b with per-sample coefficients computed from x.
+ * f_inject == NULL: f = RMSNorm(sum_i H_pre[b,i] x[b,i,:]) * w  (the layer).
+ * f_inject != NULL: f is that [B, C] tensor (kernel-level view; w is ignored, may be NULL).
+ * H_pre, H_post, M, P, r, q are outputs kept for the backward call; all six are required.
+ */
+MHC_API int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype,
+                          const void *phi, int phi_dtype, const float *bias, const float *alpha,
+                          const void *f_inject, void *y, int y_dtype, float *H_pre, float *H_post,
+                          float *M, float *P, float *r, float *q, int B, int n, int C, int iters,
+                          float eps, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Gradients of the call above for upstream gradient dy (dtype y_dtype).
+ * dx has x's dtype.  df (x's dtype) is written only when f_inject != NULL and df != NULL;
+ * dw [C] fp32 is written only when f_inject == NULL.  dphi [D, nC], dbias [D], dalpha [3] fp32.
+ * Every output is fully overwritten (no pre-zeroing needed); sums are order-deterministic.
+ */
+MHC_API int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtype, const void *w,
+                          int w_dtype, const void *phi, int phi_dtype, const float *bias,
+                          const float *alpha, const void *f_inject, const float *H_pre,
+                          const float *H_post, const float *M, const float *P, const float *r,
+                          const float *q, void *dx, void *df, float *dw, float *dphi,
+                          float *dbias, float *dalpha, int B, int n, int C, int iters, float eps,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Static-H layer.  Replaces mhc_cuda.mhc_layer_fwd / mhc_layer_fwd_inference / mhc_layer_bwd
+ * (src/python/bindings.cu:264-328, :221-262, :330-401).
+ * ---------------------------------------------------------------------------------------- */
+
+MHC_API size_t mhc_layer_static_workspace_bytes(int B, int n, int C);
+
+/*
+ * H_pre_logits, H_post_logits [n], H_res_logits [n, n] fp32 are the raw parameters.
+ * Outputs H_pre, H_post [n], M [n, n] (activated) and q [B] may each be NULL (inference):
+ * they are then kept in the workspace only.
+ */
+MHC_API int mhc_layer_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
+                  const float *H_pre_logits, const float *H_post_logits,
+                  const float *H_res_logits, const void *f_inject, void *y, int y_dtype,
+                  float *H_pre, float *H_post, float *M, float *q, int B, int n, int C,
+                  int iters, float eps, void *workspace, size_t workspace_bytes, void *stream);
+
+/* dH_pre, dH_post [n], dH_res [n, n] fp32 are gradients w.r.t. the raw logits. */
+MHC_API int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const void *w,
+                  int w_dtype, const float *H_pre_logits, const float *H_post_logits,
+                  const float *H_res_logits, const void *f_inject, const float *H_pre,
+                  const float *H_post, const float *M, const float *q, void *dx, void *df,
+                  float *dw, float *dH_pre, float *dH_post, float *dH_res, int B, int n, int C,
+                  int iters, float eps, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Stand-alone operators.  Replace mhc_cuda.sinkhorn_knopp_fwd / _bwd and rmsnorm_fwd / _bwd
+ * (src/python/bindings.cu:115-164).
+ * ---------------------------------------------------------------------------------------- */
+
+/*
+ * `batch` independent rows x cols fp32 matrices (rows, cols <= 128).  No exp; a row / column
+ * is divided by its sum only when the sum exceeds eps
+ * (src/csrc/tests/test_sinkhorn_knopp.cu:16-47).
+ */
+MHC_API int mhc_sinkhorn_knopp_fwd(const float *inp, float *out, int batch, int rows, int cols, int iters,
+                           float eps, void *stream);
+
+/* Exact gradient of the call above w.r.t. inp (recomputes the iterates from inp). */
+MHC_API int mhc_sinkhorn_knopp_bwd(const float *grad_out, const float *inp, float *d_inp, int batch,
+                           int rows, int cols, int iters, float eps, void *workspace,
+                           size_t workspace_bytes, void *stream);
+MHC_API size_t mhc_sinkhorn_knopp_bwd_workspace_bytes(int batch, int rows, int cols, int iters);
+
+/* out = inp / sqrt(mean(inp^2) + eps) * w, row-wise over [rows, C]; rms [rows] fp32 (may be NULL). */
+MHC_API int mhc_rmsnorm_fwd(const void *inp, int dtype, const void *w, int w_dtype, void *out,
+                    float *rms, int rows, int C, float eps, void *stream);
+
+/* d_inp has inp's dtype; d_w [C] fp32 (deterministic two-pass column sum through workspace). */
+MHC_API int mhc_rmsnorm_bwd(const void *grad_out, const void *inp, int dtype, const void *w, int w_dtype,
+                    const float *rms, void *d_inp, float *d_w, int rows, int C, void *workspace,
+                    size_t workspace_bytes, void *stream);
+MHC_API size_t mhc_rmsnorm_bwd_workspace_bytes(int rows, int C);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MHC_HIP_H */

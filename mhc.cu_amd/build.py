@@ -1,0 +1,66 @@
+"""Builds libmhc_hip.so (hand-written HIP kernels + C ABI) for gfx950 with hipcc.
+
+    python mhc.cu_amd/build.py [--jobs N] [--force]
+
+hipcc cross-compiles for gfx950 without a GPU.  The library lands in mhc.cu_amd/mhc/ next to
+the Python package that loads it; object files go to mhc.cu_amd/build/.
+"""
+from __future__ import annotations
+
+import argparse
+import concurrent.futures as cf
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "mhc", "libmhc_hip.so")
+
+SOURCES = ["capi.hip", "proj_fwd.hip", "coef_fwd.hip", "mix_fwd.hip", "mix_bwd_reduce.hip",
+           "mix_bwd_dx.hip", "param_grads.hip", "ops.hip"]
+
+# -packed-fp32-ops off: v_pk_*_f32 forms are not trusted on this hardware pool.
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wall", "-Wno-unused-function"]
+
+
+def _hipcc():
+    for c in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if c and (os.path.isabs(c) and os.path.exists(c) or not os.path.isabs(c)):
+            return c
+    return "hipcc"
+
+
+def _compile(src):
+    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    cmd = [_hipcc(), *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in p.stderr.splitlines() if "packed-fp32-ops" not in l)
+    return src, obj, p.returncode, err
+
+
+def build(jobs: int = 8, verbose: bool = True):
+    os.makedirs(OBJ, exist_ok=True)
+    objs = []
+    with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+        for src, obj, rc, err in ex.map(_compile, SOURCES):
+            if err.strip() and verbose:
+                print(f"[{src}]\n{err}", file=sys.stderr)
+            if rc != 0:
+                raise RuntimeError(f"hipcc failed on {src}")
+            objs.append(obj)
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    subprocess.check_call(cmd)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
+    a = ap.parse_args()
+    build(a.jobs)

@@ -1,0 +1,328 @@
+// C ABI of libmhc_hip.so (declared in include/mhc_hip.h): argument validation, workspace
+// carving and the launch sequence of each entry point.  No allocation, no synchronisation,
+// no global state; every call only enqueues kernels on the caller's stream.
+#include "../../include/mhc_hip.h"
+
+#include "launchers.h"
+
+#include <stdint.h>
+
+using namespace mhc;
+
+namespace {
+
+struct Carver {
+    char *base;
+    size_t off = 0;
+    explicit Carver(void *p) : base(static_cast<char *>(p)) {}
+    float *floats(size_t count) {
+        float *p = base ? reinterpret_cast<float *>(base + off) : nullptr;
+        off += (count * sizeof(float) + 255) / 256 * 256;
+        return p;
+    }
+};
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool valid_dtype(int d) { return d == MHC_F32 || d == MHC_BF16; }
+inline bool valid_io(int x_dtype, int y_dtype) {
+    // activations in / out: (f32, f32), (bf16, bf16), (bf16 in, f32 out)
+    return (x_dtype == MHC_F32 && y_dtype == MHC_F32) || (x_dtype == MHC_BF16 && valid_dtype(y_dtype));
+}
+
+int check_shape(int B, int n, int C, int iters) {
+    if (n < 1 || n > MHC_MAX_N) return MHC_ERR_BAD_N;
+    if (B < 1 || C < 1 || iters < 0 || iters > 1024) return MHC_ERR_BAD_SHAPE;
+    if ((long long)B * n * C > (1ll << 40)) return MHC_ERR_BAD_SHAPE;
+    return MHC_OK;
+}
+
+int ws_check(void *ws, size_t have, size_t need) {
+    if (need == 0) return MHC_OK;
+    if (!ws || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0 || have < need) return MHC_ERR_WORKSPACE;
+    return MHC_OK;
+}
+
+#define MHC_LAUNCH(expr)                              \
+    do {                                              \
+        if ((expr) != hipSuccess) return MHC_ERR_LAUNCH; \
+    } while (0)
+
+// ---- dynamic workspace layout ----------------------------------------------------------------
+struct DynFwdWs { float *Ppart, *ssqpart; size_t bytes; };
+struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *cs_dt, *cs_u, *dphi_part; size_t bytes; };
+
+int max_ksplit(int B, int n, int C) { return proj_fwd_ksplit(kBF16, kBF16, B, n, C); }
+
+DynFwdWs carve_dyn_fwd(void *ws, int B, int n, int C) {
+    Carver c(ws);
+    const int ks = max_ksplit(B, n, C);
+    DynFwdWs w;
+    w.Ppart = c.floats((size_t)ks * B * padded_D(n));
+    w.ssqpart = c.floats((size_t)ks * B);
+    w.bytes = c.off;
+    return w;
+}
+
+DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
+    Carver c(ws);
+    const int D = n * n + 2 * n, nC = n * C;
+    DynBwdWs w;
+    w.dt = c.floats((size_t)B * (D + 3));
+    w.dP = c.floats((size_t)B * padded_D(n));
+    w.cx = c.floats(B);
+    w.s1 = c.floats(B);
+    w.u = c.floats((size_t)B * C);
+    w.cs_dt = c.floats(colsum_workspace_floats(B, D + 3));
+    w.cs_u = c.floats(colsum_workspace_floats(B, C));
+    const int bs = dphi_batch_splits(B, n, C);
+    w.dphi_part = c.floats(bs > 1 ? (size_t)bs * D * nC : 0);
+    w.bytes = c.off;
+    return w;
+}
+
+// ---- static workspace layout -----------------------------------------------------------------
+struct StaFwdWs { float *Hpre, *Hpost, *M, *q; size_t bytes; };
+struct StaBwdWs { float *red, *s1, *u, *red_sum, *cs_red, *cs_u; size_t bytes; };
+
+StaFwdWs carve_sta_fwd(void *ws, int B, int n) {
+    Carver c(ws);
+    StaFwdWs w;
+    w.Hpre = c.floats(n); w.Hpost = c.floats(n); w.M = c.floats((size_t)n * n); w.q = c.floats(B);
+    w.bytes = c.off;
+    return w;
+}
+
+StaBwdWs carve_sta_bwd(void *ws, int B, int n, int C) {
+    Carver c(ws);
+    const int D = n * n + 2 * n;
+    StaBwdWs w;
+    w.red = c.floats((size_t)B * D);
+    w.s1 = c.floats(B);
+    w.u = c.floats((size_t)B * C);
+    w.red_sum = c.floats(D);
+    w.cs_red = c.floats(colsum_workspace_floats(B, D));
+    w.cs_u = c.floats(colsum_workspace_floats(B, C));
+    w.bytes = c.off;
+    return w;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mhc_abi_version(void) { return MHC_ABI_VERSION; }
+
+const char *mhc_status_string(int status) {
+    switch (status) {
+        case MHC_OK: return "ok";
+        case MHC_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case MHC_ERR_BAD_N: return "expansion rate n must be in 1..32";
+        case MHC_ERR_BAD_SHAPE: return "B, C or iters out of range";
+        case MHC_ERR_BAD_DTYPE: return "unsupported dtype combination";
+        case MHC_ERR_MISALIGNED: return "tensor base pointer is not 16-byte aligned";
+        case MHC_ERR_WORKSPACE: return "workspace NULL, not 256-byte aligned or too small";
+        case MHC_ERR_LAUNCH: return "HIP kernel launch failed";
+        default: return "unknown status";
+    }
+}
+
+// ===============================================================================================
+// dynamic H
+// ===============================================================================================
+size_t mhc_layer_dynamic_workspace_bytes(int B, int n, int C) {
+    if (check_shape(B, n, C, 0) != MHC_OK) return 0;
+    const size_t f = carve_dyn_fwd(nullptr, B, n, C).bytes;
+    const size_t b = carve_dyn_bwd(nullptr, B, n, C).bytes;
+    return f > b ? f : b;
+}
+
+int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype, const void *phi,
+                          int phi_dtype, const float *bias, const float *alpha,
+                          const void *f_inject, void *y, int y_dtype, float *H_pre, float *H_post,
+                          float *M, float *P, float *r, float *q, int B, int n, int C, int iters,
+                          float eps, void *workspace, size_t workspace_bytes, void *stream) {
+    if (int s = check_shape(B, n, C, iters)) return s;
+    if (!x || !phi || !bias || !alpha || !y || !H_pre || !H_post || !M || !P || !r || !q)
+        return MHC_ERR_NULL_POINTER;
+    if (!f_inject && !w) return MHC_ERR_NULL_POINTER;
+    if (!valid_io(x_dtype, y_dtype) || !valid_dtype(phi_dtype) || (w && !valid_dtype(w_dtype)))
+        return MHC_ERR_BAD_DTYPE;
+    if (!aligned16(x) || !aligned16(y) || !aligned16(phi) || (f_inject && !aligned16(f_inject)))
+        return MHC_ERR_MISALIGNED;
+    const DynFwdWs ws = carve_dyn_fwd(workspace, B, n, C);
+    if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int KS = proj_fwd_ksplit(x_dtype, phi_dtype, B, n, C);
+    MHC_LAUNCH(launch_proj_fwd(x, x_dtype, phi, phi_dtype, ws.Ppart, ws.ssqpart, KS, B, n, C, st));
+    MHC_LAUNCH(launch_coef_fwd(ws.Ppart, ws.ssqpart, KS, padded_D(n), alpha, bias, bias + n,
+                               bias + 2 * n, H_pre, H_post, M, P, r, B, n, n * C, iters, eps, st));
+    MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, H_pre, H_post, M, n, q,
+                              B, n, C, eps, st));
+    return MHC_OK;
+}
+
+int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtype, const void *w,
+                          int w_dtype, const void *phi, int phi_dtype, const float *bias,
+                          const float *alpha, const void *f_inject, const float *H_pre,
+                          const float *H_post, const float *M, const float *P, const float *r,
+                          const float *q, void *dx, void *df, float *dw, float *dphi,
+                          float *dbias, float *dalpha, int B, int n, int C, int iters, float eps,
+                          void *workspace, size_t workspace_bytes, void *stream) {
+    if (int s = check_shape(B, n, C, iters)) return s;
+    if (!dy || !x || !phi || !bias || !alpha || !H_pre || !H_post || !M || !P || !r || !q || !dx ||
+        !dphi || !dbias || !dalpha)
+        return MHC_ERR_NULL_POINTER;
+    if (!f_inject && (!w || !dw)) return MHC_ERR_NULL_POINTER;
+    if (!valid_io(x_dtype, y_dtype) || !valid_dtype(phi_dtype) || (w && !valid_dtype(w_dtype)))
+        return MHC_ERR_BAD_DTYPE;
+    if (!aligned16(dy) || !aligned16(x) || !aligned16(dx) || !aligned16(phi) || !aligned16(dphi) ||
+        (f_inject && !aligned16(f_inject)) || (df && !aligned16(df)))
+        return MHC_ERR_MISALIGNED;
+    const DynBwdWs ws = carve_dyn_bwd(workspace, B, n, C);
+    if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int D = n * n + 2 * n, DP = padded_D(n);
+    BwdCoefOut out{ws.dt, ws.dP, ws.cx, ws.s1, nullptr};
+    MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
+                                     n, q, P, r, alpha, bias + 2 * n, out, B, n, C, iters, eps, st));
+    MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, n,
+                                 q, ws.s1, ws.cx, ws.dP, DP, phi, phi_dtype, dx, df, ws.u, B, n, C, st));
+    MHC_LAUNCH(launch_dphi(x, x_dtype, ws.dP, DP, dphi, B, n, C, ws.dphi_part, st));
+    MHC_LAUNCH(launch_colsum_split(ws.dt, B, D + 3, D + 3, dbias, dalpha, D, ws.cs_dt, st));
+    if (!f_inject) MHC_LAUNCH(launch_colsum(ws.u, B, C, C, dw, ws.cs_u, st));
+    return MHC_OK;
+}
+
+// ===============================================================================================
+// static H
+// ===============================================================================================
+size_t mhc_layer_static_workspace_bytes(int B, int n, int C) {
+    if (check_shape(B, n, C, 0) != MHC_OK) return 0;
+    const size_t f = carve_sta_fwd(nullptr, B, n).bytes;
+    const size_t b = carve_sta_bwd(nullptr, B, n, C).bytes;
+    return f > b ? f : b;
+}
+
+int mhc_layer_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
+                  const float *H_pre_logits, const float *H_post_logits,
+                  const float *H_res_logits, const void *f_inject, void *y, int y_dtype,
+                  float *H_pre, float *H_post, float *M, float *q, int B, int n, int C, int iters,
+                  float eps, void *workspace, size_t workspace_bytes, void *stream) {
+    if (int s = check_shape(B, n, C, iters)) return s;
+    if (!x || !H_pre_logits || !H_post_logits || !H_res_logits || !y) return MHC_ERR_NULL_POINTER;
+    if (!f_inject && !w) return MHC_ERR_NULL_POINTER;
+    if (!valid_io(x_dtype, y_dtype) || (w && !valid_dtype(w_dtype))) return MHC_ERR_BAD_DTYPE;
+    if (!aligned16(x) || !aligned16(y) || (f_inject && !aligned16(f_inject))) return MHC_ERR_MISALIGNED;
+    const StaFwdWs ws = carve_sta_fwd(workspace, B, n);
+    const bool need_ws = !H_pre || !H_post || !M || !q;
+    if (need_ws)
+        if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
+    float *hp = H_pre ? H_pre : ws.Hpre, *ho = H_post ? H_post : ws.Hpost;
+    float *m = M ? M : ws.M, *qq = q ? q : ws.q;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    MHC_LAUNCH(launch_coef_fwd(nullptr, nullptr, 0, 0, nullptr, H_pre_logits, H_post_logits,
+                               H_res_logits, hp, ho, m, nullptr, nullptr, 1, n, n * C, iters, eps, st));
+    MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, hp, ho, m, 0, qq, B, n, C,
+                              eps, st));
+    return MHC_OK;
+}
+
+int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const void *w,
+                  int w_dtype, const float *H_pre_logits, const float *H_post_logits,
+                  const float *H_res_logits, const void *f_inject, const float *H_pre,
+                  const float *H_post, const float *M, const float *q, void *dx, void *df,
+                  float *dw, float *dH_pre, float *dH_post, float *dH_res, int B, int n, int C,
+                  int iters, float eps, void *workspace, size_t workspace_bytes, void *stream) {
+    if (int s = check_shape(B, n, C, iters)) return s;
+    if (!dy || !x || !H_pre_logits || !H_post_logits || !H_res_logits || !H_pre || !H_post || !M ||
+        !q || !dx || !dH_pre || !dH_post || !dH_res)
+        return MHC_ERR_NULL_POINTER;
+    if (!f_inject && (!w || !dw)) return MHC_ERR_NULL_POINTER;
+    if (!valid_io(x_dtype, y_dtype) || (w && !valid_dtype(w_dtype))) return MHC_ERR_BAD_DTYPE;
+    if (!aligned16(dy) || !aligned16(x) || !aligned16(dx) || (f_inject && !aligned16(f_inject)) ||
+        (df && !aligned16(df)))
+        return MHC_ERR_MISALIGNED;
+    const StaBwdWs ws = carve_sta_bwd(workspace, B, n, C);
+    if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int D = n * n + 2 * n;
+    BwdCoefOut out{nullptr, nullptr, nullptr, ws.s1, ws.red};
+    MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
+                                     0, q, nullptr, nullptr, nullptr, nullptr, out, B, n, C, iters,
+                                     eps, st));
+    MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, 0,
+                                 q, ws.s1, nullptr, nullptr, 0, nullptr, 0, dx, df, ws.u, B, n, C, st));
+    MHC_LAUNCH(launch_colsum(ws.red, B, D, D, ws.red_sum, ws.cs_red, st));
+    MHC_LAUNCH(launch_coef_bwd_static(ws.red_sum, H_pre, H_post, H_res_logits, dH_pre, dH_post,
+                                      dH_res, n, iters, eps, st));
+    if (!f_inject) MHC_LAUNCH(launch_colsum(ws.u, B, C, C, dw, ws.cs_u, st));
+    return MHC_OK;
+}
+
+// ===============================================================================================
+// stand-alone operators
+// ===============================================================================================
+int mhc_sinkhorn_knopp_fwd(const float *inp, float *out, int batch, int rows, int cols, int iters,
+                           float eps, void *stream) {
+    if (!inp || !out) return MHC_ERR_NULL_POINTER;
+    if (batch < 1 || rows < 1 || cols < 1 || rows > 128 || cols > 128 || iters < 0 || iters > 1024)
+        return MHC_ERR_BAD_SHAPE;
+    MHC_LAUNCH(launch_sinkhorn_plain_fwd(inp, out, batch, rows, cols, iters, eps,
+                                         static_cast<hipStream_t>(stream)));
+    return MHC_OK;
+}
+
+size_t mhc_sinkhorn_knopp_bwd_workspace_bytes(int batch, int rows, int cols, int iters) {
+    if (batch < 1 || rows < 1 || cols < 1 || rows > 128 || cols > 128 || iters < 0 || iters > 1024)
+        return 0;
+    return ((size_t)batch * (iters > 0 ? iters : 1) * 2 * 128 * sizeof(float) + 255) / 256 * 256;
+}
+
+int mhc_sinkhorn_knopp_bwd(const float *grad_out, const float *inp, float *d_inp, int batch,
+                           int rows, int cols, int iters, float eps, void *workspace,
+                           size_t workspace_bytes, void *stream) {
+    if (!grad_out || !inp || !d_inp) return MHC_ERR_NULL_POINTER;
+    const size_t need = mhc_sinkhorn_knopp_bwd_workspace_bytes(batch, rows, cols, iters);
+    if (need == 0) return MHC_ERR_BAD_SHAPE;
+    if (int s = ws_check(workspace, workspace_bytes, need)) return s;
+    MHC_LAUNCH(launch_sinkhorn_plain_bwd(grad_out, inp, d_inp, batch, rows, cols, iters, eps,
+                                         static_cast<float *>(workspace),
+                                         static_cast<hipStream_t>(stream)));
+    return MHC_OK;
+}
+
+int mhc_rmsnorm_fwd(const void *inp, int dtype, const void *w, int w_dtype, void *out, float *rms,
+                    int rows, int C, float eps, void *stream) {
+    if (!inp || !w || !out) return MHC_ERR_NULL_POINTER;
+    if (rows < 1 || C < 1) return MHC_ERR_BAD_SHAPE;
+    if (!valid_dtype(dtype) || !valid_dtype(w_dtype)) return MHC_ERR_BAD_DTYPE;
+    MHC_LAUNCH(launch_rmsnorm_fwd(inp, dtype, w, w_dtype, out, rms, rows, C, eps,
+                                  static_cast<hipStream_t>(stream)));
+    return MHC_OK;
+}
+
+size_t mhc_rmsnorm_bwd_workspace_bytes(int rows, int C) {
+    if (rows < 1 || C < 1) return 0;
+    Carver c(nullptr);
+    c.floats((size_t)rows * C);
+    c.floats(colsum_workspace_floats(rows, C));
+    return c.off;
+}
+
+int mhc_rmsnorm_bwd(const void *grad_out, const void *inp, int dtype, const void *w, int w_dtype,
+                    const float *rms, void *d_inp, float *d_w, int rows, int C, void *workspace,
+                    size_t workspace_bytes, void *stream) {
+    if (!grad_out || !inp || !w || !rms || !d_inp || !d_w) return MHC_ERR_NULL_POINTER;
+    if (rows < 1 || C < 1) return MHC_ERR_BAD_SHAPE;
+    if (!valid_dtype(dtype) || !valid_dtype(w_dtype)) return MHC_ERR_BAD_DTYPE;
+    if (int s = ws_check(workspace, workspace_bytes, mhc_rmsnorm_bwd_workspace_bytes(rows, C))) return s;
+    Carver c(workspace);
+    float *u = c.floats((size_t)rows * C);
+    float *part = c.floats(colsum_workspace_floats(rows, C));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    MHC_LAUNCH(launch_rmsnorm_bwd(grad_out, inp, dtype, w, w_dtype, rms, d_inp, u, rows, C, st));
+    MHC_LAUNCH(launch_colsum(u, rows, C, C, d_w, part, st));
+    return MHC_OK;
+}
+
+}  // extern "C"

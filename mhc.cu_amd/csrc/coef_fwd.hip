@@ -1,0 +1,130 @@
+// Coefficient kernel: per-sample H_pre = sigmoid, H_post = 2 sigmoid, M = Sinkhorn(exp(.)) from
+// the projection partial sums (dynamic H) or straight from the logits (static H).
+//
+// Replaces, in one launch: the split-K reduction of the projection, fused_h_activations
+// (reference src/csrc/include/utils.cuh:50-126) and sinkhorn_knopp_forward_batched /
+// sinkhorn_knopp_forward_fused_exp (src/csrc/kernels/sinkhorn_knopp.cuh:986-1046, :461-519).
+#include "launchers.h"
+#include "sinkhorn_device.h"
+
+namespace mhc {
+
+// Logit of projection row d for sample b:  alpha_g * (sum_ks Ppart) / r + bias_d   (dynamic)
+//                                          bias_d                                   (static)
+struct CoefArgs {
+    const float *Ppart;    // [KS][B][DP] raw dot products x_flat . phi_d, or nullptr (static)
+    const float *ssqpart;  // [KS][B] partial sums of x_flat^2
+    int KS, DP;
+    const float *alpha;    // [3]
+    const float *b_pre, *b_post, *b_res;
+    float *Hpre, *Hpost, *M;  // [B,n], [B,n], [B,n,n]
+    float *P, *r;             // [B,D], [B]  (dynamic only)
+    int B, n, nC, T;
+    float eps;
+};
+
+__device__ __forceinline__ float reduce_partials(const float *part, int KS, size_t stride, size_t idx) {
+    float acc = 0.f;
+    for (int k = 0; k < KS; k++) acc += part[k * stride + idx];
+    return acc;
+}
+
+template <int NP> __global__ __launch_bounds__(64) void coef_fwd_small_kernel(CoefArgs a) {
+    using SK = SkSmall<NP>;
+    const int lane = threadIdx.x;
+    const int g = lane & 15;
+    const int b = blockIdx.x * 4 + (lane >> 4);
+    if (b >= a.B) return;  // whole 16-lane groups leave together; DPP never crosses groups
+    const int n = a.n, D = n * n + 2 * n;
+    const bool dyn = a.Ppart != nullptr;
+    float rinv = 0.f, al[3] = {0.f, 0.f, 0.f};
+    if (dyn) {
+        const float ssq = reduce_partials(a.ssqpart, a.KS, a.B, b);
+        const float r = sqrtf(ssq / (float)a.nC + a.eps);
+        rinv = 1.0f / r;
+        al[0] = a.alpha[0]; al[1] = a.alpha[1]; al[2] = a.alpha[2];
+        if (g == 0) a.r[b] = r;
+    }
+    const size_t pstride = (size_t)a.B * a.DP;
+    auto logit = [&](int d, float alpha_g, float bias) -> float {
+        if (!dyn) return bias;
+        const float p = reduce_partials(a.Ppart, a.KS, pstride, (size_t)b * a.DP + d) * rinv;
+        a.P[(size_t)b * D + d] = p;
+        return alpha_g * p + bias;
+    };
+    if (g < n) {
+        a.Hpre[b * n + g] = sigmoidf_acc(logit(g, al[0], a.b_pre[g]));
+        a.Hpost[b * n + g] = 2.0f * sigmoidf_acc(logit(n + g, al[1], a.b_post[g]));
+    }
+    const int r0 = SK::row(g), c0 = SK::col0(g);
+    float m[SK::EPL];
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++) {
+        const int c = c0 + e;
+        m[e] = (r0 < n && c < n) ? expf(logit(2 * n + r0 * n + c, al[2], a.b_res[r0 * n + c])) : 0.f;
+    }
+    SK::forward(m, g, n, a.T, a.eps, nullptr, lane);
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++) {
+        const int c = c0 + e;
+        if (r0 < n && c < n) a.M[(size_t)b * n * n + r0 * n + c] = m[e];
+    }
+}
+
+template <int NP> __global__ __launch_bounds__(64) void coef_fwd_lds_kernel(CoefArgs a) {
+    using SK = SkLds<NP>;
+    __shared__ float lds[SK::forward_floats()];
+    float *Es = lds, *u = Es + NP * SK::LD, *v = u + NP;
+    const int lane = threadIdx.x;
+    const int b = blockIdx.x;
+    const int n = a.n, D = n * n + 2 * n;
+    const bool dyn = a.Ppart != nullptr;
+    float rinv = 0.f, al[3] = {0.f, 0.f, 0.f};
+    if (dyn) {
+        const float ssq = reduce_partials(a.ssqpart, a.KS, a.B, b);
+        const float r = sqrtf(ssq / (float)a.nC + a.eps);
+        rinv = 1.0f / r;
+        al[0] = a.alpha[0]; al[1] = a.alpha[1]; al[2] = a.alpha[2];
+        if (lane == 0) a.r[b] = r;
+    }
+    const size_t pstride = (size_t)a.B * a.DP;
+    auto logit = [&](int d, float alpha_g, float bias) -> float {
+        if (!dyn) return bias;
+        const float p = reduce_partials(a.Ppart, a.KS, pstride, (size_t)b * a.DP + d) * rinv;
+        a.P[(size_t)b * D + d] = p;
+        return alpha_g * p + bias;
+    };
+    if (lane < n) {
+        a.Hpre[b * n + lane] = sigmoidf_acc(logit(lane, al[0], a.b_pre[lane]));
+        a.Hpost[b * n + lane] = 2.0f * sigmoidf_acc(logit(n + lane, al[1], a.b_post[lane]));
+    }
+    for (int e = lane; e < NP * NP; e += kWave) {
+        const int r0 = e / NP, c = e % NP;
+        Es[r0 * SK::LD + c] =
+            (r0 < n && c < n) ? expf(logit(2 * n + r0 * n + c, al[2], a.b_res[r0 * n + c])) : 0.f;
+    }
+    __syncthreads();
+    SK::forward(Es, u, v, n, a.T, a.eps, nullptr, nullptr, lane);
+    for (int e = lane; e < n * n; e += kWave) {
+        const int r0 = e / n, c = e % n;
+        a.M[(size_t)b * n * n + e] = u[r0] * Es[r0 * SK::LD + c] * v[c];
+    }
+}
+
+hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int DP,
+                           const float *alpha, const float *b_pre, const float *b_post,
+                           const float *b_res, float *Hpre, float *Hpost, float *M, float *P,
+                           float *r, int B, int n, int nC, int T, float eps, hipStream_t stream) {
+    CoefArgs a{Ppart, ssqpart, KS, DP, alpha, b_pre, b_post, b_res, Hpre, Hpost, M, P, r, B, n, nC, T, eps};
+    if (n <= 4)
+        coef_fwd_small_kernel<4><<<(B + 3) / 4, 64, 0, stream>>>(a);
+    else if (n <= 8)
+        coef_fwd_small_kernel<8><<<(B + 3) / 4, 64, 0, stream>>>(a);
+    else if (n <= 16)
+        coef_fwd_lds_kernel<16><<<B, 64, 0, stream>>>(a);
+    else
+        coef_fwd_lds_kernel<32><<<B, 64, 0, stream>>>(a);
+    return hipGetLastError();
+}
+
+}  // namespace mhc

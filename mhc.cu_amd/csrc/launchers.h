@@ -1,0 +1,101 @@
+// Host-side launch functions of the individual kernels (internal to the library).
+// Every function only enqueues work on `stream` and returns hipGetLastError().
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+namespace mhc {
+
+enum DType { kF32 = 0, kBF16 = 1 };
+
+inline size_t dtype_size(int dt) { return dt == kBF16 ? 2 : 4; }
+
+// Projection row count padded to whole 32-wide MFMA tiles.
+inline int padded_D(int n) { return ((n * n + 2 * n) + 31) / 32 * 32; }
+
+// ---- forward ---------------------------------------------------------------------------------
+
+// Number of K-splits launch_proj_fwd produces for this shape and dtype pair (never more than
+// kMaxKSplit, which sizes the workspace).
+constexpr int kMaxKSplit = 64;
+int proj_fwd_ksplit(int x_dtype, int phi_dtype, int B, int n, int C);
+
+// Ppart[ks][b][d] = sum over K-slab ks of x_flat[b,k] * phi[d,k]   (d < D; padded rows zero)
+// ssqpart[ks][b]  = sum over the slab of x_flat[b,k]^2
+hipError_t launch_proj_fwd(const void *x, int x_dtype, const void *phi, int phi_dtype, float *Ppart,
+                           float *ssqpart, int KS, int B, int n, int C, hipStream_t stream);
+
+// Coefficients from projection partials (dynamic: Ppart != nullptr) or logits (static: B == 1).
+hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int DP,
+                           const float *alpha, const float *b_pre, const float *b_post,
+                           const float *b_res, float *Hpre, float *Hpost, float *M, float *P,
+                           float *r, int B, int n, int nC, int T, float eps, hipStream_t stream);
+
+// y = M x + Hpost (x) f, f = RMSNorm(Hpre . x) * w or f_inject.  hstride = n (per-sample
+// coefficients) or 0 (shared); the M stride is hstride * n.
+hipError_t launch_mix_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
+                          const void *f_inject, void *y, int y_dtype, const float *Hpre,
+                          const float *Hpost, const float *M, int hstride, float *q, int B, int n,
+                          int C, float eps, hipStream_t stream);
+
+// ---- backward --------------------------------------------------------------------------------
+
+struct BwdCoefOut {
+    float *dt;    // [B, D+3] dL/dlogits per sample, then sum_d dt_d p_d per alpha group (dynamic only)
+    float *dP;    // [B, DP]  dL/d(raw dot product) = dt * alpha_g / r, zero padded (dynamic only)
+    float *cx;    // [B]      sum_d dt_d alpha_g p_d / (nC r^2)                    (dynamic only)
+    float *s1;    // [B]      sum_c df_c w_c a_c
+    float *red;   // [B, n*n + 2n] raw per-sample (dM | dHpre | dHpost)             (static only)
+};
+
+// Per-sample reductions over c (dM, dHpost, dHpre, s1) and, for dynamic H, the coefficient
+// backward (activation derivatives + exact Sinkhorn backward) in the same launch.
+hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int x_dtype,
+                                 const void *w, int w_dtype, const void *f_inject,
+                                 const float *Hpre, const float *Hpost, const float *M, int hstride,
+                                 const float *q, const float *P, const float *r, const float *alpha,
+                                 const float *b_res, BwdCoefOut out, int B, int n, int C, int T,
+                                 float eps, hipStream_t stream);
+
+// dx = M^T dy + Hpre (x) da - cx * x  [+ dP phi when phi != nullptr], df, and u = df * a / q
+// (the per-sample summand of dw).
+hipError_t launch_mix_bwd_dx(const void *dy, int y_dtype, const void *x, int x_dtype, const void *w,
+                             int w_dtype, const void *f_inject, const float *Hpre,
+                             const float *Hpost, const float *M, int hstride, const float *q,
+                             const float *s1, const float *cx, const float *dP, int DP,
+                             const void *phi, int phi_dtype, void *dx, void *df, float *u, int B,
+                             int n, int C, hipStream_t stream);
+
+// dphi[d, k] = sum_b dP[b, d] * x_flat[b, k].  `partial` holds dphi_batch_splits() copies of
+// dphi when that is > 1.
+int dphi_batch_splits(int B, int n, int C);
+hipError_t launch_dphi(const void *x, int x_dtype, const float *dP, int DP, float *dphi, int B,
+                       int n, int C, float *partial, hipStream_t stream);
+
+// out[j] = sum_b in[b * ld + j] for j < cols  (deterministic two-level sum through `partial`,
+// colsum_workspace_floats() floats).  The _split form sends columns >= split_col to out2.
+size_t colsum_workspace_floats(int rows, int cols);
+hipError_t launch_colsum(const float *in, int rows, int cols, int ld, float *out, float *partial,
+                         hipStream_t stream);
+hipError_t launch_colsum_split(const float *in, int rows, int cols, int ld, float *out, float *out2,
+                               int split_col, float *partial, hipStream_t stream);
+
+// Static H: coefficient backward on the sample-summed raw gradients.
+hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const float *Hpost,
+                                  const float *H_res_logits, float *dH_pre, float *dH_post,
+                                  float *dH_res, int n, int T, float eps, hipStream_t stream);
+
+// ---- stand-alone operators -------------------------------------------------------------------
+hipError_t launch_sinkhorn_plain_fwd(const float *inp, float *out, int batch, int rows, int cols,
+                                     int T, float eps, hipStream_t stream);
+hipError_t launch_sinkhorn_plain_bwd(const float *grad, const float *inp, float *d_inp, int batch,
+                                     int rows, int cols, int T, float eps, float *scal,
+                                     hipStream_t stream);
+hipError_t launch_rmsnorm_fwd(const void *inp, int dtype, const void *w, int w_dtype, void *out,
+                              float *rms, int rows, int C, float eps, hipStream_t stream);
+hipError_t launch_rmsnorm_bwd(const void *grad, const void *inp, int dtype, const void *w,
+                              int w_dtype, const float *rms, void *d_inp, float *u, int rows, int C,
+                              hipStream_t stream);
+
+}  // namespace mhc

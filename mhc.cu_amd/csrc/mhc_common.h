@@ -1,0 +1,165 @@
+// Device-side helpers shared by every kernel of the mHC library (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <type_traits>
+
+namespace mhc {
+
+typedef uint16_t bf16_t;  // raw bf16 storage; arithmetic is always fp32
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------------------------------------
+// bf16 <-> fp32
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+    return __uint_as_float(static_cast<uint32_t>(v) << 16);
+}
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t pair) {
+    return __uint_as_float(pair & 0xffff0000u);
+}
+// round-to-nearest-even; the compiler selects the gfx950 hardware conversion for __bf16 casts
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+    __bf16 b = static_cast<__bf16>(f);
+    return __builtin_bit_cast(bf16_t, b);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
+}
+
+template <typename T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<bf16_t>(bf16_t v) { return bf16_to_f32(v); }
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return f32_to_bf16(v); }
+
+// ---------------------------------------------------------------------------------------------
+// Vector loads/stores of V consecutive elements (V * sizeof(T) <= 32 bytes), converted to fp32.
+// The pointer must be aligned to min(V * sizeof(T), 16) bytes.
+// ---------------------------------------------------------------------------------------------
+template <typename T, int V>
+__device__ __forceinline__ void load_vec(const T *__restrict__ p, float (&out)[V]) {
+    if constexpr (std::is_same<T, float>::value) {
+        if constexpr (V % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < V / 4; i++) {
+                float4 t = reinterpret_cast<const float4 *>(p)[i];
+                out[4 * i] = t.x; out[4 * i + 1] = t.y; out[4 * i + 2] = t.z; out[4 * i + 3] = t.w;
+            }
+        } else if constexpr (V == 2) {
+            float2 t = *reinterpret_cast<const float2 *>(p);
+            out[0] = t.x; out[1] = t.y;
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; i++) out[i] = p[i];
+        }
+    } else {
+        if constexpr (V % 8 == 0) {
+#pragma unroll
+            for (int i = 0; i < V / 8; i++) {
+                uint4 t = reinterpret_cast<const uint4 *>(p)[i];
+                out[8 * i] = bf16lo_to_f32(t.x); out[8 * i + 1] = bf16hi_to_f32(t.x);
+                out[8 * i + 2] = bf16lo_to_f32(t.y); out[8 * i + 3] = bf16hi_to_f32(t.y);
+                out[8 * i + 4] = bf16lo_to_f32(t.z); out[8 * i + 5] = bf16hi_to_f32(t.z);
+                out[8 * i + 6] = bf16lo_to_f32(t.w); out[8 * i + 7] = bf16hi_to_f32(t.w);
+            }
+        } else if constexpr (V == 4) {
+            uint2 t = *reinterpret_cast<const uint2 *>(p);
+            out[0] = bf16lo_to_f32(t.x); out[1] = bf16hi_to_f32(t.x);
+            out[2] = bf16lo_to_f32(t.y); out[3] = bf16hi_to_f32(t.y);
+        } else if constexpr (V == 2) {
+            uint32_t t = *reinterpret_cast<const uint32_t *>(p);
+            out[0] = bf16lo_to_f32(t); out[1] = bf16hi_to_f32(t);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; i++) out[i] = bf16_to_f32(p[i]);
+        }
+    }
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void store_vec(T *__restrict__ p, const float (&v)[V]) {
+    if constexpr (std::is_same<T, float>::value) {
+        if constexpr (V % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < V / 4; i++)
+                reinterpret_cast<float4 *>(p)[i] =
+                    make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+        } else if constexpr (V == 2) {
+            *reinterpret_cast<float2 *>(p) = make_float2(v[0], v[1]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; i++) p[i] = v[i];
+        }
+    } else {
+        if constexpr (V % 8 == 0) {
+#pragma unroll
+            for (int i = 0; i < V / 8; i++)
+                reinterpret_cast<uint4 *>(p)[i] =
+                    make_uint4(pack_bf16x2(v[8 * i], v[8 * i + 1]), pack_bf16x2(v[8 * i + 2], v[8 * i + 3]),
+                               pack_bf16x2(v[8 * i + 4], v[8 * i + 5]), pack_bf16x2(v[8 * i + 6], v[8 * i + 7]));
+        } else if constexpr (V == 4) {
+            *reinterpret_cast<uint2 *>(p) =
+                make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        } else if constexpr (V == 2) {
+            *reinterpret_cast<uint32_t *>(p) = pack_bf16x2(v[0], v[1]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; i++) p[i] = f32_to_bf16(v[i]);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Cross-lane primitives
+// ---------------------------------------------------------------------------------------------
+// DPP controls (GFX9 encoding): quad_perm = 8-bit selector, row_ror:n = 0x120 + n
+constexpr int kDppQuadXor1 = 0xB1;   // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;   // quad_perm:[2,3,0,1]
+constexpr int kDppRowRor4 = 0x124;
+constexpr int kDppRowRor8 = 0x128;
+
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+    int iv = __float_as_int(v);
+    return __int_as_float(__builtin_amdgcn_update_dpp(iv, iv, CTRL, 0xF, 0xF, false));
+}
+
+// Sum over all 64 lanes; every lane gets the total.
+__device__ __forceinline__ float wave_allreduce_sum(float v) {
+    v += dpp_mov<kDppQuadXor1>(v);
+    v += dpp_mov<kDppQuadXor2>(v);
+    v += dpp_mov<kDppRowRor4>(v);
+    v += dpp_mov<kDppRowRor8>(v);
+    v += __shfl_xor(v, 16, kWave);
+    v += __shfl_xor(v, 32, kWave);
+    return v;
+}
+
+// Sum over the whole workgroup (NT threads, multiple of 64); every thread gets the total.
+// `red` is LDS scratch of at least NT/64 floats; safe to call repeatedly with the same scratch.
+template <int NT> __device__ __forceinline__ float block_allreduce_sum(float v, float *red) {
+    v = wave_allreduce_sum(v);
+    if constexpr (NT == kWave) return v;
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();  // previous readers of red are done
+    if ((threadIdx.x & (kWave - 1)) == 0) red[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int i = 0; i < NT / kWave; i++) total += red[i];
+    return total;
+}
+
+__device__ __forceinline__ float sigmoidf_acc(float t) { return 1.0f / (1.0f + expf(-t)); }
+
+// Index of the alpha group of projection row d: 0 = pre, 1 = post, 2 = res.
+__device__ __forceinline__ int alpha_group(int d, int n) { return d < n ? 0 : (d < 2 * n ? 1 : 2); }
+
+__host__ __device__ constexpr int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+}  // namespace mhc

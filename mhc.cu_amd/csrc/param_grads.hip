@@ -1,0 +1,187 @@
+// Parameter gradients that sum over the batch: dphi = dP^T x_flat (reference ops.py:332-334),
+// dbias / dalpha (ops.py:319-325), dw (reference rmsnorm.cuh:282-294, without its atomics) and the
+// static-H coefficient backward (reference bindings.cu:372-396).  All sums are order-deterministic:
+// per-split partial sums followed by a second pass, no atomics.
+#include "launchers.h"
+#include "sinkhorn_device.h"
+
+namespace mhc {
+
+// --------------------------------------------------------------------------------------------
+// column sums: out[j] = sum_b in[b * ld + j]
+// --------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void colsum_kernel(const float *__restrict__ in, int rows, int cols,
+                                                     int ld, int rows_per_split,
+                                                     float *__restrict__ out, float *__restrict__ out2,
+                                                     int split_col) {
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= cols) return;
+    const int r0 = blockIdx.y * rows_per_split;
+    const int r1 = min(rows, r0 + rows_per_split);
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int r = r0;
+    for (; r + 3 < r1; r += 4) {
+        a0 += in[(size_t)r * ld + j];
+        a1 += in[(size_t)(r + 1) * ld + j];
+        a2 += in[(size_t)(r + 2) * ld + j];
+        a3 += in[(size_t)(r + 3) * ld + j];
+    }
+    for (; r < r1; r++) a0 += in[(size_t)r * ld + j];
+    const float v = (a0 + a1) + (a2 + a3);
+    if (gridDim.y > 1) out[(size_t)blockIdx.y * cols + j] = v;   // partial [split][cols]
+    else if (j < split_col) out[j] = v;
+    else out2[j - split_col] = v;
+}
+
+static int colsum_splits(int rows, int cols) {
+    const int col_blocks = (cols + 255) / 256;
+    int rs = 256 / col_blocks;
+    if (rs > rows / 8) rs = rows / 8;
+    if (rs > 64) rs = 64;
+    if (rs < 1) rs = 1;
+    return rs;
+}
+
+size_t colsum_workspace_floats(int rows, int cols) {
+    const int rs = colsum_splits(rows, cols);
+    return rs > 1 ? (size_t)rs * cols : 0;
+}
+
+// out2 / split_col: columns >= split_col go to out2[j - split_col] (pass cols and nullptr for none)
+static hipError_t colsum2(const float *in, int rows, int cols, int ld, float *out, float *out2,
+                          int split_col, float *partial, hipStream_t stream) {
+    const int rs = colsum_splits(rows, cols);
+    const int cb = (cols + 255) / 256;
+    if (rs == 1) {
+        colsum_kernel<<<dim3(cb, 1), 256, 0, stream>>>(in, rows, cols, ld, rows, out, out2, split_col);
+        return hipGetLastError();
+    }
+    const int rps = (rows + rs - 1) / rs;
+    colsum_kernel<<<dim3(cb, rs), 256, 0, stream>>>(in, rows, cols, ld, rps, partial, nullptr, cols);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    colsum_kernel<<<dim3(cb, 1), 256, 0, stream>>>(partial, rs, cols, cols, rs, out, out2, split_col);
+    return hipGetLastError();
+}
+
+hipError_t launch_colsum(const float *in, int rows, int cols, int ld, float *out, float *partial,
+                         hipStream_t stream) {
+    return colsum2(in, rows, cols, ld, out, nullptr, cols, partial, stream);
+}
+
+hipError_t launch_colsum_split(const float *in, int rows, int cols, int ld, float *out, float *out2,
+                               int split_col, float *partial, hipStream_t stream) {
+    return colsum2(in, rows, cols, ld, out, out2, split_col, partial, stream);
+}
+
+// --------------------------------------------------------------------------------------------
+// dphi, generic path: thread = one column k of x_flat, 32 projection rows per workgroup,
+// batch optionally split (partials summed by colsum).
+// --------------------------------------------------------------------------------------------
+constexpr int kDphiDB = 32;
+
+template <typename TX>
+__global__ __launch_bounds__(256) void dphi_generic_kernel(const TX *__restrict__ x,
+                                                           const float *__restrict__ dP, int DP,
+                                                           float *__restrict__ out, int B, int D,
+                                                           int nC, int b_per_split) {
+    const int k = blockIdx.x * 256 + threadIdx.x;
+    const int d0 = blockIdx.y * kDphiDB;
+    const int b0 = blockIdx.z * b_per_split, b1 = min(B, b0 + b_per_split);
+    if (k >= nC) return;
+    float acc[kDphiDB];
+#pragma unroll
+    for (int j = 0; j < kDphiDB; j++) acc[j] = 0.f;
+    for (int b = b0; b < b1; b++) {
+        const float xv = to_f32<TX>(x[(size_t)b * nC + k]);
+        const float *dPb = dP + (size_t)b * DP + d0;  // padded rows of dP are zero
+#pragma unroll
+        for (int j = 0; j < kDphiDB; j++) acc[j] += dPb[j] * xv;
+    }
+    float *o = out + (size_t)blockIdx.z * D * nC;
+#pragma unroll
+    for (int j = 0; j < kDphiDB; j++)
+        if (d0 + j < D) o[(size_t)(d0 + j) * nC + k] = acc[j];
+}
+
+int dphi_batch_splits(int B, int n, int C) {
+    const int nC = n * C, D = n * n + 2 * n;
+    const int wgs = ((nC + 255) / 256) * ((D + kDphiDB - 1) / kDphiDB);
+    int bs = 512 / wgs;
+    if (bs > B / 16) bs = B / 16;
+    if (bs > 16) bs = 16;
+    if (bs < 1) bs = 1;
+    return bs;
+}
+
+hipError_t launch_dphi(const void *x, int x_dtype, const float *dP, int DP, float *dphi, int B,
+                       int n, int C, float *partial, hipStream_t stream) {
+    const int nC = n * C, D = n * n + 2 * n;
+    const int bs = dphi_batch_splits(B, n, C);
+    const int bps = (B + bs - 1) / bs;
+    dim3 grid((nC + 255) / 256, (D + kDphiDB - 1) / kDphiDB, bs);
+    float *out = bs > 1 ? partial : dphi;
+    if (x_dtype == kBF16)
+        dphi_generic_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t *>(x), dP, DP, out, B, D, nC, bps);
+    else
+        dphi_generic_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float *>(x), dP, DP, out, B, D, nC, bps);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || bs == 1) return e;
+    const int cols = D * nC;
+    colsum_kernel<<<dim3((cols + 255) / 256, 1), 256, 0, stream>>>(partial, bs, cols, cols, bs, dphi, nullptr, cols);
+    return hipGetLastError();
+}
+
+// --------------------------------------------------------------------------------------------
+// static H: coefficient backward on the batch-summed raw gradients (one wave)
+//   red_sum = (dM [n*n] | dHpre [n] | dHpost [n])
+// --------------------------------------------------------------------------------------------
+template <int NP>
+__global__ __launch_bounds__(64) void coef_bwd_static_kernel(const float *__restrict__ red_sum,
+                                                             const float *__restrict__ Hpre,
+                                                             const float *__restrict__ Hpost,
+                                                             const float *__restrict__ H_res_logits,
+                                                             float *__restrict__ dH_pre,
+                                                             float *__restrict__ dH_post,
+                                                             float *__restrict__ dH_res, int n, int T,
+                                                             float eps) {
+    using SK = SkLds<NP>;
+    extern __shared__ float lds[];
+    float *Es = lds, *dO = Es + NP * SK::LD;
+    float *u = dO + NP * SK::LD, *v = u + NP, *tmp = v + NP;
+    float *rho = tmp + NP, *ssc = rho + T * NP;
+    const int lane = threadIdx.x;
+    if (lane < n) {
+        const float hp = Hpre[lane], ho = Hpost[lane];
+        dH_pre[lane] = red_sum[n * n + lane] * hp * (1.0f - hp);
+        dH_post[lane] = red_sum[n * n + n + lane] * ho * (1.0f - 0.5f * ho);
+    }
+    for (int e = lane; e < NP * NP; e += kWave) {
+        const int r0 = e / NP, c = e % NP;
+        const bool ok = r0 < n && c < n;
+        Es[r0 * SK::LD + c] = ok ? expf(H_res_logits[r0 * n + c]) : 0.f;
+        dO[r0 * SK::LD + c] = ok ? red_sum[r0 * n + c] : 0.f;
+    }
+    __syncthreads();
+    SK::forward(Es, u, v, n, T, eps, rho, ssc, lane);
+    SK::backward(Es, dO, u, v, tmp, n, T, rho, ssc, lane);
+    for (int e = lane; e < n * n; e += kWave) {
+        const int r0 = e / n, c = e % n;
+        dH_res[e] = dO[r0 * SK::LD + c] * Es[r0 * SK::LD + c];
+    }
+}
+
+hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const float *Hpost,
+                                  const float *H_res_logits, float *dH_pre, float *dH_post,
+                                  float *dH_res, int n, int T, float eps, hipStream_t stream) {
+    if (n <= 16) {
+        const size_t smem = sizeof(float) * SkLds<16>::backward_floats(T);
+        coef_bwd_static_kernel<16><<<1, 64, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
+    } else {
+        const size_t smem = sizeof(float) * SkLds<32>::backward_floats(T);
+        coef_bwd_static_kernel<32><<<1, 64, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace mhc

@@ -1,0 +1,241 @@
+// Projection of the dynamic-H path: raw dot products x_flat[b,:] . phi[d,:] for all D = n^2+2n
+// rows of phi, plus sum(x_flat^2), as split-K partial sums.  The coefficient kernel finishes
+// the reduction, divides by the RMS and applies alpha / bias / activations.
+//
+// Replaces compute_rms (reference src/csrc/kernels/fused_rmsnorm_matmul.cuh:119-153) and the
+// cuBLASLt projection GEMM (src/python/bindings.cu:34-81, :436-443) with one pass over x.
+//
+// Two kernels:
+//   proj_fwd_mfma_kernel    x and phi both bf16, C % 8 == 0: v_mfma_f32_32x32x16_bf16 tiles
+//                           (32 samples x 32 projection rows), operands loaded straight from
+//                           global memory in MFMA layout (16-byte loads, no LDS staging).
+//   proj_fwd_generic_kernel any dtype / any C: fp32 FMA, exact products (the fp32 parity tier).
+#include "launchers.h"
+#include "mhc_common.h"
+
+namespace mhc {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+static inline bool use_mfma(int x_dtype, int phi_dtype, int C) {
+    return x_dtype == kBF16 && phi_dtype == kBF16 && C % 8 == 0;
+}
+
+// --------------------------------------------------------------------------------------------
+// generic path
+// --------------------------------------------------------------------------------------------
+constexpr int kGenDB = 16;  // projection rows per workgroup
+
+template <typename TX, typename TP>
+__global__ __launch_bounds__(256) void proj_fwd_generic_kernel(const TX *__restrict__ x,
+                                                               const TP *__restrict__ phi,
+                                                               float *__restrict__ Ppart,
+                                                               float *__restrict__ ssqpart, int B,
+                                                               int D, int DP, int nC) {
+    __shared__ float red[4][kGenDB + 1];
+    const int b = blockIdx.x, d0 = blockIdx.y * kGenDB, tid = threadIdx.x;
+    const TX *xb = x + (size_t)b * nC;
+    float acc[kGenDB], ssq = 0.f;
+#pragma unroll
+    for (int j = 0; j < kGenDB; j++) acc[j] = 0.f;
+    for (int k = tid; k < nC; k += 256) {
+        const float xv = to_f32<TX>(xb[k]);
+        ssq += xv * xv;
+#pragma unroll
+        for (int j = 0; j < kGenDB; j++)
+            if (d0 + j < D) acc[j] += xv * to_f32<TP>(phi[(size_t)(d0 + j) * nC + k]);
+    }
+#pragma unroll
+    for (int j = 0; j < kGenDB; j++) acc[j] = wave_allreduce_sum(acc[j]);
+    ssq = wave_allreduce_sum(ssq);
+    if ((tid & 63) == 0) {
+#pragma unroll
+        for (int j = 0; j < kGenDB; j++) red[tid >> 6][j] = acc[j];
+        red[tid >> 6][kGenDB] = ssq;
+    }
+    __syncthreads();
+    if (tid <= kGenDB) {
+        const float v = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+        if (tid < kGenDB) {
+            if (d0 + tid < D) Ppart[(size_t)b * DP + d0 + tid] = v;
+        } else if (blockIdx.y == 0) {
+            ssqpart[b] = v;
+        }
+    }
+}
+
+// --------------------------------------------------------------------------------------------
+// MFMA path.  Workgroup = 4 waves on the same 32-sample tile, each wave on its own K sub-slab;
+// the four partial tiles are summed through LDS, so one partial per workgroup reaches memory.
+// grid.x = sample_tiles * KS (sample tile fastest), grid.y = groups of NT projection tiles.
+// --------------------------------------------------------------------------------------------
+template <int NT>
+__global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__restrict__ x,
+                                                            const bf16_t *__restrict__ phi,
+                                                            float *__restrict__ Ppart,
+                                                            float *__restrict__ ssqpart, int B,
+                                                            int D, int DP, int nC, int tiles_s,
+                                                            int sub /* K per wave, multiple of 16 */) {
+    extern __shared__ float lds[];  // [3][NT*16 + 1][64]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int st = blockIdx.x % tiles_s, ks = blockIdx.x / tiles_s;
+    const int row = lane & 31, kh = lane >> 5;
+    const int b = st * 32 + row;
+    const int dbase = blockIdx.y * NT * 32;
+    const int kbeg = (ks * 4 + wave) * sub;
+    const int kend = min(kbeg + sub, nC);
+
+    const bool bvalid = b < B;
+    const uint4 *xrow = reinterpret_cast<const uint4 *>(x + (size_t)(bvalid ? b : 0) * nC);
+    const uint4 *prow[NT];
+    bool dvalid[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int d = dbase + t * 32 + row;
+        dvalid[t] = d < D;
+        prow[t] = reinterpret_cast<const uint4 *>(phi + (size_t)(dvalid[t] ? d : 0) * nC);
+    }
+
+    f32x16_t acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[t][i] = 0.f;
+    float ssq = 0.f;
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+
+    constexpr int U = 4;  // k-steps in flight
+    for (int k0 = kbeg; k0 < kend; k0 += 16 * U) {
+        uint4 av[U], bv[U][NT];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int k = k0 + u * 16 + kh * 8;
+            const bool kv = k < kend;  // kend and k are multiples of 8
+            av[u] = (kv && bvalid) ? xrow[k >> 3] : zero4;
+#pragma unroll
+            for (int t = 0; t < NT; t++) bv[u][t] = (kv && dvalid[t]) ? prow[t][k >> 3] : zero4;
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const bf16x8_t af = __builtin_bit_cast(bf16x8_t, av[u]);
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    af, __builtin_bit_cast(bf16x8_t, bv[u][t]), acc[t], 0, 0, 0);
+            if (blockIdx.y == 0) {
+                const uint32_t w4[4] = {av[u].x, av[u].y, av[u].z, av[u].w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float lo = bf16lo_to_f32(w4[i]), hi = bf16hi_to_f32(w4[i]);
+                    ssq += lo * lo + hi * hi;
+                }
+            }
+        }
+    }
+    ssq += __shfl_xor(ssq, 32, kWave);  // both K halves of the row
+
+    // cross-wave sum: waves 1..3 park their tiles in LDS, wave 0 adds and writes
+    constexpr int R = NT * 16 + 1;
+    if (wave > 0) {
+        float *dst = lds + (size_t)(wave - 1) * R * 64;
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) dst[(t * 16 + i) * 64 + lane] = acc[t][i];
+        dst[(R - 1) * 64 + lane] = ssq;
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int w = 0; w < 3; w++) {
+            const float *src = lds + (size_t)w * R * 64;
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[t][i] += src[(t * 16 + i) * 64 + lane];
+            ssq += src[(R - 1) * 64 + lane];
+        }
+        // accumulator layout of the 32x32 tile: lane -> column (lane & 31),
+        // register i -> row 8 * (i / 4) + 4 * (lane / 32) + (i % 4)
+        float *out = Ppart + (size_t)ks * B * DP;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int d = dbase + t * 32 + row;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int bs = st * 32 + 8 * (i >> 2) + 4 * kh + (i & 3);
+                if (bs < B && d < DP) out[(size_t)bs * DP + d] = acc[t][i];
+            }
+        }
+        if (blockIdx.y == 0 && kh == 0 && bvalid) ssqpart[(size_t)ks * B + b] = ssq;
+    }
+}
+
+// --------------------------------------------------------------------------------------------
+// shape-dependent split and launch
+// --------------------------------------------------------------------------------------------
+static int mfma_nt(int n) {
+    const int tiles = padded_D(n) / 32;
+    return tiles <= 4 ? tiles : 2;
+}
+
+int proj_fwd_ksplit(int x_dtype, int phi_dtype, int B, int n, int C) {
+    // The generic path always uses one split.  MFMA path: enough workgroups to fill 256 CUs,
+    // at least 64 K elements per wave, partial sums at most ~1/4 of x's bytes.
+    if (!use_mfma(x_dtype, phi_dtype, C)) return 1;
+    const int nC = n * C, DP = padded_D(n);
+    const int tiles_s = (B + 31) / 32;
+    const int groups = DP / 32 / mfma_nt(n);
+    int ks = (512 + tiles_s * groups - 1) / (tiles_s * groups);
+    const int cap_slab = nC / 256;
+    const int cap_bytes = (int)((0.25 * nC * 2.0) / (DP * 4.0));
+    if (ks > cap_slab) ks = cap_slab;
+    if (ks > cap_bytes) ks = cap_bytes;
+    if (ks > 64) ks = 64;
+    if (ks < 1) ks = 1;
+    return ks;
+}
+
+template <typename TX, typename TP>
+static hipError_t launch_generic(const void *x, const void *phi, float *Ppart, float *ssqpart, int B,
+                                 int D, int DP, int nC, hipStream_t stream) {
+    dim3 grid(B, (D + kGenDB - 1) / kGenDB);
+    proj_fwd_generic_kernel<TX, TP><<<grid, 256, 0, stream>>>(
+        static_cast<const TX *>(x), static_cast<const TP *>(phi), Ppart, ssqpart, B, D, DP, nC);
+    return hipGetLastError();
+}
+
+template <int NT>
+static hipError_t launch_mfma(const void *x, const void *phi, float *Ppart, float *ssqpart, int KS,
+                              int B, int D, int DP, int nC, hipStream_t stream) {
+    const int tiles_s = (B + 31) / 32;
+    const int groups = (DP / 32 + NT - 1) / NT;
+    const int sub = round_up((nC + KS * 4 - 1) / (KS * 4), 16);
+    dim3 grid(tiles_s * KS, groups);
+    const size_t smem = sizeof(float) * 3 * (NT * 16 + 1) * 64;
+    proj_fwd_mfma_kernel<NT><<<grid, 256, smem, stream>>>(static_cast<const bf16_t *>(x),
+                                                           static_cast<const bf16_t *>(phi), Ppart,
+                                                           ssqpart, B, D, DP, nC, tiles_s, sub);
+    return hipGetLastError();
+}
+
+hipError_t launch_proj_fwd(const void *x, int x_dtype, const void *phi, int phi_dtype, float *Ppart,
+                           float *ssqpart, int KS, int B, int n, int C, hipStream_t stream) {
+    const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
+    if (use_mfma(x_dtype, phi_dtype, C)) {
+        switch (mfma_nt(n)) {
+            case 1: return launch_mfma<1>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
+            case 2: return launch_mfma<2>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
+            case 3: return launch_mfma<3>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
+            default: return launch_mfma<4>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
+        }
+    }
+    if (KS != 1) return hipErrorInvalidValue;  // the generic path produces exactly one split
+    if (x_dtype == kF32 && phi_dtype == kF32) return launch_generic<float, float>(x, phi, Ppart, ssqpart, B, D, DP, nC, stream);
+    if (x_dtype == kF32 && phi_dtype == kBF16) return launch_generic<float, bf16_t>(x, phi, Ppart, ssqpart, B, D, DP, nC, stream);
+    if (x_dtype == kBF16 && phi_dtype == kF32) return launch_generic<bf16_t, float>(x, phi, Ppart, ssqpart, B, D, DP, nC, stream);
+    return launch_generic<bf16_t, bf16_t>(x, phi, Ppart, ssqpart, B, D, DP, nC, stream);
+}
+
+}  // namespace mhc

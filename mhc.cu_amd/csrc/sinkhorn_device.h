@@ -1,0 +1,183 @@
+// Sinkhorn-Knopp on one n x n matrix (n <= 32), forward and exact backward, as device routines.
+//
+// Semantics (reference: src/python/benchmarks/bench_layer.py:48-53 / :112-117): start from
+// E = exp(logits); T times: divide every row by (row sum + eps), then every column by
+// (column sum + eps).  The backward is the exact reverse sweep through all T iterations; the
+// per-iteration denominators rho_t[r], s_t[c] are kept in LDS during the forward recompute.
+//
+// Two layouts:
+//   SkSmall<NP> (NP = 4, 8): a matrix lives in the registers of 16 consecutive lanes
+//       (NP*NP/16 elements per lane); all reductions are DPP moves, no LDS traffic on the
+//       forward path.  Four matrices per wave.
+//   SkLds<NP>   (NP = 16, 32): one wave per matrix, E and the running scalings u, v in LDS
+//       (iterate = diag(u) E diag(v)); a half-step is one mat-vec product.
+#pragma once
+
+#include "mhc_common.h"
+
+namespace mhc {
+
+// =============================================================================================
+// SkSmall
+// =============================================================================================
+template <int NP> struct SkSmall {
+    static_assert(NP == 4 || NP == 8, "SkSmall handles 4x4 and 8x8 tiles");
+    static constexpr int EPL = NP * NP / 16;  // elements per lane (contiguous columns of one row)
+    static constexpr int LPR = NP / EPL;      // lanes per row
+    static constexpr int kGroup = 16;         // lanes per matrix
+
+    __device__ static __forceinline__ int row(int g) { return g / LPR; }
+    __device__ static __forceinline__ int col0(int g) { return (g % LPR) * EPL; }
+
+    // sum over the lanes that hold the same row
+    __device__ static __forceinline__ float row_allreduce(float v) {
+        v += dpp_mov<kDppQuadXor1>(v);
+        if constexpr (NP == 4) v += dpp_mov<kDppQuadXor2>(v);
+        return v;
+    }
+    // sum over the lanes that hold the same columns
+    __device__ static __forceinline__ float col_allreduce(float v) {
+        if constexpr (NP == 8) v += dpp_mov<kDppQuadXor2>(v);
+        v += dpp_mov<kDppRowRor4>(v);
+        v += dpp_mov<kDppRowRor8>(v);
+        return v;
+    }
+
+    // m: in = exp(logits) (0 outside n x n), out = final iterate.
+    // sc != nullptr: keep rho_t (this lane's row) and s_t (this lane's EPL columns) at
+    // sc[(t * (1 + EPL) + k) * 64 + lane].
+    __device__ static __forceinline__ void forward(float (&m)[EPL], int g, int n, int T, float eps,
+                                                   float *sc, int lane) {
+        const bool rv = row(g) < n;
+        bool cv[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; e++) cv[e] = col0(g) + e < n;
+        for (int t = 0; t < T; t++) {
+            float rs = 0.f;
+#pragma unroll
+            for (int e = 0; e < EPL; e++) rs += m[e];
+            rs = row_allreduce(rs) + eps;
+            rs = rv ? rs : 1.0f;
+            const float rinv = 1.0f / rs;
+            if (sc) sc[(t * (1 + EPL)) * kWave + lane] = rs;
+#pragma unroll
+            for (int e = 0; e < EPL; e++) {
+                m[e] *= rinv;
+                float cs = col_allreduce(m[e]) + eps;
+                cs = cv[e] ? cs : 1.0f;
+                if (sc) sc[(t * (1 + EPL) + 1 + e) * kWave + lane] = cs;
+                m[e] *= 1.0f / cs;
+            }
+        }
+    }
+
+    // m: final iterate (from forward); d: in = dL/dM, out = dL/dE.  sc as written by forward.
+    __device__ static __forceinline__ void backward(float (&m)[EPL], float (&d)[EPL], int T,
+                                                    const float *sc, int lane) {
+        for (int t = T - 1; t >= 0; t--) {
+            const float rs = sc[(t * (1 + EPL)) * kWave + lane];
+            float rdot = 0.f;
+            float dR[EPL];
+#pragma unroll
+            for (int e = 0; e < EPL; e++) {
+                const float cs = sc[(t * (1 + EPL) + 1 + e) * kWave + lane];
+                const float cdot = col_allreduce(d[e] * m[e]);
+                dR[e] = (d[e] - cdot) / cs;
+                m[e] *= cs;  // row-normalised iterate R_t
+                rdot += dR[e] * m[e];
+            }
+            rdot = row_allreduce(rdot);
+#pragma unroll
+            for (int e = 0; e < EPL; e++) {
+                d[e] = (dR[e] - rdot) / rs;
+                m[e] *= rs;  // iterate before row step t
+            }
+        }
+    }
+    __host__ __device__ static constexpr int scaling_floats(int T) { return T * (1 + EPL) * kWave; }
+};
+
+// =============================================================================================
+// SkLds: one wave, matrix in LDS.  LD = NP + 1 keeps row and column walks conflict-free.
+// =============================================================================================
+template <int NP> struct SkLds {
+    static constexpr int LD = NP + 1;
+    // LDS floats: E [NP*LD], u [NP], v [NP], tmp [NP], (backward) dO [NP*LD], rho [T*NP], s [T*NP]
+    __host__ __device__ static constexpr int forward_floats() { return NP * LD + 3 * NP; }
+    __host__ __device__ static constexpr int backward_floats(int T) {
+        return 2 * NP * LD + 3 * NP + 2 * T * NP;
+    }
+
+    // Es holds E (0 outside n x n).  On return u, v hold the final scalings: M = u_r E_rc v_c.
+    // rho/s (optional): per-iteration denominators [T][NP].
+    __device__ static __forceinline__ void forward(const float *Es, float *u, float *v, int n, int T,
+                                                   float eps, float *rho, float *s, int lane) {
+        if (lane < NP) { u[lane] = 1.0f; v[lane] = 1.0f; }
+        __syncthreads();
+        for (int t = 0; t < T; t++) {
+            if (lane < n) {
+                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+                for (int c = 0; c < NP; c += 4) {
+                    a0 += Es[lane * LD + c] * v[c];
+                    a1 += Es[lane * LD + c + 1] * v[c + 1];
+                    a2 += Es[lane * LD + c + 2] * v[c + 2];
+                    a3 += Es[lane * LD + c + 3] * v[c + 3];
+                }
+                const float ur = u[lane];
+                const float r = ur * ((a0 + a1) + (a2 + a3)) + eps;
+                if (rho) rho[t * NP + lane] = r;
+                u[lane] = ur / r;
+            }
+            __syncthreads();
+            if (lane < n) {
+                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+                for (int r = 0; r < NP; r += 4) {
+                    a0 += Es[r * LD + lane] * u[r];
+                    a1 += Es[(r + 1) * LD + lane] * u[r + 1];
+                    a2 += Es[(r + 2) * LD + lane] * u[r + 2];
+                    a3 += Es[(r + 3) * LD + lane] * u[r + 3];
+                }
+                const float vc = v[lane];
+                const float sc = vc * ((a0 + a1) + (a2 + a3)) + eps;
+                if (s) s[t * NP + lane] = sc;
+                v[lane] = vc / sc;
+            }
+            __syncthreads();
+        }
+    }
+
+    // dO: in = dL/dM, out = dL/dE ([NP][LD]).  u, v: final scalings (destroyed).  tmp: [NP].
+    __device__ static __forceinline__ void backward(const float *Es, float *dO, float *u, float *v,
+                                                    float *tmp, int n, int T, const float *rho,
+                                                    const float *s, int lane) {
+        for (int t = T - 1; t >= 0; t--) {
+            // column dots with the iterate after column step t: Out = u E v
+            if (lane < n) {
+                float acc = 0.f;
+                for (int k = 0; k < n; k++) acc += dO[k * LD + lane] * u[k] * Es[k * LD + lane];
+                tmp[lane] = acc * v[lane];
+            }
+            __syncthreads();
+            // row lane r: dR = (dO - cdot)/s ; rdot = sum_k dR_k R_k, R = u E v s ; dIn = (dR - rdot)/rho
+            if (lane < n) {
+                const float ur = u[lane];
+                float acc = 0.f;
+                for (int k = 0; k < n; k++)
+                    acc += (dO[lane * LD + k] - tmp[k]) * Es[lane * LD + k] * v[k];
+                const float rdot = acc * ur;
+                const float rinv = 1.0f / rho[t * NP + lane];
+                for (int k = 0; k < n; k++)
+                    dO[lane * LD + k] =
+                        ((dO[lane * LD + k] - tmp[k]) / s[t * NP + k] - rdot) * rinv;
+            }
+            __syncthreads();
+            if (lane < n) {
+                u[lane] *= rho[t * NP + lane];
+                v[lane] *= s[t * NP + lane];
+            }
+            __syncthreads();
+        }
+    }
+};
+
+}  // namespace mhc

@@ -1,0 +1,190 @@
+"""GPU parity: the HIP path, called through the C ABI, against the oracle.
+
+fp32 tier:  max|got - ref| / max|ref| <= 1e-5 on y and every gradient (ref = oracle in fp64).
+bf16 tier:  |got - ref| <= 2e-2 |ref| + 1e-2 elementwise (the stated tolerance) AND
+            max|got - ref| / max|ref| <= 2e-2, so that small-magnitude gradients are not
+            passed by the absolute term alone (ref = oracle in fp32 on the bf16-rounded inputs).
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import hip_dynamic, hip_static
+from helpers import golden, rel_err
+from oracle import naive_mhc as nm
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5
+BF16_RTOL, BF16_ATOL = 2e-2, 1e-2
+
+
+def _check(got, ref, tier, what):
+    ref = torch.as_tensor(ref).double()
+    got = torch.as_tensor(got).double()
+    e = rel_err(got, ref)
+    if tier == "fp32":
+        assert e <= FP32_TOL, f"{what}: rel err {e:.3e} > {FP32_TOL}"
+    else:
+        assert e <= BF16_RTOL, f"{what}: normalised err {e:.3e} > {BF16_RTOL}"
+        bad = (got - ref).abs() > BF16_RTOL * ref.abs() + BF16_ATOL
+        assert not bad.any(), f"{what}: {int(bad.sum())} elements outside rtol/atol"
+
+
+def _t(a):
+    return torch.from_numpy(np.asarray(a))
+
+
+# ------------------------------------------------------------------------------------------------
+# golden vectors written from the reference's own naive layers
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("tag", ["n4", "n16"])
+def test_golden_functional_fp32(tag):
+    g = golden("functional_" + tag)
+    p = {k: _t(g[k]) for k in nm.DYN_PARAM_NAMES}
+    y, grads = hip_dynamic(_t(g["x"]), p, _t(g["dy"]), int(g["T"]), float(g["eps"]))
+    _check(y, g["y"], "fp32", "y")
+    _check(grads["x"], g["dx"], "fp32", "dx")
+    for k in nm.DYN_PARAM_NAMES:
+        _check(grads[k], g["d" + k], "fp32", "d" + k)
+
+
+@pytest.mark.parametrize("tag", ["n4", "n8", "n3"])
+def test_golden_dynamic_module_fp32(tag):
+    g = golden("dynamic_" + tag)
+    p = {k: _t(g[k]) for k in nm.DYN_PARAM_NAMES}
+    for k in ("phi_pre", "phi_post", "phi_res"):
+        p[k] = p[k].t().contiguous()
+    y, grads = hip_dynamic(_t(g["x"]), p, _t(g["dy"]), int(g["T"]), float(g["eps"]))
+    _check(y, g["y"], "fp32", "y")
+    _check(grads["x"], g["dx"], "fp32", "dx")
+    for k in nm.DYN_PARAM_NAMES:
+        ref = g["d" + k].T if k.startswith("phi") else g["d" + k]
+        _check(grads[k], ref, "fp32", "d" + k)
+
+
+@pytest.mark.parametrize("tag", ["n4", "n8"])
+def test_golden_static_fp32(tag):
+    g = golden("static_" + tag)
+    p = {k: _t(g[k]) for k in nm.STATIC_PARAM_NAMES}
+    y, grads = hip_static(_t(g["x"]), p, _t(g["dy"]), int(g["T"]), float(g["eps"]))
+    _check(y, g["y"], "fp32", "y")
+    _check(grads["x"], g["dx"], "fp32", "dx")
+    for k in nm.STATIC_PARAM_NAMES:
+        _check(grads[k], g["d" + k], "fp32", "d" + k)
+
+
+# ------------------------------------------------------------------------------------------------
+# seeded inputs against the oracle: small shapes, ragged shapes, every layout of the kernels
+# ------------------------------------------------------------------------------------------------
+def _rand_params(p, n, C, seed=7):
+    """Move every parameter away from its init value so that no gradient path is trivially zero."""
+    g = torch.Generator().manual_seed(seed)
+    p = dict(p)
+    p["w"] = 1.0 + 0.3 * torch.randn(C, generator=g)
+    p["b_pre"] = 0.3 * torch.randn(n, generator=g)
+    p["b_post"] = 0.3 * torch.randn(n, generator=g)
+    p["b_res"] = 0.5 * torch.randn(n, n, generator=g)
+    p["alpha_pre"] = torch.tensor(0.05)
+    p["alpha_post"] = torch.tensor(-0.03)
+    p["alpha_res"] = torch.tensor(0.04)
+    return p
+
+
+DYN_SHAPES = [
+    (32, 4, 1280), (5, 4, 64), (1, 4, 128), (3, 2, 40), (2, 3, 20), (7, 1, 36),
+    (16, 8, 256), (3, 6, 72), (4, 16, 64), (3, 12, 40), (4, 32, 64), (2, 24, 104), (2, 32, 1040),
+]
+
+
+@pytest.mark.parametrize("B,n,C", DYN_SHAPES)
+@pytest.mark.parametrize("inject", [False, True])
+def test_dynamic_fp32_vs_oracle(B, n, C, inject):
+    x, dy, f, p = nm.make_dynamic_inputs(B, n, C, with_f=inject)
+    p = _rand_params(p, n, C)
+    T, eps = 20, 1e-6
+    y_ref, g_ref = nm.mhc_dynamic_fwd_bwd(x, p, dy, T, eps, f_inject=f, dtype=torch.float64)
+    y, g = hip_dynamic(x, p, dy, T, eps, f_inject=f)
+    _check(y, y_ref, "fp32", "y")
+    for k, ref in g_ref.items():
+        assert k in g, f"missing gradient {k}"
+        if n == 1 and k in ("phi_pre", "b_pre", "alpha_pre"):
+            # one stream: f = RMSNorm(H_pre x) w does not depend on H_pre except through eps, so
+            # the true gradient is O(eps) and a relative comparison is meaningless
+            assert float(g[k].abs().max()) < 1e-4
+            continue
+        _check(g[k], ref, "fp32", "d" + k)
+
+
+@pytest.mark.parametrize("B,n,C", [(32, 4, 1280), (5, 4, 64), (16, 8, 256), (3, 6, 72), (4, 16, 64),
+                                   (4, 32, 64), (2, 32, 1040), (3, 4, 20)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_dynamic_bf16_vs_oracle(B, n, C, out_dtype):
+    x, dy, _, p = nm.make_dynamic_inputs(B, n, C, bf16_round=True)
+    p = _rand_params(p, n, C)
+    for k in ("w", "phi_pre", "phi_post", "phi_res"):
+        p[k] = p[k].bfloat16().float()
+    if out_dtype == torch.float32:
+        dy_used = dy
+    else:
+        dy_used = dy.bfloat16().float()
+    T, eps = 20, 1e-6
+    y_ref, g_ref = nm.mhc_dynamic_fwd_bwd(x, p, dy_used, T, eps, dtype=torch.float32)
+    y, g = hip_dynamic(x, p, dy_used, T, eps, act_dtype=torch.bfloat16, out_dtype=out_dtype,
+                       w_dtype=torch.bfloat16)
+    _check(y, y_ref, "bf16", "y")
+    for k, ref in g_ref.items():
+        _check(g[k], ref, "bf16", "d" + k)
+
+
+@pytest.mark.parametrize("B,n,C", [(32, 4, 1280), (3, 4, 20), (8, 8, 128), (4, 16, 64), (3, 32, 72)])
+@pytest.mark.parametrize("inject", [False, True])
+def test_static_fp32_vs_oracle(B, n, C, inject):
+    x, dy, f, p = nm.make_static_inputs(B, n, C, with_f=inject)
+    p["w"] = 1.0 + 0.3 * torch.randn(C, generator=torch.Generator().manual_seed(3))
+    T, eps = 20, 1e-6
+    y_ref, g_ref = nm.mhc_static_fwd_bwd(x, p, dy, T, eps, f_inject=f, dtype=torch.float64)
+    y, g = hip_static(x, p, dy, T, eps, f_inject=f)
+    _check(y, y_ref, "fp32", "y")
+    for k, ref in g_ref.items():
+        _check(g[k], ref, "fp32", "d" + k)
+
+
+# ------------------------------------------------------------------------------------------------
+# the benchmark configurations at full size
+# ------------------------------------------------------------------------------------------------
+def test_config1_static_fp32_full_size():
+    B, n, C = 320, 4, 1280
+    x, dy, f, p = nm.make_static_inputs(B, n, C, with_f=True)
+    T, eps = 20, 1e-6
+    for inj in (None, f):
+        y_ref, g_ref = nm.mhc_static_fwd_bwd(x, p, dy, T, eps, f_inject=inj, dtype=torch.float64)
+        y, g = hip_static(x, p, dy, T, eps, f_inject=inj)
+        _check(y, y_ref, "fp32", "y")
+        for k, ref in g_ref.items():
+            _check(g[k], ref, "fp32", "d" + k)
+
+
+@pytest.mark.parametrize("B,n,C", [(320, 4, 1280), (1280, 4, 2560), (256, 8, 1280), (128, 32, 1280)])
+@pytest.mark.parametrize("inject", [False, True])
+def test_configs_2_to_5_bf16_full_size(B, n, C, inject):
+    x, dy, f, p = nm.make_dynamic_inputs(B, n, C, bf16_round=True, with_f=inject)
+    T, eps = 20, 1e-6
+    y_ref, g_ref = nm.mhc_dynamic_fwd_bwd(x, p, dy, T, eps, f_inject=f, dtype=torch.float32)
+    y, g = hip_dynamic(x, p, dy, T, eps, f_inject=f, act_dtype=torch.bfloat16,
+                       out_dtype=torch.bfloat16, w_dtype=torch.bfloat16)
+    _check(y, y_ref, "bf16", "y")
+    for k, ref in g_ref.items():
+        _check(g[k], ref, "bf16", "d" + k)
+
+
+def test_config2_fp32_full_size():
+    """The headline shape in the fp32 tier (1e-5)."""
+    B, n, C = 320, 4, 1280
+    x, dy, _, p = nm.make_dynamic_inputs(B, n, C)
+    T, eps = 20, 1e-6
+    y_ref, g_ref = nm.mhc_dynamic_fwd_bwd(x, p, dy, T, eps, dtype=torch.float64)
+    y, g = hip_dynamic(x, p, dy, T, eps)
+    _check(y, y_ref, "fp32", "y")
+    for k, ref in g_ref.items():
+        _check(g[k], ref, "fp32", "d" + k)
