@@ -49,7 +49,7 @@ int ws_check(void *ws, size_t have, size_t need) {
 
 // ---- dynamic workspace layout ----------------------------------------------------------------
 struct DynFwdWs { float *Ppart, *ssqpart; size_t bytes; };
-struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *cs_dt, *cs_u, *dphi_part; size_t bytes; };
+struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *cs_dt, *cs_u, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
 
 int max_ksplit(int B, int n, int C) { return proj_fwd_ksplit(kBF16, kBF16, B, n, C); }
 
@@ -74,8 +74,13 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
     w.u = c.floats((size_t)B * C);
     w.cs_dt = c.floats(colsum_workspace_floats(B, D + 3));
     w.cs_u = c.floats(colsum_workspace_floats(B, C));
-    const int bs = dphi_batch_splits(B, n, C);
+    int bs = dphi_batch_splits(B, n, C);
+    const int bs2 = proj_bwd_batch_splits(B, n, C);
+    if (bs2 > bs) bs = bs2;
     w.dphi_part = c.floats(bs > 1 ? (size_t)bs * D * nC : 0);
+    w.BP = (B + 31) / 32 * 32;
+    w.dPb = reinterpret_cast<unsigned short *>(c.floats(((size_t)B * padded_D(n) + 1) / 2));
+    w.dPT = reinterpret_cast<unsigned short *>(c.floats((size_t)padded_D(n) * w.BP));  // two bf16 planes
     w.bytes = c.off;
     return w;
 }
@@ -182,12 +187,22 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int D = n * n + 2 * n, DP = padded_D(n);
-    BwdCoefOut out{ws.dt, ws.dP, ws.cx, ws.s1, nullptr};
+    const bool mfma = proj_bwd_mfma_supported(x_dtype, phi_dtype, C);
+    BwdCoefOut out{ws.dt, ws.dP, ws.cx, ws.s1, nullptr, mfma ? ws.dPb : nullptr, ws.dPT, ws.BP};
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      n, q, P, r, alpha, bias + 2 * n, out, B, n, C, iters, eps, st));
-    MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, n,
-                                 q, ws.s1, ws.cx, ws.dP, DP, phi, phi_dtype, dx, df, ws.u, B, n, C, st));
-    MHC_LAUNCH(launch_dphi(x, x_dtype, ws.dP, DP, dphi, B, n, C, ws.dphi_part, st));
+    if (mfma) {
+        // matrix cores: dphi and the projection term of dx (written into dx, then completed in place)
+        MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st));
+        MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
+                                     n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, B, n,
+                                     C, st));
+    } else {
+        MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
+                                     n, q, ws.s1, ws.cx, ws.dP, DP, phi, phi_dtype, nullptr, dx, df,
+                                     ws.u, B, n, C, st));
+        MHC_LAUNCH(launch_dphi(x, x_dtype, ws.dP, DP, dphi, B, n, C, ws.dphi_part, st));
+    }
     MHC_LAUNCH(launch_colsum_split(ws.dt, B, D + 3, D + 3, dbias, dalpha, D, ws.cs_dt, st));
     if (!f_inject) MHC_LAUNCH(launch_colsum(ws.u, B, C, C, dw, ws.cs_u, st));
     return MHC_OK;
@@ -246,12 +261,13 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
     if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int D = n * n + 2 * n;
-    BwdCoefOut out{nullptr, nullptr, nullptr, ws.s1, ws.red};
+    BwdCoefOut out{nullptr, nullptr, nullptr, ws.s1, ws.red, nullptr, nullptr, 0};
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      0, q, nullptr, nullptr, nullptr, nullptr, out, B, n, C, iters,
                                      eps, st));
     MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, 0,
-                                 q, ws.s1, nullptr, nullptr, 0, nullptr, 0, dx, df, ws.u, B, n, C, st));
+                                 q, ws.s1, nullptr, nullptr, 0, nullptr, 0, nullptr, dx, df, ws.u, B, n, C,
+                                 st));
     MHC_LAUNCH(launch_colsum(ws.red, B, D, D, ws.red_sum, ws.cs_red, st));
     MHC_LAUNCH(launch_coef_bwd_static(ws.red_sum, H_pre, H_post, H_res_logits, dH_pre, dH_post,
                                       dH_res, n, iters, eps, st));

@@ -47,6 +47,9 @@ struct BwdCoefOut {
     float *cx;    // [B]      sum_d dt_d alpha_g p_d / (nC r^2)                    (dynamic only)
     float *s1;    // [B]      sum_c df_c w_c a_c
     float *red;   // [B, n*n + 2n] raw per-sample (dM | dHpre | dHpost)             (static only)
+    unsigned short *dPb;  // [B, DP]  bf16 copy of dP, or nullptr                     (dynamic only)
+    unsigned short *dPT;  // [2][DP, BP] bf16 transpose of dP (high part, remainder), pad zeroed
+    int BP;               // row pitch of dPT, a multiple of 32 that is >= B
 };
 
 // Per-sample reductions over c (dM, dHpost, dHpre, s1) and, for dynamic H, the coefficient
@@ -58,14 +61,23 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
                                  const float *b_res, BwdCoefOut out, int B, int n, int C, int T,
                                  float eps, hipStream_t stream);
 
-// dx = M^T dy + Hpre (x) da - cx * x  [+ dP phi when phi != nullptr], df, and u = df * a / q
-// (the per-sample summand of dw).
+// dx = M^T dy + Hpre (x) da - cx * x  [+ dP phi when phi != nullptr] [+ dx_in when != nullptr;
+// may alias dx], df, and u = df * a / q (the per-sample summand of dw).
 hipError_t launch_mix_bwd_dx(const void *dy, int y_dtype, const void *x, int x_dtype, const void *w,
                              int w_dtype, const void *f_inject, const float *Hpre,
                              const float *Hpost, const float *M, int hstride, const float *q,
                              const float *s1, const float *cx, const float *dP, int DP,
-                             const void *phi, int phi_dtype, void *dx, void *df, float *u, int B,
-                             int n, int C, hipStream_t stream);
+                             const void *phi, int phi_dtype, const void *dx_in, void *dx, void *df,
+                             float *u, int B, int n, int C, hipStream_t stream);
+
+// Matrix-core projection backward (x and phi bf16, C % 8 == 0): dphi = dP^T x_flat and
+// dxflat = dP phi (bf16 [B, nC]) in one pass over x and phi.  dphi_part: proj_bwd_batch_splits()
+// copies of dphi when that is > 1.
+bool proj_bwd_mfma_supported(int x_dtype, int phi_dtype, int C);
+int proj_bwd_batch_splits(int B, int n, int C);
+hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,
+                                int BP, float *dphi, float *dphi_part, void *dxflat, int B, int n,
+                                int C, hipStream_t stream);
 
 // dphi[d, k] = sum_b dP[b, d] * x_flat[b, k].  `partial` holds dphi_batch_splits() copies of
 // dphi when that is > 1.

@@ -13,7 +13,7 @@
 namespace mhc {
 
 struct BwdDxArgs {
-    const void *dy, *x, *w, *f_inject, *phi;
+    const void *dy, *x, *w, *f_inject, *phi, *dx_in;
     const float *Hpre, *Hpost, *M, *q, *s1, *cx, *dP;
     void *dx, *df;
     float *u;
@@ -115,6 +115,12 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
                         for (int v = 0; v < V; v++) out[v] += dp * pv[v];
                     }
                 }
+                if (a.dx_in) {
+                    float prev[V];
+                    load_vec<TX, V>(static_cast<const TX *>(a.dx_in) + ((size_t)b * n + j) * C + c, prev);
+#pragma unroll
+                    for (int v = 0; v < V; v++) out[v] += prev[v];
+                }
                 store_vec<TX, V>(dxb + (size_t)j * C + c, out);
             }
         }
@@ -152,9 +158,9 @@ hipError_t launch_mix_bwd_dx(const void *dy, int y_dtype, const void *x, int x_d
                              int w_dtype, const void *f_inject, const float *Hpre,
                              const float *Hpost, const float *M, int hstride, const float *q,
                              const float *s1, const float *cx, const float *dP, int DP,
-                             const void *phi, int phi_dtype, void *dx, void *df, float *u, int B,
-                             int n, int C, hipStream_t stream) {
-    BwdDxArgs a{dy, x, w, f_inject, phi, Hpre, Hpost, M, q, s1, cx, dP, dx, df, u,
+                             const void *phi, int phi_dtype, const void *dx_in, void *dx, void *df,
+                             float *u, int B, int n, int C, hipStream_t stream) {
+    BwdDxArgs a{dy, x, w, f_inject, phi, dx_in, Hpre, Hpost, M, q, s1, cx, dP, dx, df, u,
                 hstride, w_dtype == kBF16, phi_dtype == kBF16, B, n, C, DP};
     if (y_dtype == kF32 && x_dtype == kF32) return launch_t<float, float>(a, stream);
     if (y_dtype == kBF16 && x_dtype == kBF16) return launch_t<bf16_t, bf16_t>(a, stream);

@@ -43,6 +43,46 @@ __device__ __forceinline__ float row16_allreduce(float v) {
     return v;
 }
 
+// Writes dP[b, d] in every layout the later kernels read: fp32 [B, DP] (generic kernels),
+// bf16 [B, DP] and bf16 transposed [2][DP, BP] (MFMA operands; plane 0 = value rounded to
+// bf16, plane 1 = the rounding remainder, so that dphi keeps ~16 mantissa bits of dP).  Padded
+// rows d >= D and, from the last sample's workgroup, padded columns b >= B are zeroed.
+struct DPWriter {
+    BwdCoefOut o;
+    int b, B, DP;
+    __device__ __forceinline__ void put(int d, float v) const {
+        o.dP[(size_t)b * DP + d] = v;
+        if (o.dPb) {
+            const bf16_t h = f32_to_bf16(v);
+            const size_t plane = (size_t)DP * o.BP;
+            o.dPb[(size_t)b * DP + d] = h;
+            o.dPT[(size_t)d * o.BP + b] = h;
+            o.dPT[plane + (size_t)d * o.BP + b] = f32_to_bf16(v - bf16_to_f32(h));
+            if (b == B - 1)
+                for (int bb = B; bb < o.BP; bb++) {
+                    o.dPT[(size_t)d * o.BP + bb] = 0;
+                    o.dPT[plane + (size_t)d * o.BP + bb] = 0;
+                }
+        }
+    }
+    __device__ __forceinline__ void pad(int D, int first, int step) const {
+        for (int d = D + first; d < DP; d += step) {
+            o.dP[(size_t)b * DP + d] = 0.f;
+            if (o.dPb) {
+                const size_t plane = (size_t)DP * o.BP;
+                o.dPb[(size_t)b * DP + d] = 0;
+                o.dPT[(size_t)d * o.BP + b] = 0;
+                o.dPT[plane + (size_t)d * o.BP + b] = 0;
+                if (b == B - 1)
+                    for (int bb = B; bb < o.BP; bb++) {
+                        o.dPT[(size_t)d * o.BP + bb] = 0;
+                        o.dPT[plane + (size_t)d * o.BP + bb] = 0;
+                    }
+            }
+        }
+    }
+};
+
 // =============================================================================================
 // n <= 8
 // =============================================================================================
@@ -160,14 +200,14 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
     const float al0 = a.alpha[0], al1 = a.alpha[1], al2 = a.alpha[2];
     const float rinv = 1.0f / a.r[b];
     float *dt = a.out.dt + (size_t)b * (D + 3);
-    float *dP = a.out.dP + (size_t)b * a.DP;
+    const DPWriter dpw{a.out, b, a.B, a.DP};
     float S0 = 0.f, S1 = 0.f, S2 = 0.f;  // sum_d dt_d p_d per alpha group
     if (g < n) {
         const float hp = Hpre[g], ho = Hpost[g];
         const float dtp = dHpre * hp * (1.0f - hp);
         const float dto = dHpost * ho * (1.0f - 0.5f * ho);
         dt[g] = dtp; dt[n + g] = dto;
-        dP[g] = dtp * al0 * rinv; dP[n + g] = dto * al1 * rinv;
+        dpw.put(g, dtp * al0 * rinv); dpw.put(n + g, dto * al1 * rinv);
         S0 = dtp * Pb[g]; S1 = dto * Pb[n + g];
     }
     float E[SK::EPL], m[SK::EPL], d[SK::EPL];
@@ -188,7 +228,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
             const int di = 2 * n + r0 * n + c;
             const float dtr = d[e] * E[e];
             dt[di] = dtr;
-            dP[di] = dtr * al2 * rinv;
+            dpw.put(di, dtr * al2 * rinv);
             S2 += dtr * Pb[di];
         }
     }
@@ -197,7 +237,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
         dt[D] = S0; dt[D + 1] = S1; dt[D + 2] = S2;
         a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv / (float)(n * C);
     }
-    for (int di = D + g; di < a.DP; di += 16) dP[di] = 0.f;
+    dpw.pad(D, g, 16);
 }
 
 // =============================================================================================
@@ -417,7 +457,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_large_kernel(BwdReduceArgs
     const float al0 = a.alpha[0], al1 = a.alpha[1], al2 = a.alpha[2];
     const float rinv = 1.0f / a.r[b];
     float *dt = a.out.dt + (size_t)b * (D + 3);
-    float *dP = a.out.dP + (size_t)b * a.DP;
+    const DPWriter dpw{a.out, b, a.B, a.DP};
     float S0 = 0.f, S1 = 0.f, S2 = 0.f;  // sum_d dt_d p_d per alpha group
     if (w0) {
         if (lane < n) {
@@ -425,7 +465,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_large_kernel(BwdReduceArgs
             const float dtp = dHpre * hp * (1.0f - hp);
             const float dto = dHpost * ho * (1.0f - 0.5f * ho);
             dt[lane] = dtp; dt[n + lane] = dto;
-            dP[lane] = dtp * al0 * rinv; dP[n + lane] = dto * al1 * rinv;
+            dpw.put(lane, dtp * al0 * rinv); dpw.put(n + lane, dto * al1 * rinv);
             S0 = dtp * Pb[lane]; S1 = dto * Pb[n + lane];
         }
         for (int e = lane; e < NP * NP; e += kWave) {
@@ -443,7 +483,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_large_kernel(BwdReduceArgs
             const int di = 2 * n + e;
             const float dtr = dO[r0 * SK::LD + c] * Es[r0 * SK::LD + c];
             dt[di] = dtr;
-            dP[di] = dtr * al2 * rinv;
+            dpw.put(di, dtr * al2 * rinv);
             S2 += dtr * Pb[di];
         }
         S0 = wave_allreduce_sum(S0); S1 = wave_allreduce_sum(S1); S2 = wave_allreduce_sum(S2);
@@ -451,7 +491,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_large_kernel(BwdReduceArgs
             dt[D] = S0; dt[D + 1] = S1; dt[D + 2] = S2;
             a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv / (float)(n * C);
         }
-        for (int di = D + lane; di < a.DP; di += kWave) dP[di] = 0.f;
+        dpw.pad(D, lane, kWave);
     }
 }
 

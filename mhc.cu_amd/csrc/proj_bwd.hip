@@ -1,0 +1,234 @@
+// Projection backward on the matrix cores (bf16 tier): for one slab of x_flat / phi columns,
+//   dphi[d, k]   = sum_b dP[b, d] x_flat[b, k]        (reference ops.py:332-334)
+//   dxflat[b, k] = sum_d dP[b, d] phi[d, k]           (reference ops.py:336-338)
+// Both products share the slab's x and phi tiles, so phi and x are read from HBM once here.
+//
+// A workgroup (4 waves) owns 32*NTK columns k and walks the samples of its batch split in
+// blocks of 128/NTK.  v_mfma_f32_32x32x16_bf16 contracts over the index that each lane holds
+// 8 consecutive values of; for dphi that index is b and for dxflat it is d, while x and phi are
+// stored with k contiguous.  The tiles are therefore staged row-major in LDS with 16-byte
+// stores and read back transposed (8 two-byte reads per fragment).  The other operand (dP as
+// [B, DP] and as its transpose [DP, BP], both bf16, written by the reduce kernel) is loaded
+// straight from global memory in MFMA layout.  dP^T comes as a bf16 high part plus a bf16
+// remainder (two MFMAs per step), which keeps dphi at fp32-like accuracy; x is exact in bf16.
+#include "launchers.h"
+#include "mhc_common.h"
+
+namespace mhc {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+struct ProjBwdArgs {
+    const bf16_t *x;     // [B][nC]
+    const bf16_t *phi;   // [D][nC]
+    const bf16_t *dPb;   // [B][DP]   (columns >= D are zero)
+    const bf16_t *dPT;   // [2][DP][BP] high and low bf16 parts of dP^T (rows >= D, columns >= B zero)
+    float *dphi;         // [S][D][nC]  (S = gridDim.y batch splits)
+    bf16_t *dxflat;      // [B][nC]
+    int B, BP, D, DP, nC, b_per_split;
+};
+
+// Transposed fragment: lane (n = lane & 31, kg = lane >> 5) gets tile[k0 + kg*8 + i][col0 + n], i = 0..7
+__device__ __forceinline__ bf16x8_t lds_frag_t(const bf16_t *tile, int ld, int k0, int col0, int lane) {
+    const bf16_t *p = tile + (size_t)(k0 + (lane >> 5) * 8) * ld + col0 + (lane & 31);
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t lo = p[(2 * i) * ld], hi = p[(2 * i + 1) * ld];
+        w[i] = lo | (hi << 16);
+    }
+    return __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
+}
+
+template <int NTK, int TPW, bool PHI_REGS>
+__global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
+    constexpr int NSB = 4 / NTK;         // 32-sample tiles per block
+    constexpr int KW = 32 * NTK;         // slab width
+    constexpr int LD = KW + 8;           // LDS row pitch (elements), keeps 16-byte alignment
+    constexpr int SBR = 32 * NSB;        // samples per block
+    constexpr int CPR = KW / 8;          // 16-byte chunks per tile row
+    extern __shared__ bf16_t lds_bf[];
+    bf16_t *phi_s = lds_bf;                       // [DP][LD]
+    bf16_t *x_s = phi_s + (size_t)a.DP * LD;      // [SBR][LD]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int k0 = blockIdx.x * KW;
+    const int nt = wave % NTK, bt = wave / NTK;
+    const int NTD = a.DP / 32;
+    const int b_begin = blockIdx.y * a.b_per_split;
+    const int b_end = min(a.B, b_begin + a.b_per_split);
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+
+    // ---- phi slab -> LDS (rows >= D and columns >= nC read as zero) ------------------------
+    for (int ch = tid; ch < a.DP * CPR; ch += 256) {
+        const int d = ch / CPR, k = k0 + (ch % CPR) * 8;
+        const uint4 v = (d < a.D && k < a.nC)
+                            ? *reinterpret_cast<const uint4 *>(a.phi + (size_t)d * a.nC + k) : zero4;
+        *reinterpret_cast<uint4 *>(phi_s + (size_t)d * LD + (ch % CPR) * 8) = v;
+    }
+    __syncthreads();
+    bf16x8_t phif[PHI_REGS ? 2 * TPW * 4 / NTK : 1];  // fragments (nt, ks) for ks < 2*NTD
+    if constexpr (PHI_REGS) {
+#pragma unroll
+        for (int ks = 0; ks < 2 * TPW * 4 / NTK; ks++)
+            if (ks < 2 * NTD) phif[ks] = lds_frag_t(phi_s, LD, ks * 16, nt * 32, lane);
+    }
+
+    f32x16_t acc[TPW];
+#pragma unroll
+    for (int m = 0; m < TPW; m++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[m][i] = 0.f;
+
+    const int row = lane & 31, kg = lane >> 5;
+    for (int sb = b_begin; sb < b_end; sb += SBR) {
+        // ---- x block -> LDS ------------------------------------------------------------------
+        if (sb != b_begin) __syncthreads();  // previous block's fragment reads are done
+        for (int ch = tid; ch < SBR * CPR; ch += 256) {
+            const int bl = ch / CPR, b = sb + bl, k = k0 + (ch % CPR) * 8;
+            const uint4 v = (b < b_end && k < a.nC)
+                                ? *reinterpret_cast<const uint4 *>(a.x + (size_t)b * a.nC + k) : zero4;
+            *reinterpret_cast<uint4 *>(x_s + (size_t)bl * LD + (ch % CPR) * 8) = v;
+        }
+        __syncthreads();
+
+        // ---- dphi tiles of this wave: (dt, nt), dt = (wave + 4m) / NTK -------------------------
+#pragma unroll
+        for (int ks = 0; ks < 2 * NSB; ks++) {
+            if (sb + ks * 16 < b_end) {
+                const bf16x8_t xf = lds_frag_t(x_s, LD, ks * 16, nt * 32, lane);
+#pragma unroll
+                for (int m = 0; m < TPW; m++) {
+                    const int dt = (wave + 4 * m) / NTK;
+                    if (dt < NTD) {
+                        // dP^T rows d, 8 consecutive samples; the pad columns [B, BP) are zero
+                        const bf16_t *ap = a.dPT + (size_t)(dt * 32 + row) * a.BP + sb + ks * 16 + kg * 8;
+                        const uint4 ah = *reinterpret_cast<const uint4 *>(ap);
+                        const uint4 al = *reinterpret_cast<const uint4 *>(ap + (size_t)a.DP * a.BP);
+                        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(bf16x8_t, ah), xf, acc[m], 0, 0, 0);
+                        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(bf16x8_t, al), xf, acc[m], 0, 0, 0);
+                    }
+                }
+            }
+        }
+
+        // ---- dxflat tile of this wave: samples sb + 32 bt .. +32, columns nt ------------------
+        const int bs0 = sb + 32 * bt;
+        if (bs0 < b_end) {
+            f32x16_t o;
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[i] = 0.f;
+            const int b = bs0 + row;
+            const bf16_t *dprow = a.dPb + (size_t)(b < a.B ? b : 0) * a.DP + kg * 8;
+            if constexpr (PHI_REGS) {
+#pragma unroll
+                for (int ks = 0; ks < 2 * TPW * 4 / NTK; ks++) {
+                    if (ks < 2 * NTD) {
+                        const uint4 av = b < b_end ? *reinterpret_cast<const uint4 *>(dprow + ks * 16) : zero4;
+                        o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                    phif[ks], o, 0, 0, 0);
+                    }
+                }
+            } else {
+                for (int ks = 0; ks < 2 * NTD; ks++) {
+                    const uint4 av = b < b_end ? *reinterpret_cast<const uint4 *>(dprow + ks * 16) : zero4;
+                    const bf16x8_t pf = lds_frag_t(phi_s, LD, ks * 16, nt * 32, lane);
+                    o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pf, o, 0, 0, 0);
+                }
+            }
+            // accumulator layout: column = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4
+            const int k = k0 + nt * 32 + row;
+            if (k < a.nC) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int bo = bs0 + 8 * (i >> 2) + 4 * kg + (i & 3);
+                    if (bo < b_end) a.dxflat[(size_t)bo * a.nC + k] = f32_to_bf16(o[i]);
+                }
+            }
+        }
+    }
+
+    // ---- dphi out (this split's partial) -------------------------------------------------------
+    float *out = a.dphi + (size_t)blockIdx.y * a.D * a.nC;
+    const int k = k0 + nt * 32 + row;
+#pragma unroll
+    for (int m = 0; m < TPW; m++) {
+        const int dt = (wave + 4 * m) / NTK;
+        if (dt < NTD && k < a.nC) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int d = dt * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
+                if (d < a.D) out[(size_t)d * a.nC + k] = acc[m][i];
+            }
+        }
+    }
+}
+
+// --------------------------------------------------------------------------------------------
+// shape selection
+// --------------------------------------------------------------------------------------------
+bool proj_bwd_mfma_supported(int x_dtype, int phi_dtype, int C) {
+    return x_dtype == kBF16 && phi_dtype == kBF16 && C % 8 == 0;
+}
+
+// Slab width (in 32-column tiles) for this shape.
+static int proj_bwd_ntk(int B, int n, int C) {
+    (void)B; (void)n; (void)C;
+    return 1;
+}
+
+int proj_bwd_batch_splits(int B, int n, int C) {
+    const int NTK = proj_bwd_ntk(B, n, C);
+    const int nC = n * C, D = n * n + 2 * n;
+    const int slabs = (nC + 32 * NTK - 1) / (32 * NTK);
+    const int sbr = 32 * (4 / NTK);
+    const int nblocks = (B + sbr - 1) / sbr;
+    int S = (512 + slabs - 1) / slabs;
+    if (S > nblocks) S = nblocks;
+    // keep the partial sums below ~1/4 of the activation bytes this kernel moves
+    const double cap = 0.25 * (2.0 * 2.0 * B * nC) / (4.0 * D * nC);
+    if (S > (int)cap) S = (int)cap;
+    if (S < 1) S = 1;
+    return S;
+}
+
+template <int NTK, int TPW, bool PHI_REGS>
+static hipError_t launch_shape(const ProjBwdArgs &a, int S, hipStream_t stream) {
+    constexpr int LD = 32 * NTK + 8;
+    const size_t smem = sizeof(bf16_t) * (size_t)LD * (a.DP + 32 * (4 / NTK));
+    auto kern = proj_bwd_mfma_kernel<NTK, TPW, PHI_REGS>;
+    if (smem > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return e;
+    }
+    dim3 grid((a.nC + 32 * NTK - 1) / (32 * NTK), S);
+    kern<<<grid, 256, smem, stream>>>(a);
+    return hipGetLastError();
+}
+
+hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,
+                                int BP, float *dphi, float *dphi_part, void *dxflat, int B, int n,
+                                int C, hipStream_t stream) {
+    const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
+    const int S = proj_bwd_batch_splits(B, n, C);
+    const int NTK = proj_bwd_ntk(B, n, C);
+    const int sbr = 32 * (4 / NTK);
+    const int nblocks = (B + sbr - 1) / sbr;
+    const int bps = (nblocks + S - 1) / S * sbr;
+    ProjBwdArgs a{static_cast<const bf16_t *>(x), static_cast<const bf16_t *>(phi),
+                  static_cast<const bf16_t *>(dPb), static_cast<const bf16_t *>(dPT),
+                  S > 1 ? dphi_part : dphi, static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, bps};
+    const int NTD = DP / 32;
+    hipError_t e;
+    // NTK == 1: dphi tiles per wave = ceil(NTD / 4); phi fragments in registers when 2*NTD <= 8
+    if (NTD <= 4) e = launch_shape<1, 1, true>(a, S, stream);
+    else if (NTD <= 12) e = launch_shape<1, 3, false>(a, S, stream);
+    else e = launch_shape<1, 9, false>(a, S, stream);
+    if (e != hipSuccess || S == 1) return e;
+    return launch_colsum(dphi_part, S, D * nC, D * nC, dphi, nullptr, stream);
+}
+
+}  // namespace mhc
