@@ -159,6 +159,13 @@ int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int KS = proj_fwd_ksplit(x_dtype, phi_dtype, B, n, C);
     MHC_LAUNCH(launch_proj_fwd(x, x_dtype, phi, phi_dtype, ws.Ppart, ws.ssqpart, KS, B, n, C, st));
+    if (layer_fwd_fused_supported(n, C, x_dtype)) {
+        MHC_LAUNCH(launch_layer_fwd_fused(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, ws.Ppart,
+                                          ws.ssqpart, KS, padded_D(n), alpha, bias, bias + n,
+                                          bias + 2 * n, H_pre, H_post, M, P, r, q, B, n, C, iters, eps,
+                                          st));
+        return MHC_OK;
+    }
     MHC_LAUNCH(launch_coef_fwd(ws.Ppart, ws.ssqpart, KS, padded_D(n), alpha, bias, bias + n,
                                bias + 2 * n, H_pre, H_post, M, P, r, B, n, n * C, iters, eps, st));
     MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, H_pre, H_post, M, n, q,
@@ -228,13 +235,20 @@ int mhc_layer_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
     if (!f_inject && !w) return MHC_ERR_NULL_POINTER;
     if (!valid_io(x_dtype, y_dtype) || (w && !valid_dtype(w_dtype))) return MHC_ERR_BAD_DTYPE;
     if (!aligned16(x) || !aligned16(y) || (f_inject && !aligned16(f_inject))) return MHC_ERR_MISALIGNED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (layer_fwd_fused_supported(n, C, x_dtype)) {
+        // one launch; every workgroup derives the shared coefficients itself, none need storing
+        MHC_LAUNCH(launch_layer_fwd_fused(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, nullptr, nullptr,
+                                          0, 0, nullptr, H_pre_logits, H_post_logits, H_res_logits,
+                                          H_pre, H_post, M, nullptr, nullptr, q, B, n, C, iters, eps, st));
+        return MHC_OK;
+    }
     const StaFwdWs ws = carve_sta_fwd(workspace, B, n);
     const bool need_ws = !H_pre || !H_post || !M || !q;
     if (need_ws)
         if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
     float *hp = H_pre ? H_pre : ws.Hpre, *ho = H_post ? H_post : ws.Hpost;
     float *m = M ? M : ws.M, *qq = q ? q : ws.q;
-    hipStream_t st = static_cast<hipStream_t>(stream);
     MHC_LAUNCH(launch_coef_fwd(nullptr, nullptr, 0, 0, nullptr, H_pre_logits, H_post_logits,
                                H_res_logits, hp, ho, m, nullptr, nullptr, 1, n, n * C, iters, eps, st));
     MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, hp, ho, m, 0, qq, B, n, C,

@@ -39,6 +39,17 @@ hipError_t launch_mix_fwd(const void *x, int x_dtype, const void *w, int w_dtype
                           const float *Hpost, const float *M, int hstride, float *q, int B, int n,
                           int C, float eps, hipStream_t stream);
 
+// Fused coefficients + mix for n <= 8 when the sample's tile fits in registers
+// (layer_fwd_fused_supported).  Ppart == nullptr selects static H (logits in b_pre/b_post/b_res,
+// outputs Hpre/Hpost/M shared and optional).
+bool layer_fwd_fused_supported(int n, int C, int x_dtype);
+hipError_t launch_layer_fwd_fused(const void *x, int x_dtype, const void *w, int w_dtype,
+                                  const void *f_inject, void *y, int y_dtype, const float *Ppart,
+                                  const float *ssqpart, int KS, int DP, const float *alpha,
+                                  const float *b_pre, const float *b_post, const float *b_res,
+                                  float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
+                                  int B, int n, int C, int T, float eps, hipStream_t stream);
+
 // ---- backward --------------------------------------------------------------------------------
 
 struct BwdCoefOut {

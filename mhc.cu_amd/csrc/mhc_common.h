@@ -157,6 +157,10 @@ template <int NT> __device__ __forceinline__ float block_allreduce_sum(float v, 
 
 __device__ __forceinline__ float sigmoidf_acc(float t) { return 1.0f / (1.0f + expf(-t)); }
 
+// v_rcp_f32: 1 ulp, one instruction (an IEEE division costs ~10 dependent instructions, which
+// matters on the serial Sinkhorn chain).
+__device__ __forceinline__ float fast_rcp(float v) { return __builtin_amdgcn_rcpf(v); }
+
 // Index of the alpha group of projection row d: 0 = pre, 1 = post, 2 = res.
 __device__ __forceinline__ int alpha_group(int d, int n) { return d < n ? 0 : (d < 2 * n ? 1 : 2); }
 

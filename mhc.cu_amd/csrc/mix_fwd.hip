@@ -5,7 +5,7 @@
 // a and f never leave the chip; x is fetched from HBM once (the second sweep over the sample's
 // tile hits L1/L2).  With an injected f the first sweep is skipped.
 #include "launchers.h"
-#include "mhc_common.h"
+#include "sinkhorn_device.h"
 
 namespace mhc {
 
@@ -124,6 +124,269 @@ __global__ __launch_bounds__(256) void mix_fwd_kernel(MixFwdArgs a) {
             }
         }
     }
+}
+
+// =============================================================================================
+// Fused layer forward for n <= 8: coefficients + mix in one launch, x read from HBM exactly once.
+//
+// Every workgroup first issues the loads of its sample's whole [n, C] tile (kept in registers),
+// then 16 lanes of wave 0 turn the projection partial sums (dynamic H) or the shared logits
+// (static H) into H_pre, H_post and M - the Sinkhorn chain runs while the x loads are in
+// flight - and finally all threads aggregate, normalise and mix out of registers.
+// Replaces fused_h_activations + sinkhorn_knopp_forward_batched + stream_aggregate +
+// rmsnorm_forward_with_rms + stream_distribute_mix_add of the reference
+// (bindings.cu:449-477) by one kernel.
+// =============================================================================================
+struct LayerFwdArgs {
+    const void *x, *w, *f_inject;
+    void *y;
+    const float *Ppart, *ssqpart;   // dynamic: [KS][B][DP], [KS][B]; static: nullptr
+    const float *alpha, *b_pre, *b_post, *b_res;
+    float *Hpre, *Hpost, *M, *P, *r, *q;  // outputs (static: shared [n], [n], [n,n]; may be null)
+    int KS, DP, w_bf16, B, n, C, T;
+    float eps;
+};
+
+template <typename TX, typename TY, int NP, int V, int CPT>
+__global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
+    using SK = SkSmall<NP>;
+    __shared__ float coef_s[NP * NP + 2 * NP];  // M | Hpre | Hpost
+    __shared__ float red[4];
+    const int b = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x;
+    const TX *__restrict__ xb = static_cast<const TX *>(a.x) + (size_t)b * n * C;
+    TY *__restrict__ yb = static_cast<TY *>(a.y) + (size_t)b * n * C;
+    const bool inject = a.f_inject != nullptr;
+    const bool dyn = a.Ppart != nullptr;
+    const int nch = C / V;
+
+    // ---- 1. loads.  Wave 0 first asks for the small coefficient inputs (they return ahead of
+    // the bulk data, so the Sinkhorn chain below runs while the tile is still streaming in),
+    // then every thread issues the loads of the sample's whole tile. ------------------------------
+    const int g = tid & 15, part = (tid >> 4) & 3;  // wave 0: 4 lanes share each partial-sum reduction
+    const int D = n * n + 2 * n;
+    const int r0 = SK::row(g), c0 = SK::col0(g);
+    float al0 = 0.f, al1 = 0.f, al2 = 0.f, bpre = 0.f, bpost = 0.f, bres[SK::EPL];
+    float t_ssq[4], t_pre[4], t_post[4], t_e[4][SK::EPL];
+    const size_t ps = (size_t)a.B * a.DP;
+    const float *Pb = dyn ? a.Ppart + (size_t)b * a.DP : nullptr;
+    if (tid < 64) {
+        if (dyn) { al0 = a.alpha[0]; al1 = a.alpha[1]; al2 = a.alpha[2]; }
+        if (g < n) { bpre = a.b_pre[g]; bpost = a.b_post[g]; }
+#pragma unroll
+        for (int e = 0; e < SK::EPL; e++) bres[e] = (r0 < n && c0 + e < n) ? a.b_res[r0 * n + c0 + e] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {  // first batch of K-split partials: ks = part*4 + u
+            const int ks = part * 4 + u;
+            const bool ok = dyn && ks < a.KS;
+            t_ssq[u] = ok ? a.ssqpart[(size_t)ks * a.B + b] : 0.f;
+            t_pre[u] = (ok && g < n) ? Pb[ks * ps + g] : 0.f;
+            t_post[u] = (ok && g < n) ? Pb[ks * ps + n + g] : 0.f;
+#pragma unroll
+            for (int e = 0; e < SK::EPL; e++)
+                t_e[u][e] = (ok && r0 < n && c0 + e < n) ? Pb[ks * ps + 2 * n + r0 * n + c0 + e] : 0.f;
+        }
+    }
+    float xv[CPT][NP][V];
+#pragma unroll
+    for (int k = 0; k < CPT; k++) {
+        const int ch = tid + k * 256;
+#pragma unroll
+        for (int i = 0; i < NP; i++) {
+            if (ch < nch && i < n) {
+                load_vec<TX, V>(xb + (size_t)i * C + ch * V, xv[k][i]);
+            } else {
+#pragma unroll
+                for (int v = 0; v < V; v++) xv[k][i][v] = 0.f;
+            }
+        }
+    }
+    float fin[CPT][V];
+    if (inject) {
+#pragma unroll
+        for (int k = 0; k < CPT; k++) {
+            const int ch = tid + k * 256;
+            if (ch < nch) load_vec<TX, V>(static_cast<const TX *>(a.f_inject) + (size_t)b * C + ch * V, fin[k]);
+        }
+    }
+
+    // ---- 2. coefficients on wave 0 -----------------------------------------------------------
+    if (tid < 64) {
+        float pe[SK::EPL], ppre = 0.f, ppost = 0.f, ssq = 0.f;
+#pragma unroll
+        for (int e = 0; e < SK::EPL; e++) pe[e] = 0.f;
+        if (dyn) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                ssq += t_ssq[u]; ppre += t_pre[u]; ppost += t_post[u];
+#pragma unroll
+                for (int e = 0; e < SK::EPL; e++) pe[e] += t_e[u][e];
+            }
+            for (int ks0 = 16 + part * 4; ks0 < a.KS; ks0 += 16) {  // more than 16 K-splits: rare
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int ks = ks0 + u;
+                    if (ks < a.KS) {
+                        ssq += a.ssqpart[(size_t)ks * a.B + b];
+                        if (g < n) { ppre += Pb[ks * ps + g]; ppost += Pb[ks * ps + n + g]; }
+#pragma unroll
+                        for (int e = 0; e < SK::EPL; e++)
+                            if (r0 < n && c0 + e < n) pe[e] += Pb[ks * ps + 2 * n + r0 * n + c0 + e];
+                    }
+                }
+            }
+            ssq += __shfl_xor(ssq, 16, kWave); ssq += __shfl_xor(ssq, 32, kWave);
+            ppre += __shfl_xor(ppre, 16, kWave); ppre += __shfl_xor(ppre, 32, kWave);
+            ppost += __shfl_xor(ppost, 16, kWave); ppost += __shfl_xor(ppost, 32, kWave);
+#pragma unroll
+            for (int e = 0; e < SK::EPL; e++) {
+                pe[e] += __shfl_xor(pe[e], 16, kWave);
+                pe[e] += __shfl_xor(pe[e], 32, kWave);
+            }
+        }
+        if (tid < 16) {
+            float rinv = 0.f;
+            if (dyn) {
+                const float r = sqrtf(ssq / (float)(n * C) + a.eps);
+                rinv = 1.0f / r;
+                if (g == 0) a.r[b] = r;
+            }
+            const bool wr = dyn || b == 0;  // static coefficients are written once
+            const size_t hs = dyn ? (size_t)b * n : 0, ms = dyn ? (size_t)b * n * n : 0;
+            if (g < n) {
+                const float p0 = ppre * rinv, p1 = ppost * rinv;
+                const float hp = sigmoidf_acc(al0 * p0 + bpre);
+                const float ho = 2.0f * sigmoidf_acc(al1 * p1 + bpost);
+                coef_s[NP * NP + g] = hp;
+                coef_s[NP * NP + NP + g] = ho;
+                if (wr && a.Hpre) a.Hpre[hs + g] = hp;
+                if (wr && a.Hpost) a.Hpost[hs + g] = ho;
+                if (dyn) { a.P[(size_t)b * D + g] = p0; a.P[(size_t)b * D + n + g] = p1; }
+            } else if (g < NP) {
+                coef_s[NP * NP + g] = 0.f;
+                coef_s[NP * NP + NP + g] = 0.f;
+            }
+            float m[SK::EPL];
+#pragma unroll
+            for (int e = 0; e < SK::EPL; e++) {
+                const int c = c0 + e;
+                if (r0 < n && c < n) {
+                    const float p = pe[e] * rinv;
+                    if (dyn) a.P[(size_t)b * D + 2 * n + r0 * n + c] = p;
+                    m[e] = expf(al2 * p + bres[e]);
+                } else {
+                    m[e] = 0.f;
+                }
+            }
+            SK::forward(m, g, n, a.T, a.eps, nullptr, tid);
+#pragma unroll
+            for (int e = 0; e < SK::EPL; e++) {
+                const int c = c0 + e;
+                coef_s[r0 * NP + c] = m[e];
+                if (wr && a.M && r0 < n && c < n) a.M[ms + r0 * n + c] = m[e];
+            }
+        }
+    }
+    __syncthreads();
+    float hpre[NP], hpost[NP], Mr[NP][NP];
+#pragma unroll
+    for (int i = 0; i < NP; i++) {
+        hpre[i] = coef_s[NP * NP + i];
+        hpost[i] = coef_s[NP * NP + NP + i];
+#pragma unroll
+        for (int j = 0; j < NP; j++) Mr[i][j] = coef_s[i * NP + j];
+    }
+
+    // ---- 3. aggregate + RMS ------------------------------------------------------------------
+    float av[CPT][V];
+    float qinv = 1.0f;
+    if (!inject) {
+        float ssq = 0.f;
+#pragma unroll
+        for (int k = 0; k < CPT; k++)
+#pragma unroll
+            for (int v = 0; v < V; v++) {
+                float s_a = 0.f;
+#pragma unroll
+                for (int i = 0; i < NP; i++) s_a += hpre[i] * xv[k][i][v];
+                av[k][v] = s_a;
+                ssq += s_a * s_a;
+            }
+        ssq = block_allreduce_sum<256>(ssq, red);
+        const float q = sqrtf(ssq / (float)C + a.eps);
+        qinv = 1.0f / q;
+        if (tid == 0 && a.q) a.q[b] = q;
+    } else if (tid == 0 && a.q) {
+        a.q[b] = 1.0f;
+    }
+
+    // ---- 4. mix + distribute -------------------------------------------------------------------
+#pragma unroll
+    for (int k = 0; k < CPT; k++) {
+        const int ch = tid + k * 256;
+        if (ch < nch) {
+            const int c = ch * V;
+            float f[V];
+#pragma unroll
+            for (int v = 0; v < V; v++)
+                f[v] = inject ? fin[k][v] : av[k][v] * qinv * load_w(a.w, a.w_bf16, c + v);
+#pragma unroll
+            for (int i = 0; i < NP; i++) {
+                if (i < n) {
+                    float out[V];
+#pragma unroll
+                    for (int v = 0; v < V; v++) out[v] = hpost[i] * f[v];
+#pragma unroll
+                    for (int j = 0; j < NP; j++)
+#pragma unroll
+                        for (int v = 0; v < V; v++) out[v] += Mr[i][j] * xv[k][j][v];
+                    store_vec<TY, V>(yb + (size_t)i * C + c, out);
+                }
+            }
+        }
+    }
+}
+
+// Largest CPT instantiated: tiles with more than 4 * 256 vector chunks per stream take the
+// two-kernel path (coefficient kernel + streaming mix kernel).
+template <typename TX, typename TY, int NP>
+static bool launch_fused_small(const LayerFwdArgs &a, hipStream_t stream, hipError_t *err) {
+    constexpr int V = 16 / (int)sizeof(TX);
+    if (a.C % V != 0) return false;
+    const int nch = a.C / V;
+    const int cpt = (nch + 255) / 256;
+    if (cpt == 1) layer_fwd_small_kernel<TX, TY, NP, V, 1><<<a.B, 256, 0, stream>>>(a);
+    else if (cpt == 2) layer_fwd_small_kernel<TX, TY, NP, V, 2><<<a.B, 256, 0, stream>>>(a);
+    else if (cpt <= 4 && NP == 4) layer_fwd_small_kernel<TX, TY, 4, V, 4><<<a.B, 256, 0, stream>>>(a);
+    else return false;
+    *err = hipGetLastError();
+    return true;
+}
+
+bool layer_fwd_fused_supported(int n, int C, int x_dtype) {
+    if (n > 8) return false;
+    const int V = x_dtype == kBF16 ? 8 : 4;
+    if (C % V != 0) return false;
+    const int cpt = (C / V + 255) / 256;
+    return cpt <= 2 || (cpt <= 4 && n <= 4);
+}
+
+hipError_t launch_layer_fwd_fused(const void *x, int x_dtype, const void *w, int w_dtype,
+                                  const void *f_inject, void *y, int y_dtype, const float *Ppart,
+                                  const float *ssqpart, int KS, int DP, const float *alpha,
+                                  const float *b_pre, const float *b_post, const float *b_res,
+                                  float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
+                                  int B, int n, int C, int T, float eps, hipStream_t stream) {
+    LayerFwdArgs a{x, w, f_inject, y, Ppart, ssqpart, alpha, b_pre, b_post, b_res, Hpre, Hpost, M, P, r, q,
+                   KS, DP, w_dtype == kBF16, B, n, C, T, eps};
+    hipError_t err = hipErrorInvalidValue;
+    bool ok = false;
+#define MHC_FUSED(TX, TY)                                                        \
+    ok = n <= 4 ? launch_fused_small<TX, TY, 4>(a, stream, &err) : launch_fused_small<TX, TY, 8>(a, stream, &err)
+    if (x_dtype == kF32 && y_dtype == kF32) MHC_FUSED(float, float);
+    else if (x_dtype == kBF16 && y_dtype == kBF16) MHC_FUSED(bf16_t, bf16_t);
+    else if (x_dtype == kBF16 && y_dtype == kF32) MHC_FUSED(bf16_t, float);
+#undef MHC_FUSED
+    return ok ? err : hipErrorInvalidValue;
 }
 
 template <typename TX, typename TY, int NP, int V>

@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
                                                             float *__restrict__ Ppart,
                                                             float *__restrict__ ssqpart, int B,
                                                             int D, int DP, int nC, int tiles_s,
-                                                            int sub /* K per wave, multiple of 16 */) {
+                                                            int sub /* K per wave, multiple of 64 */) {
     extern __shared__ float lds[];  // [3][NT*16 + 1][64]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int st = blockIdx.x % tiles_s, ks = blockIdx.x / tiles_s;
@@ -110,7 +110,9 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
         uint4 av[U], bv[U][NT];
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int k = k0 + u * 16 + kh * 8;
+            // each lane walks 8*U contiguous elements per outer step (one 64-byte segment of a
+            // 128-byte line for U = 4); A and B use the same k grouping, which is all MFMA needs
+            const int k = k0 + kh * (8 * U) + u * 8;
             const bool kv = k < kend;  // kend and k are multiples of 8
             av[u] = (kv && bvalid) ? xrow[k >> 3] : zero4;
 #pragma unroll
@@ -211,7 +213,7 @@ static hipError_t launch_mfma(const void *x, const void *phi, float *Ppart, floa
                               int B, int D, int DP, int nC, hipStream_t stream) {
     const int tiles_s = (B + 31) / 32;
     const int groups = (DP / 32 + NT - 1) / NT;
-    const int sub = round_up((nC + KS * 4 - 1) / (KS * 4), 16);
+    const int sub = round_up((nC + KS * 4 - 1) / (KS * 4), 64);  // whole 128-byte lines per lane pair
     dim3 grid(tiles_s * KS, groups);
     const size_t smem = sizeof(float) * 3 * (NT * 16 + 1) * 64;
     proj_fwd_mfma_kernel<NT><<<grid, 256, smem, stream>>>(static_cast<const bf16_t *>(x),

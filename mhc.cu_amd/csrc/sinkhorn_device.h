@@ -58,7 +58,7 @@ template <int NP> struct SkSmall {
             for (int e = 0; e < EPL; e++) rs += m[e];
             rs = row_allreduce(rs) + eps;
             rs = rv ? rs : 1.0f;
-            const float rinv = 1.0f / rs;
+            const float rinv = fast_rcp(rs);
             if (sc) sc[(t * (1 + EPL)) * kWave + lane] = rs;
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
@@ -66,7 +66,7 @@ template <int NP> struct SkSmall {
                 float cs = col_allreduce(m[e]) + eps;
                 cs = cv[e] ? cs : 1.0f;
                 if (sc) sc[(t * (1 + EPL) + 1 + e) * kWave + lane] = cs;
-                m[e] *= 1.0f / cs;
+                m[e] *= fast_rcp(cs);
             }
         }
     }
@@ -82,14 +82,15 @@ template <int NP> struct SkSmall {
             for (int e = 0; e < EPL; e++) {
                 const float cs = sc[(t * (1 + EPL) + 1 + e) * kWave + lane];
                 const float cdot = col_allreduce(d[e] * m[e]);
-                dR[e] = (d[e] - cdot) / cs;
+                dR[e] = (d[e] - cdot) * fast_rcp(cs);
                 m[e] *= cs;  // row-normalised iterate R_t
                 rdot += dR[e] * m[e];
             }
             rdot = row_allreduce(rdot);
+            const float rinv = fast_rcp(rs);
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
-                d[e] = (dR[e] - rdot) / rs;
+                d[e] = (dR[e] - rdot) * rinv;
                 m[e] *= rs;  // iterate before row step t
             }
         }
