@@ -49,7 +49,7 @@ int ws_check(void *ws, size_t have, size_t need) {
 
 // ---- dynamic workspace layout ----------------------------------------------------------------
 struct DynFwdWs { float *Ppart, *ssqpart; size_t bytes; };
-struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *cs_dt, *cs_u, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
+struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
 
 int max_ksplit(int B, int n, int C) { return proj_fwd_ksplit(kBF16, kBF16, B, n, C); }
 
@@ -72,8 +72,7 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
     w.cx = c.floats(B);
     w.s1 = c.floats(B);
     w.u = c.floats((size_t)B * C);
-    w.cs_dt = c.floats(colsum_workspace_floats(B, D + 3));
-    w.cs_u = c.floats(colsum_workspace_floats(B, C));
+    w.dtpart = c.floats((size_t)B * (D + 3));
     int bs = dphi_batch_splits(B, n, C);
     const int bs2 = proj_bwd_batch_splits(B, n, C);
     if (bs2 > bs) bs = bs2;
@@ -198,20 +197,24 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     BwdCoefOut out{ws.dt, ws.dP, ws.cx, ws.s1, nullptr, mfma ? ws.dPb : nullptr, ws.dPT, ws.BP};
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      n, q, P, r, alpha, bias + 2 * n, out, B, n, C, iters, eps, st));
+    const int spg = bwd_dx_samples_per_group(B, n);
+    const int groups = (B + spg - 1) / spg;
+    int S = 1;
     if (mfma) {
         // matrix cores: dphi and the projection term of dx (written into dx, then completed in place)
+        S = proj_bwd_batch_splits(B, n, C);
         MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st));
         MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
-                                     n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, B, n,
-                                     C, st));
+                                     n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, ws.dt,
+                                     ws.dtpart, spg, B, n, C, st));
     } else {
         MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      n, q, ws.s1, ws.cx, ws.dP, DP, phi, phi_dtype, nullptr, dx, df,
-                                     ws.u, B, n, C, st));
+                                     ws.u, ws.dt, ws.dtpart, spg, B, n, C, st));
         MHC_LAUNCH(launch_dphi(x, x_dtype, ws.dP, DP, dphi, B, n, C, ws.dphi_part, st));
     }
-    MHC_LAUNCH(launch_colsum_split(ws.dt, B, D + 3, D + 3, dbias, dalpha, D, ws.cs_dt, st));
-    if (!f_inject) MHC_LAUNCH(launch_colsum(ws.u, B, C, C, dw, ws.cs_u, st));
+    MHC_LAUNCH(launch_finalize(ws.u, groups, C, f_inject ? nullptr : dw, ws.dtpart, groups, D, dbias,
+                               dalpha, ws.dphi_part, S, (size_t)D * n * C, dphi, st));
     return MHC_OK;
 }
 
@@ -280,8 +283,8 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
                                      0, q, nullptr, nullptr, nullptr, nullptr, out, B, n, C, iters,
                                      eps, st));
     MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, 0,
-                                 q, ws.s1, nullptr, nullptr, 0, nullptr, 0, nullptr, dx, df, ws.u, B, n, C,
-                                 st));
+                                 q, ws.s1, nullptr, nullptr, 0, nullptr, 0, nullptr, dx, df, ws.u, nullptr,
+                                 nullptr, 1, B, n, C, st));
     MHC_LAUNCH(launch_colsum(ws.red, B, D, D, ws.red_sum, ws.cs_red, st));
     MHC_LAUNCH(launch_coef_bwd_static(ws.red_sum, H_pre, H_post, H_res_logits, dH_pre, dH_post,
                                       dH_res, n, iters, eps, st));

@@ -79,11 +79,21 @@ hipError_t launch_mix_bwd_dx(const void *dy, int y_dtype, const void *x, int x_d
                              const float *Hpost, const float *M, int hstride, const float *q,
                              const float *s1, const float *cx, const float *dP, int DP,
                              const void *phi, int phi_dtype, const void *dx_in, void *dx, void *df,
-                             float *u, int B, int n, int C, hipStream_t stream);
+                             float *u, const float *dt, float *dtpart, int spg, int B, int n, int C,
+                             hipStream_t stream);
+
+// Samples per workgroup of launch_mix_bwd_dx and the resulting row count of u / dtpart.
+int bwd_dx_samples_per_group(int B, int n);
+
+// One launch for all remaining batch sums: u [rows_u, C] -> dw (skipped when dw == nullptr),
+// dt [rows_dt, D+3] -> dbias, dalpha, and (S > 1) dphi_part [S, dphi_elems] -> dphi.
+hipError_t launch_finalize(const float *u, int rows_u, int C, float *dw, const float *dt, int rows_dt,
+                           int D, float *dbias, float *dalpha, const float *dphi_part, int S,
+                           size_t dphi_elems, float *dphi, hipStream_t stream);
 
 // Matrix-core projection backward (x and phi bf16, C % 8 == 0): dphi = dP^T x_flat and
-// dxflat = dP phi (bf16 [B, nC]) in one pass over x and phi.  dphi_part: proj_bwd_batch_splits()
-// copies of dphi when that is > 1.
+// dxflat = dP phi (bf16 [B, nC]) in one pass over x and phi.  With S = proj_bwd_batch_splits() > 1
+// the S partial copies land in dphi_part and the caller's finalize launch sums them.
 bool proj_bwd_mfma_supported(int x_dtype, int phi_dtype, int C);
 int proj_bwd_batch_splits(int B, int n, int C);
 hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,

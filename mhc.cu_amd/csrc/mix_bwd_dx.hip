@@ -16,8 +16,10 @@ struct BwdDxArgs {
     const void *dy, *x, *w, *f_inject, *phi, *dx_in;
     const float *Hpre, *Hpost, *M, *q, *s1, *cx, *dP;
     void *dx, *df;
-    float *u;
-    int hstride, w_bf16, phi_bf16, B, n, C, DP;
+    float *u;            // [G, C] per-group sums of df a / q (the summands of dw)
+    const float *dt;     // [B, D+3] per-sample logit gradients (dynamic) or nullptr
+    float *dtpart;       // [G, D+3] per-group sums of dt
+    int hstride, w_bf16, phi_bf16, B, n, C, DP, spg;  // spg = samples per workgroup
 };
 
 __device__ __forceinline__ float load_w2(const void *w, int w_bf16, int c) {
@@ -28,36 +30,41 @@ template <typename TG, typename TX, int NP, int V>
 __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
     extern __shared__ float smem[];
     float *M_s = smem;  // [NP*NP] (NP >= 16 only)
-    const int b = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x, nt = blockDim.x;
-    const TG *__restrict__ gb = static_cast<const TG *>(a.dy) + (size_t)b * n * C;
-    const TX *__restrict__ xb = static_cast<const TX *>(a.x) + (size_t)b * n * C;
-    TX *__restrict__ dxb = static_cast<TX *>(a.dx) + (size_t)b * n * C;
-    const float *__restrict__ Hpre = a.Hpre + (size_t)b * a.hstride;
-    const float *__restrict__ Hpost = a.Hpost + (size_t)b * a.hstride;
-    const float *__restrict__ M = a.M + (size_t)b * a.hstride * n;
+    const int grp = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x, nt = blockDim.x;
+    const int b_first = grp * a.spg, b_last = min(a.B, b_first + a.spg);
     const bool inject = a.f_inject != nullptr;
-    const float qinv = inject ? 0.f : 1.0f / a.q[b];
-    const float k2 = inject ? 0.f : a.s1[b] * qinv * qinv * qinv / (float)C;
-    const float cx = a.cx ? a.cx[b] : 0.f;
     const int D = n * n + 2 * n, nC = n * C;
-
-    float hpre[NP], hpost[NP];
-#pragma unroll
-    for (int i = 0; i < NP; i++) {
-        hpre[i] = i < n ? Hpre[i] : 0.f;
-        hpost[i] = i < n ? Hpost[i] : 0.f;
-    }
     if constexpr (NP >= 16) {
+        // one sample per workgroup on this path (spg == 1): stage its M once, for all threads
+        const float *M0 = a.M + (size_t)b_first * a.hstride * n;
         for (int e = tid; e < NP * NP; e += nt) {
             const int i = e / NP, j = e % NP;
-            M_s[e] = (i < n && j < n) ? M[i * n + j] : 0.f;
+            M_s[e] = (i < n && j < n) ? M0[i * n + j] : 0.f;
         }
         __syncthreads();
     }
-
     const int nch = C / V;
     for (int ch = tid; ch < nch; ch += nt) {
-        const int c = ch * V;
+      const int c = ch * V;
+      float usum[V];
+#pragma unroll
+      for (int v = 0; v < V; v++) usum[v] = 0.f;
+      for (int b = b_first; b < b_last; b++) {
+        const TG *__restrict__ gb = static_cast<const TG *>(a.dy) + (size_t)b * n * C;
+        const TX *__restrict__ xb = static_cast<const TX *>(a.x) + (size_t)b * n * C;
+        TX *__restrict__ dxb = static_cast<TX *>(a.dx) + (size_t)b * n * C;
+        const float *__restrict__ Hpre = a.Hpre + (size_t)b * a.hstride;
+        const float *__restrict__ Hpost = a.Hpost + (size_t)b * a.hstride;
+        const float *__restrict__ M = a.M + (size_t)b * a.hstride * n;
+        const float qinv = inject ? 0.f : 1.0f / a.q[b];
+        const float k2 = inject ? 0.f : a.s1[b] * qinv * qinv * qinv / (float)C;
+        const float cx = a.cx ? a.cx[b] : 0.f;
+        float hpre[NP], hpost[NP];
+#pragma unroll
+        for (int i = 0; i < NP; i++) {
+            hpre[i] = i < n ? Hpre[i] : 0.f;
+            hpost[i] = i < n ? Hpost[i] : 0.f;
+        }
         float gv[NP][V], xv[NP][V];
 #pragma unroll
         for (int i = 0; i < NP; i++) {
@@ -85,8 +92,9 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
         }
         if (inject) {
             if (a.df) store_vec<TX, V>(static_cast<TX *>(a.df) + (size_t)b * C + c, dfv);
-        } else if (a.u) {
-            store_vec<float, V>(a.u + (size_t)b * C + c, uv);
+        } else {
+#pragma unroll
+            for (int v = 0; v < V; v++) usum[v] += uv[v];
         }
 #pragma unroll
         for (int j = 0; j < NP; j++) {
@@ -124,6 +132,16 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
                 store_vec<TX, V>(dxb + (size_t)j * C + c, out);
             }
         }
+      }
+      if (!inject && a.u) store_vec<float, V>(a.u + (size_t)grp * C + c, usum);
+    }
+    // per-group sums of the logit gradients (feeds dbias / dalpha)
+    if (a.dtpart) {
+        for (int col = tid; col < D + 3; col += nt) {
+            float acc = 0.f;
+            for (int b = b_first; b < b_last; b++) acc += a.dt[(size_t)b * (D + 3) + col];
+            a.dtpart[(size_t)grp * (D + 3) + col] = acc;
+        }
     }
 }
 
@@ -133,7 +151,8 @@ static hipError_t launch_one(const BwdDxArgs &a, hipStream_t stream) {
     int nt = (nch + 63) / 64 * 64;
     if (nt > 256) nt = 256;
     const size_t smem = sizeof(float) * (NP >= 16 ? NP * NP : 1);
-    mix_bwd_dx_kernel<TG, TX, NP, V><<<a.B, nt, smem, stream>>>(a);
+    const int groups = (a.B + a.spg - 1) / a.spg;
+    mix_bwd_dx_kernel<TG, TX, NP, V><<<groups, nt, smem, stream>>>(a);
     return hipGetLastError();
 }
 
@@ -154,14 +173,24 @@ static hipError_t launch_t(const BwdDxArgs &a, hipStream_t stream) {
     return launch_np<TG, TX, 32>(a, stream);
 }
 
+int bwd_dx_samples_per_group(int B, int n) {
+    if (n > 8) return 1;
+    int spg = B / 2048;
+    if (spg < 1) spg = 1;
+    if (spg > 16) spg = 16;
+    return spg;
+}
+
 hipError_t launch_mix_bwd_dx(const void *dy, int y_dtype, const void *x, int x_dtype, const void *w,
                              int w_dtype, const void *f_inject, const float *Hpre,
                              const float *Hpost, const float *M, int hstride, const float *q,
                              const float *s1, const float *cx, const float *dP, int DP,
                              const void *phi, int phi_dtype, const void *dx_in, void *dx, void *df,
-                             float *u, int B, int n, int C, hipStream_t stream) {
-    BwdDxArgs a{dy, x, w, f_inject, phi, dx_in, Hpre, Hpost, M, q, s1, cx, dP, dx, df, u,
-                hstride, w_dtype == kBF16, phi_dtype == kBF16, B, n, C, DP};
+                             float *u, const float *dt, float *dtpart, int spg, int B, int n, int C,
+                             hipStream_t stream) {
+    if (n > 8) spg = 1;  // the large-n layout stages one sample's M in LDS per workgroup
+    BwdDxArgs a{dy, x, w, f_inject, phi, dx_in, Hpre, Hpost, M, q, s1, cx, dP, dx, df, u, dt, dtpart,
+                hstride, w_dtype == kBF16, phi_dtype == kBF16, B, n, C, DP, spg};
     if (y_dtype == kF32 && x_dtype == kF32) return launch_t<float, float>(a, stream);
     if (y_dtype == kBF16 && x_dtype == kBF16) return launch_t<bf16_t, bf16_t>(a, stream);
     if (y_dtype == kF32 && x_dtype == kBF16) return launch_t<float, bf16_t>(a, stream);

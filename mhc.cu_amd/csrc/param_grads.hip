@@ -132,6 +132,78 @@ hipError_t launch_dphi(const void *x, int x_dtype, const float *dP, int DP, floa
     return hipGetLastError();
 }
 
+
+// --------------------------------------------------------------------------------------------
+// finalize: every remaining batch reduction of the dynamic backward in ONE launch.
+//   blocks [0, nblk_a): 64 columns x 16 row groups of the virtual matrix [u | dt]
+//       u  [rows_u,  C]    -> dw[C]
+//       dt [rows_dt, D+3]  -> dbias[D], dalpha[3]
+//   blocks [nblk_a, ...): 1024 columns each of the dphi batch-split partials [S, D*nC] -> dphi
+// --------------------------------------------------------------------------------------------
+struct FinalizeArgs {
+    const float *u; int rows_u, C; float *dw;
+    const float *dt; int rows_dt, D; float *dbias, *dalpha;
+    const float *dphi_part; int S; size_t dphi_elems; float *dphi;
+    int nblk_a;
+};
+
+__global__ __launch_bounds__(1024) void finalize_kernel(FinalizeArgs a) {
+    __shared__ float red[16][65];
+    const int tid = threadIdx.x;
+    if ((int)blockIdx.x < a.nblk_a) {
+        const int cl = tid & 63, rg = tid >> 6;
+        const int col = blockIdx.x * 64 + cl;
+        const int ncol_u = a.dw ? a.C : 0;
+        const int ncols = ncol_u + a.D + 3;
+        float acc = 0.f;
+        if (col < ncols) {
+            const bool is_u = col < ncol_u;
+            const float *src = is_u ? a.u + col : a.dt + (col - ncol_u);
+            const int ld = is_u ? a.C : a.D + 3;
+            const int rows = is_u ? a.rows_u : a.rows_dt;
+            float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+            int r = rg;
+            for (; r + 48 < rows; r += 64) {
+                a0 += src[(size_t)r * ld];
+                a1 += src[(size_t)(r + 16) * ld];
+                a2 += src[(size_t)(r + 32) * ld];
+                a3 += src[(size_t)(r + 48) * ld];
+            }
+            for (; r < rows; r += 16) a0 += src[(size_t)r * ld];
+            acc = (a0 + a1) + (a2 + a3);
+        }
+        red[rg][cl] = acc;
+        __syncthreads();
+        if (rg == 0 && col < ncols) {
+            float v = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) v += red[i][cl];
+            if (col < ncol_u) a.dw[col] = v;
+            else if (col - ncol_u < a.D) a.dbias[col - ncol_u] = v;
+            else a.dalpha[col - ncol_u - a.D] = v;
+        }
+        return;
+    }
+    // dphi partial sums: one float per thread per 1024-column block (coalesced)
+    const size_t e = (size_t)(blockIdx.x - a.nblk_a) * 1024 + tid;
+    if (e < a.dphi_elems) {
+        float v = 0.f;
+        for (int s = 0; s < a.S; s++) v += a.dphi_part[(size_t)s * a.dphi_elems + e];
+        a.dphi[e] = v;
+    }
+}
+
+hipError_t launch_finalize(const float *u, int rows_u, int C, float *dw, const float *dt, int rows_dt,
+                           int D, float *dbias, float *dalpha, const float *dphi_part, int S,
+                           size_t dphi_elems, float *dphi, hipStream_t stream) {
+    const int ncols = (dw ? C : 0) + D + 3;
+    const int nblk_a = (ncols + 63) / 64;
+    const int nblk_b = S > 1 ? (int)((dphi_elems + 1023) / 1024) : 0;
+    FinalizeArgs a{u, rows_u, C, dw, dt, rows_dt, D, dbias, dalpha, dphi_part, S, dphi_elems, dphi, nblk_a};
+    finalize_kernel<<<nblk_a + nblk_b, 1024, 0, stream>>>(a);
+    return hipGetLastError();
+}
+
 // --------------------------------------------------------------------------------------------
 // static H: coefficient backward on the batch-summed raw gradients (one wave)
 //   red_sum = (dM [n*n] | dHpre [n] | dHpost [n])

@@ -227,8 +227,7 @@ hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb,
     if (NTD <= 4) e = launch_shape<1, 1, true>(a, S, stream);
     else if (NTD <= 12) e = launch_shape<1, 3, false>(a, S, stream);
     else e = launch_shape<1, 9, false>(a, S, stream);
-    if (e != hipSuccess || S == 1) return e;
-    return launch_colsum(dphi_part, S, D * nC, D * nC, dphi, nullptr, stream);
+    return e;  // with S > 1 the caller's finalize launch sums the S partial copies
 }
 
 }  // namespace mhc
