@@ -1,0 +1,136 @@
+"""The reference's own Python tests for the layer (src/python/tests/test_layer.py:53-340),
+restated against this package: same shapes, same assertions, plus the numeric parity the
+reference only checks at 5e-2."""
+import pytest
+import torch
+
+from helpers import rel_err
+from oracle import naive_mhc as nm
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_layer_forward(dynamic):
+    from mhc import MHCLayer
+    B, n, C = 8, 4, 128
+    layer = MHCLayer(hidden_dim=C, expansion_rate=n, use_dynamic_h=dynamic).cuda()
+    x = torch.randn(B, n, C, device="cuda")
+    out = layer(x)
+    assert out.shape == (B, n, C) and out.dtype == torch.float32
+    assert not torch.isnan(out).any() and not torch.isinf(out).any()
+
+
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_layer_backward_all_params_get_gradients(dynamic):
+    from mhc import MHCLayer
+    B, n, C = 4, 4, 64
+    layer = MHCLayer(hidden_dim=C, expansion_rate=n, use_dynamic_h=dynamic).cuda()
+    x = (torch.randn(B, n, C, device="cuda") + 0.1).requires_grad_(True)
+    layer(x).sum().backward()
+    assert x.grad is not None and not torch.isnan(x.grad).any()
+    for name, p in layer.named_parameters():
+        assert p.grad is not None, f"{name} has no gradient"
+        assert p.grad.dtype == p.dtype and p.grad.shape == p.shape
+        assert not torch.isnan(p.grad).any(), f"{name} has NaN gradient"
+        if dynamic and name != "rmsnorm_weight":
+            assert p.grad.abs().sum() > 0, f"{name} gradient is zero"
+
+
+def test_layer_dynamic_matches_naive_small():
+    """test_layer.py:145-193 at its own shape (B=2, n=4, C=16, 3 iterations), but at 1e-5."""
+    from mhc import MHCLayer
+    B, n, C = 2, 4, 16
+    torch.manual_seed(42)
+    layer = MHCLayer(hidden_dim=C, expansion_rate=n, sinkhorn_iters=3, use_dynamic_h=True).cuda()
+    x = torch.randn(B, n, C, device="cuda", requires_grad=True)
+    dy = torch.randn(B, n, C, device="cuda")
+    out = layer(x)
+    # (the reference test uses out.sum(); under that loss the true phi_res gradient is ~0 because
+    # the Sinkhorn output's column sums are constant, so a random upstream gradient is used here)
+    out.backward(dy)
+    p = {k: getattr(layer, k).detach().cpu().float() for k in nm.DYN_PARAM_NAMES if k != "w"}
+    p["w"] = layer.rmsnorm_weight.detach().cpu().float()
+    y_ref, g_ref = nm.mhc_dynamic_fwd_bwd(x.detach().cpu(), p, dy.cpu(), 3, layer.eps, dtype=torch.float64)
+    assert rel_err(out, y_ref) < 1e-5
+    assert rel_err(x.grad, g_ref["x"]) < 1e-5
+    assert rel_err(layer.phi_res.grad, g_ref["phi_res"]) < 1e-5
+    # and the reference's own assertion, at its tolerance, under its loss
+    layer.zero_grad()
+    x2 = x.detach().clone().requires_grad_(True)
+    layer(x2).sum().backward()
+    _, g_sum = nm.mhc_dynamic_fwd_bwd(x.detach().cpu(), p, torch.ones(B, n, C), 3, layer.eps, dtype=torch.float64)
+    torch.testing.assert_close(x2.grad.cpu().double(), g_sum["x"], rtol=1e-1, atol=1e-1)
+    torch.testing.assert_close(layer.phi_res.grad.cpu().double(), g_sum["phi_res"], rtol=1e-1, atol=1e-1)
+
+
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_training_steps_and_batch_sizes(dynamic):
+    from mhc import MHCLayer
+    n, C = 4, 128
+    layer = MHCLayer(hidden_dim=C, expansion_rate=n, use_dynamic_h=dynamic).cuda()
+    opt = torch.optim.Adam(layer.parameters(), lr=1e-3)
+    x, target = torch.randn(8, n, C, device="cuda"), torch.randn(8, n, C, device="cuda")
+    losses = []
+    for _ in range(3):
+        opt.zero_grad()
+        loss = ((layer(x) - target) ** 2).mean()
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert all(l == l for l in losses) and losses[-1] < losses[0]
+    for B in [1, 4, 16, 32]:
+        assert layer(torch.randn(B, n, C, device="cuda")).shape == (B, n, C)
+
+
+def test_numerical_stability_and_determinism():
+    from mhc import MHCLayer
+    B, n, C = 8, 4, 128
+    for dynamic in (False, True):
+        layer = MHCLayer(hidden_dim=C, expansion_rate=n, use_dynamic_h=dynamic).cuda()
+        for scale in (100.0, 0.001):
+            out = layer(torch.randn(B, n, C, device="cuda") * scale)
+            assert not torch.isnan(out).any() and not torch.isinf(out).any()
+        x = torch.randn(B, n, C, device="cuda")
+        assert torch.equal(layer(x), layer(x))
+
+
+def test_static_inference_path_matches_training_path():
+    from mhc import MHCLayer
+    B, n, C = 8, 4, 128
+    layer = MHCLayer(hidden_dim=C, expansion_rate=n, use_dynamic_h=False).cuda()
+    with torch.no_grad():
+        layer.H_res.copy_(torch.randn(n, n))
+        layer.H_pre.copy_(torch.randn(n))
+    x = torch.randn(B, n, C, device="cuda")
+    y_train = layer(x)
+    layer.eval()
+    with torch.no_grad():
+        y_inf = layer(x)
+    assert torch.equal(y_train, y_inf)
+
+
+def test_bf16_input_and_output_dtype_option():
+    from mhc import MHCLayer
+    B, n, C = 8, 4, 128
+    layer = MHCLayer(hidden_dim=C, expansion_rate=n).cuda()
+    x = torch.randn(B, n, C, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    y = layer(x)
+    assert y.dtype == torch.float32          # the reference's contract
+    y.sum().backward()
+    assert x.grad.dtype == torch.bfloat16
+    layer2 = MHCLayer(hidden_dim=C, expansion_rate=n, output_dtype=torch.bfloat16).cuda()
+    assert layer2(x.detach()).dtype == torch.bfloat16
+
+
+def test_phi_cache_follows_parameter_updates():
+    """The concatenated phi is cached between calls and must be rebuilt after an in-place update."""
+    from mhc import MHCLayer
+    B, n, C = 4, 4, 64
+    layer = MHCLayer(hidden_dim=C, expansion_rate=n, alpha_init=1.0).cuda()
+    x = torch.randn(B, n, C, device="cuda")
+    y0 = layer(x).detach().clone()
+    with torch.no_grad():
+        layer.phi_res.mul_(-3.0)
+    y1 = layer(x).detach()
+    assert (y0 - y1).abs().max() > 1e-4
