@@ -49,7 +49,7 @@ int ws_check(void *ws, size_t have, size_t need) {
 
 // ---- dynamic workspace layout ----------------------------------------------------------------
 struct DynFwdWs { float *Ppart, *ssqpart; size_t bytes; };
-struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
+struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *raw, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
 
 int max_ksplit(int B, int n, int C) { return proj_fwd_ksplit(kBF16, kBF16, B, n, C); }
 
@@ -73,9 +73,12 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
     w.s1 = c.floats(B);
     w.u = c.floats((size_t)B * C);
     w.dtpart = c.floats((size_t)B * (D + 3));
+    w.raw = c.floats(n <= 8 ? (size_t)B * bwd_reduce_parts(B, n, C) * (8 * 8 + 3 * 8 + 1) : 0);
     int bs = dphi_batch_splits(B, n, C);
     const int bs2 = proj_bwd_batch_splits(B, n, C);
     if (bs2 > bs) bs = bs2;
+    const int bs3 = n <= 4 ? bwd_slab_batch_splits(B, n, C) : 1;
+    if (bs3 > bs) bs = bs3;
     w.dphi_part = c.floats(bs > 1 ? (size_t)bs * D * nC : 0);
     w.BP = (B + 31) / 32 * 32;
     w.dPb = reinterpret_cast<unsigned short *>(c.floats(((size_t)B * padded_D(n) + 1) / 2));
@@ -196,7 +199,17 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     const bool mfma = proj_bwd_mfma_supported(x_dtype, phi_dtype, C);
     BwdCoefOut out{ws.dt, ws.dP, ws.cx, ws.s1, nullptr, mfma ? ws.dPb : nullptr, ws.dPT, ws.BP};
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
-                                     n, q, P, r, alpha, bias + 2 * n, out, B, n, C, iters, eps, st));
+                                     n, q, P, r, alpha, bias + 2 * n, out, ws.raw, B, n, C, iters, eps, st));
+    if (mfma && bwd_slab_supported(x_dtype, y_dtype, phi_dtype, n, C)) {
+        // n <= 4: one slab kernel finishes dx and produces every batch-split partial sum
+        const int S = bwd_slab_batch_splits(B, n, C);
+        MHC_LAUNCH(launch_bwd_slab(dy, y_dtype, x, w, w_dtype, f_inject, phi, H_pre, H_post, M, q, ws.s1,
+                                   ws.cx, ws.dPb, ws.dPT, ws.BP, ws.dt, dx, df,
+                                   S > 1 ? ws.dphi_part : dphi, ws.u, ws.dtpart, S, B, n, C, st));
+        MHC_LAUNCH(launch_finalize(ws.u, S, C, f_inject ? nullptr : dw, ws.dtpart, S, D, dbias, dalpha,
+                                   ws.dphi_part, S, (size_t)D * n * C, dphi, st));
+        return MHC_OK;
+    }
     const int spg = bwd_dx_samples_per_group(B, n);
     const int groups = (B + spg - 1) / spg;
     int S = 1;
@@ -280,8 +293,8 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
     const int D = n * n + 2 * n;
     BwdCoefOut out{nullptr, nullptr, nullptr, ws.s1, ws.red, nullptr, nullptr, 0};
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
-                                     0, q, nullptr, nullptr, nullptr, nullptr, out, B, n, C, iters,
-                                     eps, st));
+                                     0, q, nullptr, nullptr, nullptr, nullptr, out, nullptr, B, n, C,
+                                     iters, eps, st));
     MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, 0,
                                  q, ws.s1, nullptr, nullptr, 0, nullptr, 0, nullptr, dx, df, ws.u, nullptr,
                                  nullptr, 1, B, n, C, st));

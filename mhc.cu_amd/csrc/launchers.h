@@ -69,8 +69,11 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
                                  const void *w, int w_dtype, const void *f_inject,
                                  const float *Hpre, const float *Hpost, const float *M, int hstride,
                                  const float *q, const float *P, const float *r, const float *alpha,
-                                 const float *b_res, BwdCoefOut out, int B, int n, int C, int T,
-                                 float eps, hipStream_t stream);
+                                 const float *b_res, BwdCoefOut out, float *raw, int B, int n, int C,
+                                 int T, float eps, hipStream_t stream);
+// raw (optional, dynamic H, n <= 8): scratch of B * bwd_reduce_parts() * (NP*NP + 3*NP + 1) floats;
+// when given, the channel sums and the coefficient backward run as two launches.
+int bwd_reduce_parts(int B, int n, int C);
 
 // dx = M^T dy + Hpre (x) da - cx * x  [+ dP phi when phi != nullptr] [+ dx_in when != nullptr;
 // may alias dx], df, and u = df * a / q (the per-sample summand of dw).
@@ -81,6 +84,18 @@ hipError_t launch_mix_bwd_dx(const void *dy, int y_dtype, const void *x, int x_d
                              const void *phi, int phi_dtype, const void *dx_in, void *dx, void *df,
                              float *u, const float *dt, float *dtpart, int spg, int B, int n, int C,
                              hipStream_t stream);
+
+// Slab kernel for n <= 4 in the bf16 tier: dx (complete), df, and the batch-split partial sums of
+// dphi [S][D][nC], dw [S][C] and dt [S][D+3] in one pass over dy and x.  With S == 1 pass the final
+// dphi as dphi_part.
+bool bwd_slab_supported(int x_dtype, int y_dtype, int phi_dtype, int n, int C);
+int bwd_slab_batch_splits(int B, int n, int C);
+hipError_t launch_bwd_slab(const void *dy, int y_dtype, const void *x, const void *w, int w_dtype,
+                           const void *f_inject, const void *phi, const float *Hpre,
+                           const float *Hpost, const float *M, const float *q, const float *s1,
+                           const float *cx, const void *dPb, const void *dPT, int BP, const float *dt,
+                           void *dx, void *df, float *dphi_part, float *dw_part, float *dt_part, int S,
+                           int B, int n, int C, hipStream_t stream);
 
 // Samples per workgroup of launch_mix_bwd_dx and the resulting row count of u / dtpart.
 int bwd_dx_samples_per_group(int B, int n);

@@ -124,9 +124,10 @@ constexpr int kDppQuadXor2 = 0x4E;   // quad_perm:[2,3,0,1]
 constexpr int kDppRowRor4 = 0x124;
 constexpr int kDppRowRor8 = 0x128;
 
+// All controls used here read a valid lane for every lane, so `old` is irrelevant; passing 0 with
+// bound_ctrl lets the compiler fold the move into the consuming VALU instruction (v_add_f32_dpp).
 template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
-    int iv = __float_as_int(v);
-    return __int_as_float(__builtin_amdgcn_update_dpp(iv, iv, CTRL, 0xF, 0xF, false));
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
 
 // Sum over all 64 lanes; every lane gets the total.

@@ -28,6 +28,8 @@ struct BwdReduceArgs {
     BwdCoefOut out;
     int hstride, w_bf16, B, n, C, T, DP;
     float eps;
+    float *raw;   // n <= 8: when set, write the raw channel sums [B][parts][K] and stop
+    int parts;    // column parts per sample (gridDim.y)
 };
 
 __device__ __forceinline__ float load_w_(const void *w, int w_bf16, int c) {
@@ -91,8 +93,8 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
     using SK = SkSmall<NP>;
     constexpr int K = NP * NP + 3 * NP + 1;  // dM | dHpost | A1 | A2 | s1
     extern __shared__ float smem[];
-    float *part = smem;            // [K][16]  one slot per 16-lane row of the workgroup
-    float *tot = part + K * 16;    // [K]
+    float *slot_s = smem;          // [K][16]  one slot per 16-lane row of the workgroup
+    float *tot = slot_s + K * 16;  // [K]
     float *sc = tot + K;           // Sinkhorn denominators, SK::scaling_floats(T)
     const int b = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x, nt = blockDim.x;
     const TG *__restrict__ gb = static_cast<const TG *>(a.dy) + (size_t)b * n * C;
@@ -113,7 +115,9 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
     for (int k = 0; k < K; k++) acc[k] = 0.f;
 
     const int nch = C / V;
-    for (int ch = tid; ch < nch; ch += nt) {
+    const int part = blockIdx.y, cpp = (nch + a.parts - 1) / a.parts;  // chunks per part
+    const int ch_end = min(nch, (part + 1) * cpp);
+    for (int ch = part * cpp + tid; ch < ch_end; ch += nt) {
         const int c = ch * V;
         float gv[NP][V], xv[NP][V];
 #pragma unroll
@@ -163,14 +167,16 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
 #pragma unroll
     for (int k = 0; k < K; k++) {
         const float v = row16_allreduce(acc[k]);
-        if ((tid & 15) == 0) part[k * 16 + slot] = v;
+        if ((tid & 15) == 0) slot_s[k * 16 + slot] = v;
     }
     __syncthreads();
     for (int k = tid; k < K; k += nt) {
         float v = 0.f;
-        for (int s = 0; s < nslots; s++) v += part[k * 16 + s];
+        for (int s = 0; s < nslots; s++) v += slot_s[k * 16 + s];
         tot[k] = v;
+        if (a.raw) a.raw[((size_t)b * a.parts + blockIdx.y) * K + k] = v;
     }
+    if (a.raw) return;  // the coefficient backward runs as its own small launch
     __syncthreads();
     if (tid >= 16) return;
 
@@ -219,8 +225,8 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
         m[e] = E[e];
         d[e] = ok ? tot[r0 * NP + c] : 0.f;
     }
-    SK::forward(m, g, n, a.T, a.eps, sc, tid);
-    SK::backward(m, d, a.T, sc, tid);
+    SK::template forward<false>(m, g, n, a.T, a.eps, sc, tid);
+    SK::template backward<false>(d, a.T, sc, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;
@@ -230,6 +236,92 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
             dt[di] = dtr;
             dpw.put(di, dtr * al2 * rinv);
             S2 += dtr * Pb[di];
+        }
+    }
+    S0 = row16_allreduce(S0); S1 = row16_allreduce(S1); S2 = row16_allreduce(S2);
+    if (g == 0) {
+        dt[D] = S0; dt[D + 1] = S1; dt[D + 2] = S2;
+        a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv / (float)(n * C);
+    }
+    dpw.pad(D, g, 16);
+}
+
+
+// =============================================================================================
+// n <= 8, dynamic H: coefficient backward as its own launch - one 16-lane group per sample, four
+// samples per wave, so the serial Sinkhorn chain of every sample runs concurrently instead of at
+// the tail of a bandwidth-bound workgroup.  Input: the raw channel sums written by the kernel
+// above ([B][parts][K], K = NP*NP + 3*NP + 1: dM | dHpost | A1 | A2 | s1).
+// =============================================================================================
+template <int NP, bool PRECISE>
+__global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
+    using SK = SkSmall<NP>;
+    constexpr int K = NP * NP + 3 * NP + 1;
+    extern __shared__ float sc[];  // Sinkhorn denominators, SK::scaling_floats(T)
+    const int tid = threadIdx.x, g = tid & 15;
+    const int b = blockIdx.x * 4 + (tid >> 4);
+    if (b >= a.B) return;  // whole 16-lane groups leave together; DPP never crosses groups
+    const int n = a.n, C = a.C, D = n * n + 2 * n;
+    const bool inject = a.f_inject != nullptr;
+    const int r0 = SK::row(g), c0 = SK::col0(g);
+    // everything this lane needs from memory, issued up front
+    const float *raw = a.raw + (size_t)b * a.parts * K;
+    float dMe[SK::EPL], tpost = 0.f, tA1 = 0.f, tA2 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++) dMe[e] = 0.f;
+    for (int p = 0; p < a.parts; p++) {
+        const float *rp = raw + (size_t)p * K;
+#pragma unroll
+        for (int e = 0; e < SK::EPL; e++) dMe[e] += rp[r0 * NP + c0 + e];
+        if (g < n) { tpost += rp[NP * NP + g]; tA1 += rp[NP * NP + NP + g]; tA2 += rp[NP * NP + 2 * NP + g]; }
+        s1 += rp[K - 1];
+    }
+    const float *Pb = a.P + (size_t)b * D;
+    const float al0 = a.alpha[0], al1 = a.alpha[1], al2 = a.alpha[2];
+    const float rinv = 1.0f / a.r[b];
+    const float qinv = inject ? 0.f : 1.0f / a.q[b];
+    float pres[SK::EPL], bres[SK::EPL];
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++) {
+        const bool ok = r0 < n && c0 + e < n;
+        pres[e] = ok ? Pb[2 * n + r0 * n + c0 + e] : 0.f;
+        bres[e] = ok ? a.b_res[r0 * n + c0 + e] : 0.f;
+    }
+    float hp = 0.f, ho = 0.f, ppre = 0.f, ppost = 0.f;
+    if (g < n) { hp = a.Hpre[(size_t)b * n + g]; ho = a.Hpost[(size_t)b * n + g]; ppre = Pb[g]; ppost = Pb[n + g]; }
+
+    if (g == 0) a.out.s1[b] = s1;
+    float *dt = a.out.dt + (size_t)b * (D + 3);
+    const DPWriter dpw{a.out, b, a.B, a.DP};
+    float S0 = 0.f, S1 = 0.f, S2 = 0.f;  // sum_d dt_d p_d per alpha group
+    if (g < n) {
+        const float dHpost = tpost;
+        const float dHpre = inject ? 0.f : tA1 * qinv - s1 * tA2 * qinv * qinv * qinv / (float)C;
+        const float dtp = dHpre * hp * (1.0f - hp);
+        const float dto = dHpost * ho * (1.0f - 0.5f * ho);
+        dt[g] = dtp; dt[n + g] = dto;
+        dpw.put(g, dtp * al0 * rinv); dpw.put(n + g, dto * al1 * rinv);
+        S0 = dtp * ppre; S1 = dto * ppost;
+    }
+    float E[SK::EPL], m[SK::EPL], d[SK::EPL];
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++) {
+        const bool ok = r0 < n && c0 + e < n;
+        E[e] = ok ? expf(al2 * pres[e] + bres[e]) : 0.f;
+        m[e] = E[e];
+        d[e] = ok ? dMe[e] : 0.f;
+    }
+    SK::template forward<PRECISE>(m, g, n, a.T, a.eps, sc, tid);
+    SK::template backward<PRECISE>(d, a.T, sc, tid);
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++) {
+        const int c = c0 + e;
+        if (r0 < n && c < n) {
+            const int di = 2 * n + r0 * n + c;
+            const float dtr = d[e] * E[e];
+            dt[di] = dtr;
+            dpw.put(di, dtr * al2 * rinv);
+            S2 += dtr * pres[e];
         }
     }
     S0 = row16_allreduce(S0); S1 = row16_allreduce(S1); S2 = row16_allreduce(S2);
@@ -500,12 +592,17 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_large_kernel(BwdReduceArgs
 // =============================================================================================
 template <typename TG, typename TX, int NP, int V>
 static hipError_t launch_small(const BwdReduceArgs &a, hipStream_t stream) {
-    const int nch = a.C / V;
+    const int nch = (a.C / V + a.parts - 1) / a.parts;  // chunks per column part
     int nt = (nch + 63) / 64 * 64;
     if (nt > 256) nt = 256;
     constexpr int K = NP * NP + 3 * NP + 1;
     const size_t smem = sizeof(float) * (K * 16 + K + SkSmall<NP>::scaling_floats(a.T));
-    mix_bwd_reduce_small_kernel<TG, TX, NP, V><<<a.B, nt, smem, stream>>>(a);
+    mix_bwd_reduce_small_kernel<TG, TX, NP, V><<<dim3(a.B, a.parts), nt, smem, stream>>>(a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || !a.raw) return e;
+    // fp32 activations: the parity tier, IEEE divisions in the Sinkhorn chain
+    constexpr bool kPrecise = std::is_same<TX, float>::value;
+    coef_bwd_small_kernel<NP, kPrecise><<<(a.B + 3) / 4, 64, sizeof(float) * SkSmall<NP>::scaling_floats(a.T), stream>>>(a);
     return hipGetLastError();
 }
 
@@ -528,14 +625,25 @@ static hipError_t launch_large(const BwdReduceArgs &a, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// Column parts per sample when the reduction is split from the coefficient backward.
+int bwd_reduce_parts(int B, int n, int C) {
+    (void)n;
+    if (B >= 2048 || C < 1024) return 1;
+    return 2;
+}
+
 hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int x_dtype,
                                  const void *w, int w_dtype, const void *f_inject,
                                  const float *Hpre, const float *Hpost, const float *M, int hstride,
                                  const float *q, const float *P, const float *r, const float *alpha,
-                                 const float *b_res, BwdCoefOut out, int B, int n, int C, int T,
-                                 float eps, hipStream_t stream) {
+                                 const float *b_res, BwdCoefOut out, float *raw, int B, int n, int C,
+                                 int T, float eps, hipStream_t stream) {
+    // dynamic H with n <= 8: channel sums per (sample, column part), coefficient backward as a
+    // second small launch; otherwise everything in the per-sample workgroup
+    const bool split = raw != nullptr && hstride != 0 && n <= 8;
     BwdReduceArgs a{dy, x, w, f_inject, Hpre, Hpost, M, q, P, r, alpha, b_res, out,
-                    hstride, w_dtype == kBF16, B, n, C, T, padded_D(n), eps};
+                    hstride, w_dtype == kBF16, B, n, C, T, padded_D(n), eps,
+                    split ? raw : nullptr, split ? bwd_reduce_parts(B, n, C) : 1};
     if (n <= 8) {
 #define MHC_SMALL(TG, TX)                                                   \
     return n <= 4 ? launch_small_np<TG, TX, 4>(a, stream) : launch_small_np<TG, TX, 8>(a, stream)

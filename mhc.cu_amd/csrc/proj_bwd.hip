@@ -93,23 +93,29 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
         __syncthreads();
 
         // ---- dphi tiles of this wave: (dt, nt), dt = (wave + 4m) / NTK -------------------------
+        // x fragments of the block once, then per tile all dP^T operands in one batch of loads
+        bf16x8_t xf[2 * NSB];
 #pragma unroll
-        for (int ks = 0; ks < 2 * NSB; ks++) {
-            if (sb + ks * 16 < b_end) {
-                const bf16x8_t xf = lds_frag_t(x_s, LD, ks * 16, nt * 32, lane);
+        for (int ks = 0; ks < 2 * NSB; ks++) xf[ks] = lds_frag_t(x_s, LD, ks * 16, nt * 32, lane);
 #pragma unroll
-                for (int m = 0; m < TPW; m++) {
-                    const int dt = (wave + 4 * m) / NTK;
-                    if (dt < NTD) {
-                        // dP^T rows d, 8 consecutive samples; the pad columns [B, BP) are zero
-                        const bf16_t *ap = a.dPT + (size_t)(dt * 32 + row) * a.BP + sb + ks * 16 + kg * 8;
-                        const uint4 ah = *reinterpret_cast<const uint4 *>(ap);
-                        const uint4 al = *reinterpret_cast<const uint4 *>(ap + (size_t)a.DP * a.BP);
-                        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(bf16x8_t, ah), xf, acc[m], 0, 0, 0);
-                        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(bf16x8_t, al), xf, acc[m], 0, 0, 0);
-                    }
+        for (int m = 0; m < TPW; m++) {
+            const int dt = (wave + 4 * m) / NTK;
+            if (dt < NTD) {
+                // dP^T rows d, 8 consecutive samples; columns beyond the batch are zero padded
+                const bf16_t *ap = a.dPT + (size_t)(dt * 32 + row) * a.BP + sb + kg * 8;
+                uint4 ah[2 * NSB], al[2 * NSB];
+#pragma unroll
+                for (int ks = 0; ks < 2 * NSB; ks++) {
+                    const bool ok = sb + ks * 16 < b_end;
+                    ah[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + ks * 16) : zero4;
+                    al[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + ks * 16 + (size_t)a.DP * a.BP) : zero4;
+                }
+#pragma unroll
+                for (int ks = 0; ks < 2 * NSB; ks++) {
+                    acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8_t, ah[ks]), xf[ks], acc[m], 0, 0, 0);
+                    acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8_t, al[ks]), xf[ks], acc[m], 0, 0, 0);
                 }
             }
         }
@@ -132,10 +138,19 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
                     }
                 }
             } else {
-                for (int ks = 0; ks < 2 * NTD; ks++) {
-                    const uint4 av = b < b_end ? *reinterpret_cast<const uint4 *>(dprow + ks * 16) : zero4;
-                    const bf16x8_t pf = lds_frag_t(phi_s, LD, ks * 16, nt * 32, lane);
-                    o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pf, o, 0, 0, 0);
+                for (int ks0 = 0; ks0 < 2 * NTD; ks0 += 8) {  // 8 operand loads in flight
+                    uint4 av[8];
+#pragma unroll
+                    for (int u = 0; u < 8; u++)
+                        av[u] = (b < b_end && ks0 + u < 2 * NTD)
+                                    ? *reinterpret_cast<const uint4 *>(dprow + (ks0 + u) * 16) : zero4;
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        if (ks0 + u < 2 * NTD) {
+                            const bf16x8_t pf = lds_frag_t(phi_s, LD, (ks0 + u) * 16, nt * 32, lane);
+                            o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av[u]), pf, o, 0, 0, 0);
+                        }
+                    }
                 }
             }
             // accumulator layout: column = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4

@@ -183,15 +183,16 @@ static int mfma_nt(int n) {
 }
 
 int proj_fwd_ksplit(int x_dtype, int phi_dtype, int B, int n, int C) {
-    // The generic path always uses one split.  MFMA path: enough workgroups to fill 256 CUs,
-    // at least 64 K elements per wave, partial sums at most ~1/4 of x's bytes.
+    // The generic path always uses one split.  MFMA path: enough workgroups to fill 256 CUs
+    // several times over (the K loop is latency-bound per wave), at least 64 K elements per wave.
     if (!use_mfma(x_dtype, phi_dtype, C)) return 1;
     const int nC = n * C, DP = padded_D(n);
     const int tiles_s = (B + 31) / 32;
     const int groups = DP / 32 / mfma_nt(n);
-    int ks = (512 + tiles_s * groups - 1) / (tiles_s * groups);
+    int ks = (1024 + tiles_s * groups - 1) / (tiles_s * groups);
     const int cap_slab = nC / 256;
-    const int cap_bytes = (int)((0.25 * nC * 2.0) / (DP * 4.0));
+    // partial sums (KS * B * DP fp32) at most ~1/4 of the bytes this kernel streams (x and phi)
+    const int cap_bytes = (int)(0.25 * (2.0 * B * nC + 2.0 * DP * nC) / (4.0 * B * DP));
     if (ks > cap_slab) ks = cap_slab;
     if (ks > cap_bytes) ks = cap_bytes;
     if (ks > 64) ks = 64;

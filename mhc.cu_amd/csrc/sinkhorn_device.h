@@ -44,8 +44,12 @@ template <int NP> struct SkSmall {
     }
 
     // m: in = exp(logits) (0 outside n x n), out = final iterate.
-    // sc != nullptr: keep rho_t (this lane's row) and s_t (this lane's EPL columns) at
-    // sc[(t * (1 + EPL) + k) * 64 + lane].
+    // sc != nullptr: keep, per iteration t and lane, the row denominator, and per element the
+    // column denominator, the row-normalised iterate R_t and the iterate after the column step:
+    //   sc[(t * kRec + k) * 64 + lane], k = 0: rho | 1..EPL: s | EPL+1..2EPL: R | 2EPL+1..3EPL: Out
+    // PRECISE selects IEEE divisions (fp32 parity tier) instead of v_rcp_f32.
+    static constexpr int kRec = 1 + 3 * EPL;
+    template <bool PRECISE = false>
     __device__ static __forceinline__ void forward(float (&m)[EPL], int g, int n, int T, float eps,
                                                    float *sc, int lane) {
         const bool rv = row(g) < n;
@@ -58,44 +62,47 @@ template <int NP> struct SkSmall {
             for (int e = 0; e < EPL; e++) rs += m[e];
             rs = row_allreduce(rs) + eps;
             rs = rv ? rs : 1.0f;
-            const float rinv = fast_rcp(rs);
-            if (sc) sc[(t * (1 + EPL)) * kWave + lane] = rs;
+            const float rinv = PRECISE ? 1.0f / rs : fast_rcp(rs);
+            if (sc) sc[(t * kRec) * kWave + lane] = PRECISE ? rs : rinv;  // fast tier keeps 1/rho
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
-                m[e] *= rinv;
+                m[e] = PRECISE ? m[e] / rs : m[e] * rinv;
                 float cs = col_allreduce(m[e]) + eps;
                 cs = cv[e] ? cs : 1.0f;
-                if (sc) sc[(t * (1 + EPL) + 1 + e) * kWave + lane] = cs;
-                m[e] *= fast_rcp(cs);
+                const float cinv = PRECISE ? 0.f : fast_rcp(cs);
+                if (sc) {
+                    sc[(t * kRec + 1 + e) * kWave + lane] = PRECISE ? cs : cinv;  // fast tier keeps 1/s
+                    sc[(t * kRec + 1 + EPL + e) * kWave + lane] = m[e];
+                }
+                m[e] = PRECISE ? m[e] / cs : m[e] * cinv;
+                if (sc) sc[(t * kRec + 1 + 2 * EPL + e) * kWave + lane] = m[e];
             }
         }
     }
 
-    // m: final iterate (from forward); d: in = dL/dM, out = dL/dE.  sc as written by forward.
-    __device__ static __forceinline__ void backward(float (&m)[EPL], float (&d)[EPL], int T,
-                                                    const float *sc, int lane) {
+    // d: in = dL/dM, out = dL/dE.  sc as written by forward (the saved iterates are used as they
+    // were computed, exactly like reverse-mode autodiff of the forward loop).
+    template <bool PRECISE = false>
+    __device__ static __forceinline__ void backward(float (&d)[EPL], int T, const float *sc, int lane) {
         for (int t = T - 1; t >= 0; t--) {
-            const float rs = sc[(t * (1 + EPL)) * kWave + lane];
+            const float rs = sc[(t * kRec) * kWave + lane];
             float rdot = 0.f;
             float dR[EPL];
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
-                const float cs = sc[(t * (1 + EPL) + 1 + e) * kWave + lane];
-                const float cdot = col_allreduce(d[e] * m[e]);
-                dR[e] = (d[e] - cdot) * fast_rcp(cs);
-                m[e] *= cs;  // row-normalised iterate R_t
-                rdot += dR[e] * m[e];
+                const float cs = sc[(t * kRec + 1 + e) * kWave + lane];
+                const float R = sc[(t * kRec + 1 + EPL + e) * kWave + lane];
+                const float Out = sc[(t * kRec + 1 + 2 * EPL + e) * kWave + lane];
+                const float cdot = col_allreduce(d[e] * Out);
+                dR[e] = PRECISE ? (d[e] - cdot) / cs : (d[e] - cdot) * cs;  // fast tier: cs holds 1/s
+                rdot += dR[e] * R;
             }
             rdot = row_allreduce(rdot);
-            const float rinv = fast_rcp(rs);
 #pragma unroll
-            for (int e = 0; e < EPL; e++) {
-                d[e] = (dR[e] - rdot) * rinv;
-                m[e] *= rs;  // iterate before row step t
-            }
+            for (int e = 0; e < EPL; e++) d[e] = PRECISE ? (dR[e] - rdot) / rs : (dR[e] - rdot) * rs;
         }
     }
-    __host__ __device__ static constexpr int scaling_floats(int T) { return T * (1 + EPL) * kWave; }
+    __host__ __device__ static constexpr int scaling_floats(int T) { return T * kRec * kWave; }
 };
 
 // =============================================================================================

@@ -14,7 +14,7 @@ from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmhc_hip.so")
+LIB_PATH = os.environ.get("MHC_HIP_LIBRARY") or os.path.join(_HERE, "libmhc_hip.so")
 
 MHC_F32, MHC_BF16 = 0, 1
 MHC_MAX_N = 32
