@@ -36,8 +36,8 @@ struct BwdSlabArgs {
     const void *f_inject;    // bf16 [B, C] or nullptr
     const bf16_t *phi;       // [D, nC]
     const float *Hpre, *Hpost, *M, *q, *s1, *cx;  // per sample
-    const bf16_t *dPb;       // [B, 32]
-    const bf16_t *dPT;       // [2][32][BP]
+    const bf16_t *dPb;       // dP, fragment-major (frag_dpb, DP = 32)
+    const bf16_t *dPT;       // dP^T hi/lo planes, fragment-major (frag_dpt), plane stride 32 * BP
     const float *dt;         // [B, D+3]
     bf16_t *dx;              // [B, n, C]
     bf16_t *df;              // [B, C] or nullptr
@@ -167,12 +167,12 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
         uint4 ah[2], al[2], ap2[2];
 #pragma unroll
         for (int ks = 0; ks < 2; ks++) {
-            const bf16_t *ap = a.dPT + (size_t)row * a.BP + sb + ks * 16 + kg * 8;
+            const bf16_t *ap = a.dPT + frag_base(0, a.BP >> 4, (sb >> 4) + ks) + lane * 8;
             const bool ok = sb + ks * 16 < b_end;  // BP is padded to 32 and zero beyond B
             ah[ks] = ok ? *reinterpret_cast<const uint4 *>(ap) : zero4;
             al[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + (size_t)32 * a.BP) : zero4;
             const int bq = sb + row;
-            ap2[ks] = bq < b_end ? *reinterpret_cast<const uint4 *>(a.dPb + (size_t)bq * 32 + ks * 16 + kg * 8) : zero4;
+            ap2[ks] = bq < b_end ? *reinterpret_cast<const uint4 *>(a.dPb + frag_base(sb >> 5, 2, ks) + lane * 8) : zero4;
         }
         // x tile -> LDS (rows of samples beyond the split are zero)
 #pragma unroll

@@ -81,7 +81,7 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
     if (bs3 > bs) bs = bs3;
     w.dphi_part = c.floats(bs > 1 ? (size_t)bs * D * nC : 0);
     w.BP = (B + 31) / 32 * 32;
-    w.dPb = reinterpret_cast<unsigned short *>(c.floats(((size_t)B * padded_D(n) + 1) / 2));
+    w.dPb = reinterpret_cast<unsigned short *>(c.floats(((size_t)w.BP * padded_D(n) + 1) / 2));
     w.dPT = reinterpret_cast<unsigned short *>(c.floats((size_t)padded_D(n) * w.BP));  // two bf16 planes
     w.bytes = c.off;
     return w;

@@ -71,11 +71,15 @@ template <int NP> __global__ __launch_bounds__(64) void coef_fwd_small_kernel(Co
     }
 }
 
-template <int NP> __global__ __launch_bounds__(64) void coef_fwd_lds_kernel(CoefArgs a) {
+// One workgroup (4 waves) per sample.  All 256 threads finish the split-K sums (D = n^2 + 2n
+// logits, KS partial sums each, eight loads in flight per thread), then wave 0 runs Sinkhorn on
+// the matrix in LDS; the other waves only keep the barriers.
+template <int NP> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     using SK = SkLds<NP>;
     __shared__ float lds[SK::forward_floats()];
+    __shared__ float lg[NP * NP + 2 * NP];  // logits: pre | post | res (row-major n x n)
     float *Es = lds, *u = Es + NP * SK::LD, *v = u + NP;
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x;
     const int b = blockIdx.x;
     const int n = a.n, D = n * n + 2 * n;
     const bool dyn = a.Ppart != nullptr;
@@ -85,27 +89,41 @@ template <int NP> __global__ __launch_bounds__(64) void coef_fwd_lds_kernel(Coef
         const float r = sqrtf(ssq / (float)a.nC + a.eps);
         rinv = 1.0f / r;
         al[0] = a.alpha[0]; al[1] = a.alpha[1]; al[2] = a.alpha[2];
-        if (lane == 0) a.r[b] = r;
+        if (tid == 0) a.r[b] = r;
     }
     const size_t pstride = (size_t)a.B * a.DP;
-    auto logit = [&](int d, float alpha_g, float bias) -> float {
-        if (!dyn) return bias;
-        const float p = reduce_partials(a.Ppart, a.KS, pstride, (size_t)b * a.DP + d) * rinv;
-        a.P[(size_t)b * D + d] = p;
-        return alpha_g * p + bias;
-    };
-    if (lane < n) {
-        a.Hpre[b * n + lane] = sigmoidf_acc(logit(lane, al[0], a.b_pre[lane]));
-        a.Hpost[b * n + lane] = 2.0f * sigmoidf_acc(logit(n + lane, al[1], a.b_post[lane]));
-    }
-    for (int e = lane; e < NP * NP; e += kWave) {
-        const int r0 = e / NP, c = e % NP;
-        Es[r0 * SK::LD + c] =
-            (r0 < n && c < n) ? expf(logit(2 * n + r0 * n + c, al[2], a.b_res[r0 * n + c])) : 0.f;
+    for (int d = tid; d < D; d += 256) {
+        const int grp = alpha_group(d, n);
+        const float bias = grp == 0 ? a.b_pre[d] : (grp == 1 ? a.b_post[d - n] : a.b_res[d - 2 * n]);
+        float t = bias;
+        if (dyn) {
+            const float *pp = a.Ppart + (size_t)b * a.DP + d;
+            float acc = 0.f;
+            for (int k0 = 0; k0 < a.KS; k0 += 8) {
+                float tv[8];
+#pragma unroll
+                for (int q = 0; q < 8; q++) tv[q] = k0 + q < a.KS ? pp[(size_t)(k0 + q) * pstride] : 0.f;
+#pragma unroll
+                for (int q = 0; q < 8; q++) acc += tv[q];
+            }
+            const float p = acc * rinv;
+            a.P[(size_t)b * D + d] = p;
+            t = al[grp] * p + bias;
+        }
+        lg[d] = t;
     }
     __syncthreads();
-    SK::forward(Es, u, v, n, a.T, a.eps, nullptr, nullptr, lane);
-    for (int e = lane; e < n * n; e += kWave) {
+    if (tid < n) {
+        a.Hpre[b * n + tid] = sigmoidf_acc(lg[tid]);
+        a.Hpost[b * n + tid] = 2.0f * sigmoidf_acc(lg[n + tid]);
+    }
+    for (int e = tid; e < NP * NP; e += 256) {
+        const int r0 = e / NP, c = e % NP;
+        Es[r0 * SK::LD + c] = (r0 < n && c < n) ? expf(lg[2 * n + r0 * n + c]) : 0.f;
+    }
+    __syncthreads();
+    SK::forward(Es, u, v, n, a.T, a.eps, nullptr, nullptr, tid);
+    for (int e = tid; e < n * n; e += 256) {
         const int r0 = e / n, c = e % n;
         a.M[(size_t)b * n * n + e] = u[r0] * Es[r0 * SK::LD + c] * v[c];
     }
@@ -121,9 +139,9 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
     else if (n <= 8)
         coef_fwd_small_kernel<8><<<(B + 3) / 4, 64, 0, stream>>>(a);
     else if (n <= 16)
-        coef_fwd_lds_kernel<16><<<B, 64, 0, stream>>>(a);
+        coef_fwd_lds_kernel<16><<<B, 256, 0, stream>>>(a);
     else
-        coef_fwd_lds_kernel<32><<<B, 64, 0, stream>>>(a);
+        coef_fwd_lds_kernel<32><<<B, 256, 0, stream>>>(a);
     return hipGetLastError();
 }
 

@@ -58,8 +58,8 @@ struct BwdCoefOut {
     float *cx;    // [B]      sum_d dt_d alpha_g p_d / (nC r^2)                    (dynamic only)
     float *s1;    // [B]      sum_c df_c w_c a_c
     float *red;   // [B, n*n + 2n] raw per-sample (dM | dHpre | dHpost)             (static only)
-    unsigned short *dPb;  // [B, DP]  bf16 copy of dP, or nullptr                     (dynamic only)
-    unsigned short *dPT;  // [2][DP, BP] bf16 transpose of dP (high part, remainder), pad zeroed
+    unsigned short *dPb;  // BP * DP bf16, dP in MFMA fragment order (frag_dpb), or nullptr
+    unsigned short *dPT;  // 2 planes of DP * BP bf16, dP^T in fragment order (frag_dpt): value, remainder
     int BP;               // row pitch of dPT, a multiple of 32 that is >= B
 };
 
@@ -110,6 +110,9 @@ hipError_t launch_finalize(const float *u, int rows_u, int C, float *dw, const f
 // dxflat = dP phi (bf16 [B, nC]) in one pass over x and phi.  With S = proj_bwd_batch_splits() > 1
 // the S partial copies land in dphi_part and the caller's finalize launch sums them.
 bool proj_bwd_mfma_supported(int x_dtype, int phi_dtype, int C);
+hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb, const void *dPT,
+                                 int BP, float *dphi_out, void *dxflat, int S, int B, int n, int C,
+                                 hipStream_t stream);
 int proj_bwd_batch_splits(int B, int n, int C);
 hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,
                                 int BP, float *dphi, float *dphi_part, void *dxflat, int B, int n,

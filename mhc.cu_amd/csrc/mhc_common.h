@@ -167,4 +167,22 @@ __device__ __forceinline__ int alpha_group(int d, int n) { return d < n ? 0 : (d
 
 __host__ __device__ constexpr int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
+// ---------------------------------------------------------------------------------------------
+// MFMA-ready ("fragment-major") storage of the two bf16 copies of dP that the projection
+// backward consumes as A operands of v_mfma_f32_32x32x16_bf16.  One fragment = the 64 lanes x 8
+// values of one instruction, stored contiguously (1 KiB), so a wave loads it with one fully
+// coalesced 16-byte-per-lane access: lane = 32 * kgroup + row, kgroup = (k / 8) % 2.
+//   frag_dpt: rows d (tile d / 32), contraction index b (step b / 16); BP = padded batch, % 32 == 0
+//   frag_dpb: rows b (tile b / 32), contraction index d (step d / 16); DP = padded D, % 32 == 0
+// ---------------------------------------------------------------------------------------------
+__host__ __device__ inline size_t frag_base(int tile, int steps_per_tile, int step) {
+    return ((size_t)tile * steps_per_tile + step) * 512;  // elements
+}
+__host__ __device__ inline size_t frag_dpt(int d, int b, int BP) {
+    return frag_base(d >> 5, BP >> 4, b >> 4) + (size_t)((((b >> 3) & 1) * 32 + (d & 31)) * 8 + (b & 7));
+}
+__host__ __device__ inline size_t frag_dpb(int b, int d, int DP) {
+    return frag_base(b >> 5, DP >> 4, d >> 4) + (size_t)((((d >> 3) & 1) * 32 + (b & 31)) * 8 + (d & 7));
+}
+
 }  // namespace mhc

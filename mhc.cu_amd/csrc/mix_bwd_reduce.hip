@@ -46,8 +46,9 @@ __device__ __forceinline__ float row16_allreduce(float v) {
 }
 
 // Writes dP[b, d] in every layout the later kernels read: fp32 [B, DP] (generic kernels),
-// bf16 [B, DP] and bf16 transposed [2][DP, BP] (MFMA operands; plane 0 = value rounded to
-// bf16, plane 1 = the rounding remainder, so that dphi keeps ~16 mantissa bits of dP).  Padded
+// and two bf16 copies in fragment-major order (frag_dpb / frag_dpt: MFMA A operands; for the
+// transpose, plane 0 = value rounded to bf16, plane 1 = the rounding remainder, so that dphi
+// keeps ~16 mantissa bits of dP).  Padded
 // rows d >= D and, from the last sample's workgroup, padded columns b >= B are zeroed.
 struct DPWriter {
     BwdCoefOut o;
@@ -57,13 +58,13 @@ struct DPWriter {
         if (o.dPb) {
             const bf16_t h = f32_to_bf16(v);
             const size_t plane = (size_t)DP * o.BP;
-            o.dPb[(size_t)b * DP + d] = h;
-            o.dPT[(size_t)d * o.BP + b] = h;
-            o.dPT[plane + (size_t)d * o.BP + b] = f32_to_bf16(v - bf16_to_f32(h));
+            o.dPb[frag_dpb(b, d, DP)] = h;
+            o.dPT[frag_dpt(d, b, o.BP)] = h;
+            o.dPT[plane + frag_dpt(d, b, o.BP)] = f32_to_bf16(v - bf16_to_f32(h));
             if (b == B - 1)
                 for (int bb = B; bb < o.BP; bb++) {
-                    o.dPT[(size_t)d * o.BP + bb] = 0;
-                    o.dPT[plane + (size_t)d * o.BP + bb] = 0;
+                    o.dPT[frag_dpt(d, bb, o.BP)] = 0;
+                    o.dPT[plane + frag_dpt(d, bb, o.BP)] = 0;
                 }
         }
     }
@@ -72,13 +73,13 @@ struct DPWriter {
             o.dP[(size_t)b * DP + d] = 0.f;
             if (o.dPb) {
                 const size_t plane = (size_t)DP * o.BP;
-                o.dPb[(size_t)b * DP + d] = 0;
-                o.dPT[(size_t)d * o.BP + b] = 0;
-                o.dPT[plane + (size_t)d * o.BP + b] = 0;
+                o.dPb[frag_dpb(b, d, DP)] = 0;
+                o.dPT[frag_dpt(d, b, o.BP)] = 0;
+                o.dPT[plane + frag_dpt(d, b, o.BP)] = 0;
                 if (b == B - 1)
                     for (int bb = B; bb < o.BP; bb++) {
-                        o.dPT[(size_t)d * o.BP + bb] = 0;
-                        o.dPT[plane + (size_t)d * o.BP + bb] = 0;
+                        o.dPT[frag_dpt(d, bb, o.BP)] = 0;
+                        o.dPT[plane + frag_dpt(d, bb, o.BP)] = 0;
                     }
             }
         }

@@ -22,8 +22,8 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 struct ProjBwdArgs {
     const bf16_t *x;     // [B][nC]
     const bf16_t *phi;   // [D][nC]
-    const bf16_t *dPb;   // [B][DP]   (columns >= D are zero)
-    const bf16_t *dPT;   // [2][DP][BP] high and low bf16 parts of dP^T (rows >= D, columns >= B zero)
+    const bf16_t *dPb;   // dP, fragment-major (frag_dpb); columns >= D are zero
+    const bf16_t *dPT;   // dP^T hi and lo bf16 planes, fragment-major (frag_dpt); rows >= D, columns >= B zero
     float *dphi;         // [S][D][nC]  (S = gridDim.y batch splits)
     bf16_t *dxflat;      // [B][nC]
     int B, BP, D, DP, nC, b_per_split;
@@ -102,13 +102,13 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
             const int dt = (wave + 4 * m) / NTK;
             if (dt < NTD) {
                 // dP^T rows d, 8 consecutive samples; columns beyond the batch are zero padded
-                const bf16_t *ap = a.dPT + (size_t)(dt * 32 + row) * a.BP + sb + kg * 8;
+                const bf16_t *ap = a.dPT + frag_base(dt, a.BP >> 4, sb >> 4) + lane * 8;
                 uint4 ah[2 * NSB], al[2 * NSB];
 #pragma unroll
                 for (int ks = 0; ks < 2 * NSB; ks++) {
                     const bool ok = sb + ks * 16 < b_end;
-                    ah[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + ks * 16) : zero4;
-                    al[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + ks * 16 + (size_t)a.DP * a.BP) : zero4;
+                    ah[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + ks * 512) : zero4;
+                    al[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + ks * 512 + (size_t)a.DP * a.BP) : zero4;
                 }
 #pragma unroll
                 for (int ks = 0; ks < 2 * NSB; ks++) {
@@ -127,12 +127,12 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
 #pragma unroll
             for (int i = 0; i < 16; i++) o[i] = 0.f;
             const int b = bs0 + row;
-            const bf16_t *dprow = a.dPb + (size_t)(b < a.B ? b : 0) * a.DP + kg * 8;
+            const bf16_t *dprow = a.dPb + frag_base(bs0 >> 5, a.DP >> 4, 0) + lane * 8;  // + 512 per k-step
             if constexpr (PHI_REGS) {
 #pragma unroll
                 for (int ks = 0; ks < 2 * TPW * 4 / NTK; ks++) {
                     if (ks < 2 * NTD) {
-                        const uint4 av = b < b_end ? *reinterpret_cast<const uint4 *>(dprow + ks * 16) : zero4;
+                        const uint4 av = b < b_end ? *reinterpret_cast<const uint4 *>(dprow + ks * 512) : zero4;
                         o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
                                                                     phif[ks], o, 0, 0, 0);
                     }
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
 #pragma unroll
                     for (int u = 0; u < 8; u++)
                         av[u] = (b < b_end && ks0 + u < 2 * NTD)
-                                    ? *reinterpret_cast<const uint4 *>(dprow + (ks0 + u) * 16) : zero4;
+                                    ? *reinterpret_cast<const uint4 *>(dprow + (ks0 + u) * 512) : zero4;
 #pragma unroll
                     for (int u = 0; u < 8; u++) {
                         if (ks0 + u < 2 * NTD) {
@@ -238,10 +238,11 @@ hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb,
                   S > 1 ? dphi_part : dphi, static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, bps};
     const int NTD = DP / 32;
     hipError_t e;
-    // NTK == 1: dphi tiles per wave = ceil(NTD / 4); phi fragments in registers when 2*NTD <= 8
+    // NTK == 1: dphi tiles per wave = ceil(NTD / 4); phi fragments in registers when 2*NTD <= 8.
+    // Wide projections (more than 12 row tiles) run as two GEMM kernels that share no operand.
     if (NTD <= 4) e = launch_shape<1, 1, true>(a, S, stream);
     else if (NTD <= 12) e = launch_shape<1, 3, false>(a, S, stream);
-    else e = launch_shape<1, 9, false>(a, S, stream);
+    else e = launch_proj_bwd_large(x, phi, dPb, dPT, BP, S > 1 ? dphi_part : dphi, dxflat, S, B, n, C, stream);
     return e;  // with S > 1 the caller's finalize launch sums the S partial copies
 }
 
