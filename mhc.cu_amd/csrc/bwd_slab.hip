@@ -70,16 +70,14 @@ __device__ __forceinline__ void unpack8(const uint4 &r, float (&v)[8]) {
 template <typename T> struct Raw8;
 template <> struct Raw8<bf16_t> {
     uint4 r;
-    __device__ __forceinline__ void load(const bf16_t *p, bool ok) {
-        r = ok ? *reinterpret_cast<const uint4 *>(p) : make_uint4(0, 0, 0, 0);
-    }
+    __device__ __forceinline__ void load(const bf16_t *p) { r = *reinterpret_cast<const uint4 *>(p); }
     __device__ __forceinline__ void get(float (&v)[8]) const { unpack8(r, v); }
 };
 template <> struct Raw8<float> {
     float4 r0, r1;
-    __device__ __forceinline__ void load(const float *p, bool ok) {
-        r0 = ok ? reinterpret_cast<const float4 *>(p)[0] : make_float4(0.f, 0.f, 0.f, 0.f);
-        r1 = ok ? reinterpret_cast<const float4 *>(p)[1] : make_float4(0.f, 0.f, 0.f, 0.f);
+    __device__ __forceinline__ void load(const float *p) {
+        r0 = reinterpret_cast<const float4 *>(p)[0];
+        r1 = reinterpret_cast<const float4 *>(p)[1];
     }
     __device__ __forceinline__ void get(float (&v)[8]) const {
         v[0] = r0.x; v[1] = r0.y; v[2] = r0.z; v[3] = r0.w; v[4] = r1.x; v[5] = r1.y; v[6] = r1.z; v[7] = r1.w;
@@ -97,7 +95,6 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
     const int b_begin = blockIdx.y * a.b_per_split;
     const int b_end = min(a.B, b_begin + a.b_per_split);
     const bool inject = a.f_inject != nullptr;
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
     const int row = lane & 31, kg = lane >> 5;
     // VALU ownership: sample bl of the tile, channels c0 + ch*8 .. +8 of every stream
     const int bl = tid >> 3, ch = tid & 7;
@@ -110,8 +107,9 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
     for (int e = tid; e < 32 * (kSlabKW / 8); e += 256) {
         const int d = e / (kSlabKW / 8), chunk = e % (kSlabKW / 8);
         const int j = chunk / (kSlabCW / 8), c = c0 + (chunk % (kSlabCW / 8)) * 8;
-        const uint4 v = (d < D && j < n && c < C)
-                            ? *reinterpret_cast<const uint4 *>(a.phi + (size_t)d * nC + (size_t)j * C + c) : zero4;
+        const bool ok = d < D && j < n && c < C;
+        const uint4 v = load16_masked(
+            reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * nC + (size_t)j * C + c : 0)), ok);
         *reinterpret_cast<uint4 *>(phi_s + (size_t)d * kSlabLDX + chunk * 8) = v;
     }
     __syncthreads();
@@ -145,15 +143,22 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
         uint4 xr[kSlabNS];
         Raw8<TG> gr[kSlabNS];
     };
+    // Loads carry no predicate (a predicate would be applied right behind the load and make the
+    // prefetch wait): slots beyond the batch, streams >= n and channel chunks >= C alias valid
+    // data instead.  Aliased values are finite whenever the real inputs are and only ever meet
+    // zero coefficients (dP^T is zero beyond B, H and M are zero beyond n) or land in rows and
+    // columns that are never stored.
     auto load_tile = [&](int sb, TileRegs &t) {
         const int b = sb + bl;
         const bool bok = b < b_end && cok;
-        const bf16_t *xb = a.x + (size_t)(bok ? b : 0) * nC + cth;
-        const TG *gb = static_cast<const TG *>(a.dy) + (size_t)(bok ? b : 0) * nC + cth;
+        const size_t base = bok ? (size_t)b * nC + cth : 0;
+        const bf16_t *xb = a.x + base;
+        const TG *gb = static_cast<const TG *>(a.dy) + base;
 #pragma unroll
         for (int j = 0; j < kSlabNS; j++) {
-            t.xr[j] = (bok && j < n) ? *reinterpret_cast<const uint4 *>(xb + (size_t)j * C) : zero4;
-            t.gr[j].load(gb + (size_t)j * C, bok && j < n);
+            const size_t so = j < n ? (size_t)j * C : 0;
+            t.xr[j] = *reinterpret_cast<const uint4 *>(xb + so);
+            t.gr[j].load(gb + so);
         }
     };
     TileRegs cur, nxt;
@@ -168,13 +173,13 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
 #pragma unroll
         for (int ks = 0; ks < 2; ks++) {
             const bf16_t *ap = a.dPT + frag_base(0, a.BP >> 4, (sb >> 4) + ks) + lane * 8;
-            const bool ok = sb + ks * 16 < b_end;  // BP is padded to 32 and zero beyond B
-            ah[ks] = ok ? *reinterpret_cast<const uint4 *>(ap) : zero4;
-            al[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + (size_t)32 * a.BP) : zero4;
-            const int bq = sb + row;
-            ap2[ks] = bq < b_end ? *reinterpret_cast<const uint4 *>(a.dPb + frag_base(sb >> 5, 2, ks) + lane * 8) : zero4;
+            // splits are whole 32-sample tiles and BP is padded to 32 (dP^T zero beyond B), so every
+            // fragment of the tile is inside the buffers; dP rows beyond B only feed unused rows
+            ah[ks] = *reinterpret_cast<const uint4 *>(ap);
+            al[ks] = *reinterpret_cast<const uint4 *>(ap + (size_t)32 * a.BP);
+            ap2[ks] = *reinterpret_cast<const uint4 *>(a.dPb + frag_base(sb >> 5, 2, ks) + lane * 8);
         }
-        // x tile -> LDS (rows of samples beyond the split are zero)
+        // x tile -> LDS
 #pragma unroll
         for (int j = 0; j < kSlabNS; j++)
             *reinterpret_cast<uint4 *>(x_s + (size_t)bl * kSlabLDX + j * kSlabCW + ch * 8) = cur.xr[j];

@@ -115,6 +115,17 @@ __device__ __forceinline__ void store_vec(T *__restrict__ p, const float (&v)[V]
     }
 }
 
+// 16-byte global load that yields zeros when !ok.  `p` must be dereferenceable either way (callers
+// clamp the index): the load is unconditional and the value is masked afterwards, which keeps the
+// code free of per-lane branches.  Do NOT write `ok ? *p : zero_variable`: the compiler then selects
+// between two addresses (global memory and the variable's stack slot) and emits a flat load that
+// waits on both memory counters.
+__device__ __forceinline__ uint4 load16_masked(const uint4 *p, bool ok) {
+    uint4 v = *p;
+    v.x = ok ? v.x : 0u; v.y = ok ? v.y : 0u; v.z = ok ? v.z : 0u; v.w = ok ? v.w : 0u;
+    return v;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Cross-lane primitives
 // ---------------------------------------------------------------------------------------------

@@ -57,13 +57,12 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
     const int NTD = a.DP / 32;
     const int b_begin = blockIdx.y * a.b_per_split;
     const int b_end = min(a.B, b_begin + a.b_per_split);
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
 
     // ---- phi slab -> LDS (rows >= D and columns >= nC read as zero) ------------------------
     for (int ch = tid; ch < a.DP * CPR; ch += 256) {
         const int d = ch / CPR, k = k0 + (ch % CPR) * 8;
-        const uint4 v = (d < a.D && k < a.nC)
-                            ? *reinterpret_cast<const uint4 *>(a.phi + (size_t)d * a.nC + k) : zero4;
+        const bool ok = d < a.D && k < a.nC;
+        const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * a.nC + k : 0)), ok);
         *reinterpret_cast<uint4 *>(phi_s + (size_t)d * LD + (ch % CPR) * 8) = v;
     }
     __syncthreads();
@@ -86,8 +85,8 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
         if (sb != b_begin) __syncthreads();  // previous block's fragment reads are done
         for (int ch = tid; ch < SBR * CPR; ch += 256) {
             const int bl = ch / CPR, b = sb + bl, k = k0 + (ch % CPR) * 8;
-            const uint4 v = (b < b_end && k < a.nC)
-                                ? *reinterpret_cast<const uint4 *>(a.x + (size_t)b * a.nC + k) : zero4;
+            const bool ok = b < b_end && k < a.nC;
+            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(a.x + (ok ? (size_t)b * a.nC + k : 0)), ok);
             *reinterpret_cast<uint4 *>(x_s + (size_t)bl * LD + (ch % CPR) * 8) = v;
         }
         __syncthreads();
@@ -107,8 +106,9 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
 #pragma unroll
                 for (int ks = 0; ks < 2 * NSB; ks++) {
                     const bool ok = sb + ks * 16 < b_end;
-                    ah[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + ks * 512) : zero4;
-                    al[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + ks * 512 + (size_t)a.DP * a.BP) : zero4;
+                    const bf16_t *apk = ok ? ap + ks * 512 : a.dPT;
+                    ah[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk), ok);
+                    al[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk + (size_t)a.DP * a.BP), ok);
                 }
 #pragma unroll
                 for (int ks = 0; ks < 2 * NSB; ks++) {
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
 #pragma unroll
                 for (int ks = 0; ks < 2 * TPW * 4 / NTK; ks++) {
                     if (ks < 2 * NTD) {
-                        const uint4 av = b < b_end ? *reinterpret_cast<const uint4 *>(dprow + ks * 512) : zero4;
+                        const uint4 av = load16_masked(reinterpret_cast<const uint4 *>(dprow + ks * 512), b < b_end);
                         o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
                                                                     phif[ks], o, 0, 0, 0);
                     }
@@ -142,8 +142,10 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
                     uint4 av[8];
 #pragma unroll
                     for (int u = 0; u < 8; u++)
-                        av[u] = (b < b_end && ks0 + u < 2 * NTD)
-                                    ? *reinterpret_cast<const uint4 *>(dprow + (ks0 + u) * 512) : zero4;
+                    {
+                        const bool ok = b < b_end && ks0 + u < 2 * NTD;
+                        av[u] = load16_masked(reinterpret_cast<const uint4 *>(ok ? dprow + (ks0 + u) * 512 : a.dPb), ok);
+                    }
 #pragma unroll
                     for (int u = 0; u < 8; u++) {
                         if (ks0 + u < 2 * NTD) {

@@ -58,7 +58,6 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
     const int NTD = a.DP / 32;
     const int b_begin = blockIdx.z * a.b_per_split;
     const int b_end = min(a.B, b_begin + a.b_per_split);
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
 
     f32x16_t acc[kPL_TPW];
 #pragma unroll
@@ -70,8 +69,8 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
         if (sb != b_begin) __syncthreads();
         for (int ch = tid; ch < kPL_SB * (kPL_KW / 8); ch += 256) {
             const int bl = ch / (kPL_KW / 8), b = sb + bl, kc = (ch % (kPL_KW / 8)) * 8;
-            const uint4 v = (b < b_end && k0 + kc < a.nC)
-                                ? *reinterpret_cast<const uint4 *>(a.x + (size_t)b * a.nC + k0 + kc) : zero4;
+            const bool ok = b < b_end && k0 + kc < a.nC;
+            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(a.x + (ok ? (size_t)b * a.nC + k0 + kc : 0)), ok);
             *reinterpret_cast<uint4 *>(x_s + (size_t)bl * kPL_LD + kc) = v;
         }
         __syncthreads();
@@ -87,8 +86,9 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
 #pragma unroll
                 for (int ks = 0; ks < 8; ks++) {
                     const bool ok = sb + ks * 16 < b_end;  // pad columns [B, BP) are zero
-                    ah[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + ks * 512) : zero4;
-                    al[ks] = ok ? *reinterpret_cast<const uint4 *>(ap + ks * 512 + (size_t)a.DP * a.BP) : zero4;
+                    const bf16_t *apk = ok ? ap + ks * 512 : a.dPT;
+                    ah[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk), ok);
+                    al[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk + (size_t)a.DP * a.BP), ok);
                 }
 #pragma unroll
                 for (int ks = 0; ks < 8; ks++) {
@@ -130,30 +130,37 @@ __global__ __launch_bounds__(256) void dxflat_large_kernel(ProjBwdLargeArgs a, i
     const int st = (id >> 3) % tiles_s;
     if (slab >= slabs) return;
     const int k0 = slab * kPL_KW;
-    const int b = st * 32 + row;
-    const bool bok = b < a.B;
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
     const int nchunks = (a.DP + kPL_DC - 1) / kPL_DC;
     const bf16_t *dprow = a.dPb + frag_base(st, a.DP >> 4, 0) + lane * 8;  // + 512 per k-step
 
-    // this thread's four 16-byte pieces of a phi chunk: rows (tid >> 4) + 16 h, column piece tid & 15
+    // this thread's four 16-byte pieces of a phi chunk: rows (tid >> 4) + 16 h, column piece tid & 15.
+    // The prefetching loads carry no predicate (it would be applied right behind the load and stall
+    // the prefetch): out-of-range pieces alias valid memory and are zeroed when they are parked in
+    // LDS; the dP operand then only needs to be finite where phi is zero, so its out-of-range
+    // k-steps alias k-step 0.
     auto load_phi = [&](int c, uint4 (&v)[4]) {
 #pragma unroll
         for (int h = 0; h < 4; h++) {
             const int d = c * kPL_DC + (tid >> 4) + 16 * h, k = k0 + (tid & 15) * 8;
-            v[h] = (d < a.D && k < a.nC) ? *reinterpret_cast<const uint4 *>(a.phi + (size_t)d * a.nC + k) : zero4;
+            const bool ok = d < a.D && k < a.nC;
+            v[h] = *reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * a.nC + k : 0));
         }
     };
-    auto store_phi = [&](bf16_t *buf, const uint4 (&v)[4]) {
+    auto store_phi = [&](bf16_t *buf, int c, const uint4 (&v)[4]) {
 #pragma unroll
-        for (int h = 0; h < 4; h++)
-            *reinterpret_cast<uint4 *>(buf + (size_t)((tid >> 4) + 16 * h) * kPL_LD + (tid & 15) * 8) = v[h];
+        for (int h = 0; h < 4; h++) {
+            const int d = c * kPL_DC + (tid >> 4) + 16 * h, k = k0 + (tid & 15) * 8;
+            const bool ok = d < a.D && k < a.nC;
+            uint4 t = v[h];
+            t.x = ok ? t.x : 0u; t.y = ok ? t.y : 0u; t.z = ok ? t.z : 0u; t.w = ok ? t.w : 0u;
+            *reinterpret_cast<uint4 *>(buf + (size_t)((tid >> 4) + 16 * h) * kPL_LD + (tid & 15) * 8) = t;
+        }
     };
     auto load_a = [&](int c, uint4 (&v)[4]) {
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             const int d0 = c * kPL_DC + ks * 16;
-            v[ks] = (bok && d0 < a.DP) ? *reinterpret_cast<const uint4 *>(dprow + (size_t)(d0 >> 4) * 512) : zero4;
+            v[ks] = *reinterpret_cast<const uint4 *>(dprow + (d0 < a.DP ? (size_t)(d0 >> 4) * 512 : 0));
         }
     };
 
@@ -163,7 +170,7 @@ __global__ __launch_bounds__(256) void dxflat_large_kernel(ProjBwdLargeArgs a, i
     uint4 pv[4], av[4], an[4];
     load_phi(0, pv);
     load_a(0, av);
-    store_phi(phi_s0, pv);
+    store_phi(phi_s0, 0, pv);
     __syncthreads();
     for (int c = 0; c < nchunks; c++) {
         const bool more = c + 1 < nchunks;
@@ -175,7 +182,7 @@ __global__ __launch_bounds__(256) void dxflat_large_kernel(ProjBwdLargeArgs a, i
             o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av[ks]), pf, o, 0, 0, 0);
         }
         if (more) {
-            store_phi(nxt, pv);
+            store_phi(nxt, c + 1, pv);
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) av[ks] = an[ks];
         }

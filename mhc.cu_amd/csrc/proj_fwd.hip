@@ -103,7 +103,6 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[t][i] = 0.f;
     float ssq = 0.f;
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
 
     constexpr int U = 4;  // k-steps in flight
     for (int k0 = kbeg; k0 < kend; k0 += 16 * U) {
@@ -114,9 +113,10 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
             // 128-byte line for U = 4); A and B use the same k grouping, which is all MFMA needs
             const int k = k0 + kh * (8 * U) + u * 8;
             const bool kv = k < kend;  // kend and k are multiples of 8
-            av[u] = (kv && bvalid) ? xrow[k >> 3] : zero4;
+            const int off = kv ? (k >> 3) : 0;
+            av[u] = load16_masked(xrow + off, kv && bvalid);
 #pragma unroll
-            for (int t = 0; t < NT; t++) bv[u][t] = (kv && dvalid[t]) ? prow[t][k >> 3] : zero4;
+            for (int t = 0; t < NT; t++) bv[u][t] = load16_masked(prow[t] + off, kv && dvalid[t]);
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
@@ -175,6 +175,187 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
 }
 
 // --------------------------------------------------------------------------------------------
+// MFMA path for wide projections (phi is the big operand, n > 8).
+//
+// Loads where every lane addresses a different row (the MFMA operand layout) are served at a
+// fraction of the L1 rate, so here both operands are fetched with row-contiguous loads (8 lanes
+// per 128-byte line), parked in LDS and read back in MFMA layout.
+//   workgroup tile: 128 samples x (NT * 64) projection rows, K chunks of 64 elements
+//   4 waves as 2 x 2: a wave owns 64 samples x NT*32 rows (2 x NT accumulator tiles)
+//   P chunks of global loads are in flight per thread (register FIFO) ahead of the chunk being
+//   multiplied; LDS is double-buffered, one barrier per chunk.
+// Workgroups that read the same K slab sit on the same XCD (workgroup id modulo 8 selects the
+// XCD): the slab of x is pulled into that L2 once and the other row groups hit it there.
+// grid.x = 8 * groups * sample_groups * ceil(KS / 8)
+// --------------------------------------------------------------------------------------------
+constexpr int kWideLd = 72;  // LDS row stride in bf16 elements: 128 data bytes + 16 pad
+
+template <int NT, int P>
+__global__ __launch_bounds__(256) void proj_fwd_wide_kernel(const bf16_t *__restrict__ x,
+                                                            const bf16_t *__restrict__ phi,
+                                                            float *__restrict__ Ppart,
+                                                            float *__restrict__ ssqpart, int B,
+                                                            int D, int DP, int nC, int groups,
+                                                            int sgroups, int KS,
+                                                            int cpk /* chunks per K slab */) {
+    static_assert(P % 2 == 0, "buffer parity is tied to the FIFO slot");
+    constexpr int R = NT * 64;   // projection rows per workgroup
+    constexpr int XJ = 4;        // 16-byte segments of the x tile per thread (128 rows x 8 / 256)
+    constexpr int PJ = R / 32;   // same for the phi tile
+    extern __shared__ __align__(16) bf16_t lds_w[];  // [2][128 + R][kWideLd]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row = lane & 31, kh = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int group = slot % groups;
+    const int sg = (slot / groups) % sgroups;
+    const int ks = (slot / (groups * sgroups)) * 8 + xcd;
+    if (ks >= KS) return;  // whole workgroup, before any barrier
+    const int nch_all = (nC + 63) / 64;
+    const int cbeg = ks * cpk, cend = min(cbeg + cpk, nch_all);
+    const bool want_ssq = group == 0;
+
+    // global -> register stage: thread owns segment `seg` of rows lrow + 32 j
+    const int lrow = tid >> 3, seg = tid & 7;
+    const uint4 *xg[XJ], *pg[PJ];
+    bool xv[XJ], pv[PJ];
+#pragma unroll
+    for (int j = 0; j < XJ; j++) {
+        const int b = sg * 128 + lrow + 32 * j;
+        xv[j] = b < B;
+        xg[j] = reinterpret_cast<const uint4 *>(x + (size_t)(xv[j] ? b : 0) * nC) + seg;
+    }
+#pragma unroll
+    for (int j = 0; j < PJ; j++) {
+        const int d = group * R + lrow + 32 * j;
+        pv[j] = d < D;
+        pg[j] = reinterpret_cast<const uint4 *>(phi + (size_t)(pv[j] ? d : 0) * nC) + seg;
+    }
+    // No per-lane predicate on the loads: rows beyond B / D alias row 0 (their products are never
+    // stored) and nC % 64 == 0, so a loaded value is not touched until it is parked in LDS and
+    // the loads of all P slots stay in flight.
+    uint4 rg[P][XJ + PJ];  // per slot: XJ segments of x, then PJ of phi
+    auto issue = [&](int slot_, int c) {
+#pragma unroll
+        for (int j = 0; j < PJ; j++) rg[slot_][XJ + j] = pg[j][c * 8];
+#pragma unroll
+        for (int j = 0; j < XJ; j++) rg[slot_][j] = xg[j][c * 8];
+    };
+
+    f32x16_t acc[2][NT];
+#pragma unroll
+    for (int m = 0; m < 2; m++)
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[m][t][i] = 0.f;
+    float ssq[XJ];
+#pragma unroll
+    for (int j = 0; j < XJ; j++) ssq[j] = 0.f;
+
+    // park slot j in LDS buffer j & 1, then multiply that buffer; with prefetch, `next` is the
+    // chunk whose loads refill the slot
+    auto step = [&](int j, int next, auto prefetch) {
+        bf16_t *xs = lds_w + (size_t)(j & 1) * (128 + R) * kWideLd;
+        bf16_t *ps = xs + 128 * kWideLd;
+#pragma unroll
+        for (int q = 0; q < XJ; q++)
+            *reinterpret_cast<uint4 *>(xs + (lrow + 32 * q) * kWideLd + seg * 8) = rg[j][q];
+#pragma unroll
+        for (int q = 0; q < PJ; q++)
+            *reinterpret_cast<uint4 *>(ps + (lrow + 32 * q) * kWideLd + seg * 8) = rg[j][XJ + q];
+        if (want_ssq) {
+#pragma unroll
+            for (int q = 0; q < XJ; q++) {
+                const uint32_t w4[4] = {rg[j][q].x, rg[j][q].y, rg[j][q].z, rg[j][q].w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float lo = bf16lo_to_f32(w4[i]), hi = bf16hi_to_f32(w4[i]);
+                    ssq[q] += lo * lo + hi * hi;
+                }
+            }
+        }
+        __syncthreads();
+        if constexpr (decltype(prefetch)::value) issue(j, next);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            bf16x8_t af[2], bfr[NT];
+#pragma unroll
+            for (int m = 0; m < 2; m++)
+                af[m] = *reinterpret_cast<const bf16x8_t *>(
+                    xs + (wm * 64 + m * 32 + row) * kWideLd + s * 16 + kh * 8);
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+                bfr[t] = *reinterpret_cast<const bf16x8_t *>(
+                    ps + (wn * NT * 32 + t * 32 + row) * kWideLd + s * 16 + kh * 8);
+#pragma unroll
+            for (int m = 0; m < 2; m++)
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    acc[m][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[m], bfr[t], acc[m][t], 0, 0, 0);
+        }
+    };
+
+    // prologue: fill the FIFO (indices beyond the slab are clamped: redundant, never consumed)
+#pragma unroll
+    for (int j = 0; j < P; j++) issue(j, min(cbeg + j, cend - 1));
+    int c = cbeg;
+    for (; c + P <= cend; c += P) {
+#pragma unroll
+        for (int j = 0; j < P; j++) step(j, min(c + j + P, cend - 1), std::true_type{});
+    }
+    const int rem = cend - c;  // < P chunks left, all already in flight
+#pragma unroll
+    for (int j = 0; j < P - 1; j++)
+        if (j < rem) step(j, 0, std::false_type{});
+
+    // accumulator layout of a 32x32 tile: lane -> column (lane & 31),
+    // register i -> row 8 * (i / 4) + 4 * (lane / 32) + (i % 4)
+    float *out = Ppart + (size_t)ks * B * DP;
+#pragma unroll
+    for (int m = 0; m < 2; m++)
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int d = group * R + wn * NT * 32 + t * 32 + row;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int bs = sg * 128 + wm * 64 + m * 32 + 8 * (i >> 2) + 4 * kh + (i & 3);
+                if (bs < B && d < D) out[(size_t)bs * DP + d] = acc[m][t][i];
+            }
+        }
+    if (want_ssq) {
+#pragma unroll
+        for (int j = 0; j < XJ; j++) {
+            float v = ssq[j];  // the 8 lanes of one row are consecutive
+            v += __shfl_xor(v, 1, kWave);
+            v += __shfl_xor(v, 2, kWave);
+            v += __shfl_xor(v, 4, kWave);
+            if (seg == 0 && xv[j]) ssqpart[(size_t)ks * B + sg * 128 + lrow + 32 * j] = v;
+        }
+    }
+}
+
+template <int NT, int P>
+static hipError_t launch_wide(const void *x, const void *phi, float *Ppart, float *ssqpart, int KS,
+                              int B, int D, int DP, int nC, hipStream_t stream) {
+    const int sgroups = (B + 127) / 128;
+    const int groups = (DP + NT * 64 - 1) / (NT * 64);
+    const int nch_all = (nC + 63) / 64;
+    const int cpk = (nch_all + KS - 1) / KS;
+    const int grid = 8 * groups * sgroups * ((KS + 7) / 8);
+    const size_t smem = sizeof(bf16_t) * 2 * (128 + NT * 64) * kWideLd;
+    if (smem > 64 * 1024) {  // above the default dynamic-LDS limit (the CU has 160 KB)
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&proj_fwd_wide_kernel<NT, P>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return e;
+    }
+    proj_fwd_wide_kernel<NT, P><<<grid, 256, smem, stream>>>(
+        static_cast<const bf16_t *>(x), static_cast<const bf16_t *>(phi), Ppart, ssqpart, B, D, DP,
+        nC, groups, sgroups, KS, cpk);
+    return hipGetLastError();
+}
+
+// --------------------------------------------------------------------------------------------
 // shape-dependent split and launch
 // --------------------------------------------------------------------------------------------
 static int mfma_nt(int n) {
@@ -182,11 +363,28 @@ static int mfma_nt(int n) {
     return tiles <= 4 ? tiles : 2;
 }
 
+// wide projections (more than four 32-row tiles) with whole 64-element K chunks take the
+// LDS-staged kernel
+static bool use_wide(int n, int C) { return padded_D(n) / 32 > 4 && (n * C) % 64 == 0; }
+
 int proj_fwd_ksplit(int x_dtype, int phi_dtype, int B, int n, int C) {
     // The generic path always uses one split.  MFMA path: enough workgroups to fill 256 CUs
     // several times over (the K loop is latency-bound per wave), at least 64 K elements per wave.
     if (!use_mfma(x_dtype, phi_dtype, C)) return 1;
     const int nC = n * C, DP = padded_D(n);
+    if (use_wide(n, C)) {
+        // ~1.6 workgroups per CU; a slab is at least 8 chunks; the partial sums (written here, read
+        // by the coefficient kernel) stay below ~1/4 of the bytes streamed
+        const int wgs = ((DP + 63) / 64) * ((B + 127) / 128);
+        int ks = (410 + wgs / 2) / wgs;
+        const int cap_chunks = nC / 64 / 8;
+        const int cap_bytes = (int)(0.25 * (2.0 * B * nC + 2.0 * DP * nC) / (8.0 * B * DP));
+        if (ks > cap_chunks) ks = cap_chunks;
+        if (ks > cap_bytes) ks = cap_bytes;
+        if (ks > 64) ks = 64;
+        if (ks < 1) ks = 1;
+        return ks;
+    }
     const int tiles_s = (B + 31) / 32;
     const int groups = DP / 32 / mfma_nt(n);
     int ks = (1024 + tiles_s * groups - 1) / (tiles_s * groups);
@@ -227,6 +425,7 @@ hipError_t launch_proj_fwd(const void *x, int x_dtype, const void *phi, int phi_
                            float *ssqpart, int KS, int B, int n, int C, hipStream_t stream) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
     if (use_mfma(x_dtype, phi_dtype, C)) {
+        if (use_wide(n, C)) return launch_wide<1, 4>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
         switch (mfma_nt(n)) {
             case 1: return launch_mfma<1>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
             case 2: return launch_mfma<2>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
