@@ -115,6 +115,45 @@ __device__ __forceinline__ void store_vec(T *__restrict__ p, const float (&v)[V]
     }
 }
 
+// V consecutive elements kept exactly as loaded.  No conversion instruction sits behind the load,
+// so a batch of loads stays in flight across whatever code follows (another basic block
+// included); get() widens to fp32 at the point of use.  The pointer must be dereferenceable and
+// aligned to min(V * sizeof(T), 16) bytes: callers clamp out-of-range indices to a valid element
+// instead of branching around the load.
+template <typename T, int V> struct RawVec {
+    static constexpr int kBytes = V * (int)sizeof(T);
+    static constexpr int kWords = (kBytes + 3) / 4;
+    uint32_t w[kWords];
+    __device__ __forceinline__ void load(const T *__restrict__ p) {
+        if constexpr (kBytes % 16 == 0) {
+#pragma unroll
+            for (int i = 0; i < kBytes / 16; i++) {
+                const uint4 t = reinterpret_cast<const uint4 *>(p)[i];
+                w[4 * i] = t.x; w[4 * i + 1] = t.y; w[4 * i + 2] = t.z; w[4 * i + 3] = t.w;
+            }
+        } else if constexpr (kBytes == 8) {
+            const uint2 t = *reinterpret_cast<const uint2 *>(p);
+            w[0] = t.x; w[1] = t.y;
+        } else if constexpr (kBytes == 4) {
+            w[0] = *reinterpret_cast<const uint32_t *>(p);
+        } else {
+            static_assert(kBytes == 2, "unsupported vector width");
+            w[0] = *reinterpret_cast<const uint16_t *>(p);
+        }
+    }
+    __device__ __forceinline__ void get(float (&v)[V]) const {
+        if constexpr (std::is_same<T, float>::value) {
+#pragma unroll
+            for (int i = 0; i < V; i++) v[i] = __uint_as_float(w[i]);
+        } else if constexpr (V == 1) {
+            v[0] = bf16lo_to_f32(w[0]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V / 2; i++) { v[2 * i] = bf16lo_to_f32(w[i]); v[2 * i + 1] = bf16hi_to_f32(w[i]); }
+        }
+    }
+};
+
 // 16-byte global load that yields zeros when !ok.  `p` must be dereferenceable either way (callers
 // clamp the index): the load is unconditional and the value is masked afterwards, which keeps the
 // code free of per-lane branches.  Do NOT write `ok ? *p : zero_variable`: the compiler then selects

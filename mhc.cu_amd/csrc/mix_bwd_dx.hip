@@ -65,16 +65,14 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
             hpre[i] = i < n ? Hpre[i] : 0.f;
             hpost[i] = i < n ? Hpost[i] : 0.f;
         }
+        // streams >= n alias stream 0 (no branch around the loads, so all of them are in flight
+        // together); they only ever meet zero coefficients
         float gv[NP][V], xv[NP][V];
 #pragma unroll
         for (int i = 0; i < NP; i++) {
-            if (i < n) {
-                load_vec<TG, V>(gb + (size_t)i * C + c, gv[i]);
-                load_vec<TX, V>(xb + (size_t)i * C + c, xv[i]);
-            } else {
-#pragma unroll
-                for (int v = 0; v < V; v++) { gv[i][v] = 0.f; xv[i][v] = 0.f; }
-            }
+            const size_t so = (size_t)(i < n ? i : 0) * C + c;
+            load_vec<TG, V>(gb + so, gv[i]);
+            load_vec<TX, V>(xb + so, xv[i]);
         }
         float da[V], dfv[V], uv[V];
 #pragma unroll

@@ -123,13 +123,11 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
         float gv[NP][V], xv[NP][V];
 #pragma unroll
         for (int i = 0; i < NP; i++) {
-            if (i < n) {
-                load_vec<TG, V>(gb + (size_t)i * C + c, gv[i]);
-                load_vec<TX, V>(xb + (size_t)i * C + c, xv[i]);
-            } else {
-#pragma unroll
-                for (int v = 0; v < V; v++) { gv[i][v] = 0.f; xv[i][v] = 0.f; }
-            }
+            // streams >= n alias stream 0 (no branch around the loads): their sums land in entries
+            // of acc that nobody reads, and they meet zero coefficients everywhere else
+            const size_t so = (size_t)(i < n ? i : 0) * C + c;
+            load_vec<TG, V>(gb + so, gv[i]);
+            load_vec<TX, V>(xb + so, xv[i]);
         }
         float av[V], fv[V], dfw[V];
         if (inject) load_vec<TX, V>(static_cast<const TX *>(a.f_inject) + (size_t)b * C + c, fv);
@@ -404,12 +402,20 @@ __device__ __forceinline__ float bwd_large_phase0(const BwdReduceArgs &a, const 
         float sa[V], sdf[V];
 #pragma unroll
         for (int v = 0; v < V; v++) { sa[v] = 0.f; sdf[v] = 0.f; }
-        for (int i = 0; i < n; i++) {
-            float xv[V], gv[V];
-            load_vec<TX, V>(xb + (size_t)i * C + c, xv);
-            load_vec<TG, V>(gb + (size_t)i * C + c, gv);
+        for (int i0 = 0; i0 < n; i0 += 8) {  // 16 loads in flight; streams >= n alias stream 0
+            float xv[8][V], gv[8][V];
 #pragma unroll
-            for (int v = 0; v < V; v++) { sa[v] += hp_s[i] * xv[v]; sdf[v] += ho_s[i] * gv[v]; }
+            for (int u = 0; u < 8; u++) {
+                const size_t so = (size_t)(i0 + u < n ? i0 + u : 0) * C + c;
+                load_vec<TX, V>(xb + so, xv[u]);
+                load_vec<TG, V>(gb + so, gv[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const float hp = i0 + u < n ? hp_s[i0 + u] : 0.f, ho = i0 + u < n ? ho_s[i0 + u] : 0.f;
+#pragma unroll
+                for (int v = 0; v < V; v++) { sa[v] += hp * xv[u][v]; sdf[v] += ho * gv[u][v]; }
+            }
         }
         float fv[V];
         if (inject) load_vec<TX, V>(static_cast<const TX *>(a.f_inject) + (size_t)b * C + c, fv);

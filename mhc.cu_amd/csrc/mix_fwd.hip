@@ -60,12 +60,12 @@ __global__ __launch_bounds__(256) void mix_fwd_kernel(MixFwdArgs a) {
             for (int v = 0; v < V; v++) acc[v] = 0.f;
 #pragma unroll
             for (int i = 0; i < NP; i++) {
-                if (i < n) {
-                    float xv[V];
-                    load_vec<TX, V>(xb + (size_t)i * C + c, xv);
+                // streams >= n alias stream 0 and meet hpre = 0: no branch around the loads, so
+                // all of them are in flight together
+                float xv[V];
+                load_vec<TX, V>(xb + (size_t)(i < n ? i : 0) * C + c, xv);
 #pragma unroll
-                    for (int v = 0; v < V; v++) acc[v] += hpre[i] * xv[v];
-                }
+                for (int v = 0; v < V; v++) acc[v] += hpre[i] * xv[v];
             }
 #pragma unroll
             for (int v = 0; v < V; v++) {
@@ -98,14 +98,7 @@ __global__ __launch_bounds__(256) void mix_fwd_kernel(MixFwdArgs a) {
         }
         float xv[NP][V];
 #pragma unroll
-        for (int j = 0; j < NP; j++) {
-            if (j < n) {
-                load_vec<TX, V>(xb + (size_t)j * C + c, xv[j]);
-            } else {
-#pragma unroll
-                for (int v = 0; v < V; v++) xv[j][v] = 0.f;
-            }
-        }
+        for (int j = 0; j < NP; j++) load_vec<TX, V>(xb + (size_t)(j < n ? j : 0) * C + c, xv[j]);
 #pragma unroll
         for (int i = 0; i < NP; i++) {
             if (i < n) {
@@ -169,43 +162,42 @@ __global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
     float t_ssq[4], t_pre[4], t_post[4], t_e[4][SK::EPL];
     const size_t ps = (size_t)a.B * a.DP;
     const float *Pb = dyn ? a.Ppart + (size_t)b * a.DP : nullptr;
+    // None of these loads sits behind a per-lane branch or is touched before step 2 / step 3: out of
+    // range indices alias element 0 and are discarded where the value is used.
     if (tid < 64) {
         if (dyn) { al0 = a.alpha[0]; al1 = a.alpha[1]; al2 = a.alpha[2]; }
-        if (g < n) { bpre = a.b_pre[g]; bpost = a.b_post[g]; }
+        const int gc = g < n ? g : 0;
+        bpre = a.b_pre[gc]; bpost = a.b_post[gc];
 #pragma unroll
-        for (int e = 0; e < SK::EPL; e++) bres[e] = (r0 < n && c0 + e < n) ? a.b_res[r0 * n + c0 + e] : 0.f;
+        for (int e = 0; e < SK::EPL; e++) bres[e] = a.b_res[(r0 < n && c0 + e < n) ? r0 * n + c0 + e : 0];
+        if (dyn) {
 #pragma unroll
-        for (int u = 0; u < 4; u++) {  // first batch of K-split partials: ks = part*4 + u
-            const int ks = part * 4 + u;
-            const bool ok = dyn && ks < a.KS;
-            t_ssq[u] = ok ? a.ssqpart[(size_t)ks * a.B + b] : 0.f;
-            t_pre[u] = (ok && g < n) ? Pb[ks * ps + g] : 0.f;
-            t_post[u] = (ok && g < n) ? Pb[ks * ps + n + g] : 0.f;
+            for (int u = 0; u < 4; u++) {  // first batch of K-split partials: ks = part*4 + u
+                const int ks = part * 4 + u;
+                const size_t ko = ks < a.KS ? ks : 0;
+                t_ssq[u] = a.ssqpart[ko * a.B + b];
+                t_pre[u] = Pb[ko * ps + gc];
+                t_post[u] = Pb[ko * ps + n + gc];
 #pragma unroll
-            for (int e = 0; e < SK::EPL; e++)
-                t_e[u][e] = (ok && r0 < n && c0 + e < n) ? Pb[ks * ps + 2 * n + r0 * n + c0 + e] : 0.f;
-        }
-    }
-    float xv[CPT][NP][V];
-#pragma unroll
-    for (int k = 0; k < CPT; k++) {
-        const int ch = tid + k * 256;
-#pragma unroll
-        for (int i = 0; i < NP; i++) {
-            if (ch < nch && i < n) {
-                load_vec<TX, V>(xb + (size_t)i * C + ch * V, xv[k][i]);
-            } else {
-#pragma unroll
-                for (int v = 0; v < V; v++) xv[k][i][v] = 0.f;
+                for (int e = 0; e < SK::EPL; e++)
+                    t_e[u][e] = Pb[ko * ps + ((r0 < n && c0 + e < n) ? 2 * n + r0 * n + c0 + e : 0)];
             }
         }
     }
-    float fin[CPT][V];
+    RawVec<TX, V> xr[CPT][NP];
+#pragma unroll
+    for (int k = 0; k < CPT; k++) {
+        const int ch = tid + k * 256;
+        const TX *xc = xb + (size_t)(ch < nch ? ch : 0) * V;
+#pragma unroll
+        for (int i = 0; i < NP; i++) xr[k][i].load(xc + (size_t)(i < n ? i : 0) * C);
+    }
+    RawVec<TX, V> fr[CPT];
     if (inject) {
 #pragma unroll
         for (int k = 0; k < CPT; k++) {
             const int ch = tid + k * 256;
-            if (ch < nch) load_vec<TX, V>(static_cast<const TX *>(a.f_inject) + (size_t)b * C + ch * V, fin[k]);
+            fr[k].load(static_cast<const TX *>(a.f_inject) + (size_t)b * C + (size_t)(ch < nch ? ch : 0) * V);
         }
     }
 
@@ -217,9 +209,12 @@ __global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
         if (dyn) {
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                ssq += t_ssq[u]; ppre += t_pre[u]; ppost += t_post[u];
+                const bool ok = part * 4 + u < a.KS;
+                ssq += ok ? t_ssq[u] : 0.f;
+                ppre += (ok && g < n) ? t_pre[u] : 0.f;
+                ppost += (ok && g < n) ? t_post[u] : 0.f;
 #pragma unroll
-                for (int e = 0; e < SK::EPL; e++) pe[e] += t_e[u][e];
+                for (int e = 0; e < SK::EPL; e++) pe[e] += (ok && r0 < n && c0 + e < n) ? t_e[u][e] : 0.f;
             }
             for (int ks0 = 16 + part * 4; ks0 < a.KS; ks0 += 16) {  // more than 16 K-splits: rare
 #pragma unroll
@@ -297,20 +292,27 @@ __global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
     }
 
     // ---- 3. aggregate + RMS ------------------------------------------------------------------
+    float xv[CPT][NP][V];
+#pragma unroll
+    for (int k = 0; k < CPT; k++)
+#pragma unroll
+        for (int i = 0; i < NP; i++) xr[k][i].get(xv[k][i]);  // streams >= n meet zero coefficients
     float av[CPT][V];
     float qinv = 1.0f;
     if (!inject) {
         float ssq = 0.f;
 #pragma unroll
-        for (int k = 0; k < CPT; k++)
+        for (int k = 0; k < CPT; k++) {
+            const bool live = tid + k * 256 < nch;  // chunks beyond C alias chunk 0: not counted
 #pragma unroll
             for (int v = 0; v < V; v++) {
                 float s_a = 0.f;
 #pragma unroll
                 for (int i = 0; i < NP; i++) s_a += hpre[i] * xv[k][i][v];
                 av[k][v] = s_a;
-                ssq += s_a * s_a;
+                ssq += live ? s_a * s_a : 0.f;
             }
+        }
         ssq = block_allreduce_sum<256>(ssq, red);
         const float q = sqrtf(ssq / (float)C + a.eps);
         qinv = 1.0f / q;
@@ -326,9 +328,12 @@ __global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
         if (ch < nch) {
             const int c = ch * V;
             float f[V];
+            if (inject) {
+                fr[k].get(f);
+            } else {
 #pragma unroll
-            for (int v = 0; v < V; v++)
-                f[v] = inject ? fin[k][v] : av[k][v] * qinv * load_w(a.w, a.w_bf16, c + v);
+                for (int v = 0; v < V; v++) f[v] = av[k][v] * qinv * load_w(a.w, a.w_bf16, c + v);
+            }
 #pragma unroll
             for (int i = 0; i < NP; i++) {
                 if (i < n) {
