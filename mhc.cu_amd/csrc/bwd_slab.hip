@@ -179,6 +179,23 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
             al[ks] = *reinterpret_cast<const uint4 *>(ap + (size_t)32 * a.BP);
             ap2[ks] = *reinterpret_cast<const uint4 *>(a.dPb + frag_base(sb >> 5, 2, ks) + lane * 8);
         }
+        // this thread's sample coefficients for phase C: asked for here so that they arrive behind
+        // the barriers and the matrix-core phase (slots beyond the split alias sample 0, streams
+        // >= n alias stream 0; both are discarded below)
+        float hpre[kSlabNS], hpost[kSlabNS], Mr[kSlabNS][kSlabNS], cxv, qv = 1.f, s1v = 0.f;
+        {
+            const size_t bc = bok ? b : 0;
+#pragma unroll
+            for (int i = 0; i < kSlabNS; i++) {
+                hpre[i] = a.Hpre[bc * n + (i < n ? i : 0)];
+                hpost[i] = a.Hpost[bc * n + (i < n ? i : 0)];
+#pragma unroll
+                for (int j = 0; j < kSlabNS; j++)
+                    Mr[i][j] = a.M[bc * n * n + ((i < n && j < n) ? i * n + j : 0)];
+            }
+            cxv = a.cx[bc];
+            if (!inject) { qv = a.q[bc]; s1v = a.s1[bc]; }
+        }
         // x tile -> LDS
 #pragma unroll
         for (int j = 0; j < kSlabNS; j++)
@@ -226,19 +243,17 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
         const bool more = sb + 32 < b_end;
         if (more) load_tile(sb + 32, nxt);
         if (bok) {
-            float hpre[kSlabNS], hpost[kSlabNS], Mr[kSlabNS][kSlabNS], qinv = 0.f, k2 = 0.f;
+            float qinv = 0.f, k2 = 0.f;
 #pragma unroll
             for (int i = 0; i < kSlabNS; i++) {
-                hpre[i] = i < n ? a.Hpre[(size_t)b * n + i] : 0.f;
-                hpost[i] = i < n ? a.Hpost[(size_t)b * n + i] : 0.f;
+                if (i >= n) { hpre[i] = 0.f; hpost[i] = 0.f; }
 #pragma unroll
                 for (int j = 0; j < kSlabNS; j++)
-                    Mr[i][j] = (i < n && j < n) ? a.M[(size_t)b * n * n + i * n + j] : 0.f;
+                    if (i >= n || j >= n) Mr[i][j] = 0.f;
             }
-            const float cxv = a.cx[b];
             if (!inject) {
-                qinv = 1.0f / a.q[b];
-                k2 = a.s1[b] * qinv * qinv * qinv / (float)C;
+                qinv = 1.0f / qv;
+                k2 = s1v * qinv * qinv * qinv / (float)C;
             }
             float dfv[8];
             // two halves of four channels keep the live unpacked values small
