@@ -73,7 +73,7 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
     w.s1 = c.floats(B);
     w.u = c.floats((size_t)B * C);
     w.dtpart = c.floats((size_t)B * (D + 3));
-    w.raw = c.floats(n <= 8 ? (size_t)B * bwd_reduce_parts(B, n, C) * (8 * 8 + 3 * 8 + 1) : 0);
+    w.raw = c.floats(bwd_reduce_raw_floats(B, n, C));
     int bs = dphi_batch_splits(B, n, C);
     const int bs2 = proj_bwd_batch_splits(B, n, C);
     if (bs2 > bs) bs = bs2;
@@ -89,7 +89,7 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
 
 // ---- static workspace layout -----------------------------------------------------------------
 struct StaFwdWs { float *Hpre, *Hpost, *M, *q; size_t bytes; };
-struct StaBwdWs { float *red, *s1, *u, *red_sum, *cs_red, *cs_u; size_t bytes; };
+struct StaBwdWs { float *red, *s1, *u, *red_sum, *cs_red, *cs_u, *raw; size_t bytes; };
 
 StaFwdWs carve_sta_fwd(void *ws, int B, int n) {
     Carver c(ws);
@@ -109,6 +109,7 @@ StaBwdWs carve_sta_bwd(void *ws, int B, int n, int C) {
     w.red_sum = c.floats(D);
     w.cs_red = c.floats(colsum_workspace_floats(B, D));
     w.cs_u = c.floats(colsum_workspace_floats(B, C));
+    w.raw = c.floats(n > 8 ? bwd_reduce_raw_floats(B, n, C) : 0);
     w.bytes = c.off;
     return w;
 }
@@ -293,7 +294,7 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
     const int D = n * n + 2 * n;
     BwdCoefOut out{nullptr, nullptr, nullptr, ws.s1, ws.red, nullptr, nullptr, 0};
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
-                                     0, q, nullptr, nullptr, nullptr, nullptr, out, nullptr, B, n, C,
+                                     0, q, nullptr, nullptr, nullptr, nullptr, out, n > 8 ? ws.raw : nullptr, B, n, C,
                                      iters, eps, st));
     MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, 0,
                                  q, ws.s1, nullptr, nullptr, 0, nullptr, 0, nullptr, dx, df, ws.u, nullptr,

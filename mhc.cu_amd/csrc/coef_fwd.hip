@@ -23,9 +23,16 @@ struct CoefArgs {
     float eps;
 };
 
+// eight loads in flight per round (a plain loop would pay one memory latency per split)
 __device__ __forceinline__ float reduce_partials(const float *part, int KS, size_t stride, size_t idx) {
     float acc = 0.f;
-    for (int k = 0; k < KS; k++) acc += part[k * stride + idx];
+    for (int k0 = 0; k0 < KS; k0 += 8) {
+        float t[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) t[q] = part[(size_t)(k0 + q < KS ? k0 + q : 0) * stride + idx];
+#pragma unroll
+        for (int q = 0; q < 8; q++) acc += k0 + q < KS ? t[q] : 0.f;
+    }
     return acc;
 }
 
@@ -72,13 +79,13 @@ template <int NP> __global__ __launch_bounds__(64) void coef_fwd_small_kernel(Co
 }
 
 // One workgroup (4 waves) per sample.  All 256 threads finish the split-K sums (D = n^2 + 2n
-// logits, KS partial sums each, eight loads in flight per thread), then wave 0 runs Sinkhorn on
-// the matrix in LDS; the other waves only keep the barriers.
+// logits, KS partial sums each, eight loads in flight per thread), then run Sinkhorn with the
+// matrix spread over their registers (SkWg).
 template <int NP> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
-    using SK = SkLds<NP>;
-    __shared__ float lds[SK::forward_floats()];
-    __shared__ float lg[NP * NP + 2 * NP];  // logits: pre | post | res (row-major n x n)
-    float *Es = lds, *u = Es + NP * SK::LD, *v = u + NP;
+    using SK = SkWg<NP>;
+    extern __shared__ float lds[];
+    float *lg = lds;                       // [NP*NP + 2*NP] logits: pre | post | res (row-major n x n)
+    float *sk_s = lg + NP * NP + 2 * NP;   // SK::lds_floats(T)
     const int tid = threadIdx.x;
     const int b = blockIdx.x;
     const int n = a.n, D = n * n + 2 * n;
@@ -92,41 +99,59 @@ template <int NP> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(Coe
         if (tid == 0) a.r[b] = r;
     }
     const size_t pstride = (size_t)a.B * a.DP;
-    for (int d = tid; d < D; d += 256) {
-        const int grp = alpha_group(d, n);
-        const float bias = grp == 0 ? a.b_pre[d] : (grp == 1 ? a.b_post[d - n] : a.b_res[d - 2 * n]);
-        float t = bias;
-        if (dyn) {
-            const float *pp = a.Ppart + (size_t)b * a.DP + d;
-            float acc = 0.f;
-            for (int k0 = 0; k0 < a.KS; k0 += 8) {
-                float tv[8];
+    // logits d = tid + 256 m; the partial sums of all of a thread's logits are fetched together,
+    // 4 splits at a time (out-of-range slots alias element 0 and are discarded)
+    constexpr int MD = (NP * NP + 2 * NP + 255) / 256;
+    float psum[MD];
 #pragma unroll
-                for (int q = 0; q < 8; q++) tv[q] = k0 + q < a.KS ? pp[(size_t)(k0 + q) * pstride] : 0.f;
+    for (int m = 0; m < MD; m++) psum[m] = 0.f;
+    if (dyn) {
+        const float *pb = a.Ppart + (size_t)b * a.DP;
+        for (int k0 = 0; k0 < a.KS; k0 += 4) {
+            float tv[MD][4];
 #pragma unroll
-                for (int q = 0; q < 8; q++) acc += tv[q];
-            }
-            const float p = acc * rinv;
-            a.P[(size_t)b * D + d] = p;
-            t = al[grp] * p + bias;
+            for (int m = 0; m < MD; m++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int d = tid + 256 * m;
+                    const bool ok = d < D && k0 + q < a.KS;
+                    tv[m][q] = pb[ok ? (size_t)(k0 + q) * pstride + d : 0];
+                }
+#pragma unroll
+            for (int m = 0; m < MD; m++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) psum[m] += (tid + 256 * m < D && k0 + q < a.KS) ? tv[m][q] : 0.f;
         }
-        lg[d] = t;
+    }
+#pragma unroll
+    for (int m = 0; m < MD; m++) {
+        const int d = tid + 256 * m;
+        if (d < D) {
+            const int grp = alpha_group(d, n);
+            const float bias = grp == 0 ? a.b_pre[d] : (grp == 1 ? a.b_post[d - n] : a.b_res[d - 2 * n]);
+            float t = bias;
+            if (dyn) {
+                const float p = psum[m] * rinv;
+                a.P[(size_t)b * D + d] = p;
+                t = al[grp] * p + bias;
+            }
+            lg[d] = t;
+        }
     }
     __syncthreads();
     if (tid < n) {
         a.Hpre[b * n + tid] = sigmoidf_acc(lg[tid]);
         a.Hpost[b * n + tid] = 2.0f * sigmoidf_acc(lg[n + tid]);
     }
-    for (int e = tid; e < NP * NP; e += 256) {
-        const int r0 = e / NP, c = e % NP;
-        Es[r0 * SK::LD + c] = (r0 < n && c < n) ? expf(lg[2 * n + r0 * n + c]) : 0.f;
-    }
-    __syncthreads();
-    SK::forward(Es, u, v, n, a.T, a.eps, nullptr, nullptr, tid);
-    for (int e = tid; e < n * n; e += 256) {
-        const int r0 = e / n, c = e % n;
-        a.M[(size_t)b * n * n + e] = u[r0] * Es[r0 * SK::LD + c] * v[c];
-    }
+    const int r0 = SK::row(tid), c0 = SK::col0(tid);
+    float E[SK::EPL], u, v[SK::EPL];
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++)
+        E[e] = (r0 < n && c0 + e < n) ? expf(lg[2 * n + r0 * n + c0 + e]) : 0.f;
+    SK::forward(E, u, v, n, a.T, a.eps, sk_s, tid);
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++)
+        if (r0 < n && c0 + e < n) a.M[(size_t)b * n * n + r0 * n + c0 + e] = u * E[e] * v[e];
 }
 
 hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int DP,
@@ -139,9 +164,9 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
     else if (n <= 8)
         coef_fwd_small_kernel<8><<<(B + 3) / 4, 64, 0, stream>>>(a);
     else if (n <= 16)
-        coef_fwd_lds_kernel<16><<<B, 256, 0, stream>>>(a);
+        coef_fwd_lds_kernel<16><<<B, 256, sizeof(float) * (16 * 16 + 32 + SkWg<16>::lds_floats(T)), stream>>>(a);
     else
-        coef_fwd_lds_kernel<32><<<B, 256, 0, stream>>>(a);
+        coef_fwd_lds_kernel<32><<<B, 256, sizeof(float) * (32 * 32 + 64 + SkWg<32>::lds_floats(T)), stream>>>(a);
     return hipGetLastError();
 }
 

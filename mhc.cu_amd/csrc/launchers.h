@@ -74,6 +74,7 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
 // raw (optional, dynamic H, n <= 8): scratch of B * bwd_reduce_parts() * (NP*NP + 3*NP + 1) floats;
 // when given, the channel sums and the coefficient backward run as two launches.
 int bwd_reduce_parts(int B, int n, int C);
+size_t bwd_reduce_raw_floats(int B, int n, int C);  // size of `raw` (required for n > 8)
 
 // dx = M^T dy + Hpre (x) da - cx * x  [+ dP phi when phi != nullptr] [+ dx_in when != nullptr;
 // may alias dx], df, and u = df * a / q (the per-sample summand of dw).

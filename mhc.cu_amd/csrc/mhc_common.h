@@ -180,14 +180,30 @@ template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
 
+// v[lane] + v[lane ^ 16] and v[lane] + v[lane ^ 32] in every lane.  v_permlane16_swap exchanges
+// the odd 16-lane rows of its first operand with the even rows of its second, v_permlane32_swap
+// the upper half of the first with the lower half of the second; with the same value in both
+// operands the two results hold each partner pair, so their sum is the exchange-and-add - one
+// VALU instruction instead of a round trip through the LDS crossbar (ds_bpermute).
+__device__ __forceinline__ float xor16_add(float v) {
+    const unsigned b = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor32_add(float v) {
+    const unsigned b = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Sum over all 64 lanes; every lane gets the total.
 __device__ __forceinline__ float wave_allreduce_sum(float v) {
     v += dpp_mov<kDppQuadXor1>(v);
     v += dpp_mov<kDppQuadXor2>(v);
     v += dpp_mov<kDppRowRor4>(v);
     v += dpp_mov<kDppRowRor8>(v);
-    v += __shfl_xor(v, 16, kWave);
-    v += __shfl_xor(v, 32, kWave);
+    v = xor16_add(v);
+    v = xor32_add(v);
     return v;
 }
 

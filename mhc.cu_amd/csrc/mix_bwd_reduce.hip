@@ -12,8 +12,8 @@
 // followed), and dP = dt alpha / r, cx = sum_d dt alpha p / (nC r^2)  (ops.py:327-349).
 //
 // Two layouts: n <= 8 keeps n^2+3n+1 running sums per thread (thread = column chunk);
-// n > 8 computes dM on the matrix cores (one 32x32 tile per sample, operands loaded from
-// global memory in MFMA layout) and the vector sums on the VALU beside it.
+// n > 8 computes three 32x32 Gram matrices per sample on the matrix cores (operands loaded from
+// global memory in MFMA layout) from which all the sums above follow.
 #include "launchers.h"
 #include "sinkhorn_device.h"
 
@@ -272,7 +272,8 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
         const float *rp = raw + (size_t)p * K;
 #pragma unroll
         for (int e = 0; e < SK::EPL; e++) dMe[e] += rp[r0 * NP + c0 + e];
-        if (g < n) { tpost += rp[NP * NP + g]; tA1 += rp[NP * NP + NP + g]; tA2 += rp[NP * NP + 2 * NP + g]; }
+        const int gc = g < n ? g : 0;  // lanes beyond n alias entry 0 (never used): no branch around loads
+        tpost += rp[NP * NP + gc]; tA1 += rp[NP * NP + NP + gc]; tA2 += rp[NP * NP + 2 * NP + gc];
         s1 += rp[K - 1];
     }
     const float *Pb = a.P + (size_t)b * D;
@@ -332,209 +333,278 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
 }
 
 // =============================================================================================
-// n > 8: MFMA layout
+// n > 8: the channel sums as three 32x32 Gram matrices on the matrix cores
+//
+//   dM = dy x^T          W1 = dy diag(w) x^T          XX = x x^T          (contraction over channels)
+// carry everything the coefficient backward needs:
+//   dHpost[i] = sum_j Hpre[j] W1[i][j] / q       A1[j] = sum_i Hpost[i] W1[i][j]
+//   A2[j] = sum_k Hpre[k] XX[k][j]               s1 = sum_ij Hpost[i] Hpre[j] W1[i][j]
+// (with an injected f: W1 is replaced by dy [f; 0 ...]^T, whose column 0 is dHpost; XX is skipped).
+// Launch 1 (grid B x parts): a workgroup takes a column part of one sample; its 4 waves take
+// k-steps round robin and load their operands straight in MFMA layout (row = stream), several
+// steps in flight; the partial Gram matrices go to `raw`.  Both inputs bf16: v_mfma_f32_32x32x16_bf16
+// (dy*w as a rounded value plus remainder, two instructions).  Otherwise fp32 MFMAs (32x32x2) with exact products: the fp32 tier.
+// Launch 2 (grid B): sums the parts, forms the vectors above, then sigmoid derivatives, exact
+// Sinkhorn backward, dP and cx as in the n <= 8 coefficient kernel.
 // =============================================================================================
-// One k-step operand pair: VL consecutive columns of row (lane & 31) of dy and of x; the two lane
-// halves take adjacent column groups.  Both bf16: one v_mfma_f32_32x32x16_bf16 (exact products,
-// fp32 accumulate).  Otherwise VL fp32 MFMAs (32x32x2), bf16 inputs widened exactly.
-template <typename TG, typename TX> struct PairStep {
-    static constexpr bool kBf16 = std::is_same<TG, bf16_t>::value && std::is_same<TX, bf16_t>::value;
-    static constexpr int VL = kBf16 ? 8 : 4;
-    float g[VL], x[VL];
-    uint4 gbits, xbits;
+constexpr int kGramMats = 3;
+constexpr int kGramFloats = kGramMats * 1024;  // per (sample, part), row-major [m][i][j], 32 x 32
 
-    __device__ __forceinline__ void load(const TG *gp, const TX *xp, int c, int C, bool rvalid, bool vec_ok) {
-        if (rvalid && vec_ok && c + VL <= C) {
-            if constexpr (kBf16) {
-                gbits = *reinterpret_cast<const uint4 *>(gp + c);
-                xbits = *reinterpret_cast<const uint4 *>(xp + c);
-                const uint32_t gw[4] = {gbits.x, gbits.y, gbits.z, gbits.w};
-                const uint32_t xw[4] = {xbits.x, xbits.y, xbits.z, xbits.w};
+template <typename TG, typename TX>
+__global__ __launch_bounds__(256) void gram_large_kernel(BwdReduceArgs a) {
+    constexpr bool kBf16 = std::is_same<TG, bf16_t>::value && std::is_same<TX, bf16_t>::value;
+    constexpr int VL = kBf16 ? 8 : 4;  // columns per lane and k-step
+    constexpr int SW = 2 * VL;         // columns per k-step (two lane halves)
+    constexpr int U = 4;               // k-steps in flight per wave
+    extern __shared__ float smem[];
+    float *w_s = smem;  // [cols of this part] fp32 weights (zero beyond C)
+    const int b = blockIdx.x, part = blockIdx.y, n = a.n, C = a.C, tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6, row = lane & 31, kh = lane >> 5;
+    const bool inject = a.f_inject != nullptr;
+    const int nsteps = (C + SW - 1) / SW;
+    const int spp = (nsteps + a.parts - 1) / a.parts;
+    const int s_begin = part * spp, s_end = min(nsteps, s_begin + spp);
+    const int c_begin = s_begin * SW;
+    float *xw = w_s + spp * SW;  // cross-wave scratch [3][kGramMats * 16][64]
+    for (int cc = tid; cc < spp * SW; cc += 256) {
+        const int c = c_begin + cc;
+        w_s[cc] = (c < C && !inject) ? load_w_(a.w, a.w_bf16, c) : 0.f;
+    }
+    __syncthreads();
+
+    // rows >= n alias row 0: they only produce Gram rows / columns that nobody reads
+    const size_t ro = (size_t)(row < n ? row : 0) * C;
+    const TG *grow = static_cast<const TG *>(a.dy) + (size_t)b * n * C + ro;
+    const TX *xrow = static_cast<const TX *>(a.x) + (size_t)b * n * C + ro;
+    const TX *frow = inject ? static_cast<const TX *>(a.f_inject) + (size_t)b * C : xrow;
+
+    f32x16_t acc[kGramMats];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    g[2 * i] = bf16lo_to_f32(gw[i]); g[2 * i + 1] = bf16hi_to_f32(gw[i]);
-                    x[2 * i] = bf16lo_to_f32(xw[i]); x[2 * i + 1] = bf16hi_to_f32(xw[i]);
+    for (int m = 0; m < kGramMats; m++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[m][i] = 0.f;
+
+    auto mfma3 = [&](const float (&g)[VL], const float (&x)[VL], const float (&gw)[VL],
+                     const RawVec<TG, VL> &gr, const RawVec<TX, VL> &xr, bool with_xx) {
+        if constexpr (kBf16) {
+            const bf16x8_t gb = __builtin_bit_cast(bf16x8_t, make_uint4(gr.w[0], gr.w[1], gr.w[2], gr.w[3]));
+            const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, make_uint4(xr.w[0], xr.w[1], xr.w[2], xr.w[3]));
+            // dy * w as a bf16 pair (rounded value + remainder): dHpre is a difference of two
+            // sums built on W1, a single rounding of the products is not enough for it
+            float lo[VL];
+            uint32_t hw[VL / 2];
+#pragma unroll
+            for (int i = 0; i < VL / 2; i++) {
+                hw[i] = pack_bf16x2(gw[2 * i], gw[2 * i + 1]);
+                lo[2 * i] = gw[2 * i] - bf16lo_to_f32(hw[i]);
+                lo[2 * i + 1] = gw[2 * i + 1] - bf16hi_to_f32(hw[i]);
+            }
+            const bf16x8_t gwb = __builtin_bit_cast(bf16x8_t, make_uint4(hw[0], hw[1], hw[2], hw[3]));
+            const bf16x8_t gwl = __builtin_bit_cast(
+                bf16x8_t, make_uint4(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]),
+                                     pack_bf16x2(lo[4], lo[5]), pack_bf16x2(lo[6], lo[7])));
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb, xb, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gwb, xb, acc[1], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gwl, xb, acc[1], 0, 0, 0);
+            if (with_xx) acc[2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xb, xb, acc[2], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VL; i++) {
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(g[i], x[i], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(gw[i], x[i], acc[1], 0, 0, 0);
+                if (with_xx) acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(x[i], x[i], acc[2], 0, 0, 0);
+            }
+        }
+    };
+
+    // full k-steps (every column of the step inside C, rows 16-byte aligned): raw loads, U steps
+    // in flight, nothing conditional per lane
+    const bool vec_ok = C % VL == 0;
+    const int s_full = vec_ok ? min(s_end, C / SW) : s_begin;
+    int s = s_begin + wave;
+    for (; s + 4 * (U - 1) < s_full; s += 4 * U) {
+        RawVec<TG, VL> gr[U];
+        RawVec<TX, VL> xr[U], fr[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int c = (s + 4 * u) * SW + kh * VL;
+            gr[u].load(grow + c);
+            xr[u].load(xrow + c);
+            if (inject) fr[u].load(frow + c);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int cc = (s + 4 * u) * SW + kh * VL - c_begin;
+            float g[VL], x[VL], gw[VL];
+            gr[u].get(g);
+            xr[u].get(x);
+            if (inject) {
+                // B operand = [f; 0; ...]: only lane row 0 carries f, column 0 of the product is dy . f
+                float f[VL];
+                fr[u].get(f);
+                RawVec<TX, VL> fz;
+#pragma unroll
+                for (int i = 0; i < RawVec<TX, VL>::kWords; i++) fz.w[i] = row == 0 ? fr[u].w[i] : 0u;
+#pragma unroll
+                for (int i = 0; i < VL; i++) f[i] = row == 0 ? f[i] : 0.f;
+                if constexpr (kBf16) {
+                    const bf16x8_t gb = __builtin_bit_cast(bf16x8_t, make_uint4(gr[u].w[0], gr[u].w[1], gr[u].w[2], gr[u].w[3]));
+                    const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, make_uint4(xr[u].w[0], xr[u].w[1], xr[u].w[2], xr[u].w[3]));
+                    const bf16x8_t fb = __builtin_bit_cast(bf16x8_t, make_uint4(fz.w[0], fz.w[1], fz.w[2], fz.w[3]));
+                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb, xb, acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb, fb, acc[1], 0, 0, 0);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < VL; i++) {
+                        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(g[i], x[i], acc[0], 0, 0, 0);
+                        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(g[i], f[i], acc[1], 0, 0, 0);
+                    }
                 }
             } else {
-                load_vec<TG, VL>(gp + c, g);
-                load_vec<TX, VL>(xp + c, x);
+#pragma unroll
+                for (int i = 0; i < VL; i++) gw[i] = g[i] * w_s[cc + i];
+                mfma3(g, x, gw, gr[u], xr[u], true);
+            }
+        }
+    }
+    // remaining steps of this wave (fewer than U full ones, a ragged last step, unaligned rows):
+    // element-wise masked loads, fp32 operands rounded where the bf16 instruction needs them
+    for (; s < s_end; s += 4) {
+        const int c = s * SW + kh * VL, cc = c - c_begin;
+        float g[VL], x[VL], gw[VL], f[VL];
+#pragma unroll
+        for (int i = 0; i < VL; i++) {
+            const bool ok = c + i < C;
+            g[i] = ok ? to_f32<TG>(grow[c + i]) : 0.f;
+            x[i] = ok ? to_f32<TX>(xrow[c + i]) : 0.f;
+            f[i] = (ok && inject && row == 0) ? to_f32<TX>(frow[c + i]) : 0.f;
+            gw[i] = inject ? f[i] : g[i] * w_s[cc + i];
+        }
+        if constexpr (kBf16) {
+            auto pack8 = [](const float (&v)[VL]) {
+                return __builtin_bit_cast(bf16x8_t, make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]),
+                                                               pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7])));
+            };
+            const bf16x8_t gb = pack8(g), xb = pack8(x), sb = pack8(gw);  // g, x, f came from bf16: exact
+            float lo[VL];
+#pragma unroll
+            for (int i = 0; i < VL; i++) lo[i] = gw[i] - bf16_to_f32(f32_to_bf16(gw[i]));
+            if (!inject) acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pack8(lo), xb, acc[1], 0, 0, 0);
+            if (inject) {
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb, xb, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb, sb, acc[1], 0, 0, 0);
+            } else {
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb, xb, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(sb, xb, acc[1], 0, 0, 0);
+                acc[2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xb, xb, acc[2], 0, 0, 0);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < VL; i++) {
-                const bool ok = rvalid && c + i < C;
-                g[i] = ok ? to_f32<TG>(gp[c + i]) : 0.f;
-                x[i] = ok ? to_f32<TX>(xp[c + i]) : 0.f;
-            }
-            if constexpr (kBf16) {
-                gbits = make_uint4(pack_bf16x2(g[0], g[1]), pack_bf16x2(g[2], g[3]),
-                                   pack_bf16x2(g[4], g[5]), pack_bf16x2(g[6], g[7]));
-                xbits = make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]),
-                                   pack_bf16x2(x[4], x[5]), pack_bf16x2(x[6], x[7]));
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(g[i], x[i], acc[0], 0, 0, 0);
+                if (inject) {
+                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(g[i], gw[i], acc[1], 0, 0, 0);
+                } else {
+                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(gw[i], x[i], acc[1], 0, 0, 0);
+                    acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(x[i], x[i], acc[2], 0, 0, 0);
+                }
             }
         }
     }
-    // acc[i][j] += sum_k dy[i,k] x[j,k]
-    __device__ __forceinline__ void mfma(f32x16_t &acc) const {
-        if constexpr (kBf16) {
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, gbits),
-                                                          __builtin_bit_cast(bf16x8_t, xbits), acc, 0, 0, 0);
-        } else {
-#pragma unroll
-            for (int i = 0; i < VL; i++)
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(g[i], x[i], acc, 0, 0, 0);
-        }
-    }
-};
 
-constexpr int kLargeCB = 512;  // columns staged per phase
-
-// phase 0 of a column block: a, f, df*w per column into LDS; returns this thread's part of s1
-template <typename TG, typename TX, int V>
-__device__ __forceinline__ float bwd_large_phase0(const BwdReduceArgs &a, const TG *gb, const TX *xb,
-                                                  const float *hp_s, const float *ho_s, float *a_s,
-                                                  float *f_s, float *dfw_s, int b, int cb0, int cbn,
-                                                  float qinv, bool inject) {
-    const int n = a.n, C = a.C;
-    float s1 = 0.f;
-    for (int cc = threadIdx.x * V; cc < cbn; cc += 256 * V) {
-        const int c = cb0 + cc;
-        float sa[V], sdf[V];
+    // cross-wave sum in LDS, then wave 0 writes the part's Gram matrices row-major
+    if (wave > 0) {
+        float *dst = xw + (size_t)(wave - 1) * kGramMats * 16 * 64;
 #pragma unroll
-        for (int v = 0; v < V; v++) { sa[v] = 0.f; sdf[v] = 0.f; }
-        for (int i0 = 0; i0 < n; i0 += 8) {  // 16 loads in flight; streams >= n alias stream 0
-            float xv[8][V], gv[8][V];
+        for (int m = 0; m < kGramMats; m++)
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
-                const size_t so = (size_t)(i0 + u < n ? i0 + u : 0) * C + c;
-                load_vec<TX, V>(xb + so, xv[u]);
-                load_vec<TG, V>(gb + so, gv[u]);
-            }
-#pragma unroll
-            for (int u = 0; u < 8; u++) {
-                const float hp = i0 + u < n ? hp_s[i0 + u] : 0.f, ho = i0 + u < n ? ho_s[i0 + u] : 0.f;
-#pragma unroll
-                for (int v = 0; v < V; v++) { sa[v] += hp * xv[u][v]; sdf[v] += ho * gv[u][v]; }
-            }
-        }
-        float fv[V];
-        if (inject) load_vec<TX, V>(static_cast<const TX *>(a.f_inject) + (size_t)b * C + c, fv);
-#pragma unroll
-        for (int v = 0; v < V; v++) {
-            float dfw = 0.f;
-            if (!inject) {
-                const float wv = load_w_(a.w, a.w_bf16, c + v);
-                fv[v] = sa[v] * qinv * wv;
-                dfw = sdf[v] * wv;
-            }
-            a_s[cc + v] = sa[v]; f_s[cc + v] = fv[v]; dfw_s[cc + v] = dfw;
-            s1 += dfw * sa[v];
-        }
+            for (int i = 0; i < 16; i++) dst[(m * 16 + i) * 64 + lane] = acc[m][i];
     }
-    return s1;
+    __syncthreads();
+    if (wave == 0) {
+        float *out = a.raw + ((size_t)b * a.parts + part) * kGramFloats;
+#pragma unroll
+        for (int m = 0; m < kGramMats; m++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                float v = acc[m][i];
+#pragma unroll
+                for (int w = 0; w < 3; w++) v += xw[((size_t)w * kGramMats * 16 + m * 16 + i) * 64 + lane];
+                // accumulator layout: column j = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4
+                out[m * 1024 + (8 * (i >> 2) + 4 * kh + (i & 3)) * 32 + row] = v;
+            }
+    }
 }
 
-template <typename TG, typename TX, int NP>
-__global__ __launch_bounds__(256) void mix_bwd_reduce_large_kernel(BwdReduceArgs a) {
-    using SK = SkLds<NP>;
-    using PS = PairStep<TG, TX>;
-    constexpr int VL = PS::VL;
+template <int NP>
+__global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
+    using SK = SkWg<NP>;
     extern __shared__ float smem[];
-    float *a_s = smem;                 // [CB]
-    float *f_s = a_s + kLargeCB;       // [CB]
-    float *dfw_s = f_s + kLargeCB;     // [CB]
-    float *hp_s = dfw_s + kLargeCB;    // [32] Hpre
-    float *ho_s = hp_s + 32;           // [32] Hpost
-    float *vec_s = ho_s + 32;          // [3][32] dHpost | A1 | A2 totals
-    float *red_s = vec_s + 96;         // [8]
-    float *xw = red_s + 8;             // cross-wave scratch [3][19][64], later reused by Sinkhorn
-    const int b = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6, row = lane & 31, kh = lane >> 5;
-    const TG *__restrict__ gb = static_cast<const TG *>(a.dy) + (size_t)b * n * C;
-    const TX *__restrict__ xb = static_cast<const TX *>(a.x) + (size_t)b * n * C;
+    float *W_s = smem;                   // [32][33]  W1 (or dy [f;0]^T)
+    float *X_s = W_s + 32 * 33;          // [32][33]  XX
+    float *M_s = X_s + 32 * 33;          // [32][33]  dM
+    float *hp_s = M_s + 32 * 33;         // [32] Hpre
+    float *ho_s = hp_s + 32;             // [32] Hpost
+    float *vec_s = ho_s + 32;            // [3][32] dHpost | A1 | A2
+    float *red_s = vec_s + 96;           // [4]
+    float *sk_s = red_s + 4;             // SK::lds_floats(T)
+    const int b = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x, lane = tid & 63;
+    const bool w0 = tid < 64;
     const bool inject = a.f_inject != nullptr;
     const float qinv = inject ? 0.f : 1.0f / a.q[b];
     if (tid < 32) {
         hp_s[tid] = tid < n ? a.Hpre[(size_t)b * a.hstride + tid] : 0.f;
         ho_s[tid] = tid < n ? a.Hpost[(size_t)b * a.hstride + tid] : 0.f;
     }
-    __syncthreads();
-
-    f32x16_t acc;
+    // sum the column parts; rows / columns >= n hold aliased garbage and are dropped here
+    const float *raw = a.raw + (size_t)b * a.parts * kGramFloats;
+    {
+        constexpr int EPT = kGramFloats / 256;  // 12 elements per thread, all loads of a part in flight
+        float acc[EPT];
 #pragma unroll
-    for (int i = 0; i < 16; i++) acc[i] = 0.f;
-    float vpost = 0.f, vA1 = 0.f, vA2 = 0.f, s1 = 0.f;
-    const bool rvalid = row < n;
-    const bool vec_ok = C % VL == 0;
-    const TG *grow = gb + (size_t)(rvalid ? row : 0) * C;
-    const TX *xrow = xb + (size_t)(rvalid ? row : 0) * C;
-
-    for (int cb0 = 0; cb0 < C; cb0 += kLargeCB) {
-        const int cbn = min(kLargeCB, C - cb0);
-        if (C % 2 == 0)
-            s1 += bwd_large_phase0<TG, TX, 2>(a, gb, xb, hp_s, ho_s, a_s, f_s, dfw_s, b, cb0, cbn, qinv, inject);
-        else
-            s1 += bwd_large_phase0<TG, TX, 1>(a, gb, xb, hp_s, ho_s, a_s, f_s, dfw_s, b, cb0, cbn, qinv, inject);
-        __syncthreads();
-        // phase 1: dM tile on the matrix cores, vector sums beside it
-        const int nsteps = (cbn + 2 * VL - 1) / (2 * VL);
-        for (int s = wave; s < nsteps; s += 4) {
-            const int cc = s * 2 * VL + kh * VL;
-            PS ps;
-            ps.load(grow, xrow, cb0 + cc, cb0 + cbn, rvalid, vec_ok);
-            ps.mfma(acc);
+        for (int k = 0; k < EPT; k++) acc[k] = 0.f;
+        for (int p = 0; p < a.parts; p++) {
+            float t[EPT];
 #pragma unroll
-            for (int v = 0; v < VL; v++) {
-                if (cc + v < cbn) {  // operands beyond the block are zero; LDS beyond it is stale
-                    vpost += ps.g[v] * f_s[cc + v];
-                    vA1 += ps.x[v] * dfw_s[cc + v];
-                    vA2 += ps.x[v] * a_s[cc + v];
-                }
-            }
+            for (int k = 0; k < EPT; k++) t[k] = raw[(size_t)p * kGramFloats + tid + 256 * k];
+#pragma unroll
+            for (int k = 0; k < EPT; k++) acc[k] += t[k];
         }
-        __syncthreads();
-    }
-
-    // ---- cross-wave totals (wave 0 finishes; the other waves only keep the barriers) ---------
-    vpost += __shfl_xor(vpost, 32, kWave);
-    vA1 += __shfl_xor(vA1, 32, kWave);
-    vA2 += __shfl_xor(vA2, 32, kWave);
-    s1 = wave_allreduce_sum(s1);
-    if (wave > 0) {
-        float *dst = xw + (size_t)(wave - 1) * 19 * 64;
 #pragma unroll
-        for (int i = 0; i < 16; i++) dst[i * 64 + lane] = acc[i];
-        dst[16 * 64 + lane] = vpost; dst[17 * 64 + lane] = vA1; dst[18 * 64 + lane] = vA2;
-    }
-    if (lane == 0) red_s[wave] = s1;
-    __syncthreads();
-    const bool w0 = wave == 0;
-    float *Es = xw;                      // [NP][LD]
-    float *dO = Es + NP * SK::LD;        // [NP][LD]
-    float *u = dO + NP * SK::LD, *v = u + NP, *tmp = v + NP;
-    float *rho = tmp + NP, *ssc = rho + a.T * NP;
-    if (w0) {
-#pragma unroll
-        for (int w = 0; w < 3; w++) {
-            const float *src = xw + (size_t)w * 19 * 64;
-#pragma unroll
-            for (int i = 0; i < 16; i++) acc[i] += src[i * 64 + lane];
-            vpost += src[16 * 64 + lane]; vA1 += src[17 * 64 + lane]; vA2 += src[18 * 64 + lane];
-        }
-        s1 = (red_s[0] + red_s[1]) + (red_s[2] + red_s[3]);
-        if (lane < 32) { vec_s[lane] = vpost; vec_s[32 + lane] = vA1; vec_s[64 + lane] = vA2; }
-    }
-    __syncthreads();
-    // dM[i][j] sits in acc: j = lane & 31, i = 8*(reg/4) + 4*(lane/32) + reg%4.  Stage it in the
-    // Sinkhorn backward buffer (which reuses the cross-wave scratch, now fully consumed).
-    if (w0) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int ri = 8 * (i >> 2) + 4 * kh + (i & 3);
-            if (ri < NP && row < NP) dO[ri * SK::LD + row] = acc[i];
+        for (int k = 0; k < EPT; k++) {
+            const int e = tid + 256 * k;
+            const int m = e >> 10, i = (e >> 5) & 31, j = e & 31;
+            const bool ok = i < n && j < n;
+            if (m == 0) M_s[i * 33 + j] = ok ? acc[k] : 0.f;
+            else if (m == 1) W_s[i * 33 + j] = (i < n && (j < n || inject)) ? acc[k] : 0.f;
+            else X_s[i * 33 + j] = ok ? acc[k] : 0.f;
         }
     }
     __syncthreads();
+    if (tid < 32) {          // A1[j], A2[j]
+        float a1 = 0.f, a2 = 0.f;
+#pragma unroll 8
+        for (int k = 0; k < 32; k++) { a1 += ho_s[k] * W_s[k * 33 + tid]; a2 += hp_s[k] * X_s[k * 33 + tid]; }
+        vec_s[32 + tid] = a1; vec_s[64 + tid] = a2;
+    } else if (tid < 64) {   // dHpost[i]
+        const int i = tid - 32;
+        float dh = 0.f;
+        if (inject) {
+            dh = W_s[i * 33];
+        } else {
+#pragma unroll 8
+            for (int j = 0; j < 32; j++) dh += hp_s[j] * W_s[i * 33 + j];
+            dh *= qinv;
+        }
+        vec_s[i] = dh;
+    }
+    __syncthreads();
+    float s1 = 0.f;
+    if (!inject) {
+#pragma unroll 8
+        for (int i = 0; i < 32; i++) s1 += ho_s[i] * vec_s[i];
+        s1 = s1 / qinv;  // vec_s holds W1 Hpre / q
+    }
 
     const int D = n * n + 2 * n;
     float dHpre = 0.f, dHpost = 0.f;
@@ -545,11 +615,9 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_large_kernel(BwdReduceArgs
     }
     if (tid == 0) a.out.s1[b] = s1;
     if (a.hstride == 0) {
-        if (w0) {
-            float *red = a.out.red + (size_t)b * D;
-            for (int e = lane; e < n * n; e += kWave) red[e] = dO[(e / n) * SK::LD + (e % n)];
-            if (lane < n) { red[n * n + lane] = dHpre; red[n * n + n + lane] = dHpost; }
-        }
+        float *red = a.out.red + (size_t)b * D;
+        for (int e = tid; e < n * n; e += 256) red[e] = M_s[(e / n) * 33 + (e % n)];
+        if (w0 && lane < n) { red[n * n + lane] = dHpre; red[n * n + n + lane] = dHpost; }
         return;
     }
     const float *Pb = a.P + (size_t)b * D;
@@ -558,40 +626,47 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_large_kernel(BwdReduceArgs
     float *dt = a.out.dt + (size_t)b * (D + 3);
     const DPWriter dpw{a.out, b, a.B, a.DP};
     float S0 = 0.f, S1 = 0.f, S2 = 0.f;  // sum_d dt_d p_d per alpha group
-    if (w0) {
-        if (lane < n) {
-            const float hp = hp_s[lane], ho = ho_s[lane];
-            const float dtp = dHpre * hp * (1.0f - hp);
-            const float dto = dHpost * ho * (1.0f - 0.5f * ho);
-            dt[lane] = dtp; dt[n + lane] = dto;
-            dpw.put(lane, dtp * al0 * rinv); dpw.put(n + lane, dto * al1 * rinv);
-            S0 = dtp * Pb[lane]; S1 = dto * Pb[n + lane];
-        }
-        for (int e = lane; e < NP * NP; e += kWave) {
-            const int r0 = e / NP, c = e % NP;
-            Es[r0 * SK::LD + c] =
-                (r0 < n && c < n) ? expf(al2 * Pb[2 * n + r0 * n + c] + a.b_res[r0 * n + c]) : 0.f;
-        }
+    if (w0 && lane < n) {
+        const float hp = hp_s[lane], ho = ho_s[lane];
+        const float dtp = dHpre * hp * (1.0f - hp);
+        const float dto = dHpost * ho * (1.0f - 0.5f * ho);
+        dt[lane] = dtp; dt[n + lane] = dto;
+        dpw.put(lane, dtp * al0 * rinv); dpw.put(n + lane, dto * al1 * rinv);
+        S0 = dtp * Pb[lane]; S1 = dto * Pb[n + lane];
     }
-    __syncthreads();
-    SK::forward(Es, u, v, n, a.T, a.eps, rho, ssc, tid);
-    SK::backward(Es, dO, u, v, tmp, n, a.T, rho, ssc, tid);
-    if (w0) {
-        for (int e = lane; e < n * n; e += kWave) {
-            const int r0 = e / n, c = e % n;
-            const int di = 2 * n + e;
-            const float dtr = dO[r0 * SK::LD + c] * Es[r0 * SK::LD + c];
+    // Sinkhorn forward recompute + exact backward, the matrix spread over all 256 threads
+    const int r0 = SK::row(tid), c0 = SK::col0(tid);
+    float E[SK::EPL], d[SK::EPL], pres[SK::EPL], u, v[SK::EPL];
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++) {
+        const int c = c0 + e;
+        const bool ok = r0 < n && c < n;
+        pres[e] = ok ? Pb[2 * n + r0 * n + c] : 0.f;
+        E[e] = ok ? expf(al2 * pres[e] + a.b_res[r0 * n + c]) : 0.f;
+        d[e] = ok ? M_s[r0 * 33 + c] : 0.f;
+    }
+    SK::forward(E, u, v, n, a.T, a.eps, sk_s, tid);
+    SK::backward(E, d, u, v, a.T, sk_s, tid);
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++) {
+        const int c = c0 + e;
+        if (r0 < n && c < n) {
+            const int di = 2 * n + r0 * n + c;
+            const float dtr = d[e] * E[e];
             dt[di] = dtr;
             dpw.put(di, dtr * al2 * rinv);
-            S2 += dtr * Pb[di];
+            S2 += dtr * pres[e];
         }
-        S0 = wave_allreduce_sum(S0); S1 = wave_allreduce_sum(S1); S2 = wave_allreduce_sum(S2);
+    }
+    S2 = block_allreduce_sum<256>(S2, red_s);
+    if (w0) {
+        S0 = wave_allreduce_sum(S0); S1 = wave_allreduce_sum(S1);
         if (lane == 0) {
             dt[D] = S0; dt[D + 1] = S1; dt[D + 2] = S2;
             a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv / (float)(n * C);
         }
-        dpw.pad(D, lane, kWave);
     }
+    dpw.pad(D, tid, 256);
 }
 
 // =============================================================================================
@@ -622,21 +697,49 @@ static hipError_t launch_small_np(const BwdReduceArgs &a, hipStream_t stream) {
     return launch_small<TG, TX, NP, 1>(a, stream);
 }
 
-template <typename TG, typename TX, int NP>
+template <typename TG, typename TX>
 static hipError_t launch_large(const BwdReduceArgs &a, hipStream_t stream) {
-    using SK = SkLds<NP>;
-    const size_t sk = SK::backward_floats(a.T);
-    const size_t xw = 3 * 19 * 64;
-    const size_t smem = sizeof(float) * (3 * kLargeCB + 64 + 96 + 8 + (sk > xw ? sk : xw));
-    mix_bwd_reduce_large_kernel<TG, TX, NP><<<a.B, 256, smem, stream>>>(a);
+    constexpr bool kBf16 = std::is_same<TG, bf16_t>::value && std::is_same<TX, bf16_t>::value;
+    constexpr int SW = kBf16 ? 16 : 8;
+    const int nsteps = (a.C + SW - 1) / SW;
+    const int spp = (nsteps + a.parts - 1) / a.parts;
+    const size_t smem1 = sizeof(float) * ((size_t)spp * SW + 3 * kGramMats * 16 * 64);
+    if (smem1 > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gram_large_kernel<TG, TX>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1);
+        if (e != hipSuccess) return e;
+    }
+    gram_large_kernel<TG, TX><<<dim3(a.B, a.parts), 256, smem1, stream>>>(a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (a.n <= 16) {
+        const size_t smem2 = sizeof(float) * (3 * 32 * 33 + 64 + 96 + 4 + SkWg<16>::lds_floats(a.T));
+        coef_bwd_large_kernel<16><<<a.B, 256, smem2, stream>>>(a);
+    } else {
+        const size_t smem2 = sizeof(float) * (3 * 32 * 33 + 64 + 96 + 4 + SkWg<32>::lds_floats(a.T));
+        coef_bwd_large_kernel<32><<<a.B, 256, smem2, stream>>>(a);
+    }
     return hipGetLastError();
 }
 
-// Column parts per sample when the reduction is split from the coefficient backward.
+// Column parts per sample when the channel sums are a launch of their own.
 int bwd_reduce_parts(int B, int n, int C) {
-    (void)n;
+    if (n > 8) {
+        // ~512 workgroups, at least ~128 columns per part
+        int parts = (512 + B - 1) / B;
+        const int cap = C / 128 > 0 ? C / 128 : 1;
+        if (parts > cap) parts = cap;
+        if (parts > 16) parts = 16;
+        if (parts < 1) parts = 1;
+        return parts;
+    }
     if (B >= 2048 || C < 1024) return 1;
     return 2;
+}
+
+size_t bwd_reduce_raw_floats(int B, int n, int C) {
+    if (n > 8) return (size_t)B * bwd_reduce_parts(B, n, C) * kGramFloats;
+    return (size_t)B * bwd_reduce_parts(B, n, C) * (8 * 8 + 3 * 8 + 1);
 }
 
 hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int x_dtype,
@@ -645,9 +748,10 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
                                  const float *q, const float *P, const float *r, const float *alpha,
                                  const float *b_res, BwdCoefOut out, float *raw, int B, int n, int C,
                                  int T, float eps, hipStream_t stream) {
-    // dynamic H with n <= 8: channel sums per (sample, column part), coefficient backward as a
-    // second small launch; otherwise everything in the per-sample workgroup
-    const bool split = raw != nullptr && hstride != 0 && n <= 8;
+    // n <= 8, dynamic H: channel sums per (sample, column part), coefficient backward as a second
+    // small launch (static H: everything in the per-sample workgroup).  n > 8: always two launches.
+    if (n > 8 && raw == nullptr) return hipErrorInvalidValue;
+    const bool split = raw != nullptr && (n > 8 || hstride != 0);
     BwdReduceArgs a{dy, x, w, f_inject, Hpre, Hpost, M, q, P, r, alpha, b_res, out,
                     hstride, w_dtype == kBF16, B, n, C, T, padded_D(n), eps,
                     split ? raw : nullptr, split ? bwd_reduce_parts(B, n, C) : 1};
@@ -660,12 +764,9 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
 #undef MHC_SMALL
         return hipErrorInvalidValue;
     }
-#define MHC_LARGE(TG, TX)                                                   \
-    return n <= 16 ? launch_large<TG, TX, 16>(a, stream) : launch_large<TG, TX, 32>(a, stream)
-    if (y_dtype == kF32 && x_dtype == kF32) MHC_LARGE(float, float);
-    if (y_dtype == kBF16 && x_dtype == kBF16) MHC_LARGE(bf16_t, bf16_t);
-    if (y_dtype == kF32 && x_dtype == kBF16) MHC_LARGE(float, bf16_t);
-#undef MHC_LARGE
+    if (y_dtype == kF32 && x_dtype == kF32) return launch_large<float, float>(a, stream);
+    if (y_dtype == kBF16 && x_dtype == kBF16) return launch_large<bf16_t, bf16_t>(a, stream);
+    if (y_dtype == kF32 && x_dtype == kBF16) return launch_large<float, bf16_t>(a, stream);
     return hipErrorInvalidValue;
 }
 

@@ -141,7 +141,7 @@ struct LayerFwdArgs {
 };
 
 template <typename TX, typename TY, int NP, int V, int CPT>
-__global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
+__global__ __launch_bounds__(256, (CPT == 2 && NP == 4) ? 5 : 1) void layer_fwd_small_kernel(LayerFwdArgs a) {
     using SK = SkSmall<NP>;
     __shared__ float coef_s[NP * NP + 2 * NP];  // M | Hpre | Hpost
     __shared__ float red[4];
@@ -229,13 +229,12 @@ __global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
                     }
                 }
             }
-            ssq += __shfl_xor(ssq, 16, kWave); ssq += __shfl_xor(ssq, 32, kWave);
-            ppre += __shfl_xor(ppre, 16, kWave); ppre += __shfl_xor(ppre, 32, kWave);
-            ppost += __shfl_xor(ppost, 16, kWave); ppost += __shfl_xor(ppost, 32, kWave);
+            ssq = xor32_add(xor16_add(ssq));
+            ppre = xor32_add(xor16_add(ppre));
+            ppost = xor32_add(xor16_add(ppost));
 #pragma unroll
             for (int e = 0; e < SK::EPL; e++) {
-                pe[e] += __shfl_xor(pe[e], 16, kWave);
-                pe[e] += __shfl_xor(pe[e], 32, kWave);
+                pe[e] = xor32_add(xor16_add(pe[e]));
             }
         }
         if (tid < 16) {

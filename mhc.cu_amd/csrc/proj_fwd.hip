@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
             }
         }
     }
-    ssq += __shfl_xor(ssq, 32, kWave);  // both K halves of the row
+    ssq = xor32_add(ssq);  // both K halves of the row
 
     // cross-wave sum: waves 1..3 park their tiles in LDS, wave 0 adds and writes
     constexpr int R = NT * 16 + 1;

@@ -11,6 +11,7 @@
 //       forward path.  Four matrices per wave.
 //   SkLds<NP>   (NP = 16, 32): one wave per matrix, E and the running scalings u, v in LDS
 //       (iterate = diag(u) E diag(v)); a half-step is one mat-vec product.
+//   SkWg<NP>    (NP = 16, 32): one 256-thread workgroup per matrix, everything in registers.
 #pragma once
 
 #include "mhc_common.h"
@@ -184,6 +185,116 @@ template <int NP> struct SkLds {
                 v[lane] *= s[t * NP + lane];
             }
             __syncthreads();
+        }
+    }
+};
+
+// =============================================================================================
+// SkWg: one 256-thread workgroup per matrix, NP = 16 or 32.  Thread t owns EPL consecutive
+// columns of row t / LPR of E and of the running gradient in registers; the iterate is kept in
+// scaling form diag(u) E diag(v) (u replicated over the lanes of a row, v over the rows).  A
+// half-step is one cross-lane reduction: rows inside a DPP row, columns inside the wave and then
+// across the 4 waves through a double-buffered LDS slot (one barrier per iteration).
+// Same arithmetic as SkLds (IEEE divisions, denominators rho/s kept per iteration), ~30x shorter
+// critical path.  Every thread of the workgroup must call forward/backward.
+// =============================================================================================
+template <int NP> struct SkWg {
+    static_assert(NP == 16 || NP == 32, "SkWg handles 16x16 and 32x32 tiles");
+    static constexpr int EPL = NP * NP / 256;  // 1 or 4
+    static constexpr int LPR = NP / EPL;       // lanes per row: 16 or 8
+    // LDS floats: cw [2][4][NP] | rho [T][NP] | s [T][NP]
+    __host__ __device__ static constexpr int lds_floats(int T) { return 8 * NP + 2 * T * NP; }
+    __device__ static __forceinline__ int row(int tid) { return tid / LPR; }
+    __device__ static __forceinline__ int col0(int tid) { return (tid % LPR) * EPL; }
+
+    __device__ static __forceinline__ float row_allreduce(float x) {
+        x += dpp_mov<kDppQuadXor1>(x);
+        x += dpp_mov<kDppQuadXor2>(x);
+        if constexpr (LPR == 8) {
+            x += dpp_mov<0x141>(x);  // row_half_mirror: lane i <-> 7 - i, i.e. the other quad
+        } else {
+            x += dpp_mov<kDppRowRor4>(x);
+            x += dpp_mov<kDppRowRor8>(x);
+        }
+        return x;
+    }
+    // sum over all NP rows of per-column values; cw_t = this iteration's LDS slot [4][NP]
+    __device__ static __forceinline__ void col_allreduce(float (&x)[EPL], float *cw_t, int tid) {
+        const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) {
+            if constexpr (LPR == 8) x[e] += dpp_mov<kDppRowRor8>(x[e]);
+            x[e] = xor16_add(x[e]);
+            x[e] = xor32_add(x[e]);
+        }
+        if (lane < LPR) {
+#pragma unroll
+            for (int e = 0; e < EPL; e++) cw_t[wave * NP + lane * EPL + e] = x[e];
+        }
+        __syncthreads();
+        const int c0 = col0(tid);
+#pragma unroll
+        for (int e = 0; e < EPL; e++)
+            x[e] = (cw_t[c0 + e] + cw_t[NP + c0 + e]) + (cw_t[2 * NP + c0 + e] + cw_t[3 * NP + c0 + e]);
+    }
+
+    // E: exp(logits), 0 outside n x n.  On return M = u * E[e] * v[e]; rho/s hold the denominators.
+    __device__ static __forceinline__ void forward(const float (&E)[EPL], float &u, float (&v)[EPL],
+                                                   int n, int T, float eps, float *lds, int tid) {
+        float *cw = lds, *rho = lds + 8 * NP, *s = rho + T * NP;
+        const int r = row(tid), c0 = col0(tid);
+        u = 1.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) v[e] = 1.0f;
+        for (int t = 0; t < T; t++) {
+            float p = 0.f;
+#pragma unroll
+            for (int e = 0; e < EPL; e++) p += E[e] * v[e];
+            p = row_allreduce(p);
+            const float rr = r < n ? u * p + eps : 1.0f;
+            u = u / rr;
+            if ((tid % LPR) == 0) rho[t * NP + r] = rr;
+            float q[EPL];
+#pragma unroll
+            for (int e = 0; e < EPL; e++) q[e] = E[e] * u;
+            col_allreduce(q, cw + (t & 1) * 4 * NP, tid);
+#pragma unroll
+            for (int e = 0; e < EPL; e++) {
+                const float sc = c0 + e < n ? v[e] * q[e] + eps : 1.0f;
+                v[e] = v[e] / sc;
+                if (r == 0) s[t * NP + c0 + e] = sc;
+            }
+        }
+        __syncthreads();  // rho / s visible to every thread
+    }
+
+    // d: in = dL/dM, out = dL/dE.  u, v: final scalings from forward (destroyed).
+    __device__ static __forceinline__ void backward(const float (&E)[EPL], float (&d)[EPL], float u,
+                                                    float (&v)[EPL], int T, float *lds, int tid) {
+        float *cw = lds;
+        const float *rho = lds + 8 * NP, *s = rho + T * NP;
+        const int r = row(tid), c0 = col0(tid);
+        for (int t = T - 1; t >= 0; t--) {
+            // column dots with the iterate after column step t: Out = u E v
+            float cd[EPL];
+#pragma unroll
+            for (int e = 0; e < EPL; e++) cd[e] = d[e] * u * E[e];
+            col_allreduce(cd, cw + (t & 1) * 4 * NP, tid);
+            float z = 0.f, sc[EPL];
+#pragma unroll
+            for (int e = 0; e < EPL; e++) {
+                sc[e] = s[t * NP + c0 + e];
+                d[e] -= cd[e] * v[e];
+                z += d[e] * E[e] * v[e];
+            }
+            const float rdot = u * row_allreduce(z);
+            const float rr = rho[t * NP + r];
+#pragma unroll
+            for (int e = 0; e < EPL; e++) {
+                d[e] = (d[e] / sc[e] - rdot) / rr;
+                v[e] *= sc[e];
+            }
+            u *= rr;
         }
     }
 };
