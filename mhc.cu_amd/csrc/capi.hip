@@ -48,7 +48,7 @@ int ws_check(void *ws, size_t have, size_t need) {
     } while (0)
 
 // ---- dynamic workspace layout ----------------------------------------------------------------
-struct DynFwdWs { float *Ppart, *ssqpart; size_t bytes; };
+struct DynFwdWs { float *Ppart, *ssqpart, *agg; size_t bytes; };
 struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *raw, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
 
 int max_ksplit(int B, int n, int C) { return proj_fwd_ksplit(kBF16, kBF16, B, n, C); }
@@ -59,6 +59,7 @@ DynFwdWs carve_dyn_fwd(void *ws, int B, int n, int C) {
     DynFwdWs w;
     w.Ppart = c.floats((size_t)ks * B * padded_D(n));
     w.ssqpart = c.floats((size_t)ks * B);
+    w.agg = c.floats(n > 8 ? (size_t)B * C : 0);  // stream aggregate of the matrix-core mix
     w.bytes = c.off;
     return w;
 }
@@ -88,13 +89,14 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
 }
 
 // ---- static workspace layout -----------------------------------------------------------------
-struct StaFwdWs { float *Hpre, *Hpost, *M, *q; size_t bytes; };
+struct StaFwdWs { float *Hpre, *Hpost, *M, *q, *agg; size_t bytes; };
 struct StaBwdWs { float *red, *s1, *u, *red_sum, *cs_red, *cs_u, *raw; size_t bytes; };
 
-StaFwdWs carve_sta_fwd(void *ws, int B, int n) {
+StaFwdWs carve_sta_fwd(void *ws, int B, int n, int C) {
     Carver c(ws);
     StaFwdWs w;
     w.Hpre = c.floats(n); w.Hpost = c.floats(n); w.M = c.floats((size_t)n * n); w.q = c.floats(B);
+    w.agg = c.floats(n > 8 ? (size_t)B * C : 0);
     w.bytes = c.off;
     return w;
 }
@@ -172,7 +174,7 @@ int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype
     MHC_LAUNCH(launch_coef_fwd(ws.Ppart, ws.ssqpart, KS, padded_D(n), alpha, bias, bias + n,
                                bias + 2 * n, H_pre, H_post, M, P, r, B, n, n * C, iters, eps, st));
     MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, H_pre, H_post, M, n, q,
-                              B, n, C, eps, st));
+                              ws.agg, B, n, C, eps, st));
     return MHC_OK;
 }
 
@@ -237,7 +239,7 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
 // ===============================================================================================
 size_t mhc_layer_static_workspace_bytes(int B, int n, int C) {
     if (check_shape(B, n, C, 0) != MHC_OK) return 0;
-    const size_t f = carve_sta_fwd(nullptr, B, n).bytes;
+    const size_t f = carve_sta_fwd(nullptr, B, n, C).bytes;
     const size_t b = carve_sta_bwd(nullptr, B, n, C).bytes;
     return f > b ? f : b;
 }
@@ -260,16 +262,16 @@ int mhc_layer_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
                                           H_pre, H_post, M, nullptr, nullptr, q, B, n, C, iters, eps, st));
         return MHC_OK;
     }
-    const StaFwdWs ws = carve_sta_fwd(workspace, B, n);
-    const bool need_ws = !H_pre || !H_post || !M || !q;
+    const StaFwdWs ws = carve_sta_fwd(workspace, B, n, C);
+    const bool need_ws = !H_pre || !H_post || !M || !q || n > 8;
     if (need_ws)
         if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
     float *hp = H_pre ? H_pre : ws.Hpre, *ho = H_post ? H_post : ws.Hpost;
     float *m = M ? M : ws.M, *qq = q ? q : ws.q;
     MHC_LAUNCH(launch_coef_fwd(nullptr, nullptr, 0, 0, nullptr, H_pre_logits, H_post_logits,
                                H_res_logits, hp, ho, m, nullptr, nullptr, 1, n, n * C, iters, eps, st));
-    MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, hp, ho, m, 0, qq, B, n, C,
-                              eps, st));
+    MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, hp, ho, m, 0, qq,
+                              n > 8 ? ws.agg : nullptr, B, n, C, eps, st));
     return MHC_OK;
 }
 

@@ -36,8 +36,10 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
 // coefficients) or 0 (shared); the M stride is hstride * n.
 hipError_t launch_mix_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
                           const void *f_inject, void *y, int y_dtype, const float *Hpre,
-                          const float *Hpost, const float *M, int hstride, float *q, int B, int n,
-                          int C, float eps, hipStream_t stream);
+                          const float *Hpost, const float *M, int hstride, float *q, float *a_ws,
+                          int B, int n, int C, float eps, hipStream_t stream);
+// a_ws: scratch of B * C floats, needed (with q) by the matrix-core path, see mix_fwd_large_supported
+bool mix_fwd_large_supported(int n, int C, int x_dtype);
 
 // Fused coefficients + mix for n <= 8 when the sample's tile fits in registers
 // (layer_fwd_fused_supported).  Ppart == nullptr selects static H (logits in b_pre/b_post/b_res,

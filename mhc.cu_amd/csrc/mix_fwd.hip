@@ -393,6 +393,181 @@ hipError_t launch_layer_fwd_fused(const void *x, int x_dtype, const void *w, int
     return ok ? err : hipErrorInvalidValue;
 }
 
+// =============================================================================================
+// n > 8, bf16 x: the mix on the matrix cores, in two launches.
+//   agg_large_kernel       one workgroup per sample: a = Hpre^T x (fp32, to scratch) and q
+//   mix_fwd_large_kernel   workgroup = (128-channel block, sample): y = M x + Hpost (x) f with
+//                          A = M as a bf16 pair (rounded value + remainder), B = the x tile read
+//                          back transposed from LDS (the contraction runs over streams); the
+//                          result goes through LDS to a row-major epilogue with 16-byte stores.
+// =============================================================================================
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+struct MixLargeArgs {
+    const bf16_t *x;
+    const void *w;
+    const bf16_t *f_inject;
+    void *y;
+    const float *Hpre, *Hpost, *M;
+    float *q, *a_ws;  // a_ws: [B, C] fp32 aggregate (unused with an injected f)
+    int hstride, w_bf16, B, n, C;
+    float eps;
+};
+
+__global__ __launch_bounds__(256) void agg_large_kernel(MixLargeArgs a) {
+    __shared__ float hp_s[32];
+    __shared__ float red[4];
+    const int b = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x;
+    const bf16_t *xb = a.x + (size_t)b * n * C;
+    if (tid < 32) hp_s[tid] = tid < n ? a.Hpre[(size_t)b * a.hstride + tid] : 0.f;
+    __syncthreads();
+    float ssq = 0.f;
+    for (int ch = tid; ch < C / 8; ch += 256) {
+        float acc[8];
+#pragma unroll
+        for (int v = 0; v < 8; v++) acc[v] = 0.f;
+#pragma unroll
+        for (int i0 = 0; i0 < 32; i0 += 16) {  // 16 loads in flight; streams >= n alias stream 0
+            RawVec<bf16_t, 8> xr[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++) xr[u].load(xb + (size_t)(i0 + u < n ? i0 + u : 0) * C + ch * 8);
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                float xv[8];
+                xr[u].get(xv);
+                const float hp = hp_s[i0 + u];
+#pragma unroll
+                for (int v = 0; v < 8; v++) acc[v] += hp * xv[v];
+            }
+        }
+        store_vec<float, 8>(a.a_ws + (size_t)b * C + ch * 8, acc);
+#pragma unroll
+        for (int v = 0; v < 8; v++) ssq += acc[v] * acc[v];
+    }
+    ssq = block_allreduce_sum<256>(ssq, red);
+    if (tid == 0) a.q[b] = sqrtf(ssq / (float)C + a.eps);
+}
+
+constexpr int kMflCB = 128;           // channels per workgroup
+constexpr int kMflLDT = kMflCB + 8;   // LDS pitch of the bf16 tile (elements)
+constexpr int kMflLDO = kMflCB + 4;   // LDS pitch of the fp32 output tile
+
+template <typename TY>
+__global__ __launch_bounds__(256) void mix_fwd_large_kernel(MixLargeArgs a) {
+    extern __shared__ __align__(16) unsigned char mfl_smem[];
+    bf16_t *x_s = reinterpret_cast<bf16_t *>(mfl_smem);          // [32][LDT]
+    float *o_s = reinterpret_cast<float *>(x_s + 32 * kMflLDT);  // [32][LDO]
+    float *ho_s = o_s + 32 * kMflLDO;                            // [32] Hpost (0 beyond n)
+    const int b = blockIdx.y, cb0 = blockIdx.x * kMflCB, n = a.n, C = a.C, tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6, row = lane & 31, kh = lane >> 5;
+    const bool inject = a.f_inject != nullptr;
+    const bf16_t *xb = a.x + (size_t)b * n * C;
+    const float *M = a.M + (size_t)b * a.hstride * n;
+
+    // tile loads: thread owns row tid / 8, 16-byte chunks tid % 8 and tid % 8 + 8
+    const int trow = tid >> 3;
+    RawVec<bf16_t, 8> xr[2];
+    bool cok[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int c = cb0 + ((tid & 7) + 8 * h) * 8;
+        cok[h] = c < C;  // C % 8 == 0
+        xr[h].load(xb + (size_t)(trow < n ? trow : 0) * C + (cok[h] ? c : 0));
+    }
+    // A operand: lane (row i, kg) holds M[i][k], k = ks*16 + kg*8 .. +8 (zero beyond n)
+    bf16x8_t mh[2], ml[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        float mv[8];
+        uint32_t hw[4];
+        float lo[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int k = ks * 16 + kh * 8 + i;
+            const bool ok = k < n && row < n;
+            const float m = M[ok ? row * n + k : 0];
+            mv[i] = ok ? m : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            hw[i] = pack_bf16x2(mv[2 * i], mv[2 * i + 1]);
+            lo[2 * i] = mv[2 * i] - bf16lo_to_f32(hw[i]);
+            lo[2 * i + 1] = mv[2 * i + 1] - bf16hi_to_f32(hw[i]);
+        }
+        mh[ks] = __builtin_bit_cast(bf16x8_t, make_uint4(hw[0], hw[1], hw[2], hw[3]));
+        ml[ks] = __builtin_bit_cast(bf16x8_t, make_uint4(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]),
+                                                         pack_bf16x2(lo[4], lo[5]), pack_bf16x2(lo[6], lo[7])));
+    }
+    if (tid < 32) ho_s[tid] = tid < n ? a.Hpost[(size_t)b * a.hstride + tid] : 0.f;
+    if (inject && a.q && blockIdx.x == 0 && tid == 0) a.q[b] = 1.0f;  // q is defined as 1 with an injected f
+    // f of this lane's channel in the matrix-core phase
+    const int cw = cb0 + wave * 32 + row;
+    float f = 0.f;
+    if (cw < C) {
+        if (inject) f = bf16_to_f32(a.f_inject[(size_t)b * C + cw]);
+        else f = a.a_ws[(size_t)b * C + cw] * load_w(a.w, a.w_bf16, cw) / a.q[b];
+    }
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+        *reinterpret_cast<uint4 *>(x_s + trow * kMflLDT + ((tid & 7) + 8 * h) * 8) =
+            make_uint4(xr[h].w[0], xr[h].w[1], xr[h].w[2], xr[h].w[3]);
+    __syncthreads();
+
+    f32x16_t o;
+#pragma unroll
+    for (int i = 0; i < 16; i++) o[i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        // B fragment: lane (c, kg) gets x[ks*16 + kg*8 + i][c], i = 0..7
+        const bf16_t *p = x_s + (size_t)(ks * 16 + kh * 8) * kMflLDT + wave * 32 + row;
+        uint32_t wv[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t lo = p[(2 * i) * kMflLDT], hi = p[(2 * i + 1) * kMflLDT];
+            wv[i] = lo | (hi << 16);
+        }
+        const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, make_uint4(wv[0], wv[1], wv[2], wv[3]));
+        o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(mh[ks], xf, o, 0, 0, 0);
+        o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ml[ks], xf, o, 0, 0, 0);
+    }
+    // accumulator layout: column = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int r = 8 * (i >> 2) + 4 * kh + (i & 3);
+        o_s[r * kMflLDO + wave * 32 + row] = o[i] + ho_s[r] * f;
+    }
+    __syncthreads();
+    if (trow < n) {
+        TY *yb = static_cast<TY *>(a.y) + (size_t)b * n * C + (size_t)trow * C + cb0;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            if (cok[h]) {
+                const int co = ((tid & 7) + 8 * h) * 8;
+                const float4 o0 = *reinterpret_cast<const float4 *>(o_s + trow * kMflLDO + co);
+                const float4 o1 = *reinterpret_cast<const float4 *>(o_s + trow * kMflLDO + co + 4);
+                const float out[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
+                store_vec<TY, 8>(yb + co, out);
+            }
+        }
+    }
+}
+
+static hipError_t launch_large_mfma(const MixLargeArgs &a, int y_dtype, hipStream_t stream) {
+    if (!a.f_inject) {
+        agg_large_kernel<<<a.B, 256, 0, stream>>>(a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    const size_t smem = sizeof(bf16_t) * 32 * kMflLDT + sizeof(float) * (32 * kMflLDO + 32);
+    const dim3 grid((a.C + kMflCB - 1) / kMflCB, a.B);
+    if (y_dtype == kBF16) mix_fwd_large_kernel<bf16_t><<<grid, 256, smem, stream>>>(a);
+    else mix_fwd_large_kernel<float><<<grid, 256, smem, stream>>>(a);
+    return hipGetLastError();
+}
+
+bool mix_fwd_large_supported(int n, int C, int x_dtype) { return n > 8 && x_dtype == kBF16 && C % 8 == 0; }
+
 template <typename TX, typename TY, int NP, int V>
 static hipError_t launch_one(const MixFwdArgs &a, hipStream_t stream) {
     const int nch = a.C / V;
@@ -422,8 +597,13 @@ static hipError_t launch_t(const MixFwdArgs &a, hipStream_t stream) {
 
 hipError_t launch_mix_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
                           const void *f_inject, void *y, int y_dtype, const float *Hpre,
-                          const float *Hpost, const float *M, int hstride, float *q, int B, int n,
-                          int C, float eps, hipStream_t stream) {
+                          const float *Hpost, const float *M, int hstride, float *q, float *a_ws,
+                          int B, int n, int C, float eps, hipStream_t stream) {
+    if (mix_fwd_large_supported(n, C, x_dtype) && (f_inject || (a_ws && q))) {
+        MixLargeArgs la{static_cast<const bf16_t *>(x), w, static_cast<const bf16_t *>(f_inject), y, Hpre, Hpost,
+                        M, q, a_ws, hstride, w_dtype == kBF16, B, n, C, eps};
+        return launch_large_mfma(la, y_dtype, stream);
+    }
     MixFwdArgs a{x, w, f_inject, y, Hpre, Hpost, M, q, hstride, w_dtype == kBF16, B, n, C, eps};
     if (x_dtype == kF32 && y_dtype == kF32) return launch_t<float, float>(a, stream);
     if (x_dtype == kBF16 && y_dtype == kBF16) return launch_t<bf16_t, bf16_t>(a, stream);
