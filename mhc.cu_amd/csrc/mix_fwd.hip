@@ -141,7 +141,7 @@ struct LayerFwdArgs {
 };
 
 template <typename TX, typename TY, int NP, int V, int CPT>
-__global__ __launch_bounds__(256, (CPT == 2 && NP == 4) ? 5 : 1) void layer_fwd_small_kernel(LayerFwdArgs a) {
+__global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
     using SK = SkSmall<NP>;
     __shared__ float coef_s[NP * NP + 2 * NP];  // M | Hpre | Hpost
     __shared__ float red[4];

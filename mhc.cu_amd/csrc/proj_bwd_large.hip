@@ -114,95 +114,126 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// dxflat[b, k] = sum_d dP[b, d] phi[d, k]: workgroup = 32 samples x 128 columns (wave w: columns
-// 32w..), phi streamed through LDS in double-buffered chunks of 64 rows x 256 contiguous bytes.
-// grid.x enumerates (sample tile, column slab) with the sample tile fastest and slabs dealt to
-// the 8 XCDs so that the workgroups sharing a phi slab run on the same L2.
+// dxflat[b, k] = sum_d dP[b, d] phi[d, k]: workgroup = 128 samples x 64 columns, so a column slab
+// of phi is streamed exactly once per 128 samples.  The 4 waves form a 2 x 2 grid (two 32-sample
+// tiles x 32 columns each).  phi arrives in chunks of 64 rows x 128 contiguous bytes (8 lanes per
+// row), two chunks in flight per thread (register FIFO), is parked in a double-buffered LDS tile
+// and read back transposed (the contraction runs over d, the strided axis); the dP operand comes
+// fragment-major from global memory with fully coalesced 16-byte loads, prefetched with its chunk.
+// The result leaves through LDS as 16-byte pieces of 128-byte rows.
+// grid: (column slabs of 64, groups of 128 samples)
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void dxflat_large_kernel(ProjBwdLargeArgs a, int tiles_s, int slabs) {
-    extern __shared__ bf16_t pl_lds[];
-    bf16_t *phi_s0 = pl_lds, *phi_s1 = pl_lds + kPL_DC * kPL_LD;
+constexpr int kDxfCW = 64;            // columns per workgroup
+constexpr int kDxfLD = kDxfCW + 8;    // LDS row pitch (elements)
+constexpr int kDxfDC = 64;            // phi rows per chunk
+
+__global__ __launch_bounds__(256) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
+    extern __shared__ bf16_t pl_lds[];  // [2][kDxfDC][kDxfLD]; later the [128][kDxfLD] output tile
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = lane & 31, kg = lane >> 5;
-    // id = ((slab / 8) * tiles_s + st) * 8 + slab % 8  ->  XCD (id % 8) is the same for all st
-    const int id = blockIdx.x;
-    const int slab = (id / (8 * tiles_s)) * 8 + (id & 7);
-    const int st = (id >> 3) % tiles_s;
-    if (slab >= slabs) return;
-    const int k0 = slab * kPL_KW;
-    const int nchunks = (a.DP + kPL_DC - 1) / kPL_DC;
-    const bf16_t *dprow = a.dPb + frag_base(st, a.DP >> 4, 0) + lane * 8;  // + 512 per k-step
+    const int wm = wave >> 1, wn = wave & 1;
+    const int k0 = blockIdx.x * kDxfCW;
+    const int sg = blockIdx.y;                 // group of 128 samples
+    const int tiles_all = a.BP >> 5;
+    const int nchunks = (a.DP + kDxfDC - 1) / kDxfDC;
 
-    // this thread's four 16-byte pieces of a phi chunk: rows (tid >> 4) + 16 h, column piece tid & 15.
-    // The prefetching loads carry no predicate (it would be applied right behind the load and stall
-    // the prefetch): out-of-range pieces alias valid memory and are zeroed when they are parked in
-    // LDS; the dP operand then only needs to be finite where phi is zero, so its out-of-range
-    // k-steps alias k-step 0.
-    auto load_phi = [&](int c, uint4 (&v)[4]) {
+    // phi piece of this thread: rows (tid >> 3) + 32 h of the chunk, 16-byte segment tid & 7.
+    // Out-of-range rows / columns alias valid memory: rows in [D, DP) meet zero dP, rows >= DP are
+    // never multiplied, columns >= nC are never stored.
+    const int prow = tid >> 3, pseg = tid & 7;
+    const int kc = k0 + pseg * 8 < a.nC ? k0 + pseg * 8 : 0;
+    // dP fragments of this wave: sample tiles st0, st0 + 1 (clamped: surplus tiles are not stored)
+    const int st0 = sg * 4 + wm * 2;
+    const bf16_t *ap[2];
 #pragma unroll
-        for (int h = 0; h < 4; h++) {
-            const int d = c * kPL_DC + (tid >> 4) + 16 * h, k = k0 + (tid & 15) * 8;
-            const bool ok = d < a.D && k < a.nC;
-            v[h] = *reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * a.nC + k : 0));
-        }
-    };
-    auto store_phi = [&](bf16_t *buf, int c, const uint4 (&v)[4]) {
-#pragma unroll
-        for (int h = 0; h < 4; h++) {
-            const int d = c * kPL_DC + (tid >> 4) + 16 * h, k = k0 + (tid & 15) * 8;
-            const bool ok = d < a.D && k < a.nC;
-            uint4 t = v[h];
-            t.x = ok ? t.x : 0u; t.y = ok ? t.y : 0u; t.z = ok ? t.z : 0u; t.w = ok ? t.w : 0u;
-            *reinterpret_cast<uint4 *>(buf + (size_t)((tid >> 4) + 16 * h) * kPL_LD + (tid & 15) * 8) = t;
-        }
-    };
-    auto load_a = [&](int c, uint4 (&v)[4]) {
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            const int d0 = c * kPL_DC + ks * 16;
-            v[ks] = *reinterpret_cast<const uint4 *>(dprow + (d0 < a.DP ? (size_t)(d0 >> 4) * 512 : 0));
-        }
-    };
+    for (int m = 0; m < 2; m++)
+        ap[m] = a.dPb + frag_base(min(st0 + m, tiles_all - 1), a.DP >> 4, 0) + lane * 8;
 
-    f32x16_t o;
+    // register FIFO of two chunks; a slot holds 2 phi pieces and 2 x 4 dP fragments
+    // (RawVec keeps the loaded words as scalars: whole-uint4 copies of an array element can end up in
+    // scratch memory, and a scratch store waits for the load it parks)
+    struct Slot { RawVec<bf16_t, 8> p[2]; uint4 f[8]; };
+    auto issue = [&](Slot &sl, int c) {
 #pragma unroll
-    for (int i = 0; i < 16; i++) o[i] = 0.f;
-    uint4 pv[4], av[4], an[4];
-    load_phi(0, pv);
-    load_a(0, av);
-    store_phi(phi_s0, 0, pv);
-    __syncthreads();
-    for (int c = 0; c < nchunks; c++) {
-        const bool more = c + 1 < nchunks;
-        bf16_t *cur = (c & 1) ? phi_s1 : phi_s0, *nxt = (c & 1) ? phi_s0 : phi_s1;
-        if (more) { load_phi(c + 1, pv); load_a(c + 1, an); }
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            const bf16x8_t pf = pl_frag_t(cur, ks * 16, wave * 32, lane);
-            o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av[ks]), pf, o, 0, 0, 0);
+        for (int h = 0; h < 2; h++) {
+            const int d = c * kDxfDC + prow + 32 * h;
+            sl.p[h].load(a.phi + (size_t)(d < a.D ? d : 0) * a.nC + kc);
         }
-        if (more) {
-            store_phi(nxt, c + 1, pv);
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) av[ks] = an[ks];
-        }
+        for (int m = 0; m < 2; m++)
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                const int d0 = c * kDxfDC + ks * 16;
+                sl.f[m * 4 + ks] = *reinterpret_cast<const uint4 *>(ap[m] + (size_t)(d0 < a.DP ? d0 >> 4 : 0) * 512);
+            }
+    };
+    f32x16_t o[2];
+#pragma unroll
+    for (int m = 0; m < 2; m++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[m][i] = 0.f;
+
+    // park the slot's phi pieces in LDS buffer `par`, then multiply the chunk
+    auto compute = [&](const Slot &sl, int par, int c) {
+        bf16_t *buf = pl_lds + (size_t)par * kDxfDC * kDxfLD;
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+            *reinterpret_cast<uint4 *>(buf + (size_t)(prow + 32 * h) * kDxfLD + pseg * 8) =
+                make_uint4(sl.p[h].w[0], sl.p[h].w[1], sl.p[h].w[2], sl.p[h].w[3]);
         __syncthreads();
-    }
-    // accumulator layout: column = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4.
-    // Stage the 32 x 128 tile in LDS as bf16 so that it leaves as 16-byte pieces of 256-byte rows
-    // (two-byte scattered stores cost an order of magnitude more write traffic).
-    bf16_t *o_s = phi_s0;  // the last loop iteration ended with a barrier: both buffers are free
+        bf16x8_t pf[4];
 #pragma unroll
-    for (int i = 0; i < 16; i++)
-        o_s[(size_t)(8 * (i >> 2) + 4 * kg + (i & 3)) * kPL_LD + wave * 32 + row] = f32_to_bf16(o[i]);
+        for (int ks = 0; ks < 4; ks++) {
+            // B fragment: lane (col, kg) gets phi[chunk row ks*16 + kg*8 + i][wn*32 + col]
+            const bf16_t *p = buf + (size_t)(ks * 16 + kg * 8) * kDxfLD + wn * 32 + row;
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t lo = p[(2 * i) * kDxfLD], hi = p[(2 * i + 1) * kDxfLD];
+                w[i] = lo | (hi << 16);
+            }
+            pf[ks] = __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            const bool live = c * kDxfDC + ks * 16 < a.DP;  // uniform; dead k-steps get a zero A operand
+#pragma unroll
+            for (int m = 0; m < 2; m++) {
+                uint4 av = sl.f[m * 4 + ks];
+                av.x = live ? av.x : 0u; av.y = live ? av.y : 0u; av.z = live ? av.z : 0u; av.w = live ? av.w : 0u;
+                o[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pf[ks], o[m], 0, 0, 0);
+            }
+        }
+    };
+
+    Slot s0, s1;
+    issue(s0, 0);
+    issue(s1, min(1, nchunks - 1));
+    int c = 0;
+    for (; c + 2 <= nchunks; c += 2) {
+        compute(s0, 0, c);
+        issue(s0, min(c + 2, nchunks - 1));
+        compute(s1, 1, c + 1);
+        issue(s1, min(c + 3, nchunks - 1));
+    }
+    if (c < nchunks) compute(s0, 0, c);
+    __syncthreads();  // all fragment reads done: the buffers become the output tile
+
+    // accumulator layout: column = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4.
+    bf16_t *o_s = pl_lds;  // [128][kDxfLD]
+#pragma unroll
+    for (int m = 0; m < 2; m++)
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            o_s[(size_t)((wm * 2 + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3)) * kDxfLD + wn * 32 + row] = f32_to_bf16(o[m][i]);
     __syncthreads();
 #pragma unroll
-    for (int h = 0; h < 2; h++) {
-        const int r = (tid >> 4) + 16 * h, kc = (tid & 15) * 8;
-        const int bo = st * 32 + r;
-        if (bo < a.B && k0 + kc < a.nC)
-            *reinterpret_cast<uint4 *>(a.dxflat + (size_t)bo * a.nC + k0 + kc) =
-                *reinterpret_cast<const uint4 *>(o_s + (size_t)r * kPL_LD + kc);
+    for (int h = 0; h < 4; h++) {
+        const int r = prow + 32 * h;
+        const int bo = sg * 128 + r;
+        if (bo < a.B && k0 + pseg * 8 < a.nC)
+            *reinterpret_cast<uint4 *>(a.dxflat + (size_t)bo * a.nC + k0 + pseg * 8) =
+                *reinterpret_cast<const uint4 *>(o_s + (size_t)r * kDxfLD + pseg * 8);
     }
 }
 
@@ -217,9 +248,8 @@ hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb
                        static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, bps};
     const int slabs = (nC + kPL_KW - 1) / kPL_KW;
     const int NTD = DP / 32;
-    const int tiles_s = (B + 31) / 32;
-    const int slab_groups = (slabs + 7) / 8;
-    dxflat_large_kernel<<<slab_groups * tiles_s * 8, 256, sizeof(bf16_t) * 2 * kPL_DC * kPL_LD, stream>>>(a, tiles_s, slabs);
+    dxflat_wide_kernel<<<dim3((nC + kDxfCW - 1) / kDxfCW, (B + 127) / 128), 256,
+                         sizeof(bf16_t) * 128 * kDxfLD, stream>>>(a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     dphi_large_kernel<<<dim3(slabs, (NTD + kPL_TPW - 1) / kPL_TPW, S), 256,
