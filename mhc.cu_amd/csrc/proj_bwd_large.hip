@@ -19,7 +19,6 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 constexpr int kPL_KW = 128;             // columns per workgroup: wave w owns columns 32w .. 32w+32
 constexpr int kPL_LD = kPL_KW + 8;      // LDS row pitch in elements (272 bytes, 16-byte aligned)
 constexpr int kPL_SB = 128;             // samples per block of the dphi kernel
-constexpr int kPL_TPW = 3;              // dphi row tiles per workgroup (each wave: 3 tiles x its columns)
 constexpr int kPL_DC = 64;              // phi rows per LDS chunk of the dxflat kernel
 
 struct ProjBwdLargeArgs {
@@ -45,10 +44,18 @@ __device__ __forceinline__ bf16x8_t pl_frag_t(const bf16_t *tile, int k0, int co
 }
 
 // ---------------------------------------------------------------------------------------------
-// dphi[d, k] = sum_b dP[b, d] x[b, k]: workgroup = 128 columns k x 3 row tiles of d; the four
-// waves share the dP^T operands (L1) and write 512 contiguous bytes per dphi row.
-// grid: (column slabs, groups of 3 d-tiles, batch splits)
+// dphi[d, k] = sum_b dP[b, d] x[b, k]: workgroup = 128 columns k x a group of row tiles of d.
+// The [128 samples x 128 columns] block of x is fetched with all of a thread's loads in flight,
+// parked in LDS and read back transposed once (the contraction runs over samples); wave w keeps
+// the fragments of columns 32w..32w+32 in registers and walks the row tiles of the group: the
+// dP^T operands (rounded value + remainder, fragment-major, coalesced) of the next row tile are
+// requested before the current tile's MFMAs are issued.  The kernel is bound by the fp32 dphi
+// stores (512 contiguous bytes per row and workgroup).
+// grid: (column slabs, groups of kPL_TPW row tiles, batch splits)
 // ---------------------------------------------------------------------------------------------
+// SINGLE: the split holds one sample block, so a row tile is complete (and stored) right after its
+// MFMAs and one accumulator is live at a time; otherwise TPW accumulators persist over the blocks.
+template <int TPW, bool SINGLE>
 __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
     extern __shared__ bf16_t pl_lds[];
     bf16_t *x_s = pl_lds;  // [kPL_SB][kPL_LD]
@@ -56,58 +63,109 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
     const int row = lane & 31, kg = lane >> 5;
     const int k0 = blockIdx.x * kPL_KW;
     const int NTD = a.DP / 32;
+    const int dt0 = blockIdx.y * TPW, dt1 = min(NTD, dt0 + TPW);
     const int b_begin = blockIdx.z * a.b_per_split;
     const int b_end = min(a.B, b_begin + a.b_per_split);
+    float *out = a.dphi + (size_t)blockIdx.z * a.D * a.nC;
+    const int k = k0 + wave * 32 + row;
+    const size_t plane = (size_t)a.DP * a.BP;
 
-    f32x16_t acc[kPL_TPW];
+    constexpr int NACC = SINGLE ? 1 : TPW;
+    f32x16_t acc[NACC];
 #pragma unroll
-    for (int m = 0; m < kPL_TPW; m++)
+    for (int m = 0; m < NACC; m++)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[m][i] = 0.f;
 
     for (int sb = b_begin; sb < b_end; sb += kPL_SB) {
         if (sb != b_begin) __syncthreads();
-        for (int ch = tid; ch < kPL_SB * (kPL_KW / 8); ch += 256) {
-            const int bl = ch / (kPL_KW / 8), b = sb + bl, kc = (ch % (kPL_KW / 8)) * 8;
-            const bool ok = b < b_end && k0 + kc < a.nC;
-            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(a.x + (ok ? (size_t)b * a.nC + k0 + kc : 0)), ok);
-            *reinterpret_cast<uint4 *>(x_s + (size_t)bl * kPL_LD + kc) = v;
+        // thread owns 16-byte segment tid & 15 of rows (tid >> 4) + 16 q
+        const int seg = tid & 15, r0 = tid >> 4;
+        const bool kok = k0 + seg * 8 < a.nC;
+        RawVec<bf16_t, 8> xr[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const int b = sb + r0 + 16 * q;
+            xr[q].load(a.x + ((b < b_end && kok) ? (size_t)b * a.nC + k0 + seg * 8 : 0));
+        }
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const bool ok = sb + r0 + 16 * q < b_end && kok;  // rows of other splits must not count
+            *reinterpret_cast<uint4 *>(x_s + (size_t)(r0 + 16 * q) * kPL_LD + seg * 8) =
+                make_uint4(ok ? xr[q].w[0] : 0u, ok ? xr[q].w[1] : 0u, ok ? xr[q].w[2] : 0u, ok ? xr[q].w[3] : 0u);
         }
         __syncthreads();
         bf16x8_t xf[8];
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) xf[ks] = pl_frag_t(x_s, ks * 16, wave * 32, lane);
+
+        // dP^T fragments of a row tile: 8 k-steps x (rounded, remainder); k-steps beyond the padded
+        // batch alias k-step 0 of the block and meet zero rows of x
+        struct AFrag { uint32_t w[16][4]; };
+        auto load_a = [&](AFrag &f, int dt) {
+            const bf16_t *ap = a.dPT + frag_base(min(dt, NTD - 1), a.BP >> 4, sb >> 4) + lane * 8;
 #pragma unroll
-        for (int m = 0; m < kPL_TPW; m++) {
-            const int dt = blockIdx.y * kPL_TPW + m;
-            if (dt < NTD) {
-                const bf16_t *ap = a.dPT + frag_base(dt, a.BP >> 4, sb >> 4) + lane * 8;
-                uint4 ah[8], al[8];
+            for (int ks = 0; ks < 8; ks++) {
+                const bf16_t *apk = ap + (sb + ks * 16 < a.BP ? ks * 512 : 0);
+                const uint4 h = *reinterpret_cast<const uint4 *>(apk);
+                const uint4 l = *reinterpret_cast<const uint4 *>(apk + plane);
+                f.w[2 * ks][0] = h.x; f.w[2 * ks][1] = h.y; f.w[2 * ks][2] = h.z; f.w[2 * ks][3] = h.w;
+                f.w[2 * ks + 1][0] = l.x; f.w[2 * ks + 1][1] = l.y; f.w[2 * ks + 1][2] = l.z; f.w[2 * ks + 1][3] = l.w;
+            }
+        };
+        AFrag fa, fb;
+        load_a(fa, dt0);
+        // one row tile: request the next tile's operands, multiply, (SINGLE) store
+        auto do_tile = [&](const AFrag &cur, AFrag &nxt, int m, f32x16_t &am) {
+            load_a(nxt, dt0 + m + 1);  // clamped to the last tile: redundant at the end, never used
+            if (SINGLE) {
 #pragma unroll
-                for (int ks = 0; ks < 8; ks++) {
-                    const bool ok = sb + ks * 16 < b_end;  // pad columns [B, BP) are zero
-                    const bf16_t *apk = ok ? ap + ks * 512 : a.dPT;
-                    ah[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk), ok);
-                    al[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk + (size_t)a.DP * a.BP), ok);
+                for (int i = 0; i < 16; i++) am[i] = 0.f;
+            }
+#pragma unroll
+            for (int ks = 0; ks < 8; ks++) {
+                am = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[2 * ks][0], cur.w[2 * ks][1], cur.w[2 * ks][2], cur.w[2 * ks][3])),
+                    xf[ks], am, 0, 0, 0);
+                am = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[2 * ks + 1][0], cur.w[2 * ks + 1][1], cur.w[2 * ks + 1][2], cur.w[2 * ks + 1][3])),
+                    xf[ks], am, 0, 0, 0);
+            }
+            if (SINGLE && k < a.nC) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int d = (dt0 + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
+                    if (d < a.D) out[(size_t)d * a.nC + k] = am[i];
                 }
+            }
+        };
+        if constexpr (SINGLE) {
+            // rolled loop over pairs of tiles (the two operand buffers swap roles inside a pair), so
+            // that only one tile's operands are requested ahead
+#pragma unroll 1
+            for (int m = 0; dt0 + m < dt1; m += 2) {
+                do_tile(fa, fb, m, acc[0]);
+                if (dt0 + m + 1 < dt1) do_tile(fb, fa, m + 1, acc[0]);
+            }
+        } else {
 #pragma unroll
-                for (int ks = 0; ks < 8; ks++) {
-                    acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ah[ks]), xf[ks], acc[m], 0, 0, 0);
-                    acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, al[ks]), xf[ks], acc[m], 0, 0, 0);
+            for (int m = 0; m < TPW; m++) {
+                if (dt0 + m < dt1) {  // uniform
+                    if (m & 1) do_tile(fb, fa, m, acc[m < NACC ? m : 0]);
+                    else do_tile(fa, fb, m, acc[m < NACC ? m : 0]);
                 }
             }
         }
     }
-    float *out = a.dphi + (size_t)blockIdx.z * a.D * a.nC;
-    const int k = k0 + wave * 32 + row;
+    if (!SINGLE && k < a.nC) {  // several sample blocks: tiles are complete only now
 #pragma unroll
-    for (int m = 0; m < kPL_TPW; m++) {
-        const int dt = blockIdx.y * kPL_TPW + m;
-        if (dt < NTD && k < a.nC) {
+        for (int m = 0; m < NACC; m++) {
+            if (dt0 + m < dt1) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int d = dt * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
-                if (d < a.D) out[(size_t)d * a.nC + k] = acc[m][i];
+                for (int i = 0; i < 16; i++) {
+                    const int d = (dt0 + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
+                    if (d < a.D) out[(size_t)d * a.nC + k] = acc[m][i];
+                }
             }
         }
     }
@@ -252,8 +310,11 @@ hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb
                          sizeof(bf16_t) * 128 * kDxfLD, stream>>>(a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    dphi_large_kernel<<<dim3(slabs, (NTD + kPL_TPW - 1) / kPL_TPW, S), 256,
-                        sizeof(bf16_t) * kPL_SB * kPL_LD, stream>>>(a);
+    const size_t smem = sizeof(bf16_t) * kPL_SB * kPL_LD;
+    if (bps <= kPL_SB)  // one sample block per split: 9 row tiles per workgroup, stored as they complete
+        dphi_large_kernel<9, true><<<dim3(slabs, (NTD + 8) / 9, S), 256, smem, stream>>>(a);
+    else
+        dphi_large_kernel<3, false><<<dim3(slabs, (NTD + 2) / 3, S), 256, smem, stream>>>(a);
     return hipGetLastError();
 }
 

@@ -117,7 +117,10 @@ def test_dynamic_fp32_vs_oracle(B, n, C, inject):
 
 
 @pytest.mark.parametrize("B,n,C", [(32, 4, 1280), (5, 4, 64), (16, 8, 256), (3, 6, 72), (4, 16, 64),
-                                   (4, 32, 64), (2, 32, 1040), (3, 4, 20)])
+                                   (4, 32, 64), (2, 32, 1040), (3, 4, 20),
+                                   # more than 128 samples with a wide projection: several sample
+                                   # blocks / groups in the projection kernels
+                                   (160, 20, 64), (130, 32, 136)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_dynamic_bf16_vs_oracle(B, n, C, out_dtype):
     x, dy, _, p = nm.make_dynamic_inputs(B, n, C, bf16_round=True)
@@ -132,6 +135,22 @@ def test_dynamic_bf16_vs_oracle(B, n, C, out_dtype):
     y_ref, g_ref = nm.mhc_dynamic_fwd_bwd(x, p, dy_used, T, eps, dtype=torch.float32)
     y, g = hip_dynamic(x, p, dy_used, T, eps, act_dtype=torch.bfloat16, out_dtype=out_dtype,
                        w_dtype=torch.bfloat16)
+    _check(y, y_ref, "bf16", "y")
+    for k, ref in g_ref.items():
+        _check(g[k], ref, "bf16", "d" + k)
+
+
+@pytest.mark.parametrize("B,n,C", [(16, 4, 256), (8, 8, 128), (4, 16, 64), (3, 32, 72), (5, 32, 1040)])
+@pytest.mark.parametrize("inject", [False, True])
+def test_static_bf16_vs_oracle(B, n, C, inject):
+    """Static H with bf16 activations: the shared-coefficient mode of the bf16 kernels."""
+    x, dy, f, p = nm.make_static_inputs(B, n, C, with_f=inject)
+    x, dy = x.bfloat16().float(), dy.bfloat16().float()
+    f = None if f is None else f.bfloat16().float()
+    p["w"] = (1.0 + 0.3 * torch.randn(C, generator=torch.Generator().manual_seed(3))).bfloat16().float()
+    T, eps = 20, 1e-6
+    y_ref, g_ref = nm.mhc_static_fwd_bwd(x, p, dy, T, eps, f_inject=f, dtype=torch.float32)
+    y, g = hip_static(x, p, dy, T, eps, f_inject=f, act_dtype=torch.bfloat16, w_dtype=torch.bfloat16)
     _check(y, y_ref, "bf16", "y")
     for k, ref in g_ref.items():
         _check(g[k], ref, "bf16", "d" + k)
