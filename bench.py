@@ -29,6 +29,12 @@ sys.path.insert(0, os.path.join(ROOT, "mhc.cu_amd"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM bytes of one step (all launches, graph-less run), from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE summed over the step's kernels and scaled by what the same counters read for
+# `--copy-calibration` (a 64 MiB copy).  Filled from the committed counter summaries; None where
+# no counter run exists for the configuration.
+MEASURED_TRAFFIC_BYTES = {"c1": 13282107, "c2": 43058552, "c3": 251359210, "c4": 92878513, "c5": 570193781}
+
 CONFIGS = {
     "c1": dict(kind="static", B=320, n=4, C=1280, dtype="f32", bwd=False),
     "c2": dict(kind="dynamic", B=320, n=4, C=1280, dtype="bf16", bwd=True),
@@ -239,10 +245,13 @@ def main():
     ap.add_argument("--view", default="L", choices=["L", "K"])
     ap.add_argument("--mode", default="graph", choices=["graph", "eager"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run a plain 64 MiB device copy instead of the layer (reference point for the "
+                         "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 "
-              "(every sample is independent, see DESIGN.md for how the path would shard)", file=sys.stderr)
+              "(every sample is independent: the path shards over the batch)", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -251,6 +260,16 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if a.copy_calibration:
+        nbytes = 64 * 1024 * 1024
+        src = torch.arange(nbytes // 4, dtype=torch.int32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(max(a.steps, 1)):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": True, "bytes_read": nbytes, "bytes_written": nbytes,
+                          "copies": max(a.steps, 1)}))
+        return
     cfg = CONFIGS[a.config]
     step = Step(cfg, a.view, torch)
 
@@ -316,7 +335,8 @@ def main():
                                f"{cfg['dtype']} T={T_ITERS} eps={EPS}",
                    "view": a.view, "launch": mode, "cache": "warm (back-to-back steps)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.config) if a.view == "L" else None,
                      "kernel": "whole step (all launches of one forward+backward)",
                      "algorithmic_bytes": alg, "device_us": dev_step,
                      "fwd": {"algorithmic_bytes": fwd_b, "device_us": dev_fwd,
