@@ -172,7 +172,8 @@ int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype
         return MHC_OK;
     }
     MHC_LAUNCH(launch_coef_fwd(ws.Ppart, ws.ssqpart, KS, padded_D(n), alpha, bias, bias + n,
-                               bias + 2 * n, H_pre, H_post, M, P, r, B, n, n * C, iters, eps, st));
+                               bias + 2 * n, H_pre, H_post, M, P, r, B, n, n * C, iters, eps,
+                               x_dtype == kF32, st));
     MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, H_pre, H_post, M, n, q,
                               ws.agg, B, n, C, eps, st));
     return MHC_OK;
@@ -269,7 +270,8 @@ int mhc_layer_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
     float *hp = H_pre ? H_pre : ws.Hpre, *ho = H_post ? H_post : ws.Hpost;
     float *m = M ? M : ws.M, *qq = q ? q : ws.q;
     MHC_LAUNCH(launch_coef_fwd(nullptr, nullptr, 0, 0, nullptr, H_pre_logits, H_post_logits,
-                               H_res_logits, hp, ho, m, nullptr, nullptr, 1, n, n * C, iters, eps, st));
+                               H_res_logits, hp, ho, m, nullptr, nullptr, 1, n, n * C, iters, eps,
+                               x_dtype == kF32, st));
     MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, hp, ho, m, 0, qq,
                               n > 8 ? ws.agg : nullptr, B, n, C, eps, st));
     return MHC_OK;

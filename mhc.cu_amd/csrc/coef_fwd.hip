@@ -81,7 +81,7 @@ template <int NP> __global__ __launch_bounds__(64) void coef_fwd_small_kernel(Co
 // One workgroup (4 waves) per sample.  All 256 threads finish the split-K sums (D = n^2 + 2n
 // logits, KS partial sums each, eight loads in flight per thread), then run Sinkhorn with the
 // matrix spread over their registers (SkWg).
-template <int NP> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
+template <int NP, bool PRECISE> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     using SK = SkWg<NP>;
     extern __shared__ float lds[];
     float *lg = lds;                       // [NP*NP + 2*NP] logits: pre | post | res (row-major n x n)
@@ -100,19 +100,20 @@ template <int NP> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(Coe
     }
     const size_t pstride = (size_t)a.B * a.DP;
     // logits d = tid + 256 m; the partial sums of all of a thread's logits are fetched together,
-    // 4 splits at a time (out-of-range slots alias element 0 and are discarded)
+    // several splits at a time (out-of-range slots alias element 0 and are discarded)
     constexpr int MD = (NP * NP + 2 * NP + 255) / 256;
     float psum[MD];
 #pragma unroll
     for (int m = 0; m < MD; m++) psum[m] = 0.f;
     if (dyn) {
         const float *pb = a.Ppart + (size_t)b * a.DP;
-        for (int k0 = 0; k0 < a.KS; k0 += 4) {
-            float tv[MD][4];
+        constexpr int KB = MD > 2 ? 12 : 16;  // splits per round: 60 / 32 loads in flight per thread
+        for (int k0 = 0; k0 < a.KS; k0 += KB) {
+            float tv[MD][KB];
 #pragma unroll
             for (int m = 0; m < MD; m++)
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
+                for (int q = 0; q < KB; q++) {
                     const int d = tid + 256 * m;
                     const bool ok = d < D && k0 + q < a.KS;
                     tv[m][q] = pb[ok ? (size_t)(k0 + q) * pstride + d : 0];
@@ -120,7 +121,7 @@ template <int NP> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(Coe
 #pragma unroll
             for (int m = 0; m < MD; m++)
 #pragma unroll
-                for (int q = 0; q < 4; q++) psum[m] += (tid + 256 * m < D && k0 + q < a.KS) ? tv[m][q] : 0.f;
+                for (int q = 0; q < KB; q++) psum[m] += (tid + 256 * m < D && k0 + q < a.KS) ? tv[m][q] : 0.f;
         }
     }
 #pragma unroll
@@ -148,7 +149,7 @@ template <int NP> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(Coe
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         E[e] = (r0 < n && c0 + e < n) ? expf(lg[2 * n + r0 * n + c0 + e]) : 0.f;
-    SK::forward(E, u, v, n, a.T, a.eps, sk_s, tid);
+    SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         if (r0 < n && c0 + e < n) a.M[(size_t)b * n * n + r0 * n + c0 + e] = u * E[e] * v[e];
@@ -157,16 +158,22 @@ template <int NP> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(Coe
 hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int DP,
                            const float *alpha, const float *b_pre, const float *b_post,
                            const float *b_res, float *Hpre, float *Hpost, float *M, float *P,
-                           float *r, int B, int n, int nC, int T, float eps, hipStream_t stream) {
+                           float *r, int B, int n, int nC, int T, float eps, bool precise,
+                           hipStream_t stream) {
     CoefArgs a{Ppart, ssqpart, KS, DP, alpha, b_pre, b_post, b_res, Hpre, Hpost, M, P, r, B, n, nC, T, eps};
     if (n <= 4)
         coef_fwd_small_kernel<4><<<(B + 3) / 4, 64, 0, stream>>>(a);
     else if (n <= 8)
         coef_fwd_small_kernel<8><<<(B + 3) / 4, 64, 0, stream>>>(a);
-    else if (n <= 16)
-        coef_fwd_lds_kernel<16><<<B, 256, sizeof(float) * (16 * 16 + 32 + SkWg<16>::lds_floats(T)), stream>>>(a);
-    else
-        coef_fwd_lds_kernel<32><<<B, 256, sizeof(float) * (32 * 32 + 64 + SkWg<32>::lds_floats(T)), stream>>>(a);
+    else if (n <= 16) {
+        const size_t smem = sizeof(float) * (16 * 16 + 32 + SkWg<16>::lds_floats(T));
+        if (precise) coef_fwd_lds_kernel<16, true><<<B, 256, smem, stream>>>(a);
+        else coef_fwd_lds_kernel<16, false><<<B, 256, smem, stream>>>(a);
+    } else {
+        const size_t smem = sizeof(float) * (32 * 32 + 64 + SkWg<32>::lds_floats(T));
+        if (precise) coef_fwd_lds_kernel<32, true><<<B, 256, smem, stream>>>(a);
+        else coef_fwd_lds_kernel<32, false><<<B, 256, smem, stream>>>(a);
+    }
     return hipGetLastError();
 }
 

@@ -30,7 +30,9 @@ hipError_t launch_proj_fwd(const void *x, int x_dtype, const void *phi, int phi_
 hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int DP,
                            const float *alpha, const float *b_pre, const float *b_post,
                            const float *b_res, float *Hpre, float *Hpost, float *M, float *P,
-                           float *r, int B, int n, int nC, int T, float eps, hipStream_t stream);
+                           float *r, int B, int n, int nC, int T, float eps, bool precise,
+                           hipStream_t stream);
+// precise: IEEE divisions in the n > 8 Sinkhorn (fp32 parity tier); otherwise v_rcp_f32
 
 // y = M x + Hpost (x) f, f = RMSNorm(Hpre . x) * w or f_inject.  hstride = n (per-sample
 // coefficients) or 0 (shared); the M stride is hstride * n.

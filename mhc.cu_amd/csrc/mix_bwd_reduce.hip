@@ -536,7 +536,7 @@ __global__ __launch_bounds__(256) void gram_large_kernel(BwdReduceArgs a) {
     }
 }
 
-template <int NP>
+template <int NP, bool PRECISE>
 __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
     using SK = SkWg<NP>;
     extern __shared__ float smem[];
@@ -556,6 +556,18 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         hp_s[tid] = tid < n ? a.Hpre[(size_t)b * a.hstride + tid] : 0.f;
         ho_s[tid] = tid < n ? a.Hpost[(size_t)b * a.hstride + tid] : 0.f;
     }
+    // inputs of the Sinkhorn recompute, requested now so that they arrive behind the part sums
+    // (out-of-range elements alias element 0 and are masked where they are used)
+    const int D = n * n + 2 * n;
+    const int r0 = SK::row(tid), c0 = SK::col0(tid);
+    const bool dyn = a.hstride != 0;
+    float pres[SK::EPL], bres[SK::EPL];
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++) {
+        const bool ok = dyn && r0 < n && c0 + e < n;
+        pres[e] = dyn ? a.P[(size_t)b * D + (ok ? 2 * n + r0 * n + c0 + e : 0)] : 0.f;
+        bres[e] = dyn ? a.b_res[ok ? r0 * n + c0 + e : 0] : 0.f;
+    }
     // sum the column parts; rows / columns >= n hold aliased garbage and are dropped here
     const float *raw = a.raw + (size_t)b * a.parts * kGramFloats;
     {
@@ -563,12 +575,17 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         float acc[EPT];
 #pragma unroll
         for (int k = 0; k < EPT; k++) acc[k] = 0.f;
-        for (int p = 0; p < a.parts; p++) {
-            float t[EPT];
+        for (int p0 = 0; p0 < a.parts; p0 += 4) {  // 48 loads in flight; surplus parts alias part 0
+            float t[4][EPT];
 #pragma unroll
-            for (int k = 0; k < EPT; k++) t[k] = raw[(size_t)p * kGramFloats + tid + 256 * k];
+            for (int q = 0; q < 4; q++)
 #pragma unroll
-            for (int k = 0; k < EPT; k++) acc[k] += t[k];
+                for (int k = 0; k < EPT; k++)
+                    t[q][k] = raw[(size_t)(p0 + q < a.parts ? p0 + q : 0) * kGramFloats + tid + 256 * k];
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+#pragma unroll
+                for (int k = 0; k < EPT; k++) acc[k] += p0 + q < a.parts ? t[q][k] : 0.f;
         }
 #pragma unroll
         for (int k = 0; k < EPT; k++) {
@@ -606,7 +623,6 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         s1 = s1 / qinv;  // vec_s holds W1 Hpre / q
     }
 
-    const int D = n * n + 2 * n;
     float dHpre = 0.f, dHpost = 0.f;
     if (w0 && lane < n) {
         dHpost = vec_s[lane];
@@ -635,18 +651,17 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         S0 = dtp * Pb[lane]; S1 = dto * Pb[n + lane];
     }
     // Sinkhorn forward recompute + exact backward, the matrix spread over all 256 threads
-    const int r0 = SK::row(tid), c0 = SK::col0(tid);
-    float E[SK::EPL], d[SK::EPL], pres[SK::EPL], u, v[SK::EPL];
+    float E[SK::EPL], d[SK::EPL], u, v[SK::EPL];
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;
         const bool ok = r0 < n && c < n;
-        pres[e] = ok ? Pb[2 * n + r0 * n + c] : 0.f;
-        E[e] = ok ? expf(al2 * pres[e] + a.b_res[r0 * n + c]) : 0.f;
+        pres[e] = ok ? pres[e] : 0.f;
+        E[e] = ok ? expf(al2 * pres[e] + bres[e]) : 0.f;
         d[e] = ok ? M_s[r0 * 33 + c] : 0.f;
     }
-    SK::forward(E, u, v, n, a.T, a.eps, sk_s, tid);
-    SK::backward(E, d, u, v, a.T, sk_s, tid);
+    SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
+    SK::template backward<PRECISE>(E, d, u, v, a.T, sk_s, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;
@@ -712,12 +727,13 @@ static hipError_t launch_large(const BwdReduceArgs &a, hipStream_t stream) {
     gram_large_kernel<TG, TX><<<dim3(a.B, a.parts), 256, smem1, stream>>>(a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
+    constexpr bool kPrecise = std::is_same<TX, float>::value;  // fp32 activations: the parity tier
     if (a.n <= 16) {
         const size_t smem2 = sizeof(float) * (3 * 32 * 33 + 64 + 96 + 4 + SkWg<16>::lds_floats(a.T));
-        coef_bwd_large_kernel<16><<<a.B, 256, smem2, stream>>>(a);
+        coef_bwd_large_kernel<16, kPrecise><<<a.B, 256, smem2, stream>>>(a);
     } else {
         const size_t smem2 = sizeof(float) * (3 * 32 * 33 + 64 + 96 + 4 + SkWg<32>::lds_floats(a.T));
-        coef_bwd_large_kernel<32><<<a.B, 256, smem2, stream>>>(a);
+        coef_bwd_large_kernel<32, kPrecise><<<a.B, 256, smem2, stream>>>(a);
     }
     return hipGetLastError();
 }

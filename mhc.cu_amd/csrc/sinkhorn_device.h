@@ -239,6 +239,8 @@ template <int NP> struct SkWg {
     }
 
     // E: exp(logits), 0 outside n x n.  On return M = u * E[e] * v[e]; rho/s hold the denominators.
+    // PRECISE selects IEEE divisions (fp32 parity tier) instead of v_rcp_f32 (1 ulp).
+    template <bool PRECISE = true>
     __device__ static __forceinline__ void forward(const float (&E)[EPL], float &u, float (&v)[EPL],
                                                    int n, int T, float eps, float *lds, int tid) {
         float *cw = lds, *rho = lds + 8 * NP, *s = rho + T * NP;
@@ -252,7 +254,7 @@ template <int NP> struct SkWg {
             for (int e = 0; e < EPL; e++) p += E[e] * v[e];
             p = row_allreduce(p);
             const float rr = r < n ? u * p + eps : 1.0f;
-            u = u / rr;
+            u = PRECISE ? u / rr : u * fast_rcp(rr);
             if ((tid % LPR) == 0) rho[t * NP + r] = rr;
             float q[EPL];
 #pragma unroll
@@ -261,7 +263,7 @@ template <int NP> struct SkWg {
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
                 const float sc = c0 + e < n ? v[e] * q[e] + eps : 1.0f;
-                v[e] = v[e] / sc;
+                v[e] = PRECISE ? v[e] / sc : v[e] * fast_rcp(sc);
                 if (r == 0) s[t * NP + c0 + e] = sc;
             }
         }
@@ -269,6 +271,7 @@ template <int NP> struct SkWg {
     }
 
     // d: in = dL/dM, out = dL/dE.  u, v: final scalings from forward (destroyed).
+    template <bool PRECISE = true>
     __device__ static __forceinline__ void backward(const float (&E)[EPL], float (&d)[EPL], float u,
                                                     float (&v)[EPL], int T, float *lds, int tid) {
         float *cw = lds;
@@ -289,9 +292,10 @@ template <int NP> struct SkWg {
             }
             const float rdot = u * row_allreduce(z);
             const float rr = rho[t * NP + r];
+            const float rri = PRECISE ? 0.f : fast_rcp(rr);
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
-                d[e] = (d[e] / sc[e] - rdot) / rr;
+                d[e] = PRECISE ? (d[e] / sc[e] - rdot) / rr : (d[e] * fast_rcp(sc[e]) - rdot) * rri;
                 v[e] *= sc[e];
             }
             u *= rr;
