@@ -690,7 +690,9 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
 template <typename TG, typename TX, int NP, int V>
 static hipError_t launch_small(const BwdReduceArgs &a, hipStream_t stream) {
     const int nch = (a.C / V + a.parts - 1) / a.parts;  // chunks per column part
-    int nt = (nch + 63) / 64 * 64;
+    // every thread gets the same number of chunks (whole 16-lane rows: the reduction works on them)
+    const int rounds = (nch + 255) / 256;
+    int nt = round_up((nch + rounds - 1) / rounds, 16);
     if (nt > 256) nt = 256;
     constexpr int K = NP * NP + 3 * NP + 1;
     const size_t smem = sizeof(float) * (K * 16 + K + SkSmall<NP>::scaling_floats(a.T));

@@ -209,49 +209,48 @@ hipError_t launch_finalize(const float *u, int rows_u, int C, float *dw, const f
 //   red_sum = (dM [n*n] | dHpre [n] | dHpost [n])
 // --------------------------------------------------------------------------------------------
 template <int NP>
-__global__ __launch_bounds__(64) void coef_bwd_static_kernel(const float *__restrict__ red_sum,
-                                                             const float *__restrict__ Hpre,
-                                                             const float *__restrict__ Hpost,
-                                                             const float *__restrict__ H_res_logits,
-                                                             float *__restrict__ dH_pre,
-                                                             float *__restrict__ dH_post,
-                                                             float *__restrict__ dH_res, int n, int T,
-                                                             float eps) {
-    using SK = SkLds<NP>;
-    extern __shared__ float lds[];
-    float *Es = lds, *dO = Es + NP * SK::LD;
-    float *u = dO + NP * SK::LD, *v = u + NP, *tmp = v + NP;
-    float *rho = tmp + NP, *ssc = rho + T * NP;
-    const int lane = threadIdx.x;
-    if (lane < n) {
-        const float hp = Hpre[lane], ho = Hpost[lane];
-        dH_pre[lane] = red_sum[n * n + lane] * hp * (1.0f - hp);
-        dH_post[lane] = red_sum[n * n + n + lane] * ho * (1.0f - 0.5f * ho);
+__global__ __launch_bounds__(256) void coef_bwd_static_kernel(const float *__restrict__ red_sum,
+                                                              const float *__restrict__ Hpre,
+                                                              const float *__restrict__ Hpost,
+                                                              const float *__restrict__ H_res_logits,
+                                                              float *__restrict__ dH_pre,
+                                                              float *__restrict__ dH_post,
+                                                              float *__restrict__ dH_res, int n, int T,
+                                                              float eps) {
+    // one workgroup, the matrix spread over the registers of its 256 threads (IEEE divisions: this
+    // kernel serves both precision tiers and runs once per backward call)
+    using SK = SkWg<NP>;
+    extern __shared__ float lds[];  // SK::lds_floats(T)
+    const int tid = threadIdx.x;
+    if (tid < n) {
+        const float hp = Hpre[tid], ho = Hpost[tid];
+        dH_pre[tid] = red_sum[n * n + tid] * hp * (1.0f - hp);
+        dH_post[tid] = red_sum[n * n + n + tid] * ho * (1.0f - 0.5f * ho);
     }
-    for (int e = lane; e < NP * NP; e += kWave) {
-        const int r0 = e / NP, c = e % NP;
-        const bool ok = r0 < n && c < n;
-        Es[r0 * SK::LD + c] = ok ? expf(H_res_logits[r0 * n + c]) : 0.f;
-        dO[r0 * SK::LD + c] = ok ? red_sum[r0 * n + c] : 0.f;
+    const int r0 = SK::row(tid), c0 = SK::col0(tid);
+    float E[SK::EPL], d[SK::EPL], u, v[SK::EPL];
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++) {
+        const bool ok = r0 < n && c0 + e < n;
+        E[e] = ok ? expf(H_res_logits[r0 * n + c0 + e]) : 0.f;
+        d[e] = ok ? red_sum[r0 * n + c0 + e] : 0.f;
     }
-    __syncthreads();
-    SK::forward(Es, u, v, n, T, eps, rho, ssc, lane);
-    SK::backward(Es, dO, u, v, tmp, n, T, rho, ssc, lane);
-    for (int e = lane; e < n * n; e += kWave) {
-        const int r0 = e / n, c = e % n;
-        dH_res[e] = dO[r0 * SK::LD + c] * Es[r0 * SK::LD + c];
-    }
+    SK::template forward<true>(E, u, v, n, T, eps, lds, tid);
+    SK::template backward<true>(E, d, u, v, T, lds, tid);
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++)
+        if (r0 < n && c0 + e < n) dH_res[r0 * n + c0 + e] = d[e] * E[e];
 }
 
 hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const float *Hpost,
                                   const float *H_res_logits, float *dH_pre, float *dH_post,
                                   float *dH_res, int n, int T, float eps, hipStream_t stream) {
     if (n <= 16) {
-        const size_t smem = sizeof(float) * SkLds<16>::backward_floats(T);
-        coef_bwd_static_kernel<16><<<1, 64, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
+        const size_t smem = sizeof(float) * SkWg<16>::lds_floats(T);
+        coef_bwd_static_kernel<16><<<1, 256, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
     } else {
-        const size_t smem = sizeof(float) * SkLds<32>::backward_floats(T);
-        coef_bwd_static_kernel<32><<<1, 64, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
+        const size_t smem = sizeof(float) * SkWg<32>::lds_floats(T);
+        coef_bwd_static_kernel<32><<<1, 256, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
     }
     return hipGetLastError();
 }
