@@ -90,7 +90,7 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
 
 // ---- static workspace layout -----------------------------------------------------------------
 struct StaFwdWs { float *Hpre, *Hpost, *M, *q, *agg; size_t bytes; };
-struct StaBwdWs { float *red, *s1, *u, *red_sum, *cs_red, *cs_u, *raw; size_t bytes; };
+struct StaBwdWs { float *red, *s1, *u, *red_sum, *raw; size_t bytes; };
 
 StaFwdWs carve_sta_fwd(void *ws, int B, int n, int C) {
     Carver c(ws);
@@ -105,12 +105,10 @@ StaBwdWs carve_sta_bwd(void *ws, int B, int n, int C) {
     Carver c(ws);
     const int D = n * n + 2 * n;
     StaBwdWs w;
-    w.red = c.floats((size_t)B * D);
+    w.red = c.floats((size_t)B * (D + 3));
     w.s1 = c.floats(B);
     w.u = c.floats((size_t)B * C);
-    w.red_sum = c.floats(D);
-    w.cs_red = c.floats(colsum_workspace_floats(B, D));
-    w.cs_u = c.floats(colsum_workspace_floats(B, C));
+    w.red_sum = c.floats(D + 3);
     w.raw = c.floats(n > 8 ? bwd_reduce_raw_floats(B, n, C) : 0);
     w.bytes = c.off;
     return w;
@@ -303,10 +301,12 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
     MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, 0,
                                  q, ws.s1, nullptr, nullptr, 0, nullptr, 0, nullptr, dx, df, ws.u, nullptr,
                                  nullptr, 1, B, n, C, st));
-    MHC_LAUNCH(launch_colsum(ws.red, B, D, D, ws.red_sum, ws.cs_red, st));
+    // one launch for both batch sums: dw = sum_b u, red_sum = sum_b red (its 3 padding columns land
+    // in red_sum[D..D+2] and are ignored)
+    MHC_LAUNCH(launch_finalize(ws.u, B, C, f_inject ? nullptr : dw, ws.red, B, D, ws.red_sum, ws.red_sum + D,
+                               nullptr, 1, 0, nullptr, st));
     MHC_LAUNCH(launch_coef_bwd_static(ws.red_sum, H_pre, H_post, H_res_logits, dH_pre, dH_post,
                                       dH_res, n, iters, eps, st));
-    if (!f_inject) MHC_LAUNCH(launch_colsum(ws.u, B, C, C, dw, ws.cs_u, st));
     return MHC_OK;
 }
 

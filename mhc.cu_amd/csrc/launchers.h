@@ -61,7 +61,7 @@ struct BwdCoefOut {
     float *dP;    // [B, DP]  dL/d(raw dot product) = dt * alpha_g / r, zero padded (dynamic only)
     float *cx;    // [B]      sum_d dt_d alpha_g p_d / (nC r^2)                    (dynamic only)
     float *s1;    // [B]      sum_c df_c w_c a_c
-    float *red;   // [B, n*n + 2n] raw per-sample (dM | dHpre | dHpost)             (static only)
+    float *red;   // [B, n*n + 2n + 3] raw per-sample (dM | dHpre | dHpost | 3 unused)   (static only)
     unsigned short *dPb;  // BP * DP bf16, dP in MFMA fragment order (frag_dpb), or nullptr
     unsigned short *dPT;  // 2 planes of DP * BP bf16, dP^T in fragment order (frag_dpt): value, remainder
     int BP;               // row pitch of dPT, a multiple of 32 that is >= B

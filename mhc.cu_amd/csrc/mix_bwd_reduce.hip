@@ -194,7 +194,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
     const int r0 = SK::row(g), c0 = SK::col0(g);
     if (a.hstride == 0) {
         // static H: raw sums only; the coefficient backward runs once on the batch total
-        float *red = a.out.red + (size_t)b * D;
+        float *red = a.out.red + (size_t)b * (D + 3);  // rows padded like dt, for the batch-sum launch
 #pragma unroll
         for (int e = 0; e < SK::EPL; e++)
             if (r0 < n && c0 + e < n) red[r0 * n + c0 + e] = tot[r0 * NP + c0 + e];
@@ -631,7 +631,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
     }
     if (tid == 0) a.out.s1[b] = s1;
     if (a.hstride == 0) {
-        float *red = a.out.red + (size_t)b * D;
+        float *red = a.out.red + (size_t)b * (D + 3);  // rows padded like dt, for the batch-sum launch
         for (int e = tid; e < n * n; e += 256) red[e] = M_s[(e / n) * 33 + (e % n)];
         if (w0 && lane < n) { red[n * n + lane] = dHpre; red[n * n + n + lane] = dHpost; }
         return;

@@ -9,9 +9,8 @@
 //   SkSmall<NP> (NP = 4, 8): a matrix lives in the registers of 16 consecutive lanes
 //       (NP*NP/16 elements per lane); all reductions are DPP moves, no LDS traffic on the
 //       forward path.  Four matrices per wave.
-//   SkLds<NP>   (NP = 16, 32): one wave per matrix, E and the running scalings u, v in LDS
-//       (iterate = diag(u) E diag(v)); a half-step is one mat-vec product.
-//   SkWg<NP>    (NP = 16, 32): one 256-thread workgroup per matrix, everything in registers.
+//   SkWg<NP>    (NP = 16, 32): one 256-thread workgroup per matrix, everything in registers,
+//       iterate kept in scaling form diag(u) E diag(v).
 #pragma once
 
 #include "mhc_common.h"
@@ -107,96 +106,14 @@ template <int NP> struct SkSmall {
 };
 
 // =============================================================================================
-// SkLds: one wave, matrix in LDS.  LD = NP + 1 keeps row and column walks conflict-free.
-// =============================================================================================
-template <int NP> struct SkLds {
-    static constexpr int LD = NP + 1;
-    // LDS floats: E [NP*LD], u [NP], v [NP], tmp [NP], (backward) dO [NP*LD], rho [T*NP], s [T*NP]
-    __host__ __device__ static constexpr int forward_floats() { return NP * LD + 3 * NP; }
-    __host__ __device__ static constexpr int backward_floats(int T) {
-        return 2 * NP * LD + 3 * NP + 2 * T * NP;
-    }
-
-    // Es holds E (0 outside n x n).  On return u, v hold the final scalings: M = u_r E_rc v_c.
-    // rho/s (optional): per-iteration denominators [T][NP].
-    __device__ static __forceinline__ void forward(const float *Es, float *u, float *v, int n, int T,
-                                                   float eps, float *rho, float *s, int lane) {
-        if (lane < NP) { u[lane] = 1.0f; v[lane] = 1.0f; }
-        __syncthreads();
-        for (int t = 0; t < T; t++) {
-            if (lane < n) {
-                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-                for (int c = 0; c < NP; c += 4) {
-                    a0 += Es[lane * LD + c] * v[c];
-                    a1 += Es[lane * LD + c + 1] * v[c + 1];
-                    a2 += Es[lane * LD + c + 2] * v[c + 2];
-                    a3 += Es[lane * LD + c + 3] * v[c + 3];
-                }
-                const float ur = u[lane];
-                const float r = ur * ((a0 + a1) + (a2 + a3)) + eps;
-                if (rho) rho[t * NP + lane] = r;
-                u[lane] = ur / r;
-            }
-            __syncthreads();
-            if (lane < n) {
-                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-                for (int r = 0; r < NP; r += 4) {
-                    a0 += Es[r * LD + lane] * u[r];
-                    a1 += Es[(r + 1) * LD + lane] * u[r + 1];
-                    a2 += Es[(r + 2) * LD + lane] * u[r + 2];
-                    a3 += Es[(r + 3) * LD + lane] * u[r + 3];
-                }
-                const float vc = v[lane];
-                const float sc = vc * ((a0 + a1) + (a2 + a3)) + eps;
-                if (s) s[t * NP + lane] = sc;
-                v[lane] = vc / sc;
-            }
-            __syncthreads();
-        }
-    }
-
-    // dO: in = dL/dM, out = dL/dE ([NP][LD]).  u, v: final scalings (destroyed).  tmp: [NP].
-    __device__ static __forceinline__ void backward(const float *Es, float *dO, float *u, float *v,
-                                                    float *tmp, int n, int T, const float *rho,
-                                                    const float *s, int lane) {
-        for (int t = T - 1; t >= 0; t--) {
-            // column dots with the iterate after column step t: Out = u E v
-            if (lane < n) {
-                float acc = 0.f;
-                for (int k = 0; k < n; k++) acc += dO[k * LD + lane] * u[k] * Es[k * LD + lane];
-                tmp[lane] = acc * v[lane];
-            }
-            __syncthreads();
-            // row lane r: dR = (dO - cdot)/s ; rdot = sum_k dR_k R_k, R = u E v s ; dIn = (dR - rdot)/rho
-            if (lane < n) {
-                const float ur = u[lane];
-                float acc = 0.f;
-                for (int k = 0; k < n; k++)
-                    acc += (dO[lane * LD + k] - tmp[k]) * Es[lane * LD + k] * v[k];
-                const float rdot = acc * ur;
-                const float rinv = 1.0f / rho[t * NP + lane];
-                for (int k = 0; k < n; k++)
-                    dO[lane * LD + k] =
-                        ((dO[lane * LD + k] - tmp[k]) / s[t * NP + k] - rdot) * rinv;
-            }
-            __syncthreads();
-            if (lane < n) {
-                u[lane] *= rho[t * NP + lane];
-                v[lane] *= s[t * NP + lane];
-            }
-            __syncthreads();
-        }
-    }
-};
-
-// =============================================================================================
 // SkWg: one 256-thread workgroup per matrix, NP = 16 or 32.  Thread t owns EPL consecutive
 // columns of row t / LPR of E and of the running gradient in registers; the iterate is kept in
 // scaling form diag(u) E diag(v) (u replicated over the lanes of a row, v over the rows).  A
 // half-step is one cross-lane reduction: rows inside a DPP row, columns inside the wave and then
 // across the 4 waves through a double-buffered LDS slot (one barrier per iteration).
-// Same arithmetic as SkLds (IEEE divisions, denominators rho/s kept per iteration), ~30x shorter
-// critical path.  Every thread of the workgroup must call forward/backward.
+// The denominators rho/s of every iteration are kept in LDS for the backward sweep, which unwinds
+// the scalings (u *= rho, v *= s) instead of storing iterates.  Every thread of the workgroup must
+// call forward/backward.
 // =============================================================================================
 template <int NP> struct SkWg {
     static_assert(NP == 16 || NP == 32, "SkWg handles 16x16 and 32x32 tiles");
