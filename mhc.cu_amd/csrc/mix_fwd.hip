@@ -141,7 +141,8 @@ struct LayerFwdArgs {
 };
 
 template <typename TX, typename TY, int NP, int V, int CPT>
-__global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
+__global__ __launch_bounds__(256, (CPT == 2 && NP == 4 && !std::is_same<TX, float>::value) ? 5 : 1)
+void layer_fwd_small_kernel(LayerFwdArgs a) {
     using SK = SkSmall<NP>;
     __shared__ float coef_s[NP * NP + 2 * NP];  // M | Hpre | Hpost
     __shared__ float red[4];
@@ -291,11 +292,18 @@ __global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
     }
 
     // ---- 3. aggregate + RMS ------------------------------------------------------------------
-    float xv[CPT][NP][V];
+    // The tile stays in registers as raw words; LEAN (two chunks per thread) widens a stream at
+    // the point of use instead of holding the fp32 copy of the whole tile, which keeps the
+    // kernel under 96 registers, i.e. five workgroups per CU (1280 samples then fit in one round
+    // of the grid); the extra conversions are cheaper than a second round.
+    constexpr bool LEAN = CPT >= 2 && NP <= 4 && !std::is_same<TX, float>::value;
+    float xv[LEAN ? 1 : CPT][NP][V];
+    if constexpr (!LEAN) {
 #pragma unroll
-    for (int k = 0; k < CPT; k++)
+        for (int k = 0; k < CPT; k++)
 #pragma unroll
-        for (int i = 0; i < NP; i++) xr[k][i].get(xv[k][i]);  // streams >= n meet zero coefficients
+            for (int i = 0; i < NP; i++) xr[k][i].get(xv[k][i]);  // streams >= n meet zero coefficients
+    }
     float av[CPT][V];
     float qinv = 1.0f;
     if (!inject) {
@@ -303,13 +311,20 @@ __global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
         for (int k = 0; k < CPT; k++) {
             const bool live = tid + k * 256 < nch;  // chunks beyond C alias chunk 0: not counted
+            float s_a[V];
+#pragma unroll
+            for (int v = 0; v < V; v++) s_a[v] = 0.f;
+#pragma unroll
+            for (int i = 0; i < NP; i++) {
+                float t[V];
+                if constexpr (LEAN) xr[k][i].get(t);
+#pragma unroll
+                for (int v = 0; v < V; v++) s_a[v] += hpre[i] * (LEAN ? t[v] : xv[LEAN ? 0 : k][i][v]);
+            }
 #pragma unroll
             for (int v = 0; v < V; v++) {
-                float s_a = 0.f;
-#pragma unroll
-                for (int i = 0; i < NP; i++) s_a += hpre[i] * xv[k][i][v];
-                av[k][v] = s_a;
-                ssq += live ? s_a * s_a : 0.f;
+                av[k][v] = s_a[v];
+                ssq += live ? s_a[v] * s_a[v] : 0.f;
             }
         }
         ssq = block_allreduce_sum<256>(ssq, red);
@@ -340,9 +355,13 @@ __global__ __launch_bounds__(256) void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
                     for (int v = 0; v < V; v++) out[v] = hpost[i] * f[v];
 #pragma unroll
-                    for (int j = 0; j < NP; j++)
+                    for (int j = 0; j < NP; j++) {
+                        float t[V];
+                        if constexpr (LEAN) xr[k][j].get(t);
+                        const float mij = LEAN ? coef_s[i * NP + j] : Mr[i][j];
 #pragma unroll
-                        for (int v = 0; v < V; v++) out[v] += Mr[i][j] * xv[k][j][v];
+                        for (int v = 0; v < V; v++) out[v] += mij * (LEAN ? t[v] : xv[LEAN ? 0 : k][j][v]);
+                    }
                     store_vec<TY, V>(yb + (size_t)i * C + c, out);
                 }
             }
