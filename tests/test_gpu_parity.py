@@ -120,7 +120,10 @@ def test_dynamic_fp32_vs_oracle(B, n, C, inject):
                                    (4, 32, 64), (2, 32, 1040), (3, 4, 20),
                                    # more than 128 samples with a wide projection: several sample
                                    # blocks / groups in the projection kernels
-                                   (160, 20, 64), (130, 32, 136)])
+                                   (160, 20, 64), (130, 32, 136),
+                                   # two chunks per thread with a ragged chunk count and a partial sample tile;
+                                   # n between the tile sizes; one sample; C not a multiple of 8 with n > 8
+                                   (33, 4, 2568), (3, 12, 40), (2, 24, 104), (1, 32, 128), (3, 20, 36)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_dynamic_bf16_vs_oracle(B, n, C, out_dtype):
     x, dy, _, p = nm.make_dynamic_inputs(B, n, C, bf16_round=True)
