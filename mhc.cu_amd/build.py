@@ -1,6 +1,6 @@
 """Builds libmhc_hip.so (hand-written HIP kernels + C ABI) for gfx950 with hipcc.
 
-    python mhc.cu_amd/build.py [--jobs N] [--force]
+    python mhc.cu_amd/build.py [--jobs N] [--profile]
 
 hipcc cross-compiles for gfx950 without a GPU.  The library lands in mhc.cu_amd/mhc/ next to
 the Python package that loads it; object files go to mhc.cu_amd/build/.
@@ -34,33 +34,40 @@ def _hipcc():
     return "hipcc"
 
 
-def _compile(src):
-    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+PROFILE_LIB = os.path.join(HERE, "mhc", "libmhc_hip_profile.so")
+
+
+def _compile(src, extra=(), suffix=""):
+    obj = os.path.join(OBJ, os.path.splitext(src)[0] + suffix + ".o")
+    cmd = [_hipcc(), *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     p = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in p.stderr.splitlines() if "packed-fp32-ops" not in l)
     return src, obj, p.returncode, err
 
 
-def build(jobs: int = 8, verbose: bool = True):
+def build(jobs: int = 8, verbose: bool = True, profile: bool = False):
+    """profile=True builds libmhc_hip_profile.so instead: the same library with the in-kernel phase
+    profiler compiled in (csrc/phase_profiler.h) and the extra entry point mhc_phase_read."""
     os.makedirs(OBJ, exist_ok=True)
     objs = []
+    extra, suffix, lib = ((("-DMHC_PHASE_PROFILE", "-fgpu-rdc"), "_prof", PROFILE_LIB) if profile else ((), "", LIB))
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
-        for src, obj, rc, err in ex.map(_compile, SOURCES):
+        for src, obj, rc, err in ex.map(lambda s_: _compile(s_, extra, suffix), SOURCES):
             if err.strip() and verbose:
                 print(f"[{src}]\n{err}", file=sys.stderr)
             if rc != 0:
                 raise RuntimeError(f"hipcc failed on {src}")
             objs.append(obj)
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *(["-fgpu-rdc"] if profile else []), "-o", lib, *objs]
     subprocess.check_call(cmd)
     if verbose:
-        print("built", LIB)
-    return LIB
+        print("built", lib)
+    return lib
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
+    ap.add_argument("--profile", action="store_true", help="build libmhc_hip_profile.so (in-kernel phase profiler)")
     a = ap.parse_args()
-    build(a.jobs)
+    build(a.jobs, profile=a.profile)

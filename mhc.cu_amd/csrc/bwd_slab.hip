@@ -17,6 +17,7 @@
 // Per tile: two barriers, x and dy read once from HBM, dx written once; no atomics.
 #include "launchers.h"
 #include "mhc_common.h"
+#include "phase_profiler.h"
 
 namespace mhc {
 
@@ -91,6 +92,10 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
     bf16_t *x_s = reinterpret_cast<bf16_t *>(dxf_s + 32 * kSlabLDF);         // [32][LDX] bf16
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = a.n, C = a.C, nC = n * C, D = n * n + 2 * n;
+    const int pwg = blockIdx.y * gridDim.x + blockIdx.x;
+    (void)pwg;
+    MHC_PHASE_ZERO(kPhaseBwdSlab, pwg);
+    MHC_PHASE_BEGIN(pclk);
     const int c0 = blockIdx.x * kSlabCW;
     const int b_begin = blockIdx.y * a.b_per_split;
     const int b_end = min(a.B, b_begin + a.b_per_split);
@@ -164,6 +169,7 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
     TileRegs cur, nxt;
     if (b_begin < b_end) load_tile(b_begin, cur);
 
+    MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 0, pclk);
     for (int sb = b_begin; sb < b_end; sb += 32) {
         const int b = sb + bl;
         const bool bok = b < b_end && cok;
@@ -212,6 +218,7 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
             }
         }
         __syncthreads();
+        MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 1, pclk);
 
         // ---- phase B: matrix cores ----------------------------------------------------------------
         {
@@ -238,6 +245,7 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
             }
         }
         __syncthreads();
+        MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 2, pclk);
 
         // ---- prefetch the next tile, then phase C: finish dx on the VALU ---------------------------
         const bool more = sb + 32 < b_end;
@@ -301,6 +309,7 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
         // no barrier needed here: the next tile's x_s writes come after barrier 2 of this tile (all
         // fragment reads done) and its dxf_s writes come after its own barrier 1 (all phase C done)
         if (more) cur = nxt;
+        MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 3, pclk);
     }
 
     // ---- outputs of the split -----------------------------------------------------------------------
@@ -343,6 +352,7 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
             a.dt_part[(size_t)blockIdx.y * (D + 3) + tid] = s;
         }
     }
+    MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 4, pclk);
 }
 
 bool bwd_slab_supported(int x_dtype, int y_dtype, int phi_dtype, int n, int C) {

@@ -4,6 +4,7 @@
 #include "../../include/mhc_hip.h"
 
 #include "launchers.h"
+#include "phase_profiler.h"
 
 #include <stdint.h>
 
@@ -116,7 +117,24 @@ StaBwdWs carve_sta_bwd(void *ws, int B, int n, int C) {
 
 }  // namespace
 
+#ifdef MHC_PHASE_PROFILE
+namespace mhc {
+__device__ unsigned long long g_phase[kPhaseKernels][kPhaseMaxWg][kPhaseMaxMarks];
+}
+#endif
+
 extern "C" {
+
+#ifdef MHC_PHASE_PROFILE
+// Profile build only (declared in csrc/phase_profiler.h's host interface, not in the product header):
+// copies the stamp table of one instrumented kernel to host memory; returns the HIP status.
+__attribute__((visibility("default"))) int mhc_phase_read(int kernel, unsigned long long *host, int workgroups) {
+    if (kernel < 0 || kernel >= mhc::kPhaseKernels || workgroups > mhc::kPhaseMaxWg) return -1;
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mhc::g_phase),
+                                    sizeof(unsigned long long) * mhc::kPhaseMaxMarks * workgroups,
+                                    sizeof(unsigned long long) * mhc::kPhaseMaxMarks * mhc::kPhaseMaxWg * kernel);
+}
+#endif
 
 int mhc_abi_version(void) { return MHC_ABI_VERSION; }
 

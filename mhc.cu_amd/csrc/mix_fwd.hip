@@ -5,6 +5,7 @@
 // a and f never leave the chip; x is fetched from HBM once (the second sweep over the sample's
 // tile hits L1/L2).  With an injected f the first sweep is skipped.
 #include "launchers.h"
+#include "phase_profiler.h"
 #include "sinkhorn_device.h"
 
 namespace mhc {
@@ -152,6 +153,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
     const bool inject = a.f_inject != nullptr;
     const bool dyn = a.Ppart != nullptr;
     const int nch = C / V;
+    MHC_PHASE(kPhaseFwdFused, b, 0);
 
     // ---- 1. loads.  Wave 0 first asks for the small coefficient inputs (they return ahead of
     // the bulk data, so the Sinkhorn chain below runs while the tile is still streaming in),
@@ -202,6 +204,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
         }
     }
 
+    MHC_PHASE(kPhaseFwdFused, b, 1);
     // ---- 2. coefficients on wave 0 -----------------------------------------------------------
     if (tid < 64) {
         float pe[SK::EPL], ppre = 0.f, ppost = 0.f, ssq = 0.f;
@@ -238,6 +241,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
                 pe[e] = xor32_add(xor16_add(pe[e]));
             }
         }
+        MHC_PHASE(kPhaseFwdFused, b, 2);
         if (tid < 16) {
             float rinv = 0.f;
             if (dyn) {
@@ -281,7 +285,9 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             }
         }
     }
+    MHC_PHASE(kPhaseFwdFused, b, 3);
     __syncthreads();
+    MHC_PHASE(kPhaseFwdFused, b, 4);
     float hpre[NP], hpost[NP], Mr[NP][NP];
 #pragma unroll
     for (int i = 0; i < NP; i++) {
@@ -335,6 +341,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
         a.q[b] = 1.0f;
     }
 
+    MHC_PHASE(kPhaseFwdFused, b, 5);
     // ---- 4. mix + distribute -------------------------------------------------------------------
 #pragma unroll
     for (int k = 0; k < CPT; k++) {
@@ -367,6 +374,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             }
         }
     }
+    MHC_PHASE(kPhaseFwdFused, b, 6);
 }
 
 // Largest CPT instantiated: tiles with more than 4 * 256 vector chunks per stream take the

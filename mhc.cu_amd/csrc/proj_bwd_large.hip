@@ -19,7 +19,6 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 constexpr int kPL_KW = 128;             // columns per workgroup: wave w owns columns 32w .. 32w+32
 constexpr int kPL_LD = kPL_KW + 8;      // LDS row pitch in elements (272 bytes, 16-byte aligned)
 constexpr int kPL_SB = 128;             // samples per block of the dphi kernel
-constexpr int kPL_DC = 64;              // phi rows per LDS chunk of the dxflat kernel
 
 struct ProjBwdLargeArgs {
     const bf16_t *x;     // [B][nC]

@@ -1,0 +1,107 @@
+// Prints the in-kernel phase timeline of the fused forward kernel and of the slab backward kernel.
+//
+//   phase_profile [--batch B] [--hidden C] [--expansion n]          (n <= 4, C % 8 == 0, bf16)
+//
+// Links libmhc_hip_profile.so (python mhc.cu_amd/build.py --profile), the build of the library with
+// csrc/phase_profiler.h compiled in.  Counterpart of the reference's HostProfiler::print_summary
+// (src/csrc/include/utils.cuh:305-347): per phase the mean / 10th / 90th percentile over the
+// recorded workgroups, in shader-clock ticks (s_memtime) and as a share of the workgroup's life.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "../../include/mhc_hip.h"
+
+extern "C" int mhc_phase_read(int kernel, unsigned long long *host, int workgroups);
+
+#define HIP_OK(e) do { hipError_t _e = (e); if (_e != hipSuccess) { fprintf(stderr, "HIP error %s at line %d\n", hipGetErrorString(_e), __LINE__); exit(1); } } while (0)
+#define MHC_OK_(e) do { int _s = (e); if (_s != MHC_OK) { fprintf(stderr, "mhc error %d (%s) at line %d\n", _s, mhc_status_string(_s), __LINE__); exit(1); } } while (0)
+
+static uint16_t to_bf16(float f) { uint32_t u; memcpy(&u, &f, 4); u += 0x7fffu + ((u >> 16) & 1u); return (uint16_t)(u >> 16); }
+static void *dev_bf16(size_t n, float scale, std::mt19937 &g) {
+    std::normal_distribution<float> d(0.f, 1.f);
+    std::vector<uint16_t> h(n);
+    for (auto &v : h) v = to_bf16(scale * d(g));
+    void *p; HIP_OK(hipMalloc(&p, n * 2 + 16)); HIP_OK(hipMemcpy(p, h.data(), n * 2, hipMemcpyHostToDevice));
+    return p;
+}
+static float *dev_f32(size_t n, float val) {
+    std::vector<float> h(n, val);
+    float *p; HIP_OK(hipMalloc(&p, n * 4 + 16)); HIP_OK(hipMemcpy(p, h.data(), n * 4, hipMemcpyHostToDevice));
+    return p;
+}
+
+static void summary(const char *title, int kernel, int wgs, const std::vector<const char *> &names, bool stamps) {
+    constexpr int M = 8;
+    std::vector<unsigned long long> t((size_t)wgs * M);
+    if (mhc_phase_read(kernel, t.data(), wgs) != 0) { printf("%s: read failed\n", title); return; }
+    printf("\n%s (%d workgroups, shader-clock ticks)\n", title, wgs);
+    printf("%-34s %10s %10s %10s %7s\n", "phase", "mean", "p10", "p90", "share");
+    const int np = (int)names.size();
+    std::vector<std::vector<double>> d(np);
+    std::vector<double> life;
+    for (int w = 0; w < wgs; w++) {
+        double total = 0;
+        for (int i = 0; i < np; i++) {
+            const double v = stamps ? (double)(t[(size_t)w * M + i + 1] - t[(size_t)w * M + i]) : (double)t[(size_t)w * M + i];
+            d[i].push_back(v);
+            total += v;
+        }
+        life.push_back(total);
+    }
+    double life_mean = 0;
+    for (double v : life) life_mean += v;
+    life_mean /= wgs;
+    for (int i = 0; i < np; i++) {
+        std::sort(d[i].begin(), d[i].end());
+        double mean = 0;
+        for (double v : d[i]) mean += v;
+        mean /= wgs;
+        printf("%-34s %10.0f %10.0f %10.0f %6.1f%%\n", names[i], mean, d[i][wgs / 10], d[i][wgs * 9 / 10], 100.0 * mean / life_mean);
+    }
+    printf("%-34s %10.0f\n", "workgroup life", life_mean);
+}
+
+int main(int argc, char **argv) {
+    int B = 1280, C = 2560, n = 4, T = 20;
+    for (int i = 1; i < argc; i++) {
+        auto is = [&](const char *s) { return strcmp(argv[i], s) == 0; };
+        if (is("--batch") && i + 1 < argc) B = atoi(argv[++i]);
+        else if (is("--hidden") && i + 1 < argc) C = atoi(argv[++i]);
+        else if (is("--expansion") && i + 1 < argc) n = atoi(argv[++i]);
+        else { fprintf(stderr, "unknown argument %s\n", argv[i]); return 2; }
+    }
+    if (n > 4 || C % 8) { fprintf(stderr, "the instrumented kernels serve n <= 4 with C %% 8 == 0\n"); return 2; }
+    const size_t BnC = (size_t)B * n * C, nC = (size_t)n * C, D = (size_t)n * n + 2 * n;
+    std::mt19937 g(0);
+    void *x = dev_bf16(BnC, 1.f, g), *dy = dev_bf16(BnC, 1.f, g), *phi = dev_bf16(D * nC, 0.02f, g), *w = dev_bf16(C, 0.f, g);
+    { std::vector<uint16_t> one(C, to_bf16(1.f)); HIP_OK(hipMemcpy(w, one.data(), C * 2, hipMemcpyHostToDevice)); }
+    void *y, *dx; HIP_OK(hipMalloc(&y, BnC * 2)); HIP_OK(hipMalloc(&dx, BnC * 2));
+    float *bias = dev_f32(D, 0.f), *alpha = dev_f32(3, 0.01f), *Hp = dev_f32((size_t)B * n, 0.f), *Ho = dev_f32((size_t)B * n, 0.f),
+          *M = dev_f32((size_t)B * n * n, 0.f), *P = dev_f32(B * D, 0.f), *r = dev_f32(B, 0.f), *q = dev_f32(B, 0.f),
+          *dw = dev_f32(C, 0.f), *dphi = dev_f32(D * nC, 0.f), *dbias = dev_f32(D, 0.f), *dalpha = dev_f32(3, 0.f);
+    const size_t wsb = mhc_layer_dynamic_workspace_bytes(B, n, C);
+    void *ws; HIP_OK(hipMalloc(&ws, wsb + 256));
+    for (int it = 0; it < 3; it++) {
+        MHC_OK_(mhc_layer_fwd_dynamic(x, MHC_BF16, w, MHC_BF16, phi, MHC_BF16, bias, alpha, nullptr, y, MHC_BF16, Hp, Ho, M, P, r,
+                                      q, B, n, C, T, 1e-6f, ws, wsb, nullptr));
+        MHC_OK_(mhc_layer_bwd_dynamic(dy, MHC_BF16, x, MHC_BF16, w, MHC_BF16, phi, MHC_BF16, bias, alpha, nullptr, Hp, Ho, M, P, r, q,
+                                      dx, nullptr, dw, dphi, dbias, dalpha, B, n, C, T, 1e-6f, ws, wsb, nullptr));
+        HIP_OK(hipDeviceSynchronize());
+    }
+    printf("phase profile: dynamic H, bf16, B=%d C=%d n=%d (last of 3 warm calls)\n", B, C, n);
+    summary("fused forward kernel, one workgroup per sample", 0, std::min(B, 4096),
+            {"issue loads", "coefficient inputs arrive", "activations + Sinkhorn", "barrier", "tile arrives, aggregate, RMS",
+             "mix, stores issued"}, true);
+    const int slabs = (C + 63) / 64;
+    summary("slab backward kernel, one workgroup per (64 channels, batch split)", 1, std::min(slabs * 4, 4096),
+            {"prologue (phi slab, first loads)", "tile loads, LDS, barrier (all tiles)", "matrix cores, barrier (all tiles)",
+             "coefficients, VALU, stores (all)", "epilogue (partials)"}, false);
+    return 0;
+}
