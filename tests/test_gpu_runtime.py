@@ -1,0 +1,87 @@
+"""Runtime properties of the C ABI calls: HIP-graph capture and replay, bit-exact determinism,
+re-entrancy across streams with separate workspaces, and the compute_dtype option of MHCLayer."""
+import pytest
+import torch
+
+from oracle import naive_mhc as nm
+
+pytestmark = pytest.mark.gpu
+
+
+def _bf16_step(B, n, C):
+    import bench
+
+    cfg = dict(kind="dynamic", B=B, n=n, C=C, dtype="bf16", bwd=True)
+    return bench.Step(cfg, "L", torch)
+
+
+@pytest.mark.parametrize("B,n,C", [(96, 4, 512), (40, 8, 256), (24, 32, 256)])
+def test_graph_replay_matches_eager_and_is_deterministic(B, n, C):
+    """Forward + backward captured in one HIP graph; three replays, with unrelated eager work and
+    synchronisations between them, must each reproduce the eager results bit for bit."""
+    st = _bf16_step(B, n, C)
+    outs = lambda: [t.clone() for t in (st.y, st.dx, st.dw, st.dphi, st.dbias, st.dalpha)]
+    st.step()
+    torch.cuda.synchronize()
+    eager = outs()
+    st.step()
+    torch.cuda.synchronize()
+    for a, b in zip(eager, outs()):
+        assert torch.equal(a, b), "two eager runs differ"
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        st.step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        st.step()
+    scratch = torch.zeros(1 << 20, device="cuda")
+    for rep in range(3):
+        for t in (st.y, st.dx, st.dw, st.dphi, st.dbias, st.dalpha):
+            t.fill_(float("nan"))
+        scratch.add_(1.0).sum().item()  # eager work + a host sync between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("y", "dx", "dw", "dphi", "dbias", "dalpha"), eager, outs()):
+            assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager result"
+
+
+def test_two_streams_with_separate_workspaces():
+    """Two layer calls in flight on two streams, each with its own workspace, give the results of
+    running them one after the other."""
+    a, b = _bf16_step(64, 4, 512), _bf16_step(48, 4, 1024)
+    for s in (a, b):
+        s.step()
+    torch.cuda.synchronize()
+    ref = [[t.clone() for t in (s.y, s.dx, s.dphi)] for s in (a, b)]
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    for _ in range(5):
+        with torch.cuda.stream(s1):
+            a.step()
+        with torch.cuda.stream(s2):
+            b.step()
+    torch.cuda.synchronize()
+    for s, r in zip((a, b), ref):
+        for got, want in zip((s.y, s.dx, s.dphi), r):
+            assert torch.equal(got, want)
+
+
+def test_compute_dtype_casts_like_the_reference():
+    """fp32 input with compute_dtype=bf16 equals feeding the bf16-rounded input; result stays fp32."""
+    from mhc import MHCLayer
+
+    B, n, C = 16, 4, 256
+    torch.manual_seed(3)
+    layer = MHCLayer(C, n, use_dynamic_h=True, compute_dtype=torch.bfloat16).cuda()
+    x = torch.randn(B, n, C, device="cuda")
+    y = layer(x)
+    assert y.dtype == torch.float32
+    plain = MHCLayer(C, n, use_dynamic_h=True).cuda()
+    plain.load_state_dict(layer.state_dict())
+    y2 = plain(x.bfloat16())
+    assert torch.equal(y, y2)
+    xg = x.clone().requires_grad_(True)
+    layer(xg).sum().backward()
+    assert xg.grad is not None and xg.grad.dtype == torch.float32 and torch.isfinite(xg.grad).all()
