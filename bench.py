@@ -63,12 +63,42 @@ def algorithmic_bytes(cfg, view):
     return fwd, bwd
 
 
+def synthetic_inputs(torch, cfg, with_f):
+    """Seeded synthetic inputs of a configuration, on the host, as fp32 tensors: x, dy (and f) ~ N(0,1)
+    from seed 0; parameters from seed 1: phi ~ N(0, 0.02^2), bias = 0, alpha = 0.01, w = 1 (dynamic),
+    logits ~ N(0,1) (static).  For the bf16 configurations everything stored in bf16 on the device is
+    rounded to bf16 here, so the CPU baseline sees the same values as the GPU."""
+    B, n, C = cfg["B"], cfg["n"], cfg["C"]
+    gd, gp = torch.Generator().manual_seed(0), torch.Generator().manual_seed(1)
+    x = torch.randn(B, n, C, generator=gd)
+    dy = torch.randn(B, n, C, generator=gd)
+    f = torch.randn(B, C, generator=gd) if with_f else None
+    if cfg["kind"] == "dynamic":
+        nC = n * C
+        p = {"w": torch.ones(C),
+             "phi_pre": torch.randn(n, nC, generator=gp) * 0.02,
+             "phi_post": torch.randn(n, nC, generator=gp) * 0.02,
+             "phi_res": torch.randn(n * n, nC, generator=gp) * 0.02,
+             "alpha_pre": torch.tensor(0.01), "alpha_post": torch.tensor(0.01), "alpha_res": torch.tensor(0.01),
+             "b_pre": torch.zeros(n), "b_post": torch.zeros(n), "b_res": torch.zeros(n, n)}
+    else:
+        p = {"w": torch.ones(C), "H_pre": torch.randn(n, generator=gp), "H_post": torch.randn(n, generator=gp),
+             "H_res": torch.randn(n, n, generator=gp)}
+    if cfg["dtype"] == "bf16":
+        rb = lambda t: t.bfloat16().float()
+        x, dy = rb(x), rb(dy)
+        f = None if f is None else rb(f)
+        for k in ("w", "phi_pre", "phi_post", "phi_res"):
+            if k in p:
+                p[k] = rb(p[k])
+    return x, dy, f, p
+
+
 class Step:
     """Pre-allocated tensors and the two C-ABI calls of one configuration."""
 
     def __init__(self, cfg, view, torch):
         from mhc import _lib
-        from oracle import naive_mhc as nm
 
         self.torch, self.lib, self._lib = torch, _lib.lib, _lib
         self.cfg, self.view = cfg, view
@@ -77,10 +107,7 @@ class Step:
         act = torch.float32 if cfg["dtype"] == "f32" else torch.bfloat16
         bf = cfg["dtype"] == "bf16"
         self.dynamic = cfg["kind"] == "dynamic"
-        if self.dynamic:
-            x, dy, f, p = nm.make_dynamic_inputs(B, n, C, bf16_round=bf, with_f=(view == "K"))
-        else:
-            x, dy, f, p = nm.make_static_inputs(B, n, C, with_f=(view == "K"))
+        x, dy, f, p = synthetic_inputs(torch, cfg, with_f=(view == "K"))
         self.host = dict(x=x, dy=dy, f=f, p=p)
         to = lambda t, dt: t.to(dt).to(dev).contiguous()
         self.x, self.dy = to(x, act), to(dy, act)
