@@ -43,8 +43,9 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
         }
         __syncthreads();
     }
+    // grid.y workgroups share the channels of a sample group
     const int nch = C / V;
-    for (int ch = tid; ch < nch; ch += nt) {
+    for (int ch = blockIdx.y * nt + tid; ch < nch; ch += nt * gridDim.y) {
       const int c = ch * V;
       float usum[V];
 #pragma unroll
@@ -73,6 +74,14 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
             const size_t so = (size_t)(i < n ? i : 0) * C + c;
             load_vec<TG, V>(gb + so, gv[i]);
             load_vec<TX, V>(xb + so, xv[i]);
+        }
+        // dx_in may alias dx, so the compiler cannot move its loads above the stores of earlier
+        // rows: request all rows here (every thread reads exactly the elements it later writes)
+        RawVec<TX, V> prev[NP];
+        if (a.dx_in) {
+#pragma unroll
+            for (int j = 0; j < NP; j++)
+                prev[j].load(static_cast<const TX *>(a.dx_in) + ((size_t)b * n + (j < n ? j : 0)) * C + c);
         }
         float da[V], dfv[V], uv[V];
 #pragma unroll
@@ -122,10 +131,10 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
                     }
                 }
                 if (a.dx_in) {
-                    float prev[V];
-                    load_vec<TX, V>(static_cast<const TX *>(a.dx_in) + ((size_t)b * n + j) * C + c, prev);
+                    float pv[V];
+                    prev[j].get(pv);
 #pragma unroll
-                    for (int v = 0; v < V; v++) out[v] += prev[v];
+                    for (int v = 0; v < V; v++) out[v] += pv[v];
                 }
                 store_vec<TX, V>(dxb + (size_t)j * C + c, out);
             }
@@ -134,7 +143,7 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
       if (!inject && a.u) store_vec<float, V>(a.u + (size_t)grp * C + c, usum);
     }
     // per-group sums of the logit gradients (feeds dbias / dalpha)
-    if (a.dtpart) {
+    if (a.dtpart && blockIdx.y == 0) {
         for (int col = tid; col < D + 3; col += nt) {
             float acc = 0.f;
             for (int b = b_first; b < b_last; b++) acc += a.dt[(size_t)b * (D + 3) + col];
@@ -334,14 +343,22 @@ static hipError_t launch_large_mfma(const BwdDxArgs &a, hipStream_t stream) {
     return hipGetLastError();
 }
 
+static int groups_of(const BwdDxArgs &a) { return (a.B + a.spg - 1) / a.spg; }
+
 template <typename TG, typename TX, int NP, int V>
 static hipError_t launch_one(const BwdDxArgs &a, hipStream_t stream) {
     const int nch = a.C / V;
     int nt = (nch + 63) / 64 * 64;
     if (nt > 256) nt = 256;
+    int ny = 1;
+    if (NP <= 8) {
+        // one wave per workgroup and one channel chunk per thread: every lane is busy and the grid
+        // has enough workgroups to keep loads of many samples in flight on each CU
+        nt = 64;
+        ny = (nch + 63) / 64;
+    }
     const size_t smem = sizeof(float) * (NP >= 16 ? NP * NP : 1);
-    const int groups = (a.B + a.spg - 1) / a.spg;
-    mix_bwd_dx_kernel<TG, TX, NP, V><<<groups, nt, smem, stream>>>(a);
+    mix_bwd_dx_kernel<TG, TX, NP, V><<<dim3(groups_of(a), ny), nt, smem, stream>>>(a);
     return hipGetLastError();
 }
 
