@@ -264,6 +264,7 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
                 k2 = s1v * qinv * qinv * qinv / (float)C;
             }
             float dfv[8];
+            uint32_t dxw[kSlabNS][2];  // packed dx of the first half, stored with the second (16 bytes per stream)
             // two halves of four channels keep the live unpacked values small
 #pragma unroll
             for (int h = 0; h < 2; h++) {
@@ -300,7 +301,13 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
                             for (int i = 0; i < kSlabNS; i++) sacc += Mr[i][j] * gv[i][v];
                             out[v] = sacc;
                         }
-                        store_vec<bf16_t, 4>(a.dx + (size_t)b * nC + (size_t)j * C + cth + 4 * h, out);
+                        if (h == 0) {
+                            dxw[j][0] = pack_bf16x2(out[0], out[1]);
+                            dxw[j][1] = pack_bf16x2(out[2], out[3]);
+                        } else {
+                            st16<true>(a.dx + (size_t)b * nC + (size_t)j * C + cth, dxw[j][0], dxw[j][1],
+                                       pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3]));
+                        }
                     }
                 }
             }

@@ -83,7 +83,7 @@ template <int NP> __global__ __launch_bounds__(64) void coef_fwd_small_kernel(Co
 // matrix spread over their registers (SkWg).
 template <int NP, bool PRECISE> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     using SK = SkWg<NP>;
-    extern __shared__ float lds[];
+    extern __shared__ __align__(16) float lds[];
     float *lg = lds;                       // [NP*NP + 2*NP] logits: pre | post | res (row-major n x n)
     float *sk_s = lg + NP * NP + 2 * NP;   // SK::lds_floats(T)
     const int tid = threadIdx.x;
@@ -145,11 +145,11 @@ template <int NP, bool PRECISE> __global__ __launch_bounds__(256) void coef_fwd_
         a.Hpost[b * n + tid] = 2.0f * sigmoidf_acc(lg[n + tid]);
     }
     const int r0 = SK::row(tid), c0 = SK::col0(tid);
-    float E[SK::EPL], u, v[SK::EPL];
+    float E[SK::EPL], ET[SK::EPL], u, v[SK::EPL];
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         E[e] = (r0 < n && c0 + e < n) ? expf(lg[2 * n + r0 * n + c0 + e]) : 0.f;
-    SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
+    SK::template forward<PRECISE>(E, ET, u, v, n, a.T, a.eps, sk_s, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         if (r0 < n && c0 + e < n) a.M[(size_t)b * n * n + r0 * n + c0 + e] = u * E[e] * v[e];

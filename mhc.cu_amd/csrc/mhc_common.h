@@ -82,32 +82,50 @@ __device__ __forceinline__ void load_vec(const T *__restrict__ p, float (&out)[V
     }
 }
 
-template <typename T, int V>
+// Raw stores of 16 / 8 / 4 bytes.  STREAM marks the data as written once and not read again soon
+// (the `nt` bit of the store): a large output then does not push the operands that other
+// workgroups still re-read out of L2.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+template <bool STREAM> __device__ __forceinline__ void st16(void *p, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    const u32x4_t v = {a, b, c, d};
+    if constexpr (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t *>(p));
+    else *reinterpret_cast<u32x4_t *>(p) = v;
+}
+template <bool STREAM> __device__ __forceinline__ void st8(void *p, uint32_t a, uint32_t b) {
+    const u32x2_t v = {a, b};
+    if constexpr (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u32x2_t *>(p));
+    else *reinterpret_cast<u32x2_t *>(p) = v;
+}
+template <bool STREAM> __device__ __forceinline__ void st4(void *p, uint32_t a) {
+    if constexpr (STREAM) __builtin_nontemporal_store(a, reinterpret_cast<uint32_t *>(p));
+    else *reinterpret_cast<uint32_t *>(p) = a;
+}
+
+template <typename T, int V, bool STREAM = false>
 __device__ __forceinline__ void store_vec(T *__restrict__ p, const float (&v)[V]) {
     if constexpr (std::is_same<T, float>::value) {
         if constexpr (V % 4 == 0) {
 #pragma unroll
             for (int i = 0; i < V / 4; i++)
-                reinterpret_cast<float4 *>(p)[i] =
-                    make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+                st16<STREAM>(p + 4 * i, __float_as_uint(v[4 * i]), __float_as_uint(v[4 * i + 1]),
+                             __float_as_uint(v[4 * i + 2]), __float_as_uint(v[4 * i + 3]));
         } else if constexpr (V == 2) {
-            *reinterpret_cast<float2 *>(p) = make_float2(v[0], v[1]);
+            st8<STREAM>(p, __float_as_uint(v[0]), __float_as_uint(v[1]));
         } else {
 #pragma unroll
-            for (int i = 0; i < V; i++) p[i] = v[i];
+            for (int i = 0; i < V; i++) st4<STREAM>(p + i, __float_as_uint(v[i]));
         }
     } else {
         if constexpr (V % 8 == 0) {
 #pragma unroll
             for (int i = 0; i < V / 8; i++)
-                reinterpret_cast<uint4 *>(p)[i] =
-                    make_uint4(pack_bf16x2(v[8 * i], v[8 * i + 1]), pack_bf16x2(v[8 * i + 2], v[8 * i + 3]),
-                               pack_bf16x2(v[8 * i + 4], v[8 * i + 5]), pack_bf16x2(v[8 * i + 6], v[8 * i + 7]));
+                st16<STREAM>(p + 8 * i, pack_bf16x2(v[8 * i], v[8 * i + 1]), pack_bf16x2(v[8 * i + 2], v[8 * i + 3]),
+                             pack_bf16x2(v[8 * i + 4], v[8 * i + 5]), pack_bf16x2(v[8 * i + 6], v[8 * i + 7]));
         } else if constexpr (V == 4) {
-            *reinterpret_cast<uint2 *>(p) =
-                make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            st8<STREAM>(p, pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
         } else if constexpr (V == 2) {
-            *reinterpret_cast<uint32_t *>(p) = pack_bf16x2(v[0], v[1]);
+            st4<STREAM>(p, pack_bf16x2(v[0], v[1]));
         } else {
 #pragma unroll
             for (int i = 0; i < V; i++) p[i] = f32_to_bf16(v[i]);

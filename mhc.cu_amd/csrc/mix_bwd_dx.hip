@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
 #pragma unroll
                     for (int v = 0; v < V; v++) out[v] += pv[v];
                 }
-                store_vec<TX, V>(dxb + (size_t)j * C + c, out);
+                store_vec<TX, V, true>(dxb + (size_t)j * C + c, out);
             }
         }
       }
@@ -325,7 +325,7 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
 #pragma unroll
                     for (int v = 0; v < 8; v++) out[v] += pv[v];
                 }
-                store_vec<bf16_t, 8>(static_cast<bf16_t *>(a.dx) + (size_t)b * n * C + (size_t)trow * C + cb0 + co, out);
+                store_vec<bf16_t, 8, true>(static_cast<bf16_t *>(a.dx) + (size_t)b * n * C + (size_t)trow * C + cb0 + co, out);
             }
         }
     }

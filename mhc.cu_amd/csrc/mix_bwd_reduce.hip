@@ -539,7 +539,7 @@ __global__ __launch_bounds__(256) void gram_large_kernel(BwdReduceArgs a) {
 template <int NP, bool PRECISE>
 __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
     using SK = SkWg<NP>;
-    extern __shared__ float smem[];
+    extern __shared__ __align__(16) float smem[];
     float *W_s = smem;                   // [32][33]  W1 (or dy [f;0]^T)
     float *X_s = W_s + 32 * 33;          // [32][33]  XX
     float *M_s = X_s + 32 * 33;          // [32][33]  dM
@@ -651,7 +651,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         S0 = dtp * Pb[lane]; S1 = dto * Pb[n + lane];
     }
     // Sinkhorn forward recompute + exact backward, the matrix spread over all 256 threads
-    float E[SK::EPL], d[SK::EPL], u, v[SK::EPL];
+    float E[SK::EPL], ET[SK::EPL], d[SK::EPL], u, v[SK::EPL];
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;
@@ -660,8 +660,8 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         E[e] = ok ? expf(al2 * pres[e] + bres[e]) : 0.f;
         d[e] = ok ? M_s[r0 * 33 + c] : 0.f;
     }
-    SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
-    SK::template backward<PRECISE>(E, d, u, v, a.T, sk_s, tid);
+    SK::template forward<PRECISE>(E, ET, u, v, n, a.T, a.eps, sk_s, tid);
+    SK::template backward<PRECISE>(E, ET, d, u, v, a.T, sk_s, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;

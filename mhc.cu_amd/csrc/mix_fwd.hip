@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void mix_fwd_kernel(MixFwdArgs a) {
 #pragma unroll
                     for (int v = 0; v < V; v++) out[v] += mij * xv[j][v];
                 }
-                store_vec<TY, V>(yb + (size_t)i * C + c, out);
+                store_vec<TY, V, true>(yb + (size_t)i * C + c, out);
             }
         }
     }
@@ -369,7 +369,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
                         for (int v = 0; v < V; v++) out[v] += mij * (LEAN ? t[v] : xv[LEAN ? 0 : k][j][v]);
                     }
-                    store_vec<TY, V>(yb + (size_t)i * C + c, out);
+                    store_vec<TY, V, true>(yb + (size_t)i * C + c, out);
                 }
             }
         }
@@ -574,7 +574,7 @@ __global__ __launch_bounds__(256) void mix_fwd_large_kernel(MixLargeArgs a) {
                 const float4 o0 = *reinterpret_cast<const float4 *>(o_s + trow * kMflLDO + co);
                 const float4 o1 = *reinterpret_cast<const float4 *>(o_s + trow * kMflLDO + co + 4);
                 const float out[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
-                store_vec<TY, 8>(yb + co, out);
+                store_vec<TY, 8, true>(yb + co, out);
             }
         }
     }

@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
                     const int d = (dt0 + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
-                    if (d < a.D) out[(size_t)d * a.nC + k] = am[i];
+                    if (d < a.D) __builtin_nontemporal_store(am[i], out + (size_t)d * a.nC + k);
                 }
             }
         };
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
                     const int d = (dt0 + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
-                    if (d < a.D) out[(size_t)d * a.nC + k] = acc[m][i];
+                    if (d < a.D) __builtin_nontemporal_store(acc[m][i], out + (size_t)d * a.nC + k);
                 }
             }
         }

@@ -106,25 +106,30 @@ template <int NP> struct SkSmall {
 };
 
 // =============================================================================================
-// SkWg: one 256-thread workgroup per matrix, NP = 16 or 32.  Thread t owns EPL consecutive
-// columns of row t / LPR of E and of the running gradient in registers; the iterate is kept in
-// scaling form diag(u) E diag(v) (u replicated over the lanes of a row, v over the rows).  A
-// half-step is one cross-lane reduction: rows inside a DPP row, columns inside the wave and then
-// across the 4 waves through a double-buffered LDS slot (one barrier per iteration).
-// The denominators rho/s of every iteration are kept in LDS for the backward sweep, which unwinds
-// the scalings (u *= rho, v *= s) instead of storing iterates.  Every thread of the workgroup must
-// call forward/backward.
+// SkWg: one 256-thread workgroup per matrix, NP = 16 or 32, iterate kept in scaling form
+// diag(u) E diag(v) with E constant in registers.  Every thread plays two roles on the same pair of
+// numbers (a, b0) = (tid / LPR, (tid % LPR) * EPL):
+//   row role     owns E[a][b0 .. b0+EPL) (and the running gradient there), and u[a]
+//   column role  owns E[b0 .. b0+EPL)[a] (a transposed copy made once through LDS), and v[a]
+// so both the row sums and the column sums are an in-register dot product plus a reduction over
+// the LPR lanes of a DPP row; the two vectors travel through LDS (u after the row half-step, v
+// after the column half-step, one barrier each).  The denominators rho/s of every iteration stay
+// in LDS for the backward sweep, which unwinds the scalings (u *= rho, v *= s) instead of storing
+// iterates and keeps the gradient in both roles.  Every thread of the workgroup must call
+// forward/backward; `lds` must be 16-byte aligned.
 // =============================================================================================
 template <int NP> struct SkWg {
     static_assert(NP == 16 || NP == 32, "SkWg handles 16x16 and 32x32 tiles");
     static constexpr int EPL = NP * NP / 256;  // 1 or 4
     static constexpr int LPR = NP / EPL;       // lanes per row: 16 or 8
-    // LDS floats: cw [2][4][NP] | rho [T][NP] | s [T][NP]
-    __host__ __device__ static constexpr int lds_floats(int T) { return 8 * NP + 2 * T * NP; }
+    static constexpr int kTile = NP * (NP + 1);
+    // LDS floats: transpose tile | u | v | column dots | row dots | rho [T][NP] | s [T][NP]
+    __host__ __device__ static constexpr int lds_floats(int T) { return kTile + 4 * NP + 2 * T * NP; }
     __device__ static __forceinline__ int row(int tid) { return tid / LPR; }
     __device__ static __forceinline__ int col0(int tid) { return (tid % LPR) * EPL; }
 
-    __device__ static __forceinline__ float row_allreduce(float x) {
+    // sum over the LPR lanes that share tid / LPR
+    __device__ static __forceinline__ float seg_allreduce(float x) {
         x += dpp_mov<kDppQuadXor1>(x);
         x += dpp_mov<kDppQuadXor2>(x);
         if constexpr (LPR == 8) {
@@ -135,87 +140,121 @@ template <int NP> struct SkWg {
         }
         return x;
     }
-    // sum over all NP rows of per-column values; cw_t = this iteration's LDS slot [4][NP]
-    __device__ static __forceinline__ void col_allreduce(float (&x)[EPL], float *cw_t, int tid) {
-        const int lane = tid & 63, wave = tid >> 6;
+    // EPL consecutive floats at a 16-byte aligned LDS address
+    __device__ static __forceinline__ void ld_vec(const float *p, float (&x)[EPL]) {
+        if constexpr (EPL == 4) {
+            const float4 t = *reinterpret_cast<const float4 *>(p);
+            x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
+        } else {
 #pragma unroll
-        for (int e = 0; e < EPL; e++) {
-            if constexpr (LPR == 8) x[e] += dpp_mov<kDppRowRor8>(x[e]);
-            x[e] = xor16_add(x[e]);
-            x[e] = xor32_add(x[e]);
+            for (int e = 0; e < EPL; e++) x[e] = p[e];
         }
-        if (lane < LPR) {
+    }
+    // row-role values a[e] = A[a][b0+e]  ->  column-role values at[e] = A[b0+e][a]
+    __device__ static __forceinline__ void transpose(const float (&a)[EPL], float (&at)[EPL], float *tile,
+                                                     int tid) {
+        const int r = row(tid), c0 = col0(tid);
 #pragma unroll
-            for (int e = 0; e < EPL; e++) cw_t[wave * NP + lane * EPL + e] = x[e];
-        }
+        for (int e = 0; e < EPL; e++) tile[r * (NP + 1) + c0 + e] = a[e];
         __syncthreads();
-        const int c0 = col0(tid);
 #pragma unroll
-        for (int e = 0; e < EPL; e++)
-            x[e] = (cw_t[c0 + e] + cw_t[NP + c0 + e]) + (cw_t[2 * NP + c0 + e] + cw_t[3 * NP + c0 + e]);
+        for (int e = 0; e < EPL; e++) at[e] = tile[(c0 + e) * (NP + 1) + r];
+        __syncthreads();
     }
 
-    // E: exp(logits), 0 outside n x n.  On return M = u * E[e] * v[e]; rho/s hold the denominators.
+    // E: exp(logits), 0 outside n x n (row role).  On return ET is the column-role copy,
+    // M = u * E[e] * v[e], and u / v / rho / s sit in LDS for backward().
     // PRECISE selects IEEE divisions (fp32 parity tier) instead of v_rcp_f32 (1 ulp).
     template <bool PRECISE = true>
-    __device__ static __forceinline__ void forward(const float (&E)[EPL], float &u, float (&v)[EPL],
-                                                   int n, int T, float eps, float *lds, int tid) {
-        float *cw = lds, *rho = lds + 8 * NP, *s = rho + T * NP;
-        const int r = row(tid), c0 = col0(tid);
+    __device__ static __forceinline__ void forward(const float (&E)[EPL], float (&ET)[EPL], float &u,
+                                                   float (&v)[EPL], int n, int T, float eps, float *lds,
+                                                   int tid) {
+        float *ub = lds + kTile, *vb = ub + NP, *rho = vb + 3 * NP, *s = rho + T * NP;
+        const int a = row(tid), b0 = col0(tid);
+        const bool head = (tid % LPR) == 0, live = a < n;
+        transpose(E, ET, lds, tid);
         u = 1.0f;
+        float vc = 1.0f;  // v[a], column role
 #pragma unroll
         for (int e = 0; e < EPL; e++) v[e] = 1.0f;
         for (int t = 0; t < T; t++) {
             float p = 0.f;
 #pragma unroll
             for (int e = 0; e < EPL; e++) p += E[e] * v[e];
-            p = row_allreduce(p);
-            const float rr = r < n ? u * p + eps : 1.0f;
+            p = seg_allreduce(p);
+            const float rr = live ? u * p + eps : 1.0f;
             u = PRECISE ? u / rr : u * fast_rcp(rr);
-            if ((tid % LPR) == 0) rho[t * NP + r] = rr;
-            float q[EPL];
+            if (head) { rho[t * NP + a] = rr; ub[a] = u; }
+            __syncthreads();
+            float uc[EPL], q = 0.f;
+            ld_vec(ub + b0, uc);
 #pragma unroll
-            for (int e = 0; e < EPL; e++) q[e] = E[e] * u;
-            col_allreduce(q, cw + (t & 1) * 4 * NP, tid);
-#pragma unroll
-            for (int e = 0; e < EPL; e++) {
-                const float sc = c0 + e < n ? v[e] * q[e] + eps : 1.0f;
-                v[e] = PRECISE ? v[e] / sc : v[e] * fast_rcp(sc);
-                if (r == 0) s[t * NP + c0 + e] = sc;
-            }
+            for (int e = 0; e < EPL; e++) q += ET[e] * uc[e];
+            q = seg_allreduce(q);
+            const float sc = live ? vc * q + eps : 1.0f;
+            vc = PRECISE ? vc / sc : vc * fast_rcp(sc);
+            if (head) { s[t * NP + a] = sc; vb[a] = vc; }
+            __syncthreads();
+            ld_vec(vb + b0, v);
         }
-        __syncthreads();  // rho / s visible to every thread
     }
 
-    // d: in = dL/dM, out = dL/dE.  u, v: final scalings from forward (destroyed).
+    // d: in = dL/dM, out = dL/dE (row role).  E, ET, u, v, LDS contents: as left by forward()
+    // (u and v are destroyed).
     template <bool PRECISE = true>
-    __device__ static __forceinline__ void backward(const float (&E)[EPL], float (&d)[EPL], float u,
-                                                    float (&v)[EPL], int T, float *lds, int tid) {
-        float *cw = lds;
-        const float *rho = lds + 8 * NP, *s = rho + T * NP;
-        const int r = row(tid), c0 = col0(tid);
+    __device__ static __forceinline__ void backward(const float (&E)[EPL], const float (&ET)[EPL],
+                                                    float (&d)[EPL], float u, float (&v)[EPL], int T,
+                                                    float *lds, int tid) {
+        float *ub = lds + kTile, *vb = ub + NP, *cdb = vb + NP, *rdb = cdb + NP;
+        const float *rho = rdb + NP, *s = rho + T * NP;
+        const int a = row(tid), b0 = col0(tid);
+        const bool head = (tid % LPR) == 0;
+        float dT[EPL], uc[EPL];
+        transpose(d, dT, lds, tid);
+        ld_vec(ub + b0, uc);
+        float vc = vb[a];
         for (int t = T - 1; t >= 0; t--) {
-            // column dots with the iterate after column step t: Out = u E v
-            float cd[EPL];
+            // column role: dots of the gradient with the iterate after column step t
+            float x = 0.f;
 #pragma unroll
-            for (int e = 0; e < EPL; e++) cd[e] = d[e] * u * E[e];
-            col_allreduce(cd, cw + (t & 1) * 4 * NP, tid);
-            float z = 0.f, sc[EPL];
+            for (int e = 0; e < EPL; e++) x += dT[e] * uc[e] * ET[e];
+            x = seg_allreduce(x);
+            if (head) cdb[a] = x;
+            const float sc_c = s[t * NP + a];
+#pragma unroll
+            for (int e = 0; e < EPL; e++) dT[e] -= x * vc;
+            __syncthreads();
+            // row role: same update, then the row dots of row step t
+            float cdv[EPL], scv[EPL], z = 0.f;
+            ld_vec(cdb + b0, cdv);
+            ld_vec(s + t * NP + b0, scv);
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
-                sc[e] = s[t * NP + c0 + e];
-                d[e] -= cd[e] * v[e];
+                d[e] -= cdv[e] * v[e];
                 z += d[e] * E[e] * v[e];
             }
-            const float rdot = u * row_allreduce(z);
-            const float rr = rho[t * NP + r];
+            const float rdot = u * seg_allreduce(z);
+            if (head) rdb[a] = rdot;
+            const float rr = rho[t * NP + a];
             const float rri = PRECISE ? 0.f : fast_rcp(rr);
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
-                d[e] = PRECISE ? (d[e] / sc[e] - rdot) / rr : (d[e] * fast_rcp(sc[e]) - rdot) * rri;
-                v[e] *= sc[e];
+                d[e] = PRECISE ? (d[e] / scv[e] - rdot) / rr : (d[e] * fast_rcp(scv[e]) - rdot) * rri;
+                v[e] *= scv[e];
             }
             u *= rr;
+            __syncthreads();
+            // column role: finish the update with the row dots
+            float rdv[EPL], rrv[EPL];
+            ld_vec(rdb + b0, rdv);
+            ld_vec(rho + t * NP + b0, rrv);
+            const float sci = PRECISE ? 0.f : fast_rcp(sc_c);
+#pragma unroll
+            for (int e = 0; e < EPL; e++) {
+                dT[e] = PRECISE ? (dT[e] / sc_c - rdv[e]) / rrv[e] : (dT[e] * sci - rdv[e]) * fast_rcp(rrv[e]);
+                uc[e] *= rrv[e];
+            }
+            vc *= sc_c;
         }
     }
 };
