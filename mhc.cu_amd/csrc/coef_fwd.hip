@@ -90,24 +90,31 @@ template <int NP, bool PRECISE> __global__ __launch_bounds__(256) void coef_fwd_
     const int b = blockIdx.x;
     const int n = a.n, D = n * n + 2 * n;
     const bool dyn = a.Ppart != nullptr;
-    float rinv = 0.f, al[3] = {0.f, 0.f, 0.f};
+    float al[3] = {0.f, 0.f, 0.f};
+    // every wave fetches the split sums of x^2 itself (lane = split, KS <= 64): one load in flight
+    // together with the partial dot products below instead of a chain of its own
+    float ssq_l = 0.f;
     if (dyn) {
-        const float ssq = reduce_partials(a.ssqpart, a.KS, a.B, b);
-        const float r = sqrtf(ssq / (float)a.nC + a.eps);
-        rinv = 1.0f / r;
+        const int lane = tid & 63;
+        ssq_l = a.ssqpart[(size_t)(lane < a.KS ? lane : 0) * a.B + b];
+        ssq_l = lane < a.KS ? ssq_l : 0.f;
         al[0] = a.alpha[0]; al[1] = a.alpha[1]; al[2] = a.alpha[2];
-        if (tid == 0) a.r[b] = r;
     }
     const size_t pstride = (size_t)a.B * a.DP;
     // logits d = tid + 256 m; the partial sums of all of a thread's logits are fetched together,
-    // several splits at a time (out-of-range slots alias element 0 and are discarded)
+    // all splits of a round at once (out-of-range slots alias element 0 and are discarded)
     constexpr int MD = (NP * NP + 2 * NP + 255) / 256;
-    float psum[MD];
+    float psum[MD], bias[MD];
 #pragma unroll
-    for (int m = 0; m < MD; m++) psum[m] = 0.f;
+    for (int m = 0; m < MD; m++) {
+        psum[m] = 0.f;
+        const int d = tid + 256 * m < D ? tid + 256 * m : 0;
+        const int grp = alpha_group(d, n);
+        bias[m] = *(grp == 0 ? a.b_pre + d : (grp == 1 ? a.b_post + (d - n) : a.b_res + (d - 2 * n)));
+    }
     if (dyn) {
         const float *pb = a.Ppart + (size_t)b * a.DP;
-        constexpr int KB = MD > 2 ? 12 : 16;  // splits per round: 60 / 32 loads in flight per thread
+        constexpr int KB = MD > 2 ? 24 : 32;  // splits per round: up to 120 / 64 loads in flight per thread
         for (int k0 = 0; k0 < a.KS; k0 += KB) {
             float tv[MD][KB];
 #pragma unroll
@@ -124,17 +131,22 @@ template <int NP, bool PRECISE> __global__ __launch_bounds__(256) void coef_fwd_
                 for (int q = 0; q < KB; q++) psum[m] += (tid + 256 * m < D && k0 + q < a.KS) ? tv[m][q] : 0.f;
         }
     }
+    float rinv = 0.f;
+    if (dyn) {
+        const float r = sqrtf(wave_allreduce_sum(ssq_l) / (float)a.nC + a.eps);
+        rinv = 1.0f / r;
+        if (tid == 0) a.r[b] = r;
+    }
 #pragma unroll
     for (int m = 0; m < MD; m++) {
         const int d = tid + 256 * m;
         if (d < D) {
             const int grp = alpha_group(d, n);
-            const float bias = grp == 0 ? a.b_pre[d] : (grp == 1 ? a.b_post[d - n] : a.b_res[d - 2 * n]);
-            float t = bias;
+            float t = bias[m];
             if (dyn) {
                 const float p = psum[m] * rinv;
                 a.P[(size_t)b * D + d] = p;
-                t = al[grp] * p + bias;
+                t = al[grp] * p + bias[m];
             }
             lg[d] = t;
         }

@@ -561,6 +561,12 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
     const int D = n * n + 2 * n;
     const int r0 = SK::row(tid), c0 = SK::col0(tid);
     const bool dyn = a.hstride != 0;
+    // scalars of the coefficient backward, requested with everything else (used after the sums)
+    float al0 = 0.f, al1 = 0.f, al2 = 0.f, rinv = 0.f;
+    if (dyn) {
+        al0 = a.alpha[0]; al1 = a.alpha[1]; al2 = a.alpha[2];
+        rinv = 1.0f / a.r[b];
+    }
     float pres[SK::EPL], bres[SK::EPL];
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
@@ -637,8 +643,6 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         return;
     }
     const float *Pb = a.P + (size_t)b * D;
-    const float al0 = a.alpha[0], al1 = a.alpha[1], al2 = a.alpha[2];
-    const float rinv = 1.0f / a.r[b];
     float *dt = a.out.dt + (size_t)b * (D + 3);
     const DPWriter dpw{a.out, b, a.B, a.DP};
     float S0 = 0.f, S1 = 0.f, S2 = 0.f;  // sum_d dt_d p_d per alpha group
