@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "mhc", "libmhc_hip.so")
 
-SOURCES = ["capi.hip", "proj_fwd.hip", "proj_bwd.hip", "proj_bwd_large.hip", "bwd_slab.hip", "coef_fwd.hip", "mix_fwd.hip", "mix_bwd_reduce.hip",
+SOURCES = ["capi.hip", "proj_fwd.hip", "gemm_f32.hip", "proj_bwd.hip", "proj_bwd_large.hip", "bwd_slab.hip", "coef_fwd.hip", "mix_fwd.hip", "mix_bwd_reduce.hip",
            "mix_bwd_dx.hip", "param_grads.hip", "ops.hip"]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are not trusted on this hardware pool.

@@ -52,7 +52,10 @@ int ws_check(void *ws, size_t have, size_t need) {
 struct DynFwdWs { float *Ppart, *ssqpart, *agg; size_t bytes; };
 struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *raw, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
 
-int max_ksplit(int B, int n, int C) { return proj_fwd_ksplit(kBF16, kBF16, B, n, C); }
+int max_ksplit(int B, int n, int C) {
+    const int a = proj_fwd_ksplit(kBF16, kBF16, B, n, C), b = proj_fwd_ksplit(kF32, kF32, B, n, C);
+    return a > b ? a : b;
+}
 
 DynFwdWs carve_dyn_fwd(void *ws, int B, int n, int C) {
     Carver c(ws);
@@ -240,6 +243,14 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
         MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, ws.dt,
                                      ws.dtpart, spg, B, n, C, st));
+    } else if (gemm_f32_supported(x_dtype, phi_dtype, n, C)) {
+        // exact float32 tier, wide projection: both products on the fp32 matrix cores; the projection
+        // term of dx is written into dx and completed in place
+        MHC_LAUNCH(launch_gemm_f32_dxflat(ws.dP, static_cast<const float *>(phi), static_cast<float *>(dx), B, n, C, st));
+        MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
+                                     n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, ws.dt,
+                                     ws.dtpart, spg, B, n, C, st));
+        MHC_LAUNCH(launch_gemm_f32_dphi(ws.dP, static_cast<const float *>(x), dphi, B, n, C, st));
     } else {
         MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      n, q, ws.s1, ws.cx, ws.dP, DP, phi, phi_dtype, nullptr, dx, df,

@@ -54,6 +54,16 @@ hipError_t launch_layer_fwd_fused(const void *x, int x_dtype, const void *w, int
                                   float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
                                   int B, int n, int C, int T, float eps, hipStream_t stream);
 
+// fp32 matrix-core GEMMs of the exact float32 tier (wide projections): see gemm_f32.hip.
+bool gemm_f32_supported(int x_dtype, int phi_dtype, int n, int C);
+int gemm_f32_proj_ksplit(int B, int n, int C, int max_splits);
+hipError_t launch_gemm_f32_proj(const float *x, const float *phi, float *Ppart, float *ssqpart, int KS,
+                                int B, int n, int C, hipStream_t stream);
+hipError_t launch_gemm_f32_dphi(const float *dP, const float *x, float *dphi, int B, int n, int C,
+                                hipStream_t stream);
+hipError_t launch_gemm_f32_dxflat(const float *dP, const float *phi, float *dxflat, int B, int n, int C,
+                                  hipStream_t stream);
+
 // ---- backward --------------------------------------------------------------------------------
 
 struct BwdCoefOut {

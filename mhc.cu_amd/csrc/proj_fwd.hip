@@ -370,6 +370,7 @@ static bool use_wide(int n, int C) { return padded_D(n) / 32 > 4 && (n * C) % 64
 int proj_fwd_ksplit(int x_dtype, int phi_dtype, int B, int n, int C) {
     // The generic path always uses one split.  MFMA path: enough workgroups to fill 256 CUs
     // several times over (the K loop is latency-bound per wave), at least 64 K elements per wave.
+    if (gemm_f32_supported(x_dtype, phi_dtype, n, C)) return gemm_f32_proj_ksplit(B, n, C, kMaxKSplit);
     if (!use_mfma(x_dtype, phi_dtype, C)) return 1;
     const int nC = n * C, DP = padded_D(n);
     if (use_wide(n, C)) {
@@ -433,6 +434,9 @@ hipError_t launch_proj_fwd(const void *x, int x_dtype, const void *phi, int phi_
             default: return launch_mfma<4>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
         }
     }
+    if (gemm_f32_supported(x_dtype, phi_dtype, n, C))
+        return launch_gemm_f32_proj(static_cast<const float *>(x), static_cast<const float *>(phi), Ppart,
+                                    ssqpart, KS, B, n, C, stream);
     if (KS != 1) return hipErrorInvalidValue;  // the generic path produces exactly one split
     if (x_dtype == kF32 && phi_dtype == kF32) return launch_generic<float, float>(x, phi, Ppart, ssqpart, B, D, DP, nC, stream);
     if (x_dtype == kF32 && phi_dtype == kBF16) return launch_generic<float, bf16_t>(x, phi, Ppart, ssqpart, B, D, DP, nC, stream);

@@ -94,6 +94,9 @@ def _rand_params(p, n, C, seed=7):
 DYN_SHAPES = [
     (32, 4, 1280), (5, 4, 64), (1, 4, 128), (3, 2, 40), (2, 3, 20), (7, 1, 36),
     (16, 8, 256), (3, 6, 72), (4, 16, 64), (3, 12, 40), (4, 32, 64), (2, 24, 104), (2, 32, 1040),
+    # n > 8 in float32: several tiles and a ragged last slice for the fp32 matrix-core products, and
+    # a row length that is not a multiple of 4 (scalar kernels)
+    (130, 12, 36), (3, 9, 10),
 ]
 
 
