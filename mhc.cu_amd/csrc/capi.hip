@@ -32,7 +32,7 @@ inline bool valid_io(int x_dtype, int y_dtype) {
 
 int check_shape(int B, int n, int C, int iters) {
     if (n < 1 || n > MHC_MAX_N) return MHC_ERR_BAD_N;
-    if (B < 1 || C < 1 || iters < 0 || iters > 1024) return MHC_ERR_BAD_SHAPE;
+    if (B < 1 || C < 1 || iters < 0 || iters > max_layer_sinkhorn_iters(n)) return MHC_ERR_BAD_SHAPE;
     if ((long long)B * n * C > (1ll << 40)) return MHC_ERR_BAD_SHAPE;
     return MHC_OK;
 }
@@ -141,12 +141,14 @@ __attribute__((visibility("default"))) int mhc_phase_read(int kernel, unsigned l
 
 int mhc_abi_version(void) { return MHC_ABI_VERSION; }
 
+int mhc_max_sinkhorn_iters(int n) { return (n < 1 || n > MHC_MAX_N) ? 0 : max_layer_sinkhorn_iters(n); }
+
 const char *mhc_status_string(int status) {
     switch (status) {
         case MHC_OK: return "ok";
         case MHC_ERR_NULL_POINTER: return "a required pointer is NULL";
         case MHC_ERR_BAD_N: return "expansion rate n must be in 1..32";
-        case MHC_ERR_BAD_SHAPE: return "B, C or iters out of range";
+        case MHC_ERR_BAD_SHAPE: return "B, C or iters out of range (see mhc_max_sinkhorn_iters)";
         case MHC_ERR_BAD_DTYPE: return "unsupported dtype combination";
         case MHC_ERR_MISALIGNED: return "tensor base pointer is not 16-byte aligned";
         case MHC_ERR_WORKSPACE: return "workspace NULL, not 256-byte aligned or too small";

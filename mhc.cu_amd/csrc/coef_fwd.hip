@@ -179,10 +179,16 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
         coef_fwd_small_kernel<8><<<(B + 3) / 4, 64, 0, stream>>>(a);
     else if (n <= 16) {
         const size_t smem = sizeof(float) * (16 * 16 + 32 + SkWg<16>::lds_floats(T));
+        hipError_t e = precise ? allow_dynamic_lds(&coef_fwd_lds_kernel<16, true>, smem)
+                               : allow_dynamic_lds(&coef_fwd_lds_kernel<16, false>, smem);
+        if (e != hipSuccess) return e;
         if (precise) coef_fwd_lds_kernel<16, true><<<B, 256, smem, stream>>>(a);
         else coef_fwd_lds_kernel<16, false><<<B, 256, smem, stream>>>(a);
     } else {
         const size_t smem = sizeof(float) * (32 * 32 + 64 + SkWg<32>::lds_floats(T));
+        hipError_t e = precise ? allow_dynamic_lds(&coef_fwd_lds_kernel<32, true>, smem)
+                               : allow_dynamic_lds(&coef_fwd_lds_kernel<32, false>, smem);
+        if (e != hipSuccess) return e;
         if (precise) coef_fwd_lds_kernel<32, true><<<B, 256, smem, stream>>>(a);
         else coef_fwd_lds_kernel<32, false><<<B, 256, smem, stream>>>(a);
     }

@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
         d[e] = ok ? tot[r0 * NP + c] : 0.f;
     }
     SK::template forward<false>(m, g, n, a.T, a.eps, sc, tid);
-    SK::template backward<false>(d, a.T, sc, tid);
+    SK::template backward<false>(d, m, a.T, sc, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
         d[e] = ok ? dMe[e] : 0.f;
     }
     SK::template forward<PRECISE>(m, g, n, a.T, a.eps, sc, tid);
-    SK::template backward<PRECISE>(d, a.T, sc, tid);
+    SK::template backward<PRECISE>(d, m, a.T, sc, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;
@@ -702,13 +702,19 @@ static hipError_t launch_small(const BwdReduceArgs &a, hipStream_t stream) {
     int nt = round_up((nch + rounds - 1) / rounds, 16);
     if (nt > 256) nt = 256;
     constexpr int K = NP * NP + 3 * NP + 1;
-    const size_t smem = sizeof(float) * (K * 16 + K + SkSmall<NP>::scaling_floats(a.T));
+    // the Sinkhorn area is only needed when the coefficient backward runs in the same launch
+    const size_t smem = sizeof(float) * (K * 16 + K + (a.raw ? 0 : SkSmall<NP>::scaling_floats(a.T)));
+    hipError_t e = allow_dynamic_lds(&mix_bwd_reduce_small_kernel<TG, TX, NP, V>, smem);
+    if (e != hipSuccess) return e;
     mix_bwd_reduce_small_kernel<TG, TX, NP, V><<<dim3(a.B, a.parts), nt, smem, stream>>>(a);
-    hipError_t e = hipGetLastError();
+    e = hipGetLastError();
     if (e != hipSuccess || !a.raw) return e;
     // fp32 activations: the parity tier, IEEE divisions in the Sinkhorn chain
     constexpr bool kPrecise = std::is_same<TX, float>::value;
-    coef_bwd_small_kernel<NP, kPrecise><<<(a.B + 3) / 4, 64, sizeof(float) * SkSmall<NP>::scaling_floats(a.T), stream>>>(a);
+    const size_t smem2 = sizeof(float) * SkSmall<NP>::scaling_floats(a.T);
+    e = allow_dynamic_lds(&coef_bwd_small_kernel<NP, kPrecise>, smem2);
+    if (e != hipSuccess) return e;
+    coef_bwd_small_kernel<NP, kPrecise><<<(a.B + 3) / 4, 64, smem2, stream>>>(a);
     return hipGetLastError();
 }
 
@@ -739,9 +745,13 @@ static hipError_t launch_large(const BwdReduceArgs &a, hipStream_t stream) {
     constexpr bool kPrecise = std::is_same<TX, float>::value;  // fp32 activations: the parity tier
     if (a.n <= 16) {
         const size_t smem2 = sizeof(float) * (3 * 32 * 33 + 64 + 96 + 4 + SkWg<16>::lds_floats(a.T));
+        e = allow_dynamic_lds(&coef_bwd_large_kernel<16, kPrecise>, smem2);
+        if (e != hipSuccess) return e;
         coef_bwd_large_kernel<16, kPrecise><<<a.B, 256, smem2, stream>>>(a);
     } else {
         const size_t smem2 = sizeof(float) * (3 * 32 * 33 + 64 + 96 + 4 + SkWg<32>::lds_floats(a.T));
+        e = allow_dynamic_lds(&coef_bwd_large_kernel<32, kPrecise>, smem2);
+        if (e != hipSuccess) return e;
         coef_bwd_large_kernel<32, kPrecise><<<a.B, 256, smem2, stream>>>(a);
     }
     return hipGetLastError();

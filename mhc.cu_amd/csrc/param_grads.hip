@@ -247,9 +247,11 @@ hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const
                                   float *dH_res, int n, int T, float eps, hipStream_t stream) {
     if (n <= 16) {
         const size_t smem = sizeof(float) * SkWg<16>::lds_floats(T);
+        if (hipError_t e = allow_dynamic_lds(&coef_bwd_static_kernel<16>, smem); e != hipSuccess) return e;
         coef_bwd_static_kernel<16><<<1, 256, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
     } else {
         const size_t smem = sizeof(float) * SkWg<32>::lds_floats(T);
+        if (hipError_t e = allow_dynamic_lds(&coef_bwd_static_kernel<32>, smem); e != hipSuccess) return e;
         coef_bwd_static_kernel<32><<<1, 256, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
     }
     return hipGetLastError();

@@ -32,6 +32,7 @@ _P, _I, _F, _Z = c_void_p, c_int, c_float, c_size_t
 _SIGNATURES = {
     "mhc_abi_version": (c_int, []),
     "mhc_status_string": (c_char_p, [_I]),
+    "mhc_max_sinkhorn_iters": (c_int, [_I]),
     "mhc_layer_dynamic_workspace_bytes": (_Z, [_I, _I, _I]),
     "mhc_layer_fwd_dynamic": (c_int, [_P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P,
                                       _P, _I, _I, _I, _I, _F, _P, _Z, _P]),

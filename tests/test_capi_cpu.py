@@ -66,10 +66,15 @@ def test_argument_validation_happens_before_any_launch():
     odd = P(a16.value + 4)
     fwd = lambda **kw: L.mhc_layer_fwd_dynamic(
         kw.get("x", a16), kw.get("xd", 0), a16, 0, a16, 0, a16, a16, None, kw.get("y", a16), kw.get("yd", 0),
-        a16, a16, a16, a16, a16, a16, kw.get("B", 2), kw.get("n", 4), kw.get("C", 8), 20, 1e-6,
+        a16, a16, a16, a16, a16, a16, kw.get("B", 2), kw.get("n", 4), kw.get("C", 8), kw.get("T", 20), 1e-6,
         kw.get("ws", None), kw.get("wsb", 0), None)
     assert fwd(n=0) == 2 and fwd(n=33) == 2            # MHC_ERR_BAD_N
     assert fwd(B=0) == 3                               # MHC_ERR_BAD_SHAPE
+    # iteration counts beyond what the backward keeps in LDS are refused up front, per n
+    assert [L.mhc_max_sinkhorn_iters(n) for n in (0, 1, 4, 5, 8, 9, 16, 17, 32, 33)] == \
+        [0, 256, 256, 112, 112, 512, 512, 256, 256, 0]
+    assert fwd(n=4, T=257) == 3 and fwd(n=8, T=113) == 3 and fwd(n=32, T=257) == 3 and fwd(T=-1) == 3
+    assert fwd(n=4, T=256) == 6 and fwd(n=8, T=112) == 6 and fwd(n=16, T=512) == 6   # next check: workspace
     assert fwd(x=None) == 1                            # MHC_ERR_NULL_POINTER
     assert fwd(xd=7) == 4                              # MHC_ERR_BAD_DTYPE
     assert fwd(xd=0, yd=1) == 4                        # fp32 in / bf16 out is not offered

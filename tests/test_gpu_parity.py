@@ -119,6 +119,27 @@ def test_dynamic_fp32_vs_oracle(B, n, C, inject):
         _check(g[k], ref, "fp32", "d" + k)
 
 
+@pytest.mark.parametrize("B,n,C,T", [(2, 4, 16, 256), (3, 8, 16, 112), (2, 16, 8, 512), (2, 32, 8, 256),
+                                     (3, 8, 64, 60)])
+@pytest.mark.parametrize("dyn", [True, False])
+def test_largest_iteration_counts(B, n, C, T, dyn):
+    """The largest accepted iteration count of every Sinkhorn layout (LDS above 64 KB per workgroup):
+    forward and exact backward against the float64 oracle."""
+    eps = 1e-6
+    if dyn:
+        x, dy, f, p = nm.make_dynamic_inputs(B, n, C, with_f=False)
+        p = _rand_params(p, n, C)
+        y_ref, g_ref = nm.mhc_dynamic_fwd_bwd(x, p, dy, T, eps, dtype=torch.float64)
+        y, g = hip_dynamic(x, p, dy, T, eps)
+    else:
+        x, dy, f, p = nm.make_static_inputs(B, n, C, with_f=False)
+        y_ref, g_ref = nm.mhc_static_fwd_bwd(x, p, dy, T, eps, dtype=torch.float64)
+        y, g = hip_static(x, p, dy, T, eps)
+    _check(y, y_ref, "fp32", "y")
+    for k, ref in g_ref.items():
+        _check(g[k], ref, "fp32", "d" + k)
+
+
 @pytest.mark.parametrize("B,n,C", [(32, 4, 1280), (5, 4, 64), (16, 8, 256), (3, 6, 72), (4, 16, 64),
                                    (4, 32, 64), (2, 32, 1040), (3, 4, 20),
                                    # more than 128 samples with a wide projection: several sample
