@@ -162,7 +162,10 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
     const int D = n * n + 2 * n;
     const int r0 = SK::row(g), c0 = SK::col0(g);
     float al0 = 0.f, al1 = 0.f, al2 = 0.f, bpre = 0.f, bpost = 0.f, bres[SK::EPL];
-    float t_ssq[4], t_pre[4], t_post[4], t_e[4][SK::EPL];
+    // wave 0 sums 4 * SU K-splits in one round of loads (proj_fwd_ksplit caps the split count to
+    // match; the two-chunk variant has no registers to spare for more)
+    constexpr int SU = CPT == 1 ? 6 : 4;
+    float t_ssq[SU], t_pre[SU], t_post[SU], t_e[SU][SK::EPL];
     const size_t ps = (size_t)a.B * a.DP;
     const float *Pb = dyn ? a.Ppart + (size_t)b * a.DP : nullptr;
     // None of these loads sits behind a per-lane branch or is touched before step 2 / step 3: out of
@@ -175,8 +178,8 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
         for (int e = 0; e < SK::EPL; e++) bres[e] = a.b_res[(r0 < n && c0 + e < n) ? r0 * n + c0 + e : 0];
         if (dyn) {
 #pragma unroll
-            for (int u = 0; u < 4; u++) {  // first batch of K-split partials: ks = part*4 + u
-                const int ks = part * 4 + u;
+            for (int u = 0; u < SU; u++) {  // first batch of K-split partials: ks = part*SU + u
+                const int ks = part * SU + u;
                 const size_t ko = ks < a.KS ? ks : 0;
                 t_ssq[u] = a.ssqpart[ko * a.B + b];
                 t_pre[u] = Pb[ko * ps + gc];
@@ -212,17 +215,17 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
         for (int e = 0; e < SK::EPL; e++) pe[e] = 0.f;
         if (dyn) {
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const bool ok = part * 4 + u < a.KS;
+            for (int u = 0; u < SU; u++) {
+                const bool ok = part * SU + u < a.KS;
                 ssq += ok ? t_ssq[u] : 0.f;
                 ppre += (ok && g < n) ? t_pre[u] : 0.f;
                 ppost += (ok && g < n) ? t_post[u] : 0.f;
 #pragma unroll
                 for (int e = 0; e < SK::EPL; e++) pe[e] += (ok && r0 < n && c0 + e < n) ? t_e[u][e] : 0.f;
             }
-            for (int ks0 = 16 + part * 4; ks0 < a.KS; ks0 += 16) {  // more than 16 K-splits: rare
+            for (int ks0 = 4 * SU + part * SU; ks0 < a.KS; ks0 += 4 * SU) {  // never with proj_fwd_ksplit's cap
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
+                for (int u = 0; u < SU; u++) {
                     const int ks = ks0 + u;
                     if (ks < a.KS) {
                         ssq += a.ssqpart[(size_t)ks * a.B + b];

@@ -394,6 +394,11 @@ int proj_fwd_ksplit(int x_dtype, int phi_dtype, int B, int n, int C) {
     const int cap_bytes = (int)(0.25 * (2.0 * B * nC + 2.0 * DP * nC) / (4.0 * B * DP));
     if (ks > cap_slab) ks = cap_slab;
     if (ks > cap_bytes) ks = cap_bytes;
+    // the fused forward kernel (n <= 8) sums up to 24 splits (16 when a thread holds two chunks of
+    // the sample, C > 2048) with loads that it issues ahead of the sample's tile; more splits would
+    // queue behind the tile
+    const int fused_cap = C <= 2048 ? 24 : 16;
+    if (n <= 8 && ks > fused_cap) ks = fused_cap;
     if (ks > 64) ks = 64;
     if (ks < 1) ks = 1;
     return ks;
