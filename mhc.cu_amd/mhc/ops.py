@@ -10,6 +10,8 @@ Differences that a caller can observe are limited to these:
 """
 from __future__ import annotations
 
+import weakref
+
 import torch
 from torch.autograd import Function
 
@@ -178,23 +180,50 @@ def mhc_layer_fused_inference(x_expanded, rmsnorm_weight, H_pre, H_post, H_res, 
 # ----------------------------------------------------------------------------------------------
 # dynamic-H layer (reference ops.py:154-417)
 # ----------------------------------------------------------------------------------------------
-_PHI_CACHE: dict = {}
+class _DerivedCache:
+    """Small tensors derived from parameters (concatenations, casts), rebuilt only when a source
+    changed.  An entry is valid while the very same tensor objects are alive (weak references: a new
+    tensor that happens to reuse the address of a freed one never matches) and their storage address
+    and in-place version counters are unchanged."""
+
+    def __init__(self, limit):
+        self._d = {}
+        self._limit = limit
+
+    def get(self, sources, extra, build):
+        key = tuple(id(t) for t in sources) + (extra,)
+        state = tuple((t.data_ptr(), t._version, tuple(t.shape)) for t in sources)
+        hit = self._d.get(key)
+        if hit is not None and hit[0] == state and all(r() is t for r, t in zip(hit[1], sources)):
+            return hit[2]
+        with torch.no_grad():
+            value = build()
+        if len(self._d) >= self._limit:
+            self._d.clear()
+        self._d[key] = (state, tuple(weakref.ref(t) for t in sources), value)
+        return value
+
+
+_PHI_CACHE = _DerivedCache(64)
+_SMALL_CACHE = _DerivedCache(256)
 
 
 def _phi_concat(phi_pre, phi_post, phi_res, dtype):
-    """[D, nC] = rows [pre | post | res] in `dtype`, rebuilt only when a parameter changed."""
+    """[D, nC] = rows [pre | post | res] in `dtype`."""
     n = phi_pre.size(0)
-    key = (phi_pre.data_ptr(), phi_post.data_ptr(), phi_res.data_ptr(), dtype)
-    ver = (phi_pre._version, phi_post._version, phi_res._version, tuple(phi_res.shape))
-    hit = _PHI_CACHE.get(key)
-    if hit is not None and hit[0] == ver:
-        return hit[1]
-    with torch.no_grad():
-        cat = torch.cat([phi_pre, phi_post, phi_res.reshape(n * n, -1)], dim=0).to(dtype).contiguous()
-    if len(_PHI_CACHE) > 64:
-        _PHI_CACHE.clear()
-    _PHI_CACHE[key] = (ver, cat)
-    return cat
+    return _PHI_CACHE.get(
+        (phi_pre, phi_post, phi_res), dtype,
+        lambda: torch.cat([phi_pre, phi_post, phi_res.reshape(n * n, -1)], dim=0).to(dtype).contiguous())
+
+
+def _bias_alpha(b_pre, b_post, b_res, alpha_pre, alpha_post, alpha_res, dev):
+    """fp32 [D] bias (pre | post | res) and fp32 [3] alpha on the device (two small kernels and
+    their launch overhead on every call otherwise)."""
+    def build():
+        bias = torch.cat([b_pre.reshape(-1), b_post.reshape(-1), b_res.reshape(-1)]).float().to(dev)
+        alpha = torch.stack([a.to(dev).reshape(()).float() for a in (alpha_pre, alpha_post, alpha_res)])
+        return bias, alpha
+    return _SMALL_CACHE.get((b_pre, b_post, b_res, alpha_pre, alpha_post, alpha_res), str(dev), build)
 
 
 class MHCLayerDynamicFunction(Function):
@@ -209,9 +238,9 @@ class MHCLayerDynamicFunction(Function):
         D = n * n + 2 * n
         phi = _phi_concat(phi_pre, phi_post, phi_res,
                           torch.bfloat16 if x.dtype == torch.bfloat16 else torch.float32)
-        bias = torch.cat([b_pre.reshape(-1), b_post.reshape(-1), b_res.reshape(-1)]).float()
-        alpha = torch.stack([torch.as_tensor(a, device=dev).reshape(()).float()
-                             for a in (alpha_pre, alpha_post, alpha_res)])
+        alphas = tuple(a if torch.is_tensor(a) else torch.as_tensor(a, device=dev)
+                       for a in (alpha_pre, alpha_post, alpha_res))
+        bias, alpha = _bias_alpha(b_pre, b_post, b_res, *alphas, dev)
         require_gpu(x, w, phi, bias, alpha, f_inject)
         f32 = dict(dtype=torch.float32, device=dev)
         y = torch.empty((B, n, C), dtype=out_dtype or torch.float32, device=dev)
