@@ -489,6 +489,7 @@ __global__ __launch_bounds__(256) void mix_fwd_large_kernel(MixLargeArgs a) {
     bf16_t *x_s = reinterpret_cast<bf16_t *>(mfl_smem);          // [32][LDT]
     float *o_s = reinterpret_cast<float *>(x_s + 32 * kMflLDT);  // [32][LDO]
     float *ho_s = o_s + 32 * kMflLDO;                            // [32] Hpost (0 beyond n)
+    float *m_s = ho_s + 32;                                      // [32][33] M (0 beyond n x n)
     const int b = blockIdx.y, cb0 = blockIdx.x * kMflCB, n = a.n, C = a.C, tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6, row = lane & 31, kh = lane >> 5;
     const bool inject = a.f_inject != nullptr;
@@ -505,31 +506,20 @@ __global__ __launch_bounds__(256) void mix_fwd_large_kernel(MixLargeArgs a) {
         cok[h] = c < C;  // C % 8 == 0
         xr[h].load(xb + (size_t)(trow < n ? trow : 0) * C + (cok[h] ? c : 0));
     }
-    // A operand: lane (row i, kg) holds M[i][k], k = ks*16 + kg*8 .. +8 (zero beyond n)
-    bf16x8_t mh[2], ml[2];
+    // M through LDS: the operand layout below has every lane on a different row of M, which is the
+    // slow way to read global memory; here 8 lanes share a row (128 contiguous bytes)
+    float mraw[4];
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
-        float mv[8];
-        uint32_t hw[4];
-        float lo[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int k = ks * 16 + kh * 8 + i;
-            const bool ok = k < n && row < n;
-            const float m = M[ok ? row * n + k : 0];
-            mv[i] = ok ? m : 0.f;
-        }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            hw[i] = pack_bf16x2(mv[2 * i], mv[2 * i + 1]);
-            lo[2 * i] = mv[2 * i] - bf16lo_to_f32(hw[i]);
-            lo[2 * i + 1] = mv[2 * i + 1] - bf16hi_to_f32(hw[i]);
-        }
-        mh[ks] = __builtin_bit_cast(bf16x8_t, make_uint4(hw[0], hw[1], hw[2], hw[3]));
-        ml[ks] = __builtin_bit_cast(bf16x8_t, make_uint4(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]),
-                                                         pack_bf16x2(lo[4], lo[5]), pack_bf16x2(lo[6], lo[7])));
+    for (int i = 0; i < 4; i++) {
+        const int k = (tid & 7) * 4 + i;
+        mraw[i] = M[(trow < n && k < n) ? trow * n + k : 0];
     }
     if (tid < 32) ho_s[tid] = tid < n ? a.Hpost[(size_t)b * a.hstride + tid] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int k = (tid & 7) * 4 + i;
+        m_s[trow * 33 + k] = (trow < n && k < n) ? mraw[i] : 0.f;
+    }
     if (inject && a.q && blockIdx.x == 0 && tid == 0) a.q[b] = 1.0f;  // q is defined as 1 with an injected f
     // f of this lane's channel in the matrix-core phase
     const int cw = cb0 + wave * 32 + row;
@@ -544,6 +534,24 @@ __global__ __launch_bounds__(256) void mix_fwd_large_kernel(MixLargeArgs a) {
             make_uint4(xr[h].w[0], xr[h].w[1], xr[h].w[2], xr[h].w[3]);
     __syncthreads();
 
+    // A operand: lane (row i, kg) holds M[i][k], k = ks*16 + kg*8 .. +8, as a bf16 pair
+    bf16x8_t mh[2], ml[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        float mv[8], lo[8];
+        uint32_t hw[4];
+#pragma unroll
+        for (int i = 0; i < 8; i++) mv[i] = m_s[row * 33 + ks * 16 + kh * 8 + i];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            hw[i] = pack_bf16x2(mv[2 * i], mv[2 * i + 1]);
+            lo[2 * i] = mv[2 * i] - bf16lo_to_f32(hw[i]);
+            lo[2 * i + 1] = mv[2 * i + 1] - bf16hi_to_f32(hw[i]);
+        }
+        mh[ks] = __builtin_bit_cast(bf16x8_t, make_uint4(hw[0], hw[1], hw[2], hw[3]));
+        ml[ks] = __builtin_bit_cast(bf16x8_t, make_uint4(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]),
+                                                         pack_bf16x2(lo[4], lo[5]), pack_bf16x2(lo[6], lo[7])));
+    }
     f32x16_t o;
 #pragma unroll
     for (int i = 0; i < 16; i++) o[i] = 0.f;
@@ -589,7 +597,7 @@ static hipError_t launch_large_mfma(const MixLargeArgs &a, int y_dtype, hipStrea
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    const size_t smem = sizeof(bf16_t) * 32 * kMflLDT + sizeof(float) * (32 * kMflLDO + 32);
+    const size_t smem = sizeof(bf16_t) * 32 * kMflLDT + sizeof(float) * (32 * kMflLDO + 32 + 32 * 33);
     const dim3 grid((a.C + kMflCB - 1) / kMflCB, a.B);
     if (y_dtype == kBF16) mix_fwd_large_kernel<bf16_t><<<grid, 256, smem, stream>>>(a);
     else mix_fwd_large_kernel<float><<<grid, 256, smem, stream>>>(a);
