@@ -206,7 +206,7 @@ __device__ __forceinline__ float bcast_lower32(float v) {
     return __uint_as_float(r[0]);
 }
 
-__global__ __launch_bounds__(256) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
+__global__ __launch_bounds__(256, 4) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
     extern __shared__ __align__(16) unsigned char dxl_smem[];
     bf16_t *g_s = reinterpret_cast<bf16_t *>(dxl_smem);      // [32][LDT] dy tile
     bf16_t *x_s = g_s + 32 * kDxlLDT;                        // [32][LDT] x tile
