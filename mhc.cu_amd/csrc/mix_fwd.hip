@@ -141,6 +141,8 @@ struct LayerFwdArgs {
     float eps;
 };
 
+constexpr int kFwdStaggerMinB = 512;  // two or more workgroups per CU
+
 template <typename TX, typename TY, int NP, int V, int CPT>
 __global__ __launch_bounds__(256, (CPT == 2 && NP == 4 && !std::is_same<TX, float>::value) ? 5 : 1)
 void layer_fwd_small_kernel(LayerFwdArgs a) {
@@ -190,22 +192,31 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             }
         }
     }
+    // Every second workgroup of an XCD asks for its tile only after the coefficient step: with all
+    // workgroups resident at once they would otherwise move in lockstep (everybody loads, everybody
+    // runs the serial Sinkhorn chain with the memory system idle, everybody stores); the two
+    // halves now load and store at different times.  With about one workgroup per CU there is no such
+    // contention and the delay would only cost time.
+    const bool late = a.B >= kFwdStaggerMinB && ((blockIdx.x >> 3) & 1) != 0;
     RawVec<TX, V> xr[CPT][NP];
-#pragma unroll
-    for (int k = 0; k < CPT; k++) {
-        const int ch = tid + k * 256;
-        const TX *xc = xb + (size_t)(ch < nch ? ch : 0) * V;
-#pragma unroll
-        for (int i = 0; i < NP; i++) xr[k][i].load(xc + (size_t)(i < n ? i : 0) * C);
-    }
     RawVec<TX, V> fr[CPT];
-    if (inject) {
+    auto issue_tile = [&]() {
 #pragma unroll
         for (int k = 0; k < CPT; k++) {
             const int ch = tid + k * 256;
-            fr[k].load(static_cast<const TX *>(a.f_inject) + (size_t)b * C + (size_t)(ch < nch ? ch : 0) * V);
+            const TX *xc = xb + (size_t)(ch < nch ? ch : 0) * V;
+#pragma unroll
+            for (int i = 0; i < NP; i++) xr[k][i].load(xc + (size_t)(i < n ? i : 0) * C);
         }
-    }
+        if (inject) {
+#pragma unroll
+            for (int k = 0; k < CPT; k++) {
+                const int ch = tid + k * 256;
+                fr[k].load(static_cast<const TX *>(a.f_inject) + (size_t)b * C + (size_t)(ch < nch ? ch : 0) * V);
+            }
+        }
+    };
+    if (!late) issue_tile();
 
     MHC_PHASE(kPhaseFwdFused, b, 1);
     // ---- 2. coefficients on wave 0 -----------------------------------------------------------
@@ -289,6 +300,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
         }
     }
     MHC_PHASE(kPhaseFwdFused, b, 3);
+    if (late) issue_tile();
     __syncthreads();
     MHC_PHASE(kPhaseFwdFused, b, 4);
     float hpre[NP], hpost[NP], Mr[NP][NP];
