@@ -41,7 +41,7 @@ static void summary(const char *title, int kernel, int wgs, const std::vector<co
     constexpr int M = 8;
     std::vector<unsigned long long> t((size_t)wgs * M);
     if (mhc_phase_read(kernel, t.data(), wgs) != 0) { printf("%s: read failed\n", title); return; }
-    printf("\n%s (%d workgroups, shader-clock ticks)\n", title, wgs);
+    printf("\n%s (first %d workgroups of the grid, shader-clock ticks)\n", title, wgs);
     printf("%-34s %10s %10s %10s %7s\n", "phase", "mean", "p10", "p90", "share");
     const int np = (int)names.size();
     std::vector<std::vector<double>> d(np);
@@ -97,7 +97,7 @@ int main(int argc, char **argv) {
     }
     printf("phase profile: dynamic H, bf16, B=%d C=%d n=%d (last of 3 warm calls)\n", B, C, n);
     summary("fused forward kernel, one workgroup per sample", 0, std::min(B, 4096),
-            {"issue loads", "coefficient inputs arrive", "activations + Sinkhorn", "barrier", "tile arrives, aggregate, RMS",
+            {"issue loads (early half: tile too)", "coefficient inputs arrive", "activations + Sinkhorn", "tile request (late half), barrier", "tile arrives, aggregate, RMS",
              "mix, stores issued"}, true);
     const int slabs = (C + 63) / 64;
     summary("slab backward kernel, one workgroup per (64 channels, batch split)", 1, std::min(slabs * 4, 4096),
