@@ -184,7 +184,7 @@ class _DerivedCache:
     """Small tensors derived from parameters (concatenations, casts), rebuilt only when a source
     changed.  An entry is valid while the very same tensor objects are alive (weak references: a new
     tensor that happens to reuse the address of a freed one never matches) and their storage address
-    and in-place version counters are unchanged."""
+    and in-place version counters are unchanged; it is dropped when one of them is freed."""
 
     def __init__(self, limit):
         self._d = {}
@@ -200,7 +200,9 @@ class _DerivedCache:
             value = build()
         if len(self._d) >= self._limit:
             self._d.clear()
-        self._d[key] = (state, tuple(weakref.ref(t) for t in sources), value)
+        # the entry (and the derived tensor it holds) goes away with the first source that dies
+        drop = lambda _ref, d=self._d, k=key: d.pop(k, None)
+        self._d[key] = (state, tuple(weakref.ref(t, drop) for t in sources), value)
         return value
 
 
