@@ -98,37 +98,55 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) xf[ks] = pl_frag_t(x_s, ks * 16, wave * 32, lane);
 
-        // dP^T fragments of a row tile: 8 k-steps x (rounded, remainder); k-steps beyond the padded
-        // batch alias k-step 0 of the block and meet zero rows of x
-        struct AFrag { uint32_t w[16][4]; };
-        auto load_a = [&](AFrag &f, int dt) {
-            const bf16_t *ap = a.dPT + frag_base(min(dt, NTD - 1), a.BP >> 4, sb >> 4) + lane * 8;
+        // dP^T operands of a row tile: 8 k-steps x (rounded, remainder) x 64 lanes x 16 bytes = 16 KB,
+        // contiguous per plane in the fragment-major layout.  All four waves multiply the same
+        // operands (they differ in the columns they own), so the workgroup fetches a tile once,
+        // 4 x 16 bytes per thread, and shares it through a double-buffered LDS tile; k-steps beyond
+        // the padded batch alias k-step 0 of the block and meet zero rows of x.
+        // (the operand tiles reuse the LDS of the x block, which is dead once xf is in registers)
+        bf16_t *a_s = x_s;  // [2][2 planes][8 k-steps][512]
+        uint32_t ar[16];  // scalar words: whole-uint4 array elements can end up in scratch memory
+        auto fetch_a = [&](int dt) {
+            const bf16_t *ap = a.dPT + frag_base(min(dt, NTD - 1), a.BP >> 4, sb >> 4);
 #pragma unroll
-            for (int ks = 0; ks < 8; ks++) {
-                const bf16_t *apk = ap + (sb + ks * 16 < a.BP ? ks * 512 : 0);
+            for (int j = 0; j < 2; j++) {
+                const int c = tid + 256 * j, ks = c >> 6;  // 16-byte piece c of the plane's 8 KB
+                const bf16_t *apk = ap + (sb + ks * 16 < a.BP ? c * 8 : (c & 63) * 8);
                 const uint4 h = *reinterpret_cast<const uint4 *>(apk);
                 const uint4 l = *reinterpret_cast<const uint4 *>(apk + plane);
-                f.w[2 * ks][0] = h.x; f.w[2 * ks][1] = h.y; f.w[2 * ks][2] = h.z; f.w[2 * ks][3] = h.w;
-                f.w[2 * ks + 1][0] = l.x; f.w[2 * ks + 1][1] = l.y; f.w[2 * ks + 1][2] = l.z; f.w[2 * ks + 1][3] = l.w;
+                ar[8 * j] = h.x; ar[8 * j + 1] = h.y; ar[8 * j + 2] = h.z; ar[8 * j + 3] = h.w;
+                ar[8 * j + 4] = l.x; ar[8 * j + 5] = l.y; ar[8 * j + 6] = l.z; ar[8 * j + 7] = l.w;
             }
         };
-        AFrag fa, fb;
-        load_a(fa, dt0);
-        // one row tile: request the next tile's operands, multiply, (SINGLE) store
-        auto do_tile = [&](const AFrag &cur, AFrag &nxt, int m, f32x16_t &am) {
-            load_a(nxt, dt0 + m + 1);  // clamped to the last tile: redundant at the end, never used
+        auto park_a = [&](int buf) {
+            bf16_t *dst = a_s + (size_t)buf * 2 * 4096;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                *reinterpret_cast<uint4 *>(dst + (tid + 256 * j) * 8) =
+                    make_uint4(ar[8 * j], ar[8 * j + 1], ar[8 * j + 2], ar[8 * j + 3]);
+                *reinterpret_cast<uint4 *>(dst + 4096 + (tid + 256 * j) * 8) =
+                    make_uint4(ar[8 * j + 4], ar[8 * j + 5], ar[8 * j + 6], ar[8 * j + 7]);
+            }
+        };
+        fetch_a(dt0);
+        __syncthreads();  // every wave has its x fragments
+        park_a(0);
+        __syncthreads();
+        // one row tile: request the next tile's operands, multiply from LDS, (SINGLE) store, park
+        // the next tile, one barrier
+        auto do_tile = [&](int m, f32x16_t &am) {
+            fetch_a(dt0 + m + 1);  // clamped to the last tile: redundant at the end, never used
             if (SINGLE) {
 #pragma unroll
                 for (int i = 0; i < 16; i++) am[i] = 0.f;
             }
+            const bf16_t *src = a_s + (size_t)(m & 1) * 2 * 4096 + lane * 8;
 #pragma unroll
             for (int ks = 0; ks < 8; ks++) {
-                am = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[2 * ks][0], cur.w[2 * ks][1], cur.w[2 * ks][2], cur.w[2 * ks][3])),
-                    xf[ks], am, 0, 0, 0);
-                am = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[2 * ks + 1][0], cur.w[2 * ks + 1][1], cur.w[2 * ks + 1][2], cur.w[2 * ks + 1][3])),
-                    xf[ks], am, 0, 0, 0);
+                const uint4 h = *reinterpret_cast<const uint4 *>(src + ks * 512);
+                const uint4 l = *reinterpret_cast<const uint4 *>(src + 4096 + ks * 512);
+                am = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, h), xf[ks], am, 0, 0, 0);
+                am = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, l), xf[ks], am, 0, 0, 0);
             }
             if (SINGLE && k < a.nC) {
 #pragma unroll
@@ -137,23 +155,16 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
                     if (d < a.D) __builtin_nontemporal_store(am[i], out + (size_t)d * a.nC + k);
                 }
             }
+            park_a((m + 1) & 1);  // last read two tiles ago, before the previous barrier
+            __syncthreads();
         };
         if constexpr (SINGLE) {
-            // rolled loop over pairs of tiles (the two operand buffers swap roles inside a pair), so
-            // that only one tile's operands are requested ahead
 #pragma unroll 1
-            for (int m = 0; dt0 + m < dt1; m += 2) {
-                do_tile(fa, fb, m, acc[0]);
-                if (dt0 + m + 1 < dt1) do_tile(fb, fa, m + 1, acc[0]);
-            }
+            for (int m = 0; dt0 + m < dt1; m++) do_tile(m, acc[0]);
         } else {
 #pragma unroll
-            for (int m = 0; m < TPW; m++) {
-                if (dt0 + m < dt1) {  // uniform
-                    if (m & 1) do_tile(fb, fa, m, acc[m < NACC ? m : 0]);
-                    else do_tile(fa, fb, m, acc[m < NACC ? m : 0]);
-                }
-            }
+            for (int m = 0; m < TPW; m++)
+                if (dt0 + m < dt1) do_tile(m, acc[m < NACC ? m : 0]);  // uniform
         }
     }
     if (!SINGLE && k < a.nC) {  // several sample blocks: tiles are complete only now
@@ -309,11 +320,17 @@ hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb
                          sizeof(bf16_t) * 128 * kDxfLD, stream>>>(a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const size_t smem = sizeof(bf16_t) * kPL_SB * kPL_LD;
-    if (bps <= kPL_SB)  // one sample block per split: 9 row tiles per workgroup, stored as they complete
+    // the x block, later two operand tiles of 16 KB in the same memory
+    const size_t smem = sizeof(bf16_t) * (kPL_SB * kPL_LD > 2 * 2 * 4096 ? kPL_SB * kPL_LD : 2 * 2 * 4096);
+    if (bps <= kPL_SB) {  // one sample block per split: 9 row tiles per workgroup, stored as they complete
+        e = allow_dynamic_lds(&dphi_large_kernel<9, true>, smem);
+        if (e != hipSuccess) return e;
         dphi_large_kernel<9, true><<<dim3(slabs, (NTD + 8) / 9, S), 256, smem, stream>>>(a);
-    else
+    } else {
+        e = allow_dynamic_lds(&dphi_large_kernel<3, false>, smem);
+        if (e != hipSuccess) return e;
         dphi_large_kernel<3, false><<<dim3(slabs, (NTD + 2) / 3, S), 256, smem, stream>>>(a);
+    }
     return hipGetLastError();
 }
 
