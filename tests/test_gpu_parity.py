@@ -97,6 +97,8 @@ DYN_SHAPES = [
     # n > 8 in float32: several tiles and a ragged last slice for the fp32 matrix-core products, and
     # a row length that is not a multiple of 4 (scalar kernels)
     (130, 12, 36), (3, 9, 10),
+    # a batch far beyond the CU count, a row too long for the fused forward kernel, odd expansion rates
+    (2100, 4, 32), (2, 4, 4400), (3, 17, 24), (2, 31, 40),
 ]
 
 
@@ -147,7 +149,10 @@ def test_largest_iteration_counts(B, n, C, T, dyn):
                                    (160, 20, 64), (130, 32, 136),
                                    # two chunks per thread with a ragged chunk count and a partial sample tile;
                                    # n between the tile sizes; one sample; C not a multiple of 8 with n > 8
-                                   (33, 4, 2568), (3, 12, 40), (2, 24, 104), (1, 32, 128), (3, 20, 36)])
+                                   (33, 4, 2568), (3, 12, 40), (2, 24, 104), (1, 32, 128), (3, 20, 36),
+                                   # a batch far beyond the CU count (several samples per workgroup, batch
+                                   # splits), a row too long for the fused forward kernel, odd expansion rates
+                                   (4100, 4, 64), (2, 4, 8200), (3, 17, 24), (2, 31, 40), (600, 8, 64)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_dynamic_bf16_vs_oracle(B, n, C, out_dtype):
     x, dy, _, p = nm.make_dynamic_inputs(B, n, C, bf16_round=True)
