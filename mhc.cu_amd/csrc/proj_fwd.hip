@@ -390,8 +390,8 @@ int proj_fwd_ksplit(int x_dtype, int phi_dtype, int B, int n, int C) {
     const int groups = DP / 32 / mfma_nt(n);
     int ks = (1024 + tiles_s * groups - 1) / (tiles_s * groups);
     const int cap_slab = nC / 256;
-    // partial sums (KS * B * DP fp32) at most ~1/4 of the bytes this kernel streams (x and phi)
-    const int cap_bytes = (int)(0.25 * (2.0 * B * nC + 2.0 * DP * nC) / (4.0 * B * DP));
+    // partial sums (KS * B * DP fp32) at most ~1/3 of the bytes this kernel streams (x and phi)
+    const int cap_bytes = (int)(0.35 * (2.0 * B * nC + 2.0 * DP * nC) / (4.0 * B * DP));
     if (ks > cap_slab) ks = cap_slab;
     if (ks > cap_bytes) ks = cap_bytes;
     // the fused forward kernel (n <= 8) sums up to 24 splits (16 when a thread holds two chunks of
