@@ -152,7 +152,9 @@ def test_largest_iteration_counts(B, n, C, T, dyn):
                                    (33, 4, 2568), (3, 12, 40), (2, 24, 104), (1, 32, 128), (3, 20, 36),
                                    # a batch far beyond the CU count (several samples per workgroup, batch
                                    # splits), a row too long for the fused forward kernel, odd expansion rates
-                                   (4100, 4, 64), (2, 4, 8200), (3, 17, 24), (2, 31, 40), (600, 8, 64)])
+                                   (4100, 4, 64), (2, 4, 8200), (3, 17, 24), (2, 31, 40), (600, 8, 64),
+                                   # wide projection with batch splits and many sample blocks per split
+                                   (4000, 20, 32)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_dynamic_bf16_vs_oracle(B, n, C, out_dtype):
     x, dy, _, p = nm.make_dynamic_inputs(B, n, C, bf16_round=True)
