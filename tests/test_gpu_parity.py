@@ -241,3 +241,56 @@ def test_config2_fp32_full_size():
     _check(y, y_ref, "fp32", "y")
     for k, ref in g_ref.items():
         _check(g[k], ref, "fp32", "d" + k)
+
+
+def _random_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(count):
+        n = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 16, 17, 24, 31, 32]))
+        B = int(rng.choice([1, 2, 3, 5, 17, 33, 64, 129, 260]))
+        unit = int(rng.choice([1, 2, 4, 8]))
+        C = unit * int(rng.integers(1, 40))
+        if n * C * B > 600_000:   # keep the float64 oracle quick
+            B = max(1, 600_000 // (n * C))
+        T = int(rng.choice([0, 1, 3, 20]))
+        cases.append((B, n, C, T, bool(rng.integers(2)), bool(rng.integers(2)), bool(rng.integers(2))))
+    return cases
+
+
+@pytest.mark.parametrize("B,n,C,T,dyn,bf16,inject", _random_cases(40, seed=2024))
+def test_random_shapes_vs_oracle(B, n, C, T, dyn, bf16, inject):
+    """Seeded sweep over shapes, iteration counts (0 and 1 included), both coefficient modes, both
+    precision tiers and both views, against the oracle."""
+    eps = 1e-6
+    act = torch.bfloat16 if bf16 else torch.float32
+    tier = "bf16" if bf16 else "fp32"
+    make = nm.make_dynamic_inputs if dyn else nm.make_static_inputs
+    x, dy, f, p = make(B, n, C, with_f=inject)
+    if dyn:
+        p = _rand_params(p, n, C)
+    if bf16:
+        x, dy = x.bfloat16().float(), dy.bfloat16().float()
+        f = None if f is None else f.bfloat16().float()
+        for k in ("w", "phi_pre", "phi_post", "phi_res"):
+            if k in p:
+                p[k] = p[k].bfloat16().float()
+    ref_dtype = torch.float32 if bf16 else torch.float64
+    if dyn:
+        y_ref, g_ref = nm.mhc_dynamic_fwd_bwd(x, p, dy, T, eps, f_inject=f, dtype=ref_dtype)
+        y, g = hip_dynamic(x, p, dy, T, eps, f_inject=f, act_dtype=act, out_dtype=act,
+                           w_dtype=act)
+    else:
+        y_ref, g_ref = nm.mhc_static_fwd_bwd(x, p, dy, T, eps, f_inject=f, dtype=ref_dtype)
+        y, g = hip_static(x, p, dy, T, eps, f_inject=f, act_dtype=act, out_dtype=act, w_dtype=act)
+    _check(y, y_ref, tier, "y")
+    for k, ref in g_ref.items():
+        assert k in g, f"missing gradient {k}"
+        tiny = ("phi_pre", "b_pre", "alpha_pre", "H_pre") + (("phi_res", "b_res", "alpha_res", "H_res") if T > 0 else ())
+        if n == 1 and k in tiny:
+            # one stream: f does not depend on H_pre except through eps, and the 1 x 1 Sinkhorn output
+            # (after at least one iteration) is 1 / (1 + O(eps)) whatever its logit, so these gradients are O(eps) (bf16: rounding
+            # noise of that size) and a relative comparison is meaningless
+            assert float(g[k].abs().max()) < (1e-2 if bf16 else 1e-4), k
+            continue
+        _check(g[k], ref, tier, "d" + k)
