@@ -157,11 +157,11 @@ template <int NP, bool PRECISE> __global__ __launch_bounds__(256) void coef_fwd_
         a.Hpost[b * n + tid] = 2.0f * sigmoidf_acc(lg[n + tid]);
     }
     const int r0 = SK::row(tid), c0 = SK::col0(tid);
-    float E[SK::EPL], ET[SK::EPL], u, v[SK::EPL];
+    float E[SK::EPL], u, v[SK::EPL];
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         E[e] = (r0 < n && c0 + e < n) ? expf(lg[2 * n + r0 * n + c0 + e]) : 0.f;
-    SK::template forward<PRECISE>(E, ET, u, v, n, a.T, a.eps, sk_s, tid);
+    SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         if (r0 < n && c0 + e < n) a.M[(size_t)b * n * n + r0 * n + c0 + e] = u * E[e] * v[e];

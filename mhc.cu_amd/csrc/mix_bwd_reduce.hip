@@ -577,14 +577,36 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         pres[e] = dyn ? a.P[(size_t)b * D + (ok ? 2 * n + r0 * n + c0 + e : 0)] : 0.f;
         bres[e] = dyn ? a.b_res[ok ? r0 * n + c0 + e : 0] : 0.f;
     }
-    // sum the column parts; rows / columns >= n hold aliased garbage and are dropped here
+    // sum the column parts; rows / columns >= n hold aliased garbage and are dropped here.  The
+    // first four parts are requested before the Sinkhorn forward recompute (which needs none of
+    // them) and collected after it.
     const float *raw = a.raw + (size_t)b * a.parts * kGramFloats;
+    constexpr int EPT = kGramFloats / 256;  // 12 elements per thread, all loads of a part in flight
+    float t0[4][EPT];
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int k = 0; k < EPT; k++)
+            t0[q][k] = raw[(size_t)(q < a.parts ? q : 0) * kGramFloats + tid + 256 * k];
+    float E[SK::EPL], u = 1.0f, v[SK::EPL];
+    if (dyn) {
+#pragma unroll
+        for (int e = 0; e < SK::EPL; e++) {
+            const bool ok = r0 < n && c0 + e < n;
+            pres[e] = ok ? pres[e] : 0.f;
+            E[e] = ok ? expf(al2 * pres[e] + bres[e]) : 0.f;
+        }
+        SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
+    }
     {
-        constexpr int EPT = kGramFloats / 256;  // 12 elements per thread, all loads of a part in flight
         float acc[EPT];
 #pragma unroll
         for (int k = 0; k < EPT; k++) acc[k] = 0.f;
-        for (int p0 = 0; p0 < a.parts; p0 += 4) {  // 48 loads in flight; surplus parts alias part 0
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+#pragma unroll
+            for (int k = 0; k < EPT; k++) acc[k] += q < a.parts ? t0[q][k] : 0.f;
+        for (int p0 = 4; p0 < a.parts; p0 += 4) {  // 48 loads in flight; surplus parts alias part 0
             float t[4][EPT];
 #pragma unroll
             for (int q = 0; q < 4; q++)
@@ -657,18 +679,14 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         dpw.put(lane, dtp * al0 * rinv); dpw.put(n + lane, dto * al1 * rinv);
         S0 = dtp * Pb[lane]; S1 = dto * Pb[n + lane];
     }
-    // Sinkhorn forward recompute + exact backward, the matrix spread over all 256 threads
-    float E[SK::EPL], ET[SK::EPL], d[SK::EPL], u, v[SK::EPL];
+    // exact Sinkhorn backward (the forward recompute ran above), the matrix spread over all 256 threads
+    float d[SK::EPL];
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;
-        const bool ok = r0 < n && c < n;
-        pres[e] = ok ? pres[e] : 0.f;
-        E[e] = ok ? expf(al2 * pres[e] + bres[e]) : 0.f;
-        d[e] = ok ? M_s[r0 * 33 + c] : 0.f;
+        d[e] = (r0 < n && c < n) ? M_s[r0 * 33 + c] : 0.f;
     }
-    SK::template forward<PRECISE>(E, ET, u, v, n, a.T, a.eps, sk_s, tid);
-    SK::template backward<PRECISE>(E, ET, d, u, v, a.T, sk_s, tid);
+    SK::template backward<PRECISE>(E, d, u, v, a.T, sk_s, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;

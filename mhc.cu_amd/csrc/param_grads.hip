@@ -228,15 +228,15 @@ __global__ __launch_bounds__(256) void coef_bwd_static_kernel(const float *__res
         dH_post[tid] = red_sum[n * n + n + tid] * ho * (1.0f - 0.5f * ho);
     }
     const int r0 = SK::row(tid), c0 = SK::col0(tid);
-    float E[SK::EPL], ET[SK::EPL], d[SK::EPL], u, v[SK::EPL];
+    float E[SK::EPL], d[SK::EPL], u, v[SK::EPL];
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const bool ok = r0 < n && c0 + e < n;
         E[e] = ok ? expf(H_res_logits[r0 * n + c0 + e]) : 0.f;
         d[e] = ok ? red_sum[r0 * n + c0 + e] : 0.f;
     }
-    SK::template forward<true>(E, ET, u, v, n, T, eps, lds, tid);
-    SK::template backward<true>(E, ET, d, u, v, T, lds, tid);
+    SK::template forward<true>(E, u, v, n, T, eps, lds, tid);
+    SK::template backward<true>(E, d, u, v, T, lds, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         if (r0 < n && c0 + e < n) dH_res[r0 * n + c0 + e] = d[e] * E[e];

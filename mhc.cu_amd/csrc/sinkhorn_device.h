@@ -107,26 +107,28 @@ template <int NP> struct SkSmall {
 
 // =============================================================================================
 // SkWg: one 256-thread workgroup per matrix, NP = 16 or 32, iterate kept in scaling form
-// diag(u) E diag(v) with E constant in registers.  Every thread plays two roles on the same pair of
-// numbers (a, b0) = (tid / LPR, (tid % LPR) * EPL):
-//   row role     owns E[a][b0 .. b0+EPL) (and the running gradient there), and u[a]
-//   column role  owns E[b0 .. b0+EPL)[a] (a transposed copy made once through LDS), and v[a]
-// so both the row sums and the column sums are an in-register dot product plus a reduction over
-// the LPR lanes of a DPP row; the two vectors travel through LDS (u after the row half-step, v
-// after the column half-step, one barrier each).  The scalings u_t, v_t of every iteration stay in
-// LDS for the backward sweep, which rebuilds iterate t as diag(u_t) E diag(v_t) and the
-// denominators as u_{t-1} / u_t, v_{t-1} / v_t, and keeps the gradient in both roles.  Measured
-// against float64 the round-off of the backward grows by about 2e-8 per iteration (5e-7 at the
-// usual 20 iterations); the accepted iteration counts keep it below 1e-5.  Every thread of the
-// workgroup must call forward/backward; `lds` must be 16-byte aligned.
+// diag(u) E diag(v) with E constant in registers: thread t owns E[a][b0 .. b0+EPL) with
+// (a, b0) = (t / LPR, (t % LPR) * EPL), and the running gradient there.
+//
+// forward(): every thread also holds the transposed elements E[b0 .. b0+EPL)[a] (copied once
+// through LDS), so both the row sums and the column sums are an in-register dot product plus a
+// reduction over the LPR lanes of a DPP row; only the vectors u and v travel through LDS (one
+// barrier per half-step).  The denominators rho/s of every iteration stay in LDS.
+// backward(): one copy of the gradient; row dots inside a DPP row, column dots inside the wave
+// (DPP, v_permlane*_swap) and then across the 4 waves through a double-buffered LDS slot (one
+// barrier per iteration; keeping a transposed copy of the gradient as well needs two barriers and
+// measured 50 % slower); the scalings are unwound with the saved denominators (u *= rho, v *= s)
+// instead of storing iterates.  Measured against float64 the round-off of the backward grows by
+// about 2e-8 per iteration (5e-7 at the usual 20); the accepted iteration counts keep it below
+// 1e-5.  Every thread of the workgroup must call forward/backward; `lds` must be 16-byte aligned.
 // =============================================================================================
 template <int NP> struct SkWg {
     static_assert(NP == 16 || NP == 32, "SkWg handles 16x16 and 32x32 tiles");
     static constexpr int EPL = NP * NP / 256;  // 1 or 4
     static constexpr int LPR = NP / EPL;       // lanes per row: 16 or 8
     static constexpr int kTile = NP * (NP + 1);
-    // LDS floats: transpose tile | u | v | column dots | row dots | u_t [T][NP] | v_t [T][NP]
-    __host__ __device__ static constexpr int lds_floats(int T) { return kTile + 4 * NP + 2 * T * NP; }
+    // LDS floats: transpose tile (later the column slots [2][4][NP]) | u | v | rho [T][NP] | s [T][NP]
+    __host__ __device__ static constexpr int lds_floats(int T) { return kTile + 2 * NP + 2 * T * NP; }
     __device__ static __forceinline__ int row(int tid) { return tid / LPR; }
     __device__ static __forceinline__ int col0(int tid) { return (tid % LPR) * EPL; }
 
@@ -142,6 +144,25 @@ template <int NP> struct SkWg {
         }
         return x;
     }
+    // sum over all NP rows of per-column values; cw_t = this iteration's LDS slot [4][NP]
+    __device__ static __forceinline__ void col_allreduce(float (&x)[EPL], float *cw_t, int tid) {
+        const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) {
+            if constexpr (LPR == 8) x[e] += dpp_mov<kDppRowRor8>(x[e]);
+            x[e] = xor16_add(x[e]);
+            x[e] = xor32_add(x[e]);
+        }
+        if (lane < LPR) {
+#pragma unroll
+            for (int e = 0; e < EPL; e++) cw_t[wave * NP + lane * EPL + e] = x[e];
+        }
+        __syncthreads();
+        const int c0 = col0(tid);
+#pragma unroll
+        for (int e = 0; e < EPL; e++)
+            x[e] = (cw_t[c0 + e] + cw_t[NP + c0 + e]) + (cw_t[2 * NP + c0 + e] + cw_t[3 * NP + c0 + e]);
+    }
     // EPL consecutive floats at a 16-byte aligned LDS address
     __device__ static __forceinline__ void ld_vec(const float *p, float (&x)[EPL]) {
         if constexpr (EPL == 4) {
@@ -152,7 +173,7 @@ template <int NP> struct SkWg {
             for (int e = 0; e < EPL; e++) x[e] = p[e];
         }
     }
-    // row-role values a[e] = A[a][b0+e]  ->  column-role values at[e] = A[b0+e][a]
+    // a[e] = A[a][b0+e]  ->  at[e] = A[b0+e][a]
     __device__ static __forceinline__ void transpose(const float (&a)[EPL], float (&at)[EPL], float *tile,
                                                      int tid) {
         const int r = row(tid), c0 = col0(tid);
@@ -164,19 +185,18 @@ template <int NP> struct SkWg {
         __syncthreads();
     }
 
-    // E: exp(logits), 0 outside n x n (row role).  On return ET is the column-role copy,
-    // M = u * E[e] * v[e], and the scalings of every iteration sit in LDS for backward().
+    // E: exp(logits), 0 outside n x n.  On return M = u * E[e] * v[e]; rho/s hold the denominators.
     // PRECISE selects IEEE divisions (fp32 parity tier) instead of v_rcp_f32 (1 ulp).
     template <bool PRECISE = true>
-    __device__ static __forceinline__ void forward(const float (&E)[EPL], float (&ET)[EPL], float &u,
-                                                   float (&v)[EPL], int n, int T, float eps, float *lds,
-                                                   int tid) {
-        float *ub = lds + kTile, *vb = ub + NP, *uh = vb + 3 * NP, *vh = uh + T * NP;
+    __device__ static __forceinline__ void forward(const float (&E)[EPL], float &u, float (&v)[EPL], int n,
+                                                   int T, float eps, float *lds, int tid) {
+        float *ub = lds + kTile, *vb = ub + NP, *rho = vb + NP, *s = rho + T * NP;
         const int a = row(tid), b0 = col0(tid);
         const bool head = (tid % LPR) == 0, live = a < n;
+        float ET[EPL];
         transpose(E, ET, lds, tid);
         u = 1.0f;
-        float vc = 1.0f;  // v[a], column role
+        float vc = 1.0f;  // v[a]: this thread's column in the transposed role
 #pragma unroll
         for (int e = 0; e < EPL; e++) v[e] = 1.0f;
         for (int t = 0; t < T; t++) {
@@ -186,7 +206,7 @@ template <int NP> struct SkWg {
             p = seg_allreduce(p);
             const float rr = live ? u * p + eps : 1.0f;
             u = PRECISE ? u / rr : u * fast_rcp(rr);
-            if (head) { uh[t * NP + a] = u; ub[a] = u; }
+            if (head) { rho[t * NP + a] = rr; ub[a] = u; }
             __syncthreads();
             float uc[EPL], q = 0.f;
             ld_vec(ub + b0, uc);
@@ -195,86 +215,42 @@ template <int NP> struct SkWg {
             q = seg_allreduce(q);
             const float sc = live ? vc * q + eps : 1.0f;
             vc = PRECISE ? vc / sc : vc * fast_rcp(sc);
-            if (head) { vh[t * NP + a] = vc; vb[a] = vc; }
+            if (head) { s[t * NP + a] = sc; vb[a] = vc; }
             __syncthreads();
             ld_vec(vb + b0, v);
         }
     }
 
-    // d: in = dL/dM, out = dL/dE (row role).  E, ET, u, v, LDS contents: as left by forward()
-    // (u and v are destroyed).
+    // d: in = dL/dM, out = dL/dE.  E, u, v, LDS contents: as left by forward() (u and v are
+    // destroyed).
     template <bool PRECISE = true>
-    __device__ static __forceinline__ void backward(const float (&E)[EPL], const float (&ET)[EPL],
-                                                    float (&d)[EPL], float u, float (&v)[EPL], int T,
-                                                    float *lds, int tid) {
-        float *ub = lds + kTile, *vb = ub + NP, *cdb = vb + NP, *rdb = cdb + NP;
-        const float *uh = rdb + NP, *vh = uh + T * NP;
-        const int a = row(tid), b0 = col0(tid);
-        const bool head = (tid % LPR) == 0;
-        float dT[EPL], uc[EPL];
-        transpose(d, dT, lds, tid);
-        ld_vec(ub + b0, uc);
-        float vc = vb[a];
-        // scalings before iteration t (all ones before the first), fetched one iteration ahead; the
-        // denominators of iteration t are their ratios to the current ones:
-        // 1/rho = u_t / u_{t-1}, 1/s = v_t / v_{t-1}
-        float up, vpc, vp[EPL], upc[EPL];
-        auto fetch_prev = [&](int t) {
-            up = 1.0f; vpc = 1.0f;
-#pragma unroll
-            for (int e = 0; e < EPL; e++) { vp[e] = 1.0f; upc[e] = 1.0f; }
-            if (t > 0) {
-                up = uh[(t - 1) * NP + a];
-                vpc = vh[(t - 1) * NP + a];
-                ld_vec(vh + (t - 1) * NP + b0, vp);
-                ld_vec(uh + (t - 1) * NP + b0, upc);
-            }
-        };
-        fetch_prev(T - 1);
+    __device__ static __forceinline__ void backward(const float (&E)[EPL], float (&d)[EPL], float u,
+                                                    float (&v)[EPL], int T, float *lds, int tid) {
+        float *cw = lds;  // the transpose tile is dead after forward()
+        const float *rho = lds + kTile + 2 * NP, *s = rho + T * NP;
+        const int r = row(tid), c0 = col0(tid);
         for (int t = T - 1; t >= 0; t--) {
-            // column role: dots of the gradient with the iterate after column step t
-            float x = 0.f;
+            // column dots with the iterate after column step t: Out = u E v
+            float cd[EPL];
 #pragma unroll
-            for (int e = 0; e < EPL; e++) x += dT[e] * uc[e] * ET[e];
-            x = seg_allreduce(x);
-            if (head) cdb[a] = x;
-#pragma unroll
-            for (int e = 0; e < EPL; e++) dT[e] -= x * vc;
-            __syncthreads();
-            // row role: same update, then the row dots of row step t
-            float cdv[EPL], z = 0.f;
-            ld_vec(cdb + b0, cdv);
+            for (int e = 0; e < EPL; e++) cd[e] = d[e] * u * E[e];
+            col_allreduce(cd, cw + (t & 1) * 4 * NP, tid);
+            float z = 0.f, sc[EPL];
+            ld_vec(s + t * NP + c0, sc);
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
-                d[e] -= cdv[e] * v[e];
+                d[e] -= cd[e] * v[e];
                 z += d[e] * E[e] * v[e];
             }
             const float rdot = u * seg_allreduce(z);
-            if (head) rdb[a] = rdot;
-            const float irr = PRECISE ? u / up : u * fast_rcp(up);
+            const float rr = rho[t * NP + r];
+            const float rri = PRECISE ? 0.f : fast_rcp(rr);
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
-                const float isc = PRECISE ? v[e] / vp[e] : v[e] * fast_rcp(vp[e]);
-                d[e] = (d[e] * isc - rdot) * irr;
-                v[e] = vp[e];
+                d[e] = PRECISE ? (d[e] / sc[e] - rdot) / rr : (d[e] * fast_rcp(sc[e]) - rdot) * rri;
+                v[e] *= sc[e];
             }
-            u = up;
-            __syncthreads();
-            // column role: finish the update with the row dots
-            float rdv[EPL];
-            ld_vec(rdb + b0, rdv);
-            const float isc_c = PRECISE ? vc / vpc : vc * fast_rcp(vpc);
-#pragma unroll
-            for (int e = 0; e < EPL; e++) {
-                const float irr_e = PRECISE ? uc[e] / upc[e] : uc[e] * fast_rcp(upc[e]);
-                dT[e] = (dT[e] * isc_c - rdv[e]) * irr_e;
-                uc[e] = upc[e];
-            }
-            vc = vpc;
-            fetch_prev(t - 1);  // in flight across the next iteration's first reduction
-            // the two copies of the gradient can round differently; refresh the column-role copy
-            // now and then so that their difference cannot build up over hundreds of iterations
-            if ((t & 15) == 0 && t > 0) transpose(d, dT, lds, tid);
+            u *= rr;
         }
     }
 };
