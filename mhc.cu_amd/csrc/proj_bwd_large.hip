@@ -28,6 +28,7 @@ struct ProjBwdLargeArgs {
     float *dphi;         // [S][D][nC]
     bf16_t *dxflat;      // [B][nC]
     int B, BP, D, DP, nC, b_per_split;
+    int tpw;             // row tiles per workgroup of the single-block dphi kernel
 };
 
 // lane (n = lane & 31, kg = lane >> 5) gets tile[k0 + kg*8 + i][col0 + n], i = 0..7
@@ -62,7 +63,8 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
     const int row = lane & 31, kg = lane >> 5;
     const int k0 = blockIdx.x * kPL_KW;
     const int NTD = a.DP / 32;
-    const int dt0 = blockIdx.y * TPW, dt1 = min(NTD, dt0 + TPW);
+    const int tpw = SINGLE ? a.tpw : TPW;
+    const int dt0 = blockIdx.y * tpw, dt1 = min(NTD, dt0 + tpw);
     const int b_begin = blockIdx.z * a.b_per_split;
     const int b_end = min(a.B, b_begin + a.b_per_split);
     float *out = a.dphi + (size_t)blockIdx.z * a.D * a.nC;
@@ -313,7 +315,7 @@ hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb
     const int bps = (nblocks + S - 1) / S * kPL_SB;
     ProjBwdLargeArgs a{static_cast<const bf16_t *>(x), static_cast<const bf16_t *>(phi),
                        static_cast<const bf16_t *>(dPb), static_cast<const bf16_t *>(dPT), dphi_out,
-                       static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, bps};
+                       static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, bps, 9};
     const int slabs = (nC + kPL_KW - 1) / kPL_KW;
     const int NTD = DP / 32;
     dxflat_wide_kernel<<<dim3((nC + kDxfCW - 1) / kDxfCW, (B + 127) / 128), 256,
@@ -322,10 +324,19 @@ hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb
     if (e != hipSuccess) return e;
     // the x block, later two operand tiles of 16 KB in the same memory
     const size_t smem = sizeof(bf16_t) * (kPL_SB * kPL_LD > 2 * 2 * 4096 ? kPL_SB * kPL_LD : 2 * 2 * 4096);
-    if (bps <= kPL_SB) {  // one sample block per split: 9 row tiles per workgroup, stored as they complete
+    if (bps <= kPL_SB) {
+        // one sample block per split: row tiles are stored as they complete.  Tiles per workgroup:
+        // the fewest (9, 12, 17, all) with which the grid fits the chip's resident workgroups at once
+        // (4 per CU): 1280 workgroups on 1024 slots would run as two rounds, the second a quarter full.
+        const int slots = 256 * 4;
+        int tpw = NTD;
+        for (int cand : {9, 12, 17})
+            if (cand < NTD && (long long)slabs * ((NTD + cand - 1) / cand) * S <= slots) { tpw = cand; break; }
+        if ((long long)slabs * S > slots) tpw = NTD < 9 ? NTD : 9;  // more than one round anyway
+        a.tpw = tpw;
         e = allow_dynamic_lds(&dphi_large_kernel<9, true>, smem);
         if (e != hipSuccess) return e;
-        dphi_large_kernel<9, true><<<dim3(slabs, (NTD + 8) / 9, S), 256, smem, stream>>>(a);
+        dphi_large_kernel<9, true><<<dim3(slabs, (NTD + tpw - 1) / tpw, S), 256, smem, stream>>>(a);
     } else {
         e = allow_dynamic_lds(&dphi_large_kernel<3, false>, smem);
         if (e != hipSuccess) return e;
