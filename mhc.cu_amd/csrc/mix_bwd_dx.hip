@@ -158,11 +158,11 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
 // in LDS and read back transposed (the contraction runs over streams, the strided axis) as B
 // operands of v_mfma_f32_32x32x16_bf16; wave w owns channels 32w..32w+32 of the block.
 //   O   = M^T dy            A = M^T as a bf16 pair (rounded value + remainder: ~16 mantissa bits)
-//   df  = Hpost^T dy        A = [Hpost; 0; ...] (row 0 of the product)
-//   a   = Hpre^T x          A = [Hpre; 0; ...]
-// da, u = df a / q follow per channel in the lanes that hold the channel's column; O + Hpre (x) da
-// goes through LDS to a row-major epilogue that subtracts cx x, adds the projection term and
-// leaves as 16-byte stores.
+// df = Hpost^T dy and a = Hpre^T x follow per channel on the VALU from the same LDS tiles (each half
+// of the wave sums 16 streams), then da, u = df a / q; O + Hpre (x) da goes through LDS (in the
+// memory of the consumed tiles) to a row-major epilogue that subtracts cx x, adds the projection
+// term and leaves as 16-byte stores.  95 registers and 17 KB of LDS: five workgroups per CU, so
+// the 1280 workgroups of B = 128, C = 1280 are resident in one round.
 // =============================================================================================
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
@@ -206,12 +206,14 @@ __device__ __forceinline__ float bcast_lower32(float v) {
     return __uint_as_float(r[0]);
 }
 
-__global__ __launch_bounds__(256, 4) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
+__global__ __launch_bounds__(256, 5) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
     extern __shared__ __align__(16) unsigned char dxl_smem[];
     bf16_t *g_s = reinterpret_cast<bf16_t *>(dxl_smem);      // [32][LDT] dy tile
     bf16_t *x_s = g_s + 32 * kDxlLDT;                        // [32][LDT] x tile
-    float *o_s = reinterpret_cast<float *>(x_s + 32 * kDxlLDT);  // [32][LDO]
-    float *hp_s = o_s + 32 * kDxlLDO;                        // [32] Hpre (0 beyond n)
+    float *o_s = reinterpret_cast<float *>(dxl_smem);        // [32][LDO], in the two tiles once they are consumed
+    float *hp_s = reinterpret_cast<float *>(x_s + 32 * kDxlLDT);  // [32] Hpre (0 beyond n)
+    float *ho_s = hp_s + 32;                                 // [32] Hpost (0 beyond n)
+    static_assert(sizeof(float) * 32 * kDxlLDO <= sizeof(bf16_t) * 2 * 32 * kDxlLDT, "output tile must fit in the input tiles");
     const int b = blockIdx.y, cb0 = blockIdx.x * kDxlCB, n = a.n, C = a.C, tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6, row = lane & 31, kh = lane >> 5;
     const bool inject = a.f_inject != nullptr;
@@ -237,25 +239,21 @@ __global__ __launch_bounds__(256, 4) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
     }
     // ---- A operands from the coefficients (overlaps the tile loads) -----------------------------
     // lane (row j, kg): M^T[j][k] = M[k][j], k = ks*16 + kg*8 + i
-    bf16x8_t mth[2], mtl[2], hoh[2], hol[2], hph[2], hpl[2];
+    bf16x8_t mth[2], mtl[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
-        float mv[8], hov[8], hpv[8];
+        float mv[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const int k = ks * 16 + kh * 8 + i;
             const bool ok = k < n && row < n;
             const float m = M[ok ? k * n + row : 0];
-            const float ho = Hpost[k < n ? k : 0], hp = Hpre[k < n ? k : 0];
             mv[i] = ok ? m : 0.f;
-            hov[i] = (k < n && row == 0) ? ho : 0.f;
-            hpv[i] = (k < n && row == 0) ? hp : 0.f;
         }
         split_frag(mv, mth[ks], mtl[ks]);
-        split_frag(hov, hoh[ks], hol[ks]);
-        split_frag(hpv, hph[ks], hpl[ks]);
     }
     if (tid < 32) hp_s[tid] = tid < n ? Hpre[tid] : 0.f;
+    else if (tid < 64) ho_s[tid - 32] = tid - 32 < n ? Hpost[tid - 32] : 0.f;
     const float qinv = inject ? 0.f : 1.0f / a.q[b];
     const float k2 = inject ? 0.f : a.s1[b] * qinv * qinv * qinv / (float)C;
     const float cx = a.cx ? a.cx[b] : 0.f;
@@ -270,27 +268,33 @@ __global__ __launch_bounds__(256, 4) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
     }
     __syncthreads();
 
-    // ---- matrix cores -------------------------------------------------------------------------------
-    f32x16_t o, dfa, aa;
+    // ---- matrix cores: O = M^T dy ------------------------------------------------------------------
+    f32x16_t o;
 #pragma unroll
-    for (int i = 0; i < 16; i++) { o[i] = 0.f; dfa[i] = 0.f; aa[i] = 0.f; }
+    for (int i = 0; i < 16; i++) o[i] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
         const bf16x8_t gf = dxl_frag_t(g_s, ks * 16, wave * 32, lane);
-        const bf16x8_t xf = dxl_frag_t(x_s, ks * 16, wave * 32, lane);
         o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(mth[ks], gf, o, 0, 0, 0);
         o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(mtl[ks], gf, o, 0, 0, 0);
-        dfa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hoh[ks], gf, dfa, 0, 0, 0);
-        dfa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hol[ks], gf, dfa, 0, 0, 0);
-        if (!inject) {
-            aa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hph[ks], xf, aa, 0, 0, 0);
-            aa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hpl[ks], xf, aa, 0, 0, 0);
+    }
+    // df = Hpost^T dy and a = Hpre^T x of this lane's channel on the VALU, straight from the tiles
+    // (fp32 coefficients; each half of the wave sums 16 streams): as matrix-core products they
+    // cost 32 more operand registers, and this kernel needs five workgroups per CU to have its
+    // whole grid resident at once
+    float dfp = 0.f, ap = 0.f;
+    {
+        const bf16_t *gp = g_s + (size_t)(kh * 16) * kDxlLDT + wave * 32 + row;
+        const bf16_t *xp = x_s + (size_t)(kh * 16) * kDxlLDT + wave * 32 + row;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            dfp += ho_s[kh * 16 + i] * bf16_to_f32(gp[i * kDxlLDT]);
+            if (!inject) ap += hp_s[kh * 16 + i] * bf16_to_f32(xp[i * kDxlLDT]);
         }
     }
-    // accumulator layout: column = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4;
-    // row 0 of dfa / aa (register 0 of the lower half) is df / a of this lane's channel
-    const float dfc = bcast_lower32(dfa[0]);
-    const float ac = bcast_lower32(aa[0]);
+    const float dfc = xor32_add(dfp);
+    const float ac = xor32_add(ap);
+    __syncthreads();  // the tiles are consumed: their memory becomes the output tile
     const float da = inject ? 0.f : dfc * wv * qinv - ac * k2;
     if (kh == 0 && cw < C) {
         if (inject) {
@@ -338,7 +342,7 @@ __global__ __launch_bounds__(256, 4) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
 }
 
 static hipError_t launch_large_mfma(const BwdDxArgs &a, hipStream_t stream) {
-    const size_t smem = sizeof(bf16_t) * 2 * 32 * kDxlLDT + sizeof(float) * (32 * kDxlLDO + 32);
+    const size_t smem = sizeof(bf16_t) * 2 * 32 * kDxlLDT + sizeof(float) * 64;
     mix_bwd_dx_large_kernel<<<dim3((a.C + kDxlCB - 1) / kDxlCB, a.B), 256, smem, stream>>>(a);
     return hipGetLastError();
 }
