@@ -199,13 +199,6 @@ __device__ __forceinline__ bf16x8_t dxl_frag_t(const bf16_t *tile, int k0, int c
     return __builtin_bit_cast(bf16x8_t, make_uint4(wv[0], wv[1], wv[2], wv[3]));
 }
 
-// the value of lane (lane & 31) in both halves of the wave
-__device__ __forceinline__ float bcast_lower32(float v) {
-    const unsigned b = __float_as_uint(v);
-    const auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
-    return __uint_as_float(r[0]);
-}
-
 __global__ __launch_bounds__(256, 5) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
     extern __shared__ __align__(16) unsigned char dxl_smem[];
     bf16_t *g_s = reinterpret_cast<bf16_t *>(dxl_smem);      // [32][LDT] dy tile
