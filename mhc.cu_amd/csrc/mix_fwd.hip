@@ -325,7 +325,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
             for (int i = 0; i < NP; i++) xr[k][i].get(xv[k][i]);  // streams >= n meet zero coefficients
     }
-    float av[CPT][V];
+    float av[LEAN ? 1 : CPT][V];  // LEAN recomputes the aggregate in step 4 instead of keeping it
     float qinv = 1.0f;
     if (!inject) {
         float ssq = 0.f;
@@ -344,7 +344,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             }
 #pragma unroll
             for (int v = 0; v < V; v++) {
-                av[k][v] = s_a[v];
+                if constexpr (!LEAN) av[k][v] = s_a[v];
                 ssq += live ? s_a[v] * s_a[v] : 0.f;
             }
         }
@@ -367,8 +367,22 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             if (inject) {
                 fr[k].get(f);
             } else {
+                if constexpr (LEAN) {
 #pragma unroll
-                for (int v = 0; v < V; v++) f[v] = av[k][v] * qinv * load_w(a.w, a.w_bf16, c + v);
+                    for (int v = 0; v < V; v++) f[v] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < NP; i++) {
+                        float t[V];
+                        xr[k][i].get(t);
+#pragma unroll
+                        for (int v = 0; v < V; v++) f[v] += hpre[i] * t[v];
+                    }
+#pragma unroll
+                    for (int v = 0; v < V; v++) f[v] = f[v] * qinv * load_w(a.w, a.w_bf16, c + v);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < V; v++) f[v] = av[k][v] * qinv * load_w(a.w, a.w_bf16, c + v);
+                }
             }
 #pragma unroll
             for (int i = 0; i < NP; i++) {
