@@ -7,8 +7,8 @@
 //
 // Two kernels:
 //   proj_fwd_mfma_kernel    x and phi both bf16, C % 8 == 0: v_mfma_f32_32x32x16_bf16 tiles
-//                           (32 samples x 32 projection rows), operands loaded straight from
-//                           global memory in MFMA layout (16-byte loads, no LDS staging).
+//                           (32 samples x 32 projection rows), operands fetched row-contiguously
+//                           through a wave-private LDS tile.
 //   proj_fwd_generic_kernel any dtype / any C: fp32 FMA, exact products (the fp32 parity tier).
 #include "launchers.h"
 #include "mhc_common.h"
@@ -70,6 +70,8 @@ __global__ __launch_bounds__(256) void proj_fwd_generic_kernel(const TX *__restr
 // the four partial tiles are summed through LDS, so one partial per workgroup reaches memory.
 // grid.x = sample_tiles * KS (sample tile fastest), grid.y = groups of NT projection tiles.
 // --------------------------------------------------------------------------------------------
+constexpr int kNarrowPitch = 72;  // LDS row of a 64-element chunk: 128 data bytes + 16 pad (bf16 elements)
+
 template <int NT>
 __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__restrict__ x,
                                                             const bf16_t *__restrict__ phi,
@@ -77,7 +79,7 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
                                                             float *__restrict__ ssqpart, int B,
                                                             int D, int DP, int nC, int tiles_s,
                                                             int sub /* K per wave, multiple of 64 */) {
-    extern __shared__ float lds[];  // [3][NT*16 + 1][64]
+    extern __shared__ __align__(16) float lds[];  // per wave [(1 + NT) * 32][pitch] bf16; later [3][NT*16 + 1][64] fp32
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int st = blockIdx.x % tiles_s, ks = blockIdx.x / tiles_s;
     const int row = lane & 31, kh = lane >> 5;
@@ -85,17 +87,56 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
     const int dbase = blockIdx.y * NT * 32;
     const int kbeg = (ks * 4 + wave) * sub;
     const int kend = min(kbeg + sub, nC);
-
     const bool bvalid = b < B;
-    const uint4 *xrow = reinterpret_cast<const uint4 *>(x + (size_t)(bvalid ? b : 0) * nC);
-    const uint4 *prow[NT];
-    bool dvalid[NT];
+
+    // Global loads are row-contiguous (8 lanes per 128-byte row piece, rows lr + 8 j): the operand
+    // layout of the matrix cores has every lane on a different row, which the memory pipeline
+    // serves at a quarter of this rate.  The chunk goes through a wave-private LDS tile and comes
+    // back as fragments; no barrier is involved (a wave's LDS accesses complete in order).
+    bf16_t *cb = reinterpret_cast<bf16_t *>(lds) + (size_t)wave * (1 + NT) * 32 * kNarrowPitch;
+    const int lr = lane >> 3, seg = lane & 7;
+    const bf16_t *xrow[4];
+    const bf16_t *prow[NT][4];
+    bool xval[4], pval[NT][4];
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const int d = dbase + t * 32 + row;
-        dvalid[t] = d < D;
-        prow[t] = reinterpret_cast<const uint4 *>(phi + (size_t)(dvalid[t] ? d : 0) * nC);
+    for (int j = 0; j < 4; j++) {
+        const int bs = st * 32 + lr + 8 * j;
+        xval[j] = bs < B;
+        xrow[j] = x + (size_t)(xval[j] ? bs : 0) * nC;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int d = dbase + t * 32 + lr + 8 * j;
+            pval[t][j] = d < D;
+            prow[t][j] = phi + (size_t)(pval[t][j] ? d : 0) * nC;
+        }
     }
+    uint32_t xq[4][4], pq[NT][4][4];  // scalar words: whole-uint4 array elements can end up in scratch
+    auto fetch = [&](int k0) {
+        const int k = k0 + seg * 8;
+        const bool kv = k < kend;  // kend and k are multiples of 8
+        const int off = kv ? k : 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(xrow[j] + off), kv && xval[j]);
+            xq[j][0] = v.x; xq[j][1] = v.y; xq[j][2] = v.z; xq[j][3] = v.w;
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const uint4 p = load16_masked(reinterpret_cast<const uint4 *>(prow[t][j] + off), kv && pval[t][j]);
+                pq[t][j][0] = p.x; pq[t][j][1] = p.y; pq[t][j][2] = p.z; pq[t][j][3] = p.w;
+            }
+        }
+    };
+    auto park = [&]() {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            *reinterpret_cast<uint4 *>(cb + (size_t)(lr + 8 * j) * kNarrowPitch + seg * 8) =
+                make_uint4(xq[j][0], xq[j][1], xq[j][2], xq[j][3]);
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+                *reinterpret_cast<uint4 *>(cb + (size_t)(32 + t * 32 + lr + 8 * j) * kNarrowPitch + seg * 8) =
+                    make_uint4(pq[t][j][0], pq[t][j][1], pq[t][j][2], pq[t][j][3]);
+        }
+    };
 
     f32x16_t acc[NT];
 #pragma unroll
@@ -104,29 +145,22 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
         for (int i = 0; i < 16; i++) acc[t][i] = 0.f;
     float ssq = 0.f;
 
-    constexpr int U = 4;  // k-steps in flight
-    for (int k0 = kbeg; k0 < kend; k0 += 16 * U) {
-        uint4 av[U], bv[U][NT];
+    if (kbeg < kend) fetch(kbeg);
+    for (int k0 = kbeg; k0 < kend; k0 += 64) {
+        park();
+        if (k0 + 64 < kend) fetch(k0 + 64);  // in flight while this chunk is multiplied
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            // each lane walks 8*U contiguous elements per outer step (one 64-byte segment of a
-            // 128-byte line for U = 4); A and B use the same k grouping, which is all MFMA needs
-            const int k = k0 + kh * (8 * U) + u * 8;
-            const bool kv = k < kend;  // kend and k are multiples of 8
-            const int off = kv ? (k >> 3) : 0;
-            av[u] = load16_masked(xrow + off, kv && bvalid);
+        for (int u = 0; u < 4; u++) {
+            // fragment of k-step u: lane (row, kh) holds elements u*16 + kh*8 .. +8 of its row
+            const uint4 av = *reinterpret_cast<const uint4 *>(cb + (size_t)row * kNarrowPitch + u * 16 + kh * 8);
+            const bf16x8_t af = __builtin_bit_cast(bf16x8_t, av);
 #pragma unroll
-            for (int t = 0; t < NT; t++) bv[u][t] = load16_masked(prow[t] + off, kv && dvalid[t]);
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const bf16x8_t af = __builtin_bit_cast(bf16x8_t, av[u]);
-#pragma unroll
-            for (int t = 0; t < NT; t++)
-                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    af, __builtin_bit_cast(bf16x8_t, bv[u][t]), acc[t], 0, 0, 0);
+            for (int t = 0; t < NT; t++) {
+                const uint4 bv = *reinterpret_cast<const uint4 *>(cb + (size_t)(32 + t * 32 + row) * kNarrowPitch + u * 16 + kh * 8);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(bf16x8_t, bv), acc[t], 0, 0, 0);
+            }
             if (blockIdx.y == 0) {
-                const uint32_t w4[4] = {av[u].x, av[u].y, av[u].z, av[u].w};
+                const uint32_t w4[4] = {av.x, av.y, av.z, av.w};
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const float lo = bf16lo_to_f32(w4[i]), hi = bf16hi_to_f32(w4[i]);
@@ -135,6 +169,7 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
             }
         }
     }
+    __syncthreads();  // every wave is done with its chunk tile: the memory becomes the cross-wave buffer
     ssq = xor32_add(ssq);  // both K halves of the row
 
     // cross-wave sum: waves 1..3 park their tiles in LDS, wave 0 adds and writes
@@ -420,7 +455,10 @@ static hipError_t launch_mfma(const void *x, const void *phi, float *Ppart, floa
     const int groups = (DP / 32 + NT - 1) / NT;
     const int sub = round_up((nC + KS * 4 - 1) / (KS * 4), 64);  // whole 128-byte lines per lane pair
     dim3 grid(tiles_s * KS, groups);
-    const size_t smem = sizeof(float) * 3 * (NT * 16 + 1) * 64;
+    const size_t smem_chunks = sizeof(bf16_t) * 4 * (1 + NT) * 32 * kNarrowPitch;
+    const size_t smem_sum = sizeof(float) * 3 * (NT * 16 + 1) * 64;
+    const size_t smem = smem_chunks > smem_sum ? smem_chunks : smem_sum;
+    if (hipError_t e = allow_dynamic_lds(&proj_fwd_mfma_kernel<NT>, smem); e != hipSuccess) return e;
     proj_fwd_mfma_kernel<NT><<<grid, 256, smem, stream>>>(static_cast<const bf16_t *>(x),
                                                            static_cast<const bf16_t *>(phi), Ppart,
                                                            ssqpart, B, D, DP, nC, tiles_s, sub);
