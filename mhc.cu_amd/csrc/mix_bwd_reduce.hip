@@ -420,11 +420,88 @@ __global__ __launch_bounds__(256) void gram_large_kernel(BwdReduceArgs a) {
         }
     };
 
-    // full k-steps (every column of the step inside C, rows 16-byte aligned): raw loads, U steps
-    // in flight, nothing conditional per lane
+    // full k-steps (every column of the step inside C, rows 16-byte aligned)
     const bool vec_ok = C % VL == 0;
     const int s_full = vec_ok ? min(s_end, C / SW) : s_begin;
-    int s = s_begin + wave;
+    int s;
+    if constexpr (kBf16) {
+        // Chunks of 4 steps (64 channels), one chunk per wave and round: the 32 rows of dy and x are
+        // fetched row-contiguously (8 lanes per 128-byte piece, rows lr + 8 j), parked in a wave-private
+        // LDS tile (no barrier: a wave's LDS accesses complete in order) and read back in operand
+        // layout, the next chunk in flight in registers.  Loading straight in operand layout has
+        // every lane on its own row, which the memory pipeline serves at a quarter of the rate.
+        constexpr int PITCH = 72;  // 128 data bytes + 16 pad per row (bf16 elements)
+        bf16_t *cb = reinterpret_cast<bf16_t *>(xw) + (size_t)wave * (2 * 32 + 1) * PITCH;  // dy rows | x rows | f
+        const int lr = lane >> 3, seg = lane & 7;
+        const bf16_t *gq_row[4], *xq_row[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const size_t rj = (size_t)(lr + 8 * j < n ? lr + 8 * j : 0) * C;  // rows >= n alias row 0
+            gq_row[j] = static_cast<const bf16_t *>(a.dy) + (size_t)b * n * C + rj;
+            xq_row[j] = static_cast<const bf16_t *>(a.x) + (size_t)b * n * C + rj;
+        }
+        const bf16_t *fq_row = static_cast<const bf16_t *>(frow);
+        uint32_t gq[4][4], xq[4][4], fq[4];
+        auto fetch = [&](int chunk) {
+            const int col = c_begin + chunk * 64 + seg * 8;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint4 g4 = *reinterpret_cast<const uint4 *>(gq_row[j] + col);
+                const uint4 x4 = *reinterpret_cast<const uint4 *>(xq_row[j] + col);
+                gq[j][0] = g4.x; gq[j][1] = g4.y; gq[j][2] = g4.z; gq[j][3] = g4.w;
+                xq[j][0] = x4.x; xq[j][1] = x4.y; xq[j][2] = x4.z; xq[j][3] = x4.w;
+            }
+            if (inject) {
+                const uint4 f4 = *reinterpret_cast<const uint4 *>(fq_row + col);
+                fq[0] = f4.x; fq[1] = f4.y; fq[2] = f4.z; fq[3] = f4.w;
+            }
+        };
+        auto park = [&]() {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                *reinterpret_cast<uint4 *>(cb + (size_t)(lr + 8 * j) * PITCH + seg * 8) = make_uint4(gq[j][0], gq[j][1], gq[j][2], gq[j][3]);
+                *reinterpret_cast<uint4 *>(cb + (size_t)(32 + lr + 8 * j) * PITCH + seg * 8) = make_uint4(xq[j][0], xq[j][1], xq[j][2], xq[j][3]);
+            }
+            if (inject && lr == 0) *reinterpret_cast<uint4 *>(cb + (size_t)64 * PITCH + seg * 8) = make_uint4(fq[0], fq[1], fq[2], fq[3]);
+        };
+        const int nchunks = (s_full - s_begin) / 4;
+        if (wave < nchunks) fetch(wave);
+        for (int chunk = wave; chunk < nchunks; chunk += 4) {
+            park();
+            if (chunk + 4 < nchunks) fetch(chunk + 4);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                RawVec<TG, VL> gr;
+                RawVec<TX, VL> xr;
+                const uint4 g4 = *reinterpret_cast<const uint4 *>(cb + (size_t)row * PITCH + u * 16 + kh * 8);
+                const uint4 x4 = *reinterpret_cast<const uint4 *>(cb + (size_t)(32 + row) * PITCH + u * 16 + kh * 8);
+                gr.w[0] = g4.x; gr.w[1] = g4.y; gr.w[2] = g4.z; gr.w[3] = g4.w;
+                xr.w[0] = x4.x; xr.w[1] = x4.y; xr.w[2] = x4.z; xr.w[3] = x4.w;
+                if (inject) {
+                    // B operand = [f; 0; ...]: only lane row 0 carries f, column 0 of the product is dy . f
+                    const uint4 f4 = *reinterpret_cast<const uint4 *>(cb + (size_t)64 * PITCH + u * 16 + kh * 8);
+                    const bf16x8_t gb = __builtin_bit_cast(bf16x8_t, g4);
+                    const bf16x8_t xb = __builtin_bit_cast(bf16x8_t, x4);
+                    const bf16x8_t fb = __builtin_bit_cast(
+                        bf16x8_t, make_uint4(row == 0 ? f4.x : 0u, row == 0 ? f4.y : 0u, row == 0 ? f4.z : 0u, row == 0 ? f4.w : 0u));
+                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb, xb, acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb, fb, acc[1], 0, 0, 0);
+                } else {
+                    const int cc = chunk * 64 + u * 16 + kh * 8;  // relative to c_begin
+                    float g[VL], x[VL], gw[VL];
+                    gr.get(g);
+                    xr.get(x);
+#pragma unroll
+                    for (int i = 0; i < VL; i++) gw[i] = g[i] * w_s[cc + i];
+                    mfma3(g, x, gw, gr, xr, true);
+                }
+            }
+        }
+        s = s_begin + nchunks * 4 + wave;
+        __syncthreads();  // the chunk tiles live in the cross-wave scratch used below
+    } else {
+    // raw loads in operand layout, U steps in flight, nothing conditional per lane
+    s = s_begin + wave;
     for (; s + 4 * (U - 1) < s_full; s += 4 * U) {
         RawVec<TG, VL> gr[U];
         RawVec<TX, VL> xr[U], fr[U];
@@ -469,6 +546,7 @@ __global__ __launch_bounds__(256) void gram_large_kernel(BwdReduceArgs a) {
                 mfma3(g, x, gw, gr[u], xr[u], true);
             }
         }
+    }
     }
     // remaining steps of this wave (fewer than U full ones, a ragged last step, unaligned rows):
     // element-wise masked loads, fp32 operands rounded where the bf16 instruction needs them
@@ -751,7 +829,9 @@ static hipError_t launch_large(const BwdReduceArgs &a, hipStream_t stream) {
     constexpr int SW = kBf16 ? 16 : 8;
     const int nsteps = (a.C + SW - 1) / SW;
     const int spp = (nsteps + a.parts - 1) / a.parts;
-    const size_t smem1 = sizeof(float) * ((size_t)spp * SW + 3 * kGramMats * 16 * 64);
+    // weights of the part | cross-wave scratch, which first holds the four waves' chunk tiles (bf16 path)
+    const size_t scratch = sizeof(float) * 3 * kGramMats * 16 * 64, tiles = sizeof(bf16_t) * 4 * (2 * 32 + 1) * 72;
+    const size_t smem1 = sizeof(float) * (size_t)spp * SW + (kBf16 && tiles > scratch ? tiles : scratch);
     if (smem1 > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gram_large_kernel<TG, TX>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1);
