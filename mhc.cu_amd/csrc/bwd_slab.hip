@@ -106,41 +106,6 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
     const int cth = c0 + ch * 8;
     const bool cok = cth < C;  // C % 8 == 0: a chunk is entirely inside or outside
 
-    // ---- phi slab -> LDS (as [32 d][KW]) -> this wave's transposed fragments ----------------
-    // wave w owns N-tiles t = 2w, 2w+1; tile t covers stream t/2, channels c0 + (t%2)*32 .. +32
-    bf16_t *phi_s = reinterpret_cast<bf16_t *>(dxf_s);  // staged in the (not yet used) fp32 tile
-    for (int e = tid; e < 32 * (kSlabKW / 8); e += 256) {
-        const int d = e / (kSlabKW / 8), chunk = e % (kSlabKW / 8);
-        const int j = chunk / (kSlabCW / 8), c = c0 + (chunk % (kSlabCW / 8)) * 8;
-        const bool ok = d < D && j < n && c < C;
-        const uint4 v = load16_masked(
-            reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * nC + (size_t)j * C + c : 0)), ok);
-        *reinterpret_cast<uint4 *>(phi_s + (size_t)d * kSlabLDX + chunk * 8) = v;
-    }
-    __syncthreads();
-    bf16x8_t phif[2][2];
-#pragma unroll
-    for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int ks = 0; ks < 2; ks++) phif[t][ks] = slab_frag_t(phi_s, ks * 16, (2 * wave + t) * 32, lane);
-    __syncthreads();  // fragments are in registers; the region becomes dxf_s
-
-    f32x16_t acc[2];
-#pragma unroll
-    for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) acc[t][i] = 0.f;
-    float usum[8];
-#pragma unroll
-    for (int v = 0; v < 8; v++) usum[v] = 0.f;
-    float dtsum = 0.f;  // slab 0 only: thread (col = tid & 31, row group = tid >> 5)
-
-    float wv[8];
-#pragma unroll
-    for (int v = 0; v < 8; v++)
-        wv[v] = (cok && !inject) ? (a.w_bf16 ? bf16_to_f32(static_cast<const bf16_t *>(a.w)[cth + v])
-                                              : static_cast<const float *>(a.w)[cth + v]) : 0.f;
-
     // ---- software pipeline: the loads of tile t+1 are issued before the VALU phase of tile t ----
     // raw tile data of this thread (sample slot bl, 8 channels, all streams) and the MFMA operands
     // that come straight from global memory (dP^T hi/lo rows d, dP rows b)
@@ -166,8 +131,55 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
             t.gr[j].load(gb + so);
         }
     };
+    // ---- phi slab -> LDS (as [32 d][KW]) -> this wave's transposed fragments ----------------
+    // wave w owns N-tiles t = 2w, 2w+1; tile t covers stream t/2, channels c0 + (t%2)*32 .. +32
+    // The slab is requested first and the first tile right behind it, so that the tile's round
+    // trip runs under the staging of the slab.
+    bf16_t *phi_s = reinterpret_cast<bf16_t *>(dxf_s);  // staged in the (not yet used) fp32 tile
+    constexpr int kPhiIters = 32 * (kSlabKW / 8) / 256;
+    static_assert(32 * (kSlabKW / 8) % 256 == 0, "phi slab staging assumes whole rounds of 256 threads");
+    uint4 phir[kPhiIters];
+#pragma unroll
+    for (int i = 0; i < kPhiIters; i++) {
+        const int e = tid + i * 256;
+        const int d = e / (kSlabKW / 8), chunk = e % (kSlabKW / 8);
+        const int j = chunk / (kSlabCW / 8), c = c0 + (chunk % (kSlabCW / 8)) * 8;
+        const bool ok = d < D && j < n && c < C;
+        phir[i] = load16_masked(
+            reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * nC + (size_t)j * C + c : 0)), ok);
+    }
     TileRegs cur, nxt;
     if (b_begin < b_end) load_tile(b_begin, cur);
+#pragma unroll
+    for (int i = 0; i < kPhiIters; i++) {
+        const int e = tid + i * 256;
+        const int d = e / (kSlabKW / 8), chunk = e % (kSlabKW / 8);
+        *reinterpret_cast<uint4 *>(phi_s + (size_t)d * kSlabLDX + chunk * 8) = phir[i];
+    }
+    __syncthreads();
+    bf16x8_t phif[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) phif[t][ks] = slab_frag_t(phi_s, ks * 16, (2 * wave + t) * 32, lane);
+    __syncthreads();  // fragments are in registers; the region becomes dxf_s
+
+    f32x16_t acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[t][i] = 0.f;
+    float usum[8];
+#pragma unroll
+    for (int v = 0; v < 8; v++) usum[v] = 0.f;
+    float dtsum = 0.f;  // slab 0 only: thread (col = tid & 31, row group = tid >> 5)
+
+    float wv[8];
+#pragma unroll
+    for (int v = 0; v < 8; v++)
+        wv[v] = (cok && !inject) ? (a.w_bf16 ? bf16_to_f32(static_cast<const bf16_t *>(a.w)[cth + v])
+                                              : static_cast<const float *>(a.w)[cth + v]) : 0.f;
+
 
     MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 0, pclk);
     for (int sb = b_begin; sb < b_end; sb += 32) {
