@@ -255,10 +255,11 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
 // the tail of a bandwidth-bound workgroup.  Input: the raw channel sums written by the kernel
 // above ([B][parts][K], K = NP*NP + 3*NP + 1: dM | dHpost | A1 | A2 | s1).
 // =============================================================================================
-template <int NP, bool PRECISE>
+template <int NP, bool PRECISE, bool GRAM = false>
 __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
     using SK = SkSmall<NP>;
-    constexpr int K = NP * NP + 3 * NP + 1;
+    static_assert(!GRAM || NP == 4, "Gram input: 4x4 matrices only");
+    constexpr int K = GRAM ? 3 * 16 : NP * NP + 3 * NP + 1;
     extern __shared__ float sc[];  // Sinkhorn denominators, SK::scaling_floats(T)
     const int tid = threadIdx.x, g = tid & 15;
     const int b = blockIdx.x * 4 + (tid >> 4);
@@ -271,18 +272,44 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
     float dMe[SK::EPL], tpost = 0.f, tA1 = 0.f, tA2 = 0.f, s1 = 0.f;
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) dMe[e] = 0.f;
-    for (int p = 0; p < a.parts; p++) {
-        const float *rp = raw + (size_t)p * K;
+    const int gc = g < n ? g : 0;  // lanes beyond n alias entry 0 (never used): no branch around loads
+    const float qinv = inject ? 0.f : 1.0f / a.q[b];
+    if constexpr (GRAM) {
+        // input: dM | W1 | XX (4 x 4 each); lane (r0, c0) takes its element of each and the mirrored
+        // element of W1, so that every sum below runs down a column and lands in lanes 0 .. n-1:
+        //   dHpost[c] = sum_r Hpre[r] W1[c][r] / q        A1[c] = sum_r Hpost[r] W1[r][c]
+        //   A2[c] = sum_r Hpre[r] XX[r][c]                s1 = sum_c Hpost[c] (sum_r Hpre[r] W1[c][r])
+        float w1 = 0.f, w1t = 0.f, xx = 0.f;
+        for (int p = 0; p < a.parts; p++) {
+            const float *rp = raw + (size_t)p * K;
+            dMe[0] += rp[r0 * 4 + c0];
+            w1 += rp[16 + r0 * 4 + c0];
+            w1t += rp[16 + c0 * 4 + r0];
+            xx += rp[32 + r0 * 4 + c0];
+        }
+        const float hpre_r = r0 < n ? a.Hpre[(size_t)b * n + r0] : 0.f;
+        const float hpost_r = r0 < n ? a.Hpost[(size_t)b * n + r0] : 0.f;
+        if (inject) {
+            tpost = SK::col_allreduce(r0 == 0 ? w1t : 0.f);  // W1 = dy [f; 0; 0; 0]^T: column 0
+        } else {
+            const float hw = SK::col_allreduce(hpre_r * w1t);
+            tpost = hw * qinv;
+            tA1 = SK::col_allreduce(hpost_r * w1);
+            tA2 = SK::col_allreduce(hpre_r * xx);
+            s1 = row16_allreduce(g < n ? a.Hpost[(size_t)b * n + gc] * hw : 0.f);
+        }
+    } else {
+        for (int p = 0; p < a.parts; p++) {
+            const float *rp = raw + (size_t)p * K;
 #pragma unroll
-        for (int e = 0; e < SK::EPL; e++) dMe[e] += rp[r0 * NP + c0 + e];
-        const int gc = g < n ? g : 0;  // lanes beyond n alias entry 0 (never used): no branch around loads
-        tpost += rp[NP * NP + gc]; tA1 += rp[NP * NP + NP + gc]; tA2 += rp[NP * NP + 2 * NP + gc];
-        s1 += rp[K - 1];
+            for (int e = 0; e < SK::EPL; e++) dMe[e] += rp[r0 * NP + c0 + e];
+            tpost += rp[NP * NP + gc]; tA1 += rp[NP * NP + NP + gc]; tA2 += rp[NP * NP + 2 * NP + gc];
+            s1 += rp[K - 1];
+        }
     }
     const float *Pb = a.P + (size_t)b * D;
     const float al0 = a.alpha[0], al1 = a.alpha[1], al2 = a.alpha[2];
     const float rinv = 1.0f / a.r[b];
-    const float qinv = inject ? 0.f : 1.0f / a.q[b];
     float pres[SK::EPL], bres[SK::EPL];
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
@@ -333,6 +360,121 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
         a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv / (float)(n * C);
     }
     dpw.pad(D, g, 16);
+}
+
+// =============================================================================================
+// n <= 4, dynamic H, dy and x both bf16: the channel sums as three 4x4 Gram matrices per sample
+//   dM = dy x^T        W1 = dy diag(w) x^T        XX = x x^T
+// (the same three products as for n > 8; the coefficient kernel forms dHpost, A1, A2, s1 from them)
+// on v_mfma_f32_4x4x4_16b_bf16: one instruction is 16 independent 4x4x4 products, block = lane / 4,
+// a lane holding four consecutive channels of stream lane % 4 for both operands - which is how the
+// data lies in memory, so the operands are the loaded words themselves.  A step of a wave covers
+// 128 channels of all four streams (16 bytes per lane from dy and from x); nothing is unpacked
+// except dy for the product with w, and the kernel needs a third of the registers of the VALU
+// version, which is what lets enough waves be resident to keep the loads flowing.
+// With an injected f, W1 = dy [f; 0; 0; 0]^T (its column 0 is dHpost) and XX is not needed.
+// Output: raw[b][part][m][i][j], m = dM | W1 | XX.
+// =============================================================================================
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+constexpr int kGramSmallFloats = 3 * 16;
+constexpr int kGramSmallUnroll = 2;  // steps of a wave in flight
+enum { kGramInject = 0, kGramWBf16 = 1, kGramWF32 = 2 };
+
+__device__ __forceinline__ bf16x4_t bf16x4_of(uint32_t w0, uint32_t w1) {
+    return __builtin_bit_cast(bf16x4_t, make_uint2(w0, w1));
+}
+
+template <int WMODE>
+__global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
+    __shared__ float slot_s[kGramSmallFloats * 16];  // one slot per 16-lane row of the workgroup
+    const int b = blockIdx.x, part = blockIdx.y, n = a.n, C = a.C;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int blk = lane >> 2, i = lane & 3;
+    constexpr bool inject = WMODE == kGramInject;
+    const int nsteps = (C + 127) / 128, spp = (nsteps + a.parts - 1) / a.parts;
+    const int s_begin = part * spp, s_end = min(nsteps, s_begin + spp);
+    const size_t row = (size_t)b * n * C + (size_t)(i < n ? i : 0) * C;  // streams >= n: masked below
+    const bf16_t *gb = static_cast<const bf16_t *>(a.dy) + row;
+    const bf16_t *xb = static_cast<const bf16_t *>(a.x) + row;
+    const bf16_t *fb = inject ? static_cast<const bf16_t *>(a.f_inject) + (size_t)b * C : nullptr;
+
+    f32x4_t acc[3];
+#pragma unroll
+    for (int m = 0; m < 3; m++) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int s0 = s_begin + wave; s0 < s_end; s0 += 4 * kGramSmallUnroll) {
+        uint4 gr[kGramSmallUnroll], xr[kGramSmallUnroll], fr[kGramSmallUnroll];
+        RawVec<bf16_t, 8> wb[kGramSmallUnroll];
+        RawVec<float, 8> wf[kGramSmallUnroll];
+#pragma unroll
+        for (int u = 0; u < kGramSmallUnroll; u++) {
+            const int c = (s0 + 4 * u) * 128 + blk * 8;
+            const bool in = s0 + 4 * u < s_end && c < C;  // C % 8 == 0: a chunk is inside or outside
+            const bool ok = in && i < n;
+            const int cc = in ? c : 0;
+            gr[u] = load16_masked(reinterpret_cast<const uint4 *>(gb + cc), ok);
+            xr[u] = load16_masked(reinterpret_cast<const uint4 *>(xb + cc), ok);
+            if constexpr (inject) fr[u] = load16_masked(reinterpret_cast<const uint4 *>(fb + cc), in && i == 0);
+            else if constexpr (WMODE == kGramWBf16) wb[u].load(static_cast<const bf16_t *>(a.w) + cc);
+            else wf[u].load(static_cast<const float *>(a.w) + cc);
+        }
+#pragma unroll
+        for (int u = 0; u < kGramSmallUnroll; u++) {
+            const bf16x4_t g0 = bf16x4_of(gr[u].x, gr[u].y), g1 = bf16x4_of(gr[u].z, gr[u].w);
+            const bf16x4_t x0 = bf16x4_of(xr[u].x, xr[u].y), x1 = bf16x4_of(xr[u].z, xr[u].w);
+            acc[0] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(g0, x0, acc[0], 0, 0, 0);
+            acc[0] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(g1, x1, acc[0], 0, 0, 0);
+            if constexpr (inject) {
+                const bf16x4_t f0 = bf16x4_of(fr[u].x, fr[u].y), f1 = bf16x4_of(fr[u].z, fr[u].w);
+                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(g0, f0, acc[1], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(g1, f1, acc[1], 0, 0, 0);
+            } else {
+                // dy * w as a bf16 pair (rounded value + remainder): dHpre is a difference of two
+                // sums built on W1, a single rounding of the products is not enough for it
+                float gv[8], wv[8];
+                if constexpr (WMODE == kGramWBf16) wb[u].get(wv);
+                else wf[u].get(wv);
+                gv[0] = bf16lo_to_f32(gr[u].x); gv[1] = bf16hi_to_f32(gr[u].x);
+                gv[2] = bf16lo_to_f32(gr[u].y); gv[3] = bf16hi_to_f32(gr[u].y);
+                gv[4] = bf16lo_to_f32(gr[u].z); gv[5] = bf16hi_to_f32(gr[u].z);
+                gv[6] = bf16lo_to_f32(gr[u].w); gv[7] = bf16hi_to_f32(gr[u].w);
+                uint32_t hw[4], lw[4];
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const float p0 = gv[2 * k] * wv[2 * k], p1 = gv[2 * k + 1] * wv[2 * k + 1];
+                    hw[k] = pack_bf16x2(p0, p1);
+                    lw[k] = pack_bf16x2(p0 - bf16lo_to_f32(hw[k]), p1 - bf16hi_to_f32(hw[k]));
+                }
+                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(bf16x4_of(hw[0], hw[1]), x0, acc[1], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(bf16x4_of(hw[2], hw[3]), x1, acc[1], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(bf16x4_of(lw[0], lw[1]), x0, acc[1], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(bf16x4_of(lw[2], lw[3]), x1, acc[1], 0, 0, 0);
+                acc[2] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(x0, x0, acc[2], 0, 0, 0);
+                acc[2] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(x1, x1, acc[2], 0, 0, 0);
+            }
+        }
+    }
+
+    // Lane (block, j) holds column j of its block's products, register = row.  Sum over the four
+    // blocks of a 16-lane row with DPP, one LDS slot per row, then 48 lanes finish.
+    const int slot = tid >> 4;
+#pragma unroll
+    for (int m = 0; m < 3; m++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            float v = acc[m][r];
+            v += dpp_mov<kDppRowRor4>(v);
+            v += dpp_mov<kDppRowRor8>(v);
+            if ((tid & 15) < 4) slot_s[(m * 16 + r * 4 + (tid & 3)) * 16 + slot] = v;
+        }
+    __syncthreads();
+    if (tid < kGramSmallFloats) {
+        float v = 0.f;
+#pragma unroll
+        for (int sl = 0; sl < 16; sl++) v += slot_s[tid * 16 + sl];
+        a.raw[((size_t)b * a.parts + part) * kGramSmallFloats + tid] = v;
+    }
 }
 
 // =============================================================================================
@@ -790,8 +932,33 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
 // =============================================================================================
 // launch
 // =============================================================================================
+// n <= 4, dynamic H, bf16 dy and x, rows 16-byte aligned: Gram matrices on the matrix cores.
+static bool gram_small_supported(const BwdReduceArgs &a, bool both_bf16) {
+    return both_bf16 && a.raw != nullptr && a.n <= 4 && a.C % 8 == 0;
+}
+
+// Column parts of gram_small_kernel: never more than bwd_reduce_parts(), which sizes `raw`.
+static int gram_small_parts(int B, int C) { return C >= 1024 && B < 1024 ? 2 : 1; }
+
+static hipError_t launch_gram_small(BwdReduceArgs a, hipStream_t stream) {
+    a.parts = gram_small_parts(a.B, a.C);
+    const dim3 grid(a.B, a.parts);
+    if (a.f_inject) gram_small_kernel<kGramInject><<<grid, 256, 0, stream>>>(a);
+    else if (a.w_bf16) gram_small_kernel<kGramWBf16><<<grid, 256, 0, stream>>>(a);
+    else gram_small_kernel<kGramWF32><<<grid, 256, 0, stream>>>(a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const size_t smem = sizeof(float) * SkSmall<4>::scaling_floats(a.T);
+    e = allow_dynamic_lds(&coef_bwd_small_kernel<4, false, true>, smem);
+    if (e != hipSuccess) return e;
+    coef_bwd_small_kernel<4, false, true><<<(a.B + 3) / 4, 64, smem, stream>>>(a);
+    return hipGetLastError();
+}
+
 template <typename TG, typename TX, int NP, int V>
 static hipError_t launch_small(const BwdReduceArgs &a, hipStream_t stream) {
+    if constexpr (NP == 4 && std::is_same<TG, bf16_t>::value && std::is_same<TX, bf16_t>::value)
+        if (gram_small_supported(a, true)) return launch_gram_small(a, stream);
     const int nch = (a.C / V + a.parts - 1) / a.parts;  // chunks per column part
     // every thread gets the same number of chunks (whole 16-lane rows: the reduction works on them)
     const int rounds = (nch + 255) / 256;

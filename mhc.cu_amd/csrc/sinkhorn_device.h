@@ -52,23 +52,23 @@ template <int NP> struct SkSmall {
     template <bool PRECISE = false>
     __device__ static __forceinline__ void forward(float (&m)[EPL], int g, int n, int T, float eps,
                                                    float *sc, int lane) {
-        const bool rv = row(g) < n;
-        bool cv[EPL];
+        // rows and columns beyond n hold zeros: their denominator is made 1 (not eps, which may be
+        // 0) by the constant that is added, so the dependent chain carries no select
+        const float eps_r = row(g) < n ? eps : 1.0f;
+        float eps_c[EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; e++) cv[e] = col0(g) + e < n;
+        for (int e = 0; e < EPL; e++) eps_c[e] = col0(g) + e < n ? eps : 1.0f;
         for (int t = 0; t < T; t++) {
             float rs = 0.f;
 #pragma unroll
             for (int e = 0; e < EPL; e++) rs += m[e];
-            rs = row_allreduce(rs) + eps;
-            rs = rv ? rs : 1.0f;
+            rs = row_allreduce(rs) + eps_r;
             const float rinv = PRECISE ? 1.0f / rs : fast_rcp(rs);
             if (sc) sc[(t * kRec) * kWave + lane] = rs;
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
                 m[e] = PRECISE ? m[e] / rs : m[e] * rinv;
-                float cs = col_allreduce(m[e]) + eps;
-                cs = cv[e] ? cs : 1.0f;
+                const float cs = col_allreduce(m[e]) + eps_c[e];
                 if (sc) sc[(t * kRec + 1 + e) * kWave + lane] = cs;
                 m[e] = PRECISE ? m[e] / cs : m[e] * fast_rcp(cs);
             }
