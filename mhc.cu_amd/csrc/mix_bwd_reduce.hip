@@ -258,8 +258,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
 template <int NP, bool PRECISE, bool GRAM = false>
 __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
     using SK = SkSmall<NP>;
-    static_assert(!GRAM || NP == 4, "Gram input: 4x4 matrices only");
-    constexpr int K = GRAM ? 3 * 16 : NP * NP + 3 * NP + 1;
+    constexpr int K = GRAM ? 3 * NP * NP : NP * NP + 3 * NP + 1;
     extern __shared__ float sc[];  // Sinkhorn denominators, SK::scaling_floats(T)
     const int tid = threadIdx.x, g = tid & 15;
     const int b = blockIdx.x * 4 + (tid >> 4);
@@ -275,27 +274,45 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
     const int gc = g < n ? g : 0;  // lanes beyond n alias entry 0 (never used): no branch around loads
     const float qinv = inject ? 0.f : 1.0f / a.q[b];
     if constexpr (GRAM) {
-        // input: dM | W1 | XX (4 x 4 each); lane (r0, c0) takes its element of each and the mirrored
-        // element of W1, so that every sum below runs down a column and lands in lanes 0 .. n-1:
+        // input: dM | W1 | XX (NP x NP each); lane (r0, c0 ..) takes its elements of each and the
+        // mirrored elements of W1, so that every sum below runs down a column:
         //   dHpost[c] = sum_r Hpre[r] W1[c][r] / q        A1[c] = sum_r Hpost[r] W1[r][c]
         //   A2[c] = sum_r Hpre[r] XX[r][c]                s1 = sum_c Hpost[c] (sum_r Hpre[r] W1[c][r])
-        float w1 = 0.f, w1t = 0.f, xx = 0.f;
+        // The column results are handed to lanes 0 .. n-1 through LDS (same wave: no barrier).
+        float w1[SK::EPL], w1t[SK::EPL], xx[SK::EPL];
+#pragma unroll
+        for (int e = 0; e < SK::EPL; e++) w1[e] = w1t[e] = xx[e] = 0.f;
         for (int p = 0; p < a.parts; p++) {
             const float *rp = raw + (size_t)p * K;
-            dMe[0] += rp[r0 * 4 + c0];
-            w1 += rp[16 + r0 * 4 + c0];
-            w1t += rp[16 + c0 * 4 + r0];
-            xx += rp[32 + r0 * 4 + c0];
+            float t0[SK::EPL], t1[SK::EPL], t2[SK::EPL];
+            load_vec<float, SK::EPL>(rp + r0 * NP + c0, t0);
+            load_vec<float, SK::EPL>(rp + NP * NP + r0 * NP + c0, t1);
+            load_vec<float, SK::EPL>(rp + 2 * NP * NP + r0 * NP + c0, t2);
+#pragma unroll
+            for (int e = 0; e < SK::EPL; e++) {
+                dMe[e] += t0[e]; w1[e] += t1[e]; xx[e] += t2[e];
+                w1t[e] += rp[NP * NP + (c0 + e) * NP + r0];
+            }
         }
         const float hpre_r = r0 < n ? a.Hpre[(size_t)b * n + r0] : 0.f;
         const float hpost_r = r0 < n ? a.Hpost[(size_t)b * n + r0] : 0.f;
+        // with an injected f, W1 = dy [f; 0; ...]^T and dHpost is its column 0
+        const float sel = inject ? (r0 == 0 ? 1.f : 0.f) : hpre_r;
+        float *xch = sc + SK::scaling_floats(a.T) + (tid >> 4) * 3 * NP;
+#pragma unroll
+        for (int e = 0; e < SK::EPL; e++) {
+            const float x0 = SK::col_allreduce(sel * w1t[e]);
+            const float x1 = SK::col_allreduce(hpost_r * w1[e]);
+            const float x2 = SK::col_allreduce(hpre_r * xx[e]);
+            if (r0 == 0) { xch[c0 + e] = x0; xch[NP + c0 + e] = x1; xch[2 * NP + c0 + e] = x2; }
+        }
+        const float hw = xch[gc];
         if (inject) {
-            tpost = SK::col_allreduce(r0 == 0 ? w1t : 0.f);  // W1 = dy [f; 0; 0; 0]^T: column 0
+            tpost = hw;
         } else {
-            const float hw = SK::col_allreduce(hpre_r * w1t);
             tpost = hw * qinv;
-            tA1 = SK::col_allreduce(hpost_r * w1);
-            tA2 = SK::col_allreduce(hpre_r * xx);
+            tA1 = xch[NP + gc];
+            tA2 = xch[2 * NP + gc];
             s1 = row16_allreduce(g < n ? a.Hpost[(size_t)b * n + gc] * hw : 0.f);
         }
     } else {
@@ -363,117 +380,155 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
 }
 
 // =============================================================================================
-// n <= 4, dynamic H, dy and x both bf16: the channel sums as three 4x4 Gram matrices per sample
+// n <= 8, dynamic H, dy and x both bf16: the channel sums as three n x n Gram matrices per sample
 //   dM = dy x^T        W1 = dy diag(w) x^T        XX = x x^T
 // (the same three products as for n > 8; the coefficient kernel forms dHpost, A1, A2, s1 from them)
 // on v_mfma_f32_4x4x4_16b_bf16: one instruction is 16 independent 4x4x4 products, block = lane / 4,
 // a lane holding four consecutive channels of stream lane % 4 for both operands - which is how the
-// data lies in memory, so the operands are the loaded words themselves.  A step of a wave covers
-// 128 channels of all four streams (16 bytes per lane from dy and from x); nothing is unpacked
-// except dy for the product with w, and the kernel needs a third of the registers of the VALU
+// data lies in memory, so the operands are the loaded words themselves.  For n > 4 the streams
+// form two groups of four and every Gram matrix is 2 x 2 such products.  A step of a wave covers
+// 128 channels of all streams (16 bytes per lane, stream group and tensor); nothing is unpacked
+// except dy for the product with w, and the kernel needs far fewer registers than the VALU
 // version, which is what lets enough waves be resident to keep the loads flowing.
-// With an injected f, W1 = dy [f; 0; 0; 0]^T (its column 0 is dHpost) and XX is not needed.
-// Output: raw[b][part][m][i][j], m = dM | W1 | XX.
+// With an injected f, W1 = dy [f; 0; ...]^T (its column 0 is dHpost) and XX is not needed.
+// Output: raw[b][part][m][i][j] (NP x NP each), m = dM | W1 | XX.
 // =============================================================================================
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
-constexpr int kGramSmallFloats = 3 * 16;
-constexpr int kGramSmallUnroll = 2;  // steps of a wave in flight
 enum { kGramInject = 0, kGramWBf16 = 1, kGramWF32 = 2 };
 
 __device__ __forceinline__ bf16x4_t bf16x4_of(uint32_t w0, uint32_t w1) {
     return __builtin_bit_cast(bf16x4_t, make_uint2(w0, w1));
 }
+__device__ __forceinline__ f32x4_t mfma4(bf16x4_t a, bf16x4_t b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a, b, c, 0, 0, 0);
+}
 
-template <int WMODE>
+template <int NP, int WMODE>
 __global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
-    __shared__ float slot_s[kGramSmallFloats * 16];  // one slot per 16-lane row of the workgroup
+    static_assert(NP == 4 || NP == 8, "stream groups of four");
+    constexpr int NB = NP / 4;            // stream groups
+    constexpr int U = NP == 4 ? 2 : 1;    // steps of a wave in flight
+    constexpr int K = 3 * NP * NP;
+    constexpr bool inject = WMODE == kGramInject;
+    __shared__ float slot_s[K * 16];  // one slot per 16-lane row of the workgroup
     const int b = blockIdx.x, part = blockIdx.y, n = a.n, C = a.C;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int blk = lane >> 2, i = lane & 3;
-    constexpr bool inject = WMODE == kGramInject;
     const int nsteps = (C + 127) / 128, spp = (nsteps + a.parts - 1) / a.parts;
     const int s_begin = part * spp, s_end = min(nsteps, s_begin + spp);
-    const size_t row = (size_t)b * n * C + (size_t)(i < n ? i : 0) * C;  // streams >= n: masked below
-    const bf16_t *gb = static_cast<const bf16_t *>(a.dy) + row;
-    const bf16_t *xb = static_cast<const bf16_t *>(a.x) + row;
+    const bf16_t *gb[NB], *xb[NB];
+    bool sv[NB];
+#pragma unroll
+    for (int I = 0; I < NB; I++) {
+        sv[I] = 4 * I + i < n;  // streams >= n: masked below
+        const size_t row = (size_t)b * n * C + (size_t)(sv[I] ? 4 * I + i : 0) * C;
+        gb[I] = static_cast<const bf16_t *>(a.dy) + row;
+        xb[I] = static_cast<const bf16_t *>(a.x) + row;
+    }
     const bf16_t *fb = inject ? static_cast<const bf16_t *>(a.f_inject) + (size_t)b * C : nullptr;
 
-    f32x4_t acc[3];
+    f32x4_t acc[3][NB][NB];
 #pragma unroll
-    for (int m = 0; m < 3; m++) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int m = 0; m < 3; m++)
+#pragma unroll
+        for (int I = 0; I < NB; I++)
+#pragma unroll
+            for (int J = 0; J < NB; J++) acc[m][I][J] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int s0 = s_begin + wave; s0 < s_end; s0 += 4 * kGramSmallUnroll) {
-        uint4 gr[kGramSmallUnroll], xr[kGramSmallUnroll], fr[kGramSmallUnroll];
-        RawVec<bf16_t, 8> wb[kGramSmallUnroll];
-        RawVec<float, 8> wf[kGramSmallUnroll];
+    for (int s0 = s_begin + wave; s0 < s_end; s0 += 4 * U) {
+        uint4 gr[U][NB], xr[U][NB], fr[U];
+        RawVec<bf16_t, 8> wb[U];
+        RawVec<float, 8> wf[U];
 #pragma unroll
-        for (int u = 0; u < kGramSmallUnroll; u++) {
+        for (int u = 0; u < U; u++) {
             const int c = (s0 + 4 * u) * 128 + blk * 8;
             const bool in = s0 + 4 * u < s_end && c < C;  // C % 8 == 0: a chunk is inside or outside
-            const bool ok = in && i < n;
             const int cc = in ? c : 0;
-            gr[u] = load16_masked(reinterpret_cast<const uint4 *>(gb + cc), ok);
-            xr[u] = load16_masked(reinterpret_cast<const uint4 *>(xb + cc), ok);
+#pragma unroll
+            for (int I = 0; I < NB; I++) {
+                gr[u][I] = load16_masked(reinterpret_cast<const uint4 *>(gb[I] + cc), in && sv[I]);
+                xr[u][I] = load16_masked(reinterpret_cast<const uint4 *>(xb[I] + cc), in && sv[I]);
+            }
             if constexpr (inject) fr[u] = load16_masked(reinterpret_cast<const uint4 *>(fb + cc), in && i == 0);
             else if constexpr (WMODE == kGramWBf16) wb[u].load(static_cast<const bf16_t *>(a.w) + cc);
             else wf[u].load(static_cast<const float *>(a.w) + cc);
         }
 #pragma unroll
-        for (int u = 0; u < kGramSmallUnroll; u++) {
-            const bf16x4_t g0 = bf16x4_of(gr[u].x, gr[u].y), g1 = bf16x4_of(gr[u].z, gr[u].w);
-            const bf16x4_t x0 = bf16x4_of(xr[u].x, xr[u].y), x1 = bf16x4_of(xr[u].z, xr[u].w);
-            acc[0] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(g0, x0, acc[0], 0, 0, 0);
-            acc[0] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(g1, x1, acc[0], 0, 0, 0);
+        for (int u = 0; u < U; u++) {
+            bf16x4_t g0[NB], g1[NB], x0[NB], x1[NB];  // first / second group of four channels
+#pragma unroll
+            for (int I = 0; I < NB; I++) {
+                g0[I] = bf16x4_of(gr[u][I].x, gr[u][I].y); g1[I] = bf16x4_of(gr[u][I].z, gr[u][I].w);
+                x0[I] = bf16x4_of(xr[u][I].x, xr[u][I].y); x1[I] = bf16x4_of(xr[u][I].z, xr[u][I].w);
+            }
+#pragma unroll
+            for (int I = 0; I < NB; I++)
+#pragma unroll
+                for (int J = 0; J < NB; J++) {
+                    acc[0][I][J] = mfma4(g0[I], x0[J], acc[0][I][J]);
+                    acc[0][I][J] = mfma4(g1[I], x1[J], acc[0][I][J]);
+                }
             if constexpr (inject) {
                 const bf16x4_t f0 = bf16x4_of(fr[u].x, fr[u].y), f1 = bf16x4_of(fr[u].z, fr[u].w);
-                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(g0, f0, acc[1], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(g1, f1, acc[1], 0, 0, 0);
+#pragma unroll
+                for (int I = 0; I < NB; I++) {
+                    acc[1][I][0] = mfma4(g0[I], f0, acc[1][I][0]);
+                    acc[1][I][0] = mfma4(g1[I], f1, acc[1][I][0]);
+                }
             } else {
-                // dy * w as a bf16 pair (rounded value + remainder): dHpre is a difference of two
-                // sums built on W1, a single rounding of the products is not enough for it
-                float gv[8], wv[8];
+                float wv[8];
                 if constexpr (WMODE == kGramWBf16) wb[u].get(wv);
                 else wf[u].get(wv);
-                gv[0] = bf16lo_to_f32(gr[u].x); gv[1] = bf16hi_to_f32(gr[u].x);
-                gv[2] = bf16lo_to_f32(gr[u].y); gv[3] = bf16hi_to_f32(gr[u].y);
-                gv[4] = bf16lo_to_f32(gr[u].z); gv[5] = bf16hi_to_f32(gr[u].z);
-                gv[6] = bf16lo_to_f32(gr[u].w); gv[7] = bf16hi_to_f32(gr[u].w);
-                uint32_t hw[4], lw[4];
 #pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const float p0 = gv[2 * k] * wv[2 * k], p1 = gv[2 * k + 1] * wv[2 * k + 1];
-                    hw[k] = pack_bf16x2(p0, p1);
-                    lw[k] = pack_bf16x2(p0 - bf16lo_to_f32(hw[k]), p1 - bf16hi_to_f32(hw[k]));
+                for (int I = 0; I < NB; I++) {
+                    // dy * w as a bf16 pair (rounded value + remainder): dHpre is a difference of two
+                    // sums built on W1, a single rounding of the products is not enough for it
+                    const uint32_t gw[4] = {gr[u][I].x, gr[u][I].y, gr[u][I].z, gr[u][I].w};
+                    uint32_t hw[4], lw[4];
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        const float p0 = bf16lo_to_f32(gw[k]) * wv[2 * k], p1 = bf16hi_to_f32(gw[k]) * wv[2 * k + 1];
+                        hw[k] = pack_bf16x2(p0, p1);
+                        lw[k] = pack_bf16x2(p0 - bf16lo_to_f32(hw[k]), p1 - bf16hi_to_f32(hw[k]));
+                    }
+#pragma unroll
+                    for (int J = 0; J < NB; J++) {
+                        acc[1][I][J] = mfma4(bf16x4_of(hw[0], hw[1]), x0[J], acc[1][I][J]);
+                        acc[1][I][J] = mfma4(bf16x4_of(hw[2], hw[3]), x1[J], acc[1][I][J]);
+                        acc[1][I][J] = mfma4(bf16x4_of(lw[0], lw[1]), x0[J], acc[1][I][J]);
+                        acc[1][I][J] = mfma4(bf16x4_of(lw[2], lw[3]), x1[J], acc[1][I][J]);
+                        acc[2][I][J] = mfma4(x0[I], x0[J], acc[2][I][J]);
+                        acc[2][I][J] = mfma4(x1[I], x1[J], acc[2][I][J]);
+                    }
                 }
-                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(bf16x4_of(hw[0], hw[1]), x0, acc[1], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(bf16x4_of(hw[2], hw[3]), x1, acc[1], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(bf16x4_of(lw[0], lw[1]), x0, acc[1], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(bf16x4_of(lw[2], lw[3]), x1, acc[1], 0, 0, 0);
-                acc[2] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(x0, x0, acc[2], 0, 0, 0);
-                acc[2] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(x1, x1, acc[2], 0, 0, 0);
             }
         }
     }
 
     // Lane (block, j) holds column j of its block's products, register = row.  Sum over the four
-    // blocks of a 16-lane row with DPP, one LDS slot per row, then 48 lanes finish.
+    // blocks of a 16-lane row with DPP, one LDS slot per row, then K threads finish.
     const int slot = tid >> 4;
 #pragma unroll
     for (int m = 0; m < 3; m++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            float v = acc[m][r];
-            v += dpp_mov<kDppRowRor4>(v);
-            v += dpp_mov<kDppRowRor8>(v);
-            if ((tid & 15) < 4) slot_s[(m * 16 + r * 4 + (tid & 3)) * 16 + slot] = v;
-        }
+        for (int I = 0; I < NB; I++)
+#pragma unroll
+            for (int J = 0; J < NB; J++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float v = acc[m][I][J][r];
+                    v += dpp_mov<kDppRowRor4>(v);
+                    v += dpp_mov<kDppRowRor8>(v);
+                    if ((tid & 15) < 4)
+                        slot_s[(m * NP * NP + (4 * I + r) * NP + 4 * J + (tid & 3)) * 16 + slot] = v;
+                }
     __syncthreads();
-    if (tid < kGramSmallFloats) {
+    if (tid < K) {
         float v = 0.f;
 #pragma unroll
         for (int sl = 0; sl < 16; sl++) v += slot_s[tid * 16 + sl];
-        a.raw[((size_t)b * a.parts + part) * kGramSmallFloats + tid] = v;
+        a.raw[((size_t)b * a.parts + part) * K + tid] = v;
     }
 }
 
@@ -932,33 +987,32 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
 // =============================================================================================
 // launch
 // =============================================================================================
-// n <= 4, dynamic H, bf16 dy and x, rows 16-byte aligned: Gram matrices on the matrix cores.
-static bool gram_small_supported(const BwdReduceArgs &a, bool both_bf16) {
-    return both_bf16 && a.raw != nullptr && a.n <= 4 && a.C % 8 == 0;
-}
+// n <= 8, dynamic H, bf16 dy and x, rows 16-byte aligned: Gram matrices on the matrix cores.
+static bool gram_small_supported(const BwdReduceArgs &a) { return a.raw != nullptr && a.n <= 8 && a.C % 8 == 0; }
 
 // Column parts of gram_small_kernel: never more than bwd_reduce_parts(), which sizes `raw`.
 static int gram_small_parts(int B, int C) { return C >= 1024 && B < 1024 ? 2 : 1; }
 
+template <int NP>
 static hipError_t launch_gram_small(BwdReduceArgs a, hipStream_t stream) {
     a.parts = gram_small_parts(a.B, a.C);
     const dim3 grid(a.B, a.parts);
-    if (a.f_inject) gram_small_kernel<kGramInject><<<grid, 256, 0, stream>>>(a);
-    else if (a.w_bf16) gram_small_kernel<kGramWBf16><<<grid, 256, 0, stream>>>(a);
-    else gram_small_kernel<kGramWF32><<<grid, 256, 0, stream>>>(a);
+    if (a.f_inject) gram_small_kernel<NP, kGramInject><<<grid, 256, 0, stream>>>(a);
+    else if (a.w_bf16) gram_small_kernel<NP, kGramWBf16><<<grid, 256, 0, stream>>>(a);
+    else gram_small_kernel<NP, kGramWF32><<<grid, 256, 0, stream>>>(a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const size_t smem = sizeof(float) * SkSmall<4>::scaling_floats(a.T);
-    e = allow_dynamic_lds(&coef_bwd_small_kernel<4, false, true>, smem);
+    const size_t smem = sizeof(float) * (SkSmall<NP>::scaling_floats(a.T) + 4 * 3 * NP);  // + the column results
+    e = allow_dynamic_lds(&coef_bwd_small_kernel<NP, false, true>, smem);
     if (e != hipSuccess) return e;
-    coef_bwd_small_kernel<4, false, true><<<(a.B + 3) / 4, 64, smem, stream>>>(a);
+    coef_bwd_small_kernel<NP, false, true><<<(a.B + 3) / 4, 64, smem, stream>>>(a);
     return hipGetLastError();
 }
 
 template <typename TG, typename TX, int NP, int V>
 static hipError_t launch_small(const BwdReduceArgs &a, hipStream_t stream) {
-    if constexpr (NP == 4 && std::is_same<TG, bf16_t>::value && std::is_same<TX, bf16_t>::value)
-        if (gram_small_supported(a, true)) return launch_gram_small(a, stream);
+    if constexpr (std::is_same<TG, bf16_t>::value && std::is_same<TX, bf16_t>::value)
+        if (gram_small_supported(a)) return launch_gram_small<NP>(a, stream);
     const int nch = (a.C / V + a.parts - 1) / a.parts;  // chunks per column part
     // every thread gets the same number of chunks (whole 16-lane rows: the reduction works on them)
     const int rounds = (nch + 255) / 256;
@@ -1039,7 +1093,7 @@ int bwd_reduce_parts(int B, int n, int C) {
 
 size_t bwd_reduce_raw_floats(int B, int n, int C) {
     if (n > 8) return (size_t)B * bwd_reduce_parts(B, n, C) * kGramFloats;
-    return (size_t)B * bwd_reduce_parts(B, n, C) * (8 * 8 + 3 * 8 + 1);
+    return (size_t)B * bwd_reduce_parts(B, n, C) * (3 * 8 * 8);  // Gram input (the VALU sums need 8*8 + 3*8 + 1)
 }
 
 hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int x_dtype,

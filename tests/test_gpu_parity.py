@@ -174,12 +174,13 @@ def test_dynamic_bf16_vs_oracle(B, n, C, out_dtype):
         _check(g[k], ref, "bf16", "d" + k)
 
 
-# n <= 4 with bf16 activations: the channel sums of the backward are 4x4 Gram matrices on the matrix
-# cores (one to four streams, one 128-channel step with and without a tail, one and two column parts).
+# n <= 8 with bf16 activations: the channel sums of the backward are Gram matrices built from 4x4
+# matrix-core products (one to eight streams, one 128-channel step with and without a tail, one and two
+# column parts).
 # The small parameter gradients only see exact bf16 products summed in fp32, so they are held to a
 # bound far below the bf16 tolerance: a dropped remainder term or a misplaced Gram entry fails it.
 @pytest.mark.parametrize("B,n,C", [(5, 1, 8), (3, 2, 136), (6, 3, 1032), (40, 4, 1288), (7, 4, 128),
-                                   (1100, 4, 1024)])
+                                   (1100, 4, 1024), (6, 5, 136), (4, 7, 128), (9, 8, 1288), (70, 6, 1024)])
 @pytest.mark.parametrize("inject", [False, True])
 @pytest.mark.parametrize("w_dtype", [torch.bfloat16, torch.float32])
 def test_bf16_small_n_coefficient_gradients_are_tight(B, n, C, inject, w_dtype):
