@@ -68,7 +68,10 @@ __global__ __launch_bounds__(256) void proj_fwd_generic_kernel(const TX *__restr
 // --------------------------------------------------------------------------------------------
 // MFMA path.  Workgroup = 4 waves on the same 32-sample tile, each wave on its own K sub-slab;
 // the four partial tiles are summed through LDS, so one partial per workgroup reaches memory.
-// grid.x = sample_tiles * KS (sample tile fastest), grid.y = groups of NT projection tiles.
+// grid.x = sample_tiles * round_up(KS, 8), grid.y = groups of NT projection tiles.  Workgroup ids
+// go round robin over the 8 XCDs, each with its own L2: the K slab is chosen by id % 8 (plus 8 per
+// full set of sample tiles), so that all sample tiles of a slab run on one XCD and the slab of phi
+// is fetched from memory once instead of once per XCD.  Ids whose slab is beyond KS do nothing.
 // --------------------------------------------------------------------------------------------
 constexpr int kNarrowPitch = 72;  // LDS row of a 64-element chunk: 128 data bytes + 16 pad (bf16 elements)
 
@@ -77,11 +80,13 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
                                                             const bf16_t *__restrict__ phi,
                                                             float *__restrict__ Ppart,
                                                             float *__restrict__ ssqpart, int B,
-                                                            int D, int DP, int nC, int tiles_s,
+                                                            int D, int DP, int nC, int tiles_s, int KS,
                                                             int sub /* K per wave, multiple of 64 */) {
     extern __shared__ __align__(16) float lds[];  // per wave [(1 + NT) * 32][pitch] bf16; later [3][NT*16 + 1][64] fp32
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int st = blockIdx.x % tiles_s, ks = blockIdx.x / tiles_s;
+    const int set = (blockIdx.x >> 3) / tiles_s;
+    const int st = (blockIdx.x >> 3) % tiles_s, ks = (blockIdx.x & 7) + 8 * set;
+    if (ks >= KS) return;  // the whole workgroup, before any barrier
     const int row = lane & 31, kh = lane >> 5;
     const int b = st * 32 + row;
     const int dbase = blockIdx.y * NT * 32;
@@ -454,14 +459,14 @@ static hipError_t launch_mfma(const void *x, const void *phi, float *Ppart, floa
     const int tiles_s = (B + 31) / 32;
     const int groups = (DP / 32 + NT - 1) / NT;
     const int sub = round_up((nC + KS * 4 - 1) / (KS * 4), 64);  // whole 128-byte lines per lane pair
-    dim3 grid(tiles_s * KS, groups);
+    dim3 grid(tiles_s * round_up(KS, 8), groups);
     const size_t smem_chunks = sizeof(bf16_t) * 4 * (1 + NT) * 32 * kNarrowPitch;
     const size_t smem_sum = sizeof(float) * 3 * (NT * 16 + 1) * 64;
     const size_t smem = smem_chunks > smem_sum ? smem_chunks : smem_sum;
     if (hipError_t e = allow_dynamic_lds(&proj_fwd_mfma_kernel<NT>, smem); e != hipSuccess) return e;
     proj_fwd_mfma_kernel<NT><<<grid, 256, smem, stream>>>(static_cast<const bf16_t *>(x),
                                                            static_cast<const bf16_t *>(phi), Ppart,
-                                                           ssqpart, B, D, DP, nC, tiles_s, sub);
+                                                           ssqpart, B, D, DP, nC, tiles_s, KS, sub);
     return hipGetLastError();
 }
 
