@@ -52,7 +52,13 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
     bf16_t *phi_s = lds_bf;                       // [DP][LD]
     bf16_t *x_s = phi_s + (size_t)a.DP * LD;      // [SBR][LD]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int k0 = blockIdx.x * KW;
+    // Workgroup ids go round robin over the 8 XCDs (each with its own L2, 128-byte lines).  A slab
+    // row of 32 columns is half a line: neighbouring slabs are given to the same XCD (ids x and
+    // x + 8 of a group of 16), otherwise two L2s fetch every line of x and phi.
+    int slab = blockIdx.x;
+    if constexpr (NTK == 1) slab = (blockIdx.x >> 4) * 16 + (blockIdx.x & 7) * 2 + ((blockIdx.x >> 3) & 1);
+    const int k0 = slab * KW;
+    if (k0 >= a.nC) return;  // ids of the padded grid; the whole workgroup, before any barrier
     const int nt = wave % NTK, bt = wave / NTK;
     const int NTD = a.DP / 32;
     const int b_begin = blockIdx.y * a.b_per_split;
@@ -221,7 +227,8 @@ static hipError_t launch_shape(const ProjBwdArgs &a, int S, hipStream_t stream) 
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return e;
     }
-    dim3 grid((a.nC + 32 * NTK - 1) / (32 * NTK), S);
+    const int slabs = (a.nC + 32 * NTK - 1) / (32 * NTK);
+    dim3 grid(NTK == 1 ? round_up(slabs, 16) : slabs, S);
     kern<<<grid, 256, smem, stream>>>(a);
     return hipGetLastError();
 }
