@@ -39,9 +39,9 @@ __device__ __forceinline__ float reduce_partials(const float *part, int KS, size
 template <int NP> __global__ __launch_bounds__(64) void coef_fwd_small_kernel(CoefArgs a) {
     using SK = SkSmall<NP>;
     const int lane = threadIdx.x;
-    const int g = lane & 15;
-    const int b = blockIdx.x * 4 + (lane >> 4);
-    if (b >= a.B) return;  // whole 16-lane groups leave together; DPP never crosses groups
+    const int g = lane % SK::kGroup;
+    const int b = blockIdx.x * SK::kPerWave + lane / SK::kGroup;
+    if (b >= a.B) return;  // whole groups leave together; the reductions never cross groups
     const int n = a.n, D = n * n + 2 * n;
     const bool dyn = a.Ppart != nullptr;
     float rinv = 0.f, al[3] = {0.f, 0.f, 0.f};
@@ -176,7 +176,7 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
     if (n <= 4)
         coef_fwd_small_kernel<4><<<(B + 3) / 4, 64, 0, stream>>>(a);
     else if (n <= 8)
-        coef_fwd_small_kernel<8><<<(B + 3) / 4, 64, 0, stream>>>(a);
+        coef_fwd_small_kernel<8><<<B, 64, 0, stream>>>(a);
     else if (n <= 16) {
         const size_t smem = sizeof(float) * (16 * 16 + 32 + SkWg<16>::lds_floats(T));
         hipError_t e = precise ? allow_dynamic_lds(&coef_fwd_lds_kernel<16, true>, smem)

@@ -191,6 +191,7 @@ constexpr int kDppQuadXor1 = 0xB1;   // quad_perm:[1,0,3,2]
 constexpr int kDppQuadXor2 = 0x4E;   // quad_perm:[2,3,0,1]
 constexpr int kDppRowRor4 = 0x124;
 constexpr int kDppRowRor8 = 0x128;
+constexpr int kDppRowHalfMirror = 0x141;  // lane i <-> 7 - i within each 8 lanes
 
 // All controls used here read a valid lane for every lane, so `old` is irrelevant; passing 0 with
 // bound_ctrl lets the compiler fold the move into the consuming VALU instruction (v_add_f32_dpp).

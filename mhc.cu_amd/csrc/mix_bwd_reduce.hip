@@ -180,9 +180,9 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
     }
     if (a.raw) return;  // the coefficient backward runs as its own small launch
     __syncthreads();
-    if (tid >= 16) return;
+    if (tid >= SK::kGroup) return;
 
-    // ---- epilogue on one 16-lane group (SkSmall layout) -------------------------------------
+    // ---- epilogue on the lanes of one matrix (SkSmall layout) -------------------------------
     const int g = tid;
     const float s1 = tot[K - 1];
     const int D = n * n + 2 * n;
@@ -240,12 +240,12 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
             S2 += dtr * Pb[di];
         }
     }
-    S0 = row16_allreduce(S0); S1 = row16_allreduce(S1); S2 = row16_allreduce(S2);
+    S0 = SK::group_allreduce(S0); S1 = SK::group_allreduce(S1); S2 = SK::group_allreduce(S2);
     if (g == 0) {
         dt[D] = S0; dt[D + 1] = S1; dt[D + 2] = S2;
         a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv / (float)(n * C);
     }
-    dpw.pad(D, g, 16);
+    dpw.pad(D, g, SK::kGroup);
 }
 
 
@@ -260,9 +260,9 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
     using SK = SkSmall<NP>;
     constexpr int K = GRAM ? 3 * NP * NP : NP * NP + 3 * NP + 1;
     extern __shared__ float sc[];  // Sinkhorn denominators, SK::scaling_floats(T)
-    const int tid = threadIdx.x, g = tid & 15;
-    const int b = blockIdx.x * 4 + (tid >> 4);
-    if (b >= a.B) return;  // whole 16-lane groups leave together; DPP never crosses groups
+    const int tid = threadIdx.x, g = tid % SK::kGroup;
+    const int b = blockIdx.x * SK::kPerWave + tid / SK::kGroup;
+    if (b >= a.B) return;  // whole groups leave together; the reductions never cross groups
     const int n = a.n, C = a.C, D = n * n + 2 * n;
     const bool inject = a.f_inject != nullptr;
     const int r0 = SK::row(g), c0 = SK::col0(g);
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
         const float hpost_r = r0 < n ? a.Hpost[(size_t)b * n + r0] : 0.f;
         // with an injected f, W1 = dy [f; 0; ...]^T and dHpost is its column 0
         const float sel = inject ? (r0 == 0 ? 1.f : 0.f) : hpre_r;
-        float *xch = sc + SK::scaling_floats(a.T) + (tid >> 4) * 3 * NP;
+        float *xch = sc + SK::scaling_floats(a.T) + (tid / SK::kGroup) * 3 * NP;
 #pragma unroll
         for (int e = 0; e < SK::EPL; e++) {
             const float x0 = SK::col_allreduce(sel * w1t[e]);
@@ -313,7 +313,7 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
             tpost = hw * qinv;
             tA1 = xch[NP + gc];
             tA2 = xch[2 * NP + gc];
-            s1 = row16_allreduce(g < n ? a.Hpost[(size_t)b * n + gc] * hw : 0.f);
+            s1 = SK::group_allreduce(g < n ? a.Hpost[(size_t)b * n + gc] * hw : 0.f);
         }
     } else {
         for (int p = 0; p < a.parts; p++) {
@@ -371,12 +371,12 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
             S2 += dtr * pres[e];
         }
     }
-    S0 = row16_allreduce(S0); S1 = row16_allreduce(S1); S2 = row16_allreduce(S2);
+    S0 = SK::group_allreduce(S0); S1 = SK::group_allreduce(S1); S2 = SK::group_allreduce(S2);
     if (g == 0) {
         dt[D] = S0; dt[D + 1] = S1; dt[D + 2] = S2;
         a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv / (float)(n * C);
     }
-    dpw.pad(D, g, 16);
+    dpw.pad(D, g, SK::kGroup);
 }
 
 // =============================================================================================
@@ -1002,10 +1002,11 @@ static hipError_t launch_gram_small(BwdReduceArgs a, hipStream_t stream) {
     else gram_small_kernel<NP, kGramWF32><<<grid, 256, 0, stream>>>(a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const size_t smem = sizeof(float) * (SkSmall<NP>::scaling_floats(a.T) + 4 * 3 * NP);  // + the column results
+    using SK = SkSmall<NP>;
+    const size_t smem = sizeof(float) * (SK::scaling_floats(a.T) + SK::kPerWave * 3 * NP);  // + the column results
     e = allow_dynamic_lds(&coef_bwd_small_kernel<NP, false, true>, smem);
     if (e != hipSuccess) return e;
-    coef_bwd_small_kernel<NP, false, true><<<(a.B + 3) / 4, 64, smem, stream>>>(a);
+    coef_bwd_small_kernel<NP, false, true><<<(a.B + SK::kPerWave - 1) / SK::kPerWave, 64, smem, stream>>>(a);
     return hipGetLastError();
 }
 
@@ -1018,6 +1019,7 @@ static hipError_t launch_small(const BwdReduceArgs &a, hipStream_t stream) {
     const int rounds = (nch + 255) / 256;
     int nt = round_up((nch + rounds - 1) / rounds, 16);
     if (nt > 256) nt = 256;
+    if (nt < SkSmall<NP>::kGroup) nt = SkSmall<NP>::kGroup;  // the epilogue runs on the lanes of one matrix
     constexpr int K = NP * NP + 3 * NP + 1;
     // the Sinkhorn area is only needed when the coefficient backward runs in the same launch
     const size_t smem = sizeof(float) * (K * 16 + K + (a.raw ? 0 : SkSmall<NP>::scaling_floats(a.T)));
@@ -1031,7 +1033,7 @@ static hipError_t launch_small(const BwdReduceArgs &a, hipStream_t stream) {
     const size_t smem2 = sizeof(float) * SkSmall<NP>::scaling_floats(a.T);
     e = allow_dynamic_lds(&coef_bwd_small_kernel<NP, kPrecise>, smem2);
     if (e != hipSuccess) return e;
-    coef_bwd_small_kernel<NP, kPrecise><<<(a.B + 3) / 4, 64, smem2, stream>>>(a);
+    coef_bwd_small_kernel<NP, kPrecise><<<(a.B + SkSmall<NP>::kPerWave - 1) / SkSmall<NP>::kPerWave, 64, smem2, stream>>>(a);
     return hipGetLastError();
 }
 

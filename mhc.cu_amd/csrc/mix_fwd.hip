@@ -160,35 +160,33 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
     // ---- 1. loads.  Wave 0 first asks for the small coefficient inputs (they return ahead of
     // the bulk data, so the Sinkhorn chain below runs while the tile is still streaming in),
     // then every thread issues the loads of the sample's whole tile. ------------------------------
-    const int g = tid & 15, part = (tid >> 4) & 3;  // wave 0: 4 lanes share each partial-sum reduction
+    // wave 0: lane g of a group owns matrix element (r0, c0) and, for g < 2n, entry g of the vector
+    // (pre | post); with 4x4 matrices the wave holds four groups, which share the K-split sums
+    const int g = tid % SK::kGroup, part = (tid / SK::kGroup) % SK::kPerWave;
     const int D = n * n + 2 * n;
     const int r0 = SK::row(g), c0 = SK::col0(g);
-    float al0 = 0.f, al1 = 0.f, al2 = 0.f, bpre = 0.f, bpost = 0.f, bres[SK::EPL];
-    // wave 0 sums 4 * SU K-splits in one round of loads (proj_fwd_ksplit caps the split count to
-    // match; the two-chunk variant has no registers to spare for more)
-    constexpr int SU = CPT == 1 ? 6 : 4;
-    float t_ssq[SU], t_pre[SU], t_post[SU], t_e[SU][SK::EPL];
+    const bool mv = r0 < n && c0 < n, vv = g < 2 * n;
+    float al0 = 0.f, al1 = 0.f, al2 = 0.f, bvec = 0.f, bres = 0.f;
+    // wave 0 sums kPerWave * SU K-splits in one round of loads (proj_fwd_ksplit caps the split count
+    // to match; the two-chunk variant has no registers to spare for more)
+    constexpr int SU = (CPT == 1 ? 24 : 16) / SK::kPerWave;
+    float t_ssq[SU], t_vec[SU], t_e[SU];
     const size_t ps = (size_t)a.B * a.DP;
     const float *Pb = dyn ? a.Ppart + (size_t)b * a.DP : nullptr;
     // None of these loads sits behind a per-lane branch or is touched before step 2 / step 3: out of
     // range indices alias element 0 and are discarded where the value is used.
     if (tid < 64) {
         if (dyn) { al0 = a.alpha[0]; al1 = a.alpha[1]; al2 = a.alpha[2]; }
-        const int gc = g < n ? g : 0;
-        bpre = a.b_pre[gc]; bpost = a.b_post[gc];
-#pragma unroll
-        for (int e = 0; e < SK::EPL; e++) bres[e] = a.b_res[(r0 < n && c0 + e < n) ? r0 * n + c0 + e : 0];
+        bvec = g < n ? a.b_pre[g] : a.b_post[vv ? g - n : 0];
+        bres = a.b_res[mv ? r0 * n + c0 : 0];
         if (dyn) {
 #pragma unroll
             for (int u = 0; u < SU; u++) {  // first batch of K-split partials: ks = part*SU + u
                 const int ks = part * SU + u;
                 const size_t ko = ks < a.KS ? ks : 0;
                 t_ssq[u] = a.ssqpart[ko * a.B + b];
-                t_pre[u] = Pb[ko * ps + gc];
-                t_post[u] = Pb[ko * ps + n + gc];
-#pragma unroll
-                for (int e = 0; e < SK::EPL; e++)
-                    t_e[u][e] = Pb[ko * ps + ((r0 < n && c0 + e < n) ? 2 * n + r0 * n + c0 + e : 0)];
+                t_vec[u] = Pb[ko * ps + (vv ? g : 0)];
+                t_e[u] = Pb[ko * ps + (mv ? 2 * n + r0 * n + c0 : 0)];
             }
         }
     }
@@ -221,42 +219,34 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
     MHC_PHASE(kPhaseFwdFused, b, 1);
     // ---- 2. coefficients on wave 0 -----------------------------------------------------------
     if (tid < 64) {
-        float pe[SK::EPL], ppre = 0.f, ppost = 0.f, ssq = 0.f;
-#pragma unroll
-        for (int e = 0; e < SK::EPL; e++) pe[e] = 0.f;
+        float pe = 0.f, pvec = 0.f, ssq = 0.f;
         if (dyn) {
 #pragma unroll
             for (int u = 0; u < SU; u++) {
                 const bool ok = part * SU + u < a.KS;
                 ssq += ok ? t_ssq[u] : 0.f;
-                ppre += (ok && g < n) ? t_pre[u] : 0.f;
-                ppost += (ok && g < n) ? t_post[u] : 0.f;
-#pragma unroll
-                for (int e = 0; e < SK::EPL; e++) pe[e] += (ok && r0 < n && c0 + e < n) ? t_e[u][e] : 0.f;
+                pvec += (ok && vv) ? t_vec[u] : 0.f;
+                pe += (ok && mv) ? t_e[u] : 0.f;
             }
-            for (int ks0 = 4 * SU + part * SU; ks0 < a.KS; ks0 += 4 * SU) {  // never with proj_fwd_ksplit's cap
+            for (int ks0 = (SK::kPerWave + part) * SU; ks0 < a.KS; ks0 += SK::kPerWave * SU) {  // never with proj_fwd_ksplit's cap
 #pragma unroll
                 for (int u = 0; u < SU; u++) {
                     const int ks = ks0 + u;
                     if (ks < a.KS) {
                         ssq += a.ssqpart[(size_t)ks * a.B + b];
-                        if (g < n) { ppre += Pb[ks * ps + g]; ppost += Pb[ks * ps + n + g]; }
-#pragma unroll
-                        for (int e = 0; e < SK::EPL; e++)
-                            if (r0 < n && c0 + e < n) pe[e] += Pb[ks * ps + 2 * n + r0 * n + c0 + e];
+                        if (vv) pvec += Pb[ks * ps + g];
+                        if (mv) pe += Pb[ks * ps + 2 * n + r0 * n + c0];
                     }
                 }
             }
-            ssq = xor32_add(xor16_add(ssq));
-            ppre = xor32_add(xor16_add(ppre));
-            ppost = xor32_add(xor16_add(ppost));
-#pragma unroll
-            for (int e = 0; e < SK::EPL; e++) {
-                pe[e] = xor32_add(xor16_add(pe[e]));
+            if constexpr (SK::kPerWave == 4) {  // the four groups hold a quarter of the splits each
+                ssq = xor32_add(xor16_add(ssq));
+                pvec = xor32_add(xor16_add(pvec));
+                pe = xor32_add(xor16_add(pe));
             }
         }
         MHC_PHASE(kPhaseFwdFused, b, 2);
-        if (tid < 16) {
+        if (tid < SK::kGroup) {
             float rinv = 0.f;
             if (dyn) {
                 const float r = sqrtf(ssq / (float)(n * C) + a.eps);
@@ -265,38 +255,31 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             }
             const bool wr = dyn || b == 0;  // static coefficients are written once
             const size_t hs = dyn ? (size_t)b * n : 0, ms = dyn ? (size_t)b * n * n : 0;
-            if (g < n) {
-                const float p0 = ppre * rinv, p1 = ppost * rinv;
-                const float hp = sigmoidf_acc(al0 * p0 + bpre);
-                const float ho = 2.0f * sigmoidf_acc(al1 * p1 + bpost);
-                coef_s[NP * NP + g] = hp;
-                coef_s[NP * NP + NP + g] = ho;
-                if (wr && a.Hpre) a.Hpre[hs + g] = hp;
-                if (wr && a.Hpost) a.Hpost[hs + g] = ho;
-                if (dyn) { a.P[(size_t)b * D + g] = p0; a.P[(size_t)b * D + n + g] = p1; }
-            } else if (g < NP) {
-                coef_s[NP * NP + g] = 0.f;
-                coef_s[NP * NP + NP + g] = 0.f;
+            if (vv) {
+                const bool pre = g < n;
+                const int gi = pre ? g : g - n;
+                const float p = pvec * rinv;
+                const float h = pre ? sigmoidf_acc(al0 * p + bvec) : 2.0f * sigmoidf_acc(al1 * p + bvec);
+                coef_s[NP * NP + (pre ? 0 : NP) + gi] = h;
+                float *dst = pre ? a.Hpre : a.Hpost;
+                if (wr && dst) dst[hs + gi] = h;
+                if (dyn) a.P[(size_t)b * D + g] = p;
+            } else if (g < 2 * NP) {
+                // the padded entries of Hpre and Hpost: 2 (NP - n) slots, taken by lanes 2n .. 2NP-1
+                const int k = g - 2 * n;
+                coef_s[NP * NP + (k < NP - n ? n + k : NP + n + (k - (NP - n)))] = 0.f;
             }
-            float m[SK::EPL];
-#pragma unroll
-            for (int e = 0; e < SK::EPL; e++) {
-                const int c = c0 + e;
-                if (r0 < n && c < n) {
-                    const float p = pe[e] * rinv;
-                    if (dyn) a.P[(size_t)b * D + 2 * n + r0 * n + c] = p;
-                    m[e] = expf(al2 * p + bres[e]);
-                } else {
-                    m[e] = 0.f;
-                }
+            float m[1];
+            if (mv) {
+                const float p = pe * rinv;
+                if (dyn) a.P[(size_t)b * D + 2 * n + r0 * n + c0] = p;
+                m[0] = expf(al2 * p + bres);
+            } else {
+                m[0] = 0.f;
             }
             SK::forward(m, g, n, a.T, a.eps, nullptr, tid);
-#pragma unroll
-            for (int e = 0; e < SK::EPL; e++) {
-                const int c = c0 + e;
-                coef_s[r0 * NP + c] = m[e];
-                if (wr && a.M && r0 < n && c < n) a.M[ms + r0 * n + c] = m[e];
-            }
+            coef_s[r0 * NP + c0] = m[0];
+            if (wr && a.M && mv) a.M[ms + r0 * n + c0] = m[0];
         }
     }
     MHC_PHASE(kPhaseFwdFused, b, 3);

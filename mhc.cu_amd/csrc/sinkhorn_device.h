@@ -7,9 +7,11 @@
 // the iterates are rebuilt from them by undoing the scalings.
 //
 // Two layouts:
-//   SkSmall<NP> (NP = 4, 8): a matrix lives in the registers of 16 consecutive lanes
-//       (NP*NP/16 elements per lane); all reductions are DPP moves, no LDS traffic on the
-//       forward path.  Four matrices per wave.
+//   SkSmall<NP> (NP = 4, 8): one element per lane, a matrix lives in NP*NP consecutive lanes (four
+//       4x4 matrices per wave, or one 8x8 matrix); all reductions are DPP moves and lane swaps, no
+//       LDS traffic on the forward path.  The chain of an iteration is then about a dozen
+//       dependent instructions for either size (with four elements per lane an 8x8 iteration
+//       issued some 60 instructions on a wave that has the SIMD to itself).
 //   SkWg<NP>    (NP = 16, 32): one 256-thread workgroup per matrix, everything in registers,
 //       iterate kept in scaling form diag(u) E diag(v).
 #pragma once
@@ -23,26 +25,34 @@ namespace mhc {
 // =============================================================================================
 template <int NP> struct SkSmall {
     static_assert(NP == 4 || NP == 8, "SkSmall handles 4x4 and 8x8 tiles");
-    static constexpr int EPL = NP * NP / 16;  // elements per lane (contiguous columns of one row)
-    static constexpr int LPR = NP / EPL;      // lanes per row
-    static constexpr int kGroup = 16;         // lanes per matrix
+    static constexpr int EPL = 1;               // elements per lane
+    static constexpr int kGroup = NP * NP;      // lanes per matrix: 16 or the whole wave
+    static constexpr int kPerWave = kWave / kGroup;  // matrices per wave
 
-    __device__ static __forceinline__ int row(int g) { return g / LPR; }
-    __device__ static __forceinline__ int col0(int g) { return (g % LPR) * EPL; }
+    __device__ static __forceinline__ int row(int g) { return g / NP; }
+    __device__ static __forceinline__ int col0(int g) { return g % NP; }
 
-    // sum over the lanes that hold the same row
+    // sum over the NP consecutive lanes that hold a row
     __device__ static __forceinline__ float row_allreduce(float v) {
         v += dpp_mov<kDppQuadXor1>(v);
-        if constexpr (NP == 4) v += dpp_mov<kDppQuadXor2>(v);
+        v += dpp_mov<kDppQuadXor2>(v);
+        if constexpr (NP == 8) v += dpp_mov<kDppRowHalfMirror>(v);  // the other quad of the 8 lanes
         return v;
     }
-    // sum over the lanes that hold the same columns
+    // sum over the lanes that hold a column (stride NP)
     __device__ static __forceinline__ float col_allreduce(float v) {
-        if constexpr (NP == 8) v += dpp_mov<kDppQuadXor2>(v);
-        v += dpp_mov<kDppRowRor4>(v);
-        v += dpp_mov<kDppRowRor8>(v);
+        if constexpr (NP == 4) {
+            v += dpp_mov<kDppRowRor4>(v);
+            v += dpp_mov<kDppRowRor8>(v);
+        } else {
+            v += dpp_mov<kDppRowRor8>(v);
+            v = xor16_add(v);
+            v = xor32_add(v);
+        }
         return v;
     }
+    // sum over all lanes of the matrix
+    __device__ static __forceinline__ float group_allreduce(float v) { return col_allreduce(row_allreduce(v)); }
 
     // m: in = exp(logits) (0 outside n x n), out = final iterate.
     // sc != nullptr: keep, per iteration t and lane, the row denominator and per element the column
