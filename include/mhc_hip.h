@@ -64,7 +64,7 @@ MHC_API const char *mhc_status_string(int status);
 
 /*
  * Largest `iters` the layer entry points below accept for expansion rate n (0 for an invalid n):
- * 256 for n <= 4, 112 for n <= 8, 256 for n <= 32.  The exact Sinkhorn backward
+ * 256 for every n in 1..32.  The exact Sinkhorn backward
  * keeps the scalings of every iteration in LDS, and for n > 8 its float32 round-off grows with the
  * iteration count (2-3e-8 per iteration relative to float64: 5e-7 at 20, up to 8e-6 at 256).  The reference's interface states no bound
  * (sinkhorn_iters of mhc.MHCLayer, src/python/mhc/layer.py:21-29, default 20).

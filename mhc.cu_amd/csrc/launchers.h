@@ -13,7 +13,7 @@ inline size_t dtype_size(int dt) { return dt == kBF16 ? 2 : 4; }
 
 // Largest Sinkhorn iteration count of the layer entry points for this n: the per-iteration
 // denominators of the backward sweep live in LDS (160 KB per CU).
-inline int max_layer_sinkhorn_iters(int n) { return n <= 4 ? 256 : (n <= 8 ? 112 : 256); }
+inline int max_layer_sinkhorn_iters(int) { return 256; }
 
 // Dynamic LDS above 64 KB has to be enabled per kernel before the launch.
 template <typename K> inline hipError_t allow_dynamic_lds(K kernel, size_t bytes) {

@@ -72,9 +72,9 @@ def test_argument_validation_happens_before_any_launch():
     assert fwd(B=0) == 3                               # MHC_ERR_BAD_SHAPE
     # iteration counts beyond what the backward keeps in LDS are refused up front, per n
     assert [L.mhc_max_sinkhorn_iters(n) for n in (0, 1, 4, 5, 8, 9, 16, 17, 32, 33)] == \
-        [0, 256, 256, 112, 112, 256, 256, 256, 256, 0]
-    assert fwd(n=4, T=257) == 3 and fwd(n=8, T=113) == 3 and fwd(n=32, T=257) == 3 and fwd(T=-1) == 3
-    assert fwd(n=4, T=256) == 6 and fwd(n=8, T=112) == 6 and fwd(n=16, T=256) == 6   # next check: workspace
+        [0, 256, 256, 256, 256, 256, 256, 256, 256, 0]
+    assert fwd(n=4, T=257) == 3 and fwd(n=8, T=257) == 3 and fwd(n=32, T=257) == 3 and fwd(T=-1) == 3
+    assert fwd(n=4, T=256) == 6 and fwd(n=8, T=256) == 6 and fwd(n=16, T=256) == 6   # next check: workspace
     assert fwd(x=None) == 1                            # MHC_ERR_NULL_POINTER
     assert fwd(xd=7) == 4                              # MHC_ERR_BAD_DTYPE
     assert fwd(xd=0, yd=1) == 4                        # fp32 in / bf16 out is not offered

@@ -121,7 +121,7 @@ def test_dynamic_fp32_vs_oracle(B, n, C, inject):
         _check(g[k], ref, "fp32", "d" + k)
 
 
-@pytest.mark.parametrize("B,n,C,T", [(2, 4, 16, 256), (3, 8, 16, 112), (2, 16, 8, 256), (2, 32, 8, 256),
+@pytest.mark.parametrize("B,n,C,T", [(2, 4, 16, 256), (3, 8, 16, 256), (2, 5, 16, 256), (2, 16, 8, 256), (2, 32, 8, 256),
                                      (3, 8, 64, 60)])
 @pytest.mark.parametrize("dyn", [True, False])
 def test_largest_iteration_counts(B, n, C, T, dyn):
