@@ -12,7 +12,10 @@
 // straight from global memory in MFMA layout.  dP^T comes as a bf16 high part plus a bf16
 // remainder (two MFMAs per step), which keeps dphi at fp32-like accuracy; x is exact in bf16.
 #include "launchers.h"
+
+#include <type_traits>
 #include "mhc_common.h"
+#include "phase_profiler.h"
 
 namespace mhc {
 
@@ -52,6 +55,10 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
     bf16_t *phi_s = lds_bf;                       // [DP][LD]
     bf16_t *x_s = phi_s + (size_t)a.DP * LD;      // [SBR][LD]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int pwg = blockIdx.y * gridDim.x + blockIdx.x;
+    (void)pwg;
+    MHC_PHASE_ZERO(kPhaseProjBwd, pwg);
+    MHC_PHASE_BEGIN(pclk);
     // Workgroup ids go round robin over the 8 XCDs (each with its own L2, 128-byte lines).  A slab
     // row of 32 columns is half a line: neighbouring slabs are given to the same XCD (ids x and
     // x + 8 of a group of 16), otherwise two L2s fetch every line of x and phi.
@@ -63,6 +70,27 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
     const int NTD = a.DP / 32;
     const int b_begin = blockIdx.y * a.b_per_split;
     const int b_end = min(a.B, b_begin + a.b_per_split);
+
+    // x blocks travel through registers: the first one is requested here, ahead of the phi slab, and
+    // the next one as soon as the current one has been parked in LDS
+    constexpr int XCH = SBR * CPR / 256;  // 16-byte chunks of a block per thread
+    static_assert(SBR * CPR % 256 == 0, "whole rounds of 256 threads");
+    uint32_t xr[2][XCH][4];  // two blocks in flight; scalar words: whole-uint4 array elements can end up in scratch
+    auto load_x = [&](int sb, auto slot) {
+        constexpr int S = decltype(slot)::value;
+#pragma unroll
+        for (int u = 0; u < XCH; u++) {
+            const int ch = tid + u * 256;
+            const int bl = ch / CPR, b = sb + bl, k = k0 + (ch % CPR) * 8;
+            const bool ok = b < b_end && k < a.nC;
+            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(a.x + (ok ? (size_t)b * a.nC + k : 0)), ok);
+            xr[S][u][0] = v.x; xr[S][u][1] = v.y; xr[S][u][2] = v.z; xr[S][u][3] = v.w;
+        }
+    };
+    using Slot0 = std::integral_constant<int, 0>;
+    using Slot1 = std::integral_constant<int, 1>;
+    if (b_begin < b_end) load_x(b_begin, Slot0{});
+    if (b_begin + SBR < b_end) load_x(b_begin + SBR, Slot1{});
 
     // ---- phi slab -> LDS (rows >= D and columns >= nC read as zero) ------------------------
     for (int ch = tid; ch < a.DP * CPR; ch += 256) {
@@ -86,16 +114,46 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
         for (int i = 0; i < 16; i++) acc[m][i] = 0.f;
 
     const int row = lane & 31, kg = lane >> 5;
-    for (int sb = b_begin; sb < b_end; sb += SBR) {
-        // ---- x block -> LDS ------------------------------------------------------------------
+    MHC_PHASE_ADD(kPhaseProjBwd, pwg, 0, pclk);
+    auto process_block = [&](int sb, auto slot) {
+        constexpr int S = decltype(slot)::value;
+        // ---- operands that come straight from global memory (dP^T of the first dphi tile, dP of the
+        // dxflat tile): requested before the barriers, they arrive while the x block is parked ------
+        const int bs0 = sb + 32 * bt;
+        const int b = bs0 + row;
+        constexpr bool EARLY = TPW == 1;  // with more dphi tiles per wave the registers are taken by accumulators
+        static_assert(!PHI_REGS || EARLY, "the dxflat operands of the phi-in-registers variant are requested early");
+        uint4 ah0[EARLY ? 2 * NSB : 1], al0[EARLY ? 2 * NSB : 1], av0[PHI_REGS ? 2 * TPW * 4 / NTK : 1];
+        if constexpr (EARLY) {
+            const int dt = wave / NTK;
+            const bf16_t *ap = a.dPT + frag_base(dt < NTD ? dt : 0, a.BP >> 4, sb >> 4) + lane * 8;
+#pragma unroll
+            for (int ks = 0; ks < 2 * NSB; ks++) {
+                const bool ok = dt < NTD && sb + ks * 16 < b_end;
+                const bf16_t *apk = ok ? ap + ks * 512 : a.dPT;
+                ah0[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk), ok);
+                al0[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk + (size_t)a.DP * a.BP), ok);
+            }
+            if constexpr (PHI_REGS) {
+                const bool ok = bs0 < b_end && b < b_end;
+                const bf16_t *dprow = a.dPb + frag_base((ok ? bs0 : 0) >> 5, a.DP >> 4, 0) + lane * 8;  // + 512 per k-step
+#pragma unroll
+                for (int ks = 0; ks < 2 * TPW * 4 / NTK; ks++)
+                    av0[ks] = load16_masked(reinterpret_cast<const uint4 *>(ks < 2 * NTD ? dprow + ks * 512 : a.dPb),
+                                            ok && ks < 2 * NTD);
+            }
+        }
+        // ---- x block -> LDS, next block requested ----------------------------------------------
         if (sb != b_begin) __syncthreads();  // previous block's fragment reads are done
-        for (int ch = tid; ch < SBR * CPR; ch += 256) {
-            const int bl = ch / CPR, b = sb + bl, k = k0 + (ch % CPR) * 8;
-            const bool ok = b < b_end && k < a.nC;
-            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(a.x + (ok ? (size_t)b * a.nC + k : 0)), ok);
-            *reinterpret_cast<uint4 *>(x_s + (size_t)bl * LD + (ch % CPR) * 8) = v;
+#pragma unroll
+        for (int u = 0; u < XCH; u++) {
+            const int ch = tid + u * 256;
+            *reinterpret_cast<uint4 *>(x_s + (size_t)(ch / CPR) * LD + (ch % CPR) * 8) =
+                make_uint4(xr[S][u][0], xr[S][u][1], xr[S][u][2], xr[S][u][3]);
         }
         __syncthreads();
+        if (sb + 2 * SBR < b_end) load_x(sb + 2 * SBR, slot);
+        MHC_PHASE_ADD(kPhaseProjBwd, pwg, 1, pclk);
 
         // ---- dphi tiles of this wave: (dt, nt), dt = (wave + 4m) / NTK -------------------------
         // x fragments of the block once, then per tile all dP^T operands in one batch of loads
@@ -111,10 +169,14 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
                 uint4 ah[2 * NSB], al[2 * NSB];
 #pragma unroll
                 for (int ks = 0; ks < 2 * NSB; ks++) {
-                    const bool ok = sb + ks * 16 < b_end;
-                    const bf16_t *apk = ok ? ap + ks * 512 : a.dPT;
-                    ah[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk), ok);
-                    al[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk + (size_t)a.DP * a.BP), ok);
+                    if constexpr (EARLY) {  // requested ahead of the barriers
+                        ah[ks] = ah0[ks]; al[ks] = al0[ks];
+                    } else {
+                        const bool ok = sb + ks * 16 < b_end;
+                        const bf16_t *apk = ok ? ap + ks * 512 : a.dPT;
+                        ah[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk), ok);
+                        al[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk + (size_t)a.DP * a.BP), ok);
+                    }
                 }
 #pragma unroll
                 for (int ks = 0; ks < 2 * NSB; ks++) {
@@ -126,22 +188,19 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
             }
         }
 
+        MHC_PHASE_ADD(kPhaseProjBwd, pwg, 2, pclk);
         // ---- dxflat tile of this wave: samples sb + 32 bt .. +32, columns nt ------------------
-        const int bs0 = sb + 32 * bt;
         if (bs0 < b_end) {
             f32x16_t o;
 #pragma unroll
             for (int i = 0; i < 16; i++) o[i] = 0.f;
-            const int b = bs0 + row;
             const bf16_t *dprow = a.dPb + frag_base(bs0 >> 5, a.DP >> 4, 0) + lane * 8;  // + 512 per k-step
             if constexpr (PHI_REGS) {
 #pragma unroll
                 for (int ks = 0; ks < 2 * TPW * 4 / NTK; ks++) {
-                    if (ks < 2 * NTD) {
-                        const uint4 av = load16_masked(reinterpret_cast<const uint4 *>(dprow + ks * 512), b < b_end);
-                        o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av),
+                    if (ks < 2 * NTD)
+                        o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av0[ks]),
                                                                     phif[ks], o, 0, 0, 0);
-                    }
                 }
             } else {
                 for (int ks0 = 0; ks0 < 2 * NTD; ks0 += 8) {  // 8 operand loads in flight
@@ -171,8 +230,13 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
                 }
             }
         }
+    };
+    for (int sb = b_begin; sb < b_end; sb += 2 * SBR) {
+        process_block(sb, Slot0{});
+        if (sb + SBR < b_end) process_block(sb + SBR, Slot1{});
     }
 
+    MHC_PHASE_ADD(kPhaseProjBwd, pwg, 3, pclk);
     // ---- dphi out (this split's partial) -------------------------------------------------------
     float *out = a.dphi + (size_t)blockIdx.y * a.D * a.nC;
     const int k = k0 + nt * 32 + row;
@@ -187,6 +251,7 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
             }
         }
     }
+    MHC_PHASE_ADD(kPhaseProjBwd, pwg, 4, pclk);
 }
 
 // --------------------------------------------------------------------------------------------

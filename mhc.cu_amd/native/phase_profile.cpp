@@ -1,6 +1,7 @@
 // Prints the in-kernel phase timeline of the fused forward kernel and of the slab backward kernel.
 //
-//   phase_profile [--batch B] [--hidden C] [--expansion n]          (n <= 4, C % 8 == 0, bf16)
+//   phase_profile [--batch B] [--hidden C] [--expansion n]          (n <= 8, C % 8 == 0, bf16;
+//                                                                    n > 4: projection backward instead of the slab kernel)
 //
 // Links libmhc_hip_profile.so (python mhc.cu_amd/build.py --profile), the build of the library with
 // csrc/phase_profiler.h compiled in.  Counterpart of the reference's HostProfiler::print_summary
@@ -77,7 +78,7 @@ int main(int argc, char **argv) {
         else if (is("--expansion") && i + 1 < argc) n = atoi(argv[++i]);
         else { fprintf(stderr, "unknown argument %s\n", argv[i]); return 2; }
     }
-    if (n > 4 || C % 8) { fprintf(stderr, "the instrumented kernels serve n <= 4 with C %% 8 == 0\n"); return 2; }
+    if (n > 8 || C % 8) { fprintf(stderr, "the instrumented kernels serve n <= 8 with C %% 8 == 0\n"); return 2; }
     const size_t BnC = (size_t)B * n * C, nC = (size_t)n * C, D = (size_t)n * n + 2 * n;
     std::mt19937 g(0);
     void *x = dev_bf16(BnC, 1.f, g), *dy = dev_bf16(BnC, 1.f, g), *phi = dev_bf16(D * nC, 0.02f, g), *w = dev_bf16(C, 0.f, g);
@@ -99,6 +100,12 @@ int main(int argc, char **argv) {
     summary("fused forward kernel, one workgroup per sample", 0, std::min(B, 4096),
             {"issue loads (early half: tile too)", "coefficient inputs arrive", "activations + Sinkhorn", "tile request (late half), barrier", "tile arrives, aggregate, RMS",
              "mix, stores issued"}, true);
+    if (n > 4) {
+        summary("projection backward kernel, one workgroup per 32 columns of x_flat", 2, std::min((int)(nC / 32), 4096),
+                {"prologue (phi slab, first x block requested)", "operands requested, x block parked (all blocks)",
+                 "fragments, dphi on the matrix cores (all)", "dxflat on the matrix cores, stores (all)", "dphi stores"}, false);
+        return 0;
+    }
     const int slabs = (C + 63) / 64;
     summary("slab backward kernel, one workgroup per (64 channels, batch split)", 1, std::min(slabs * 4, 4096),
             {"prologue (phi slab, first loads)", "tile loads, LDS, barrier (all tiles)", "matrix cores, barrier (all tiles)",
