@@ -160,22 +160,26 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
     // ---- 1. loads.  Wave 0 first asks for the small coefficient inputs (they return ahead of
     // the bulk data, so the Sinkhorn chain below runs while the tile is still streaming in),
     // then every thread issues the loads of the sample's whole tile. ------------------------------
-    // wave 0: lane g of a group owns matrix element (r0, c0) and, for g < 2n, entry g of the vector
-    // (pre | post); with 4x4 matrices the wave holds four groups, which share the K-split sums
-    const int g = tid % SK::kGroup, part = (tid / SK::kGroup) % SK::kPerWave;
+    // Lane g of a group owns matrix element (r0, c0) and, for g < 2n, entry g of the vector (pre | post).
+    // The K-split sums are shared four ways: by the four groups of wave 0 (4x4 matrices, combined
+    // with lane swaps) or by the four waves (8x8 matrices, a whole wave per group, combined through
+    // LDS); the coefficient step itself runs on the first group.
+    constexpr int kSplitWaves = SK::kPerWave == 1 ? 4 : 1;
+    __shared__ float psum_s[kSplitWaves == 4 ? 4 * 3 * 64 : 1];
+    const int g = tid % SK::kGroup, part = (tid / SK::kGroup) % 4;
     const int D = n * n + 2 * n;
     const int r0 = SK::row(g), c0 = SK::col0(g);
     const bool mv = r0 < n && c0 < n, vv = g < 2 * n;
     float al0 = 0.f, al1 = 0.f, al2 = 0.f, bvec = 0.f, bres = 0.f;
-    // wave 0 sums kPerWave * SU K-splits in one round of loads (proj_fwd_ksplit caps the split count
-    // to match; the two-chunk variant has no registers to spare for more)
-    constexpr int SU = (CPT == 1 ? 24 : 16) / SK::kPerWave;
+    // 4 * SU K-splits are summed from one round of loads (proj_fwd_ksplit caps the split count to
+    // match; the two-chunk variant has no registers to spare for more)
+    constexpr int SU = (CPT == 1 ? 24 : 16) / 4;
     float t_ssq[SU], t_vec[SU], t_e[SU];
     const size_t ps = (size_t)a.B * a.DP;
     const float *Pb = dyn ? a.Ppart + (size_t)b * a.DP : nullptr;
     // None of these loads sits behind a per-lane branch or is touched before step 2 / step 3: out of
     // range indices alias element 0 and are discarded where the value is used.
-    if (tid < 64) {
+    if (tid < 64 * kSplitWaves) {
         if (dyn) { al0 = a.alpha[0]; al1 = a.alpha[1]; al2 = a.alpha[2]; }
         bvec = g < n ? a.b_pre[g] : a.b_post[vv ? g - n : 0];
         bres = a.b_res[mv ? r0 * n + c0 : 0];
@@ -218,33 +222,47 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 
     MHC_PHASE(kPhaseFwdFused, b, 1);
     // ---- 2. coefficients on wave 0 -----------------------------------------------------------
-    if (tid < 64) {
-        float pe = 0.f, pvec = 0.f, ssq = 0.f;
-        if (dyn) {
+    float pe = 0.f, pvec = 0.f, ssq = 0.f;
+    if (tid < 64 * kSplitWaves && dyn) {
+#pragma unroll
+        for (int u = 0; u < SU; u++) {
+            const bool ok = part * SU + u < a.KS;
+            ssq += ok ? t_ssq[u] : 0.f;
+            pvec += (ok && vv) ? t_vec[u] : 0.f;
+            pe += (ok && mv) ? t_e[u] : 0.f;
+        }
+        for (int ks0 = (4 + part) * SU; ks0 < a.KS; ks0 += 4 * SU) {  // never with proj_fwd_ksplit's cap
 #pragma unroll
             for (int u = 0; u < SU; u++) {
-                const bool ok = part * SU + u < a.KS;
-                ssq += ok ? t_ssq[u] : 0.f;
-                pvec += (ok && vv) ? t_vec[u] : 0.f;
-                pe += (ok && mv) ? t_e[u] : 0.f;
-            }
-            for (int ks0 = (SK::kPerWave + part) * SU; ks0 < a.KS; ks0 += SK::kPerWave * SU) {  // never with proj_fwd_ksplit's cap
-#pragma unroll
-                for (int u = 0; u < SU; u++) {
-                    const int ks = ks0 + u;
-                    if (ks < a.KS) {
-                        ssq += a.ssqpart[(size_t)ks * a.B + b];
-                        if (vv) pvec += Pb[ks * ps + g];
-                        if (mv) pe += Pb[ks * ps + 2 * n + r0 * n + c0];
-                    }
+                const int ks = ks0 + u;
+                if (ks < a.KS) {
+                    ssq += a.ssqpart[(size_t)ks * a.B + b];
+                    if (vv) pvec += Pb[ks * ps + g];
+                    if (mv) pe += Pb[ks * ps + 2 * n + r0 * n + c0];
                 }
             }
-            if constexpr (SK::kPerWave == 4) {  // the four groups hold a quarter of the splits each
-                ssq = xor32_add(xor16_add(ssq));
-                pvec = xor32_add(xor16_add(pvec));
-                pe = xor32_add(xor16_add(pe));
+        }
+        if constexpr (kSplitWaves == 1) {  // the four groups of wave 0 hold a quarter of the splits each
+            ssq = xor32_add(xor16_add(ssq));
+            pvec = xor32_add(xor16_add(pvec));
+            pe = xor32_add(xor16_add(pe));
+        } else {
+            psum_s[(part * 3 + 0) * 64 + g] = ssq;
+            psum_s[(part * 3 + 1) * 64 + g] = pvec;
+            psum_s[(part * 3 + 2) * 64 + g] = pe;
+        }
+    }
+    if constexpr (kSplitWaves == 4) {
+        if (dyn) {  // uniform over the workgroup
+            __syncthreads();
+            if (tid < 64) {
+                ssq = (psum_s[0 * 64 + g] + psum_s[3 * 64 + g]) + (psum_s[6 * 64 + g] + psum_s[9 * 64 + g]);
+                pvec = (psum_s[1 * 64 + g] + psum_s[4 * 64 + g]) + (psum_s[7 * 64 + g] + psum_s[10 * 64 + g]);
+                pe = (psum_s[2 * 64 + g] + psum_s[5 * 64 + g]) + (psum_s[8 * 64 + g] + psum_s[11 * 64 + g]);
             }
         }
+    }
+    if (tid < 64) {
         MHC_PHASE(kPhaseFwdFused, b, 2);
         if (tid < SK::kGroup) {
             float rinv = 0.f;
