@@ -250,133 +250,135 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
 
 
 // =============================================================================================
-// n <= 8, dynamic H: coefficient backward as its own launch - one 16-lane group per sample, four
-// samples per wave, so the serial Sinkhorn chain of every sample runs concurrently instead of at
-// the tail of a bandwidth-bound workgroup.  Input: the raw channel sums written by the kernel
-// above ([B][parts][K], K = NP*NP + 3*NP + 1: dM | dHpost | A1 | A2 | s1).
+// n <= 8, dynamic H: coefficient backward of one sample on the lanes of one SkSmall group (16 lanes
+// for 4x4, a wave for 8x8).  Input: channel sums of the sample, `parts` blocks of K floats, in
+// global memory or in LDS:
+//   GRAM:  dM | W1 | XX (NP x NP each, K = 3 NP^2)
+//   else:  dM | dHpost | A1 | A2 | s1 (K = NP^2 + 3 NP + 1)
+// prefetch() asks for everything else the sample needs (P, H, r, q, alpha, b_res), so that a caller
+// with other work to do first has those values waiting; run() then forms dHpre / dHpost, the sigmoid
+// derivatives, the exact Sinkhorn backward, dP = dt * alpha / r in all three layouts, and cx.
 // =============================================================================================
+template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
+    using SK = SkSmall<NP>;
+    static constexpr int K = GRAM ? 3 * NP * NP : NP * NP + 3 * NP + 1;
+    // LDS floats next to the Sinkhorn denominators, per group: the column results of the Gram sums
+    static constexpr int kXch = GRAM ? 3 * NP : 0;
+
+    int r0, c0, gc;
+    bool inject, mv;
+    float qinv, rinv, al0, al1, al2, pres, bres, hp, ho, ppre, ppost, hpre_r, hpost_r;
+
+    __device__ __forceinline__ void prefetch(const BwdReduceArgs &a, int b, int g) {
+        const int n = a.n, D = n * n + 2 * n;
+        r0 = SK::row(g); c0 = SK::col0(g);
+        gc = g < n ? g : 0;  // lanes beyond n alias entry 0 (never used): no branch around loads
+        mv = r0 < n && c0 < n;
+        inject = a.f_inject != nullptr;
+        qinv = inject ? 0.f : 1.0f / a.q[b];
+        const float *Pb = a.P + (size_t)b * D;
+        al0 = a.alpha[0]; al1 = a.alpha[1]; al2 = a.alpha[2];
+        rinv = 1.0f / a.r[b];
+        pres = Pb[mv ? 2 * n + r0 * n + c0 : 0];
+        bres = a.b_res[mv ? r0 * n + c0 : 0];
+        hp = a.Hpre[(size_t)b * n + gc]; ho = a.Hpost[(size_t)b * n + gc];
+        ppre = Pb[gc]; ppost = Pb[n + gc];
+        hpre_r = a.Hpre[(size_t)b * n + (r0 < n ? r0 : 0)];
+        hpost_r = a.Hpost[(size_t)b * n + (r0 < n ? r0 : 0)];
+    }
+
+    // g: lane within the group; lane: lane within the wave (indexes the denominators in sc);
+    // xch: kXch floats of LDS private to the group
+    __device__ __forceinline__ void run(const BwdReduceArgs &a, int b, int g, int lane, const float *sums,
+                                        int parts, float *sc, float *xch) {
+        const int n = a.n, C = a.C, D = n * n + 2 * n;
+        float dMe = 0.f, tpost = 0.f, tA1 = 0.f, tA2 = 0.f, s1 = 0.f;
+        if constexpr (GRAM) {
+            // lane (r0, c0) takes its element of each matrix and the mirrored element of W1, so that
+            // every sum below runs down a column:
+            //   dHpost[c] = sum_r Hpre[r] W1[c][r] / q        A1[c] = sum_r Hpost[r] W1[r][c]
+            //   A2[c] = sum_r Hpre[r] XX[r][c]                s1 = sum_c Hpost[c] (sum_r Hpre[r] W1[c][r])
+            // The column results are handed to lanes 0 .. n-1 through LDS (same wave: no barrier).
+            float w1 = 0.f, w1t = 0.f, xx = 0.f;
+            for (int p = 0; p < parts; p++) {
+                const float *rp = sums + (size_t)p * K;
+                dMe += rp[r0 * NP + c0];
+                w1 += rp[NP * NP + r0 * NP + c0];
+                w1t += rp[NP * NP + c0 * NP + r0];
+                xx += rp[2 * NP * NP + r0 * NP + c0];
+            }
+            const float hr = r0 < n ? hpre_r : 0.f, hor = r0 < n ? hpost_r : 0.f;
+            // with an injected f, W1 = dy [f; 0; ...]^T and dHpost is its column 0
+            const float sel = inject ? (r0 == 0 ? 1.f : 0.f) : hr;
+            const float x0 = SK::col_allreduce(sel * w1t);
+            const float x1 = SK::col_allreduce(hor * w1);
+            const float x2 = SK::col_allreduce(hr * xx);
+            if (r0 == 0) { xch[c0] = x0; xch[NP + c0] = x1; xch[2 * NP + c0] = x2; }
+            const float hw = xch[gc];
+            if (inject) {
+                tpost = hw;
+            } else {
+                tpost = hw * qinv;
+                tA1 = xch[NP + gc];
+                tA2 = xch[2 * NP + gc];
+                s1 = SK::group_allreduce(g < n ? ho * hw : 0.f);
+            }
+        } else {
+            for (int p = 0; p < parts; p++) {
+                const float *rp = sums + (size_t)p * K;
+                dMe += rp[r0 * NP + c0];
+                tpost += rp[NP * NP + gc]; tA1 += rp[NP * NP + NP + gc]; tA2 += rp[NP * NP + 2 * NP + gc];
+                s1 += rp[K - 1];
+            }
+        }
+        if (g == 0) a.out.s1[b] = s1;
+        float *dt = a.out.dt + (size_t)b * (D + 3);
+        const DPWriter dpw{a.out, b, a.B, a.DP};
+        float S0 = 0.f, S1 = 0.f, S2 = 0.f;  // sum_d dt_d p_d per alpha group
+        if (g < n) {
+            const float dHpost = tpost;
+            const float dHpre = inject ? 0.f : tA1 * qinv - s1 * tA2 * qinv * qinv * qinv / (float)C;
+            const float dtp = dHpre * hp * (1.0f - hp);
+            const float dto = dHpost * ho * (1.0f - 0.5f * ho);
+            dt[g] = dtp; dt[n + g] = dto;
+            dpw.put(g, dtp * al0 * rinv); dpw.put(n + g, dto * al1 * rinv);
+            S0 = dtp * ppre; S1 = dto * ppost;
+        }
+        const float E = mv ? expf(al2 * pres + bres) : 0.f;
+        float m[1] = {E}, d[1] = {mv ? dMe : 0.f};
+        SK::template forward<PRECISE>(m, g, n, a.T, a.eps, sc, lane);
+        SK::template backward<PRECISE>(d, m, a.T, sc, lane);
+        if (mv) {
+            const int di = 2 * n + r0 * n + c0;
+            const float dtr = d[0] * E;
+            dt[di] = dtr;
+            dpw.put(di, dtr * al2 * rinv);
+            S2 = dtr * pres;
+        }
+        S0 = SK::group_allreduce(S0); S1 = SK::group_allreduce(S1); S2 = SK::group_allreduce(S2);
+        if (g == 0) {
+            dt[D] = S0; dt[D + 1] = S1; dt[D + 2] = S2;
+            a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv / (float)(n * C);
+        }
+        dpw.pad(D, g, SK::kGroup);
+    }
+};
+
+// The coefficient backward as its own launch: every sample's serial Sinkhorn chain runs concurrently
+// (four 4x4 samples or one 8x8 sample per wave) instead of at the tail of a bandwidth-bound workgroup.
+// Input: the channel sums written by a kernel above or below ([B][parts][K]).
 template <int NP, bool PRECISE, bool GRAM = false>
 __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
     using SK = SkSmall<NP>;
-    constexpr int K = GRAM ? 3 * NP * NP : NP * NP + 3 * NP + 1;
-    extern __shared__ float sc[];  // Sinkhorn denominators, SK::scaling_floats(T)
+    using CB = CoefBwdSmall<NP, PRECISE, GRAM>;
+    extern __shared__ float sc[];  // Sinkhorn denominators, SK::scaling_floats(T), then CB::kXch per group
     const int tid = threadIdx.x, g = tid % SK::kGroup;
     const int b = blockIdx.x * SK::kPerWave + tid / SK::kGroup;
     if (b >= a.B) return;  // whole groups leave together; the reductions never cross groups
-    const int n = a.n, C = a.C, D = n * n + 2 * n;
-    const bool inject = a.f_inject != nullptr;
-    const int r0 = SK::row(g), c0 = SK::col0(g);
-    // everything this lane needs from memory, issued up front
-    const float *raw = a.raw + (size_t)b * a.parts * K;
-    float dMe[SK::EPL], tpost = 0.f, tA1 = 0.f, tA2 = 0.f, s1 = 0.f;
-#pragma unroll
-    for (int e = 0; e < SK::EPL; e++) dMe[e] = 0.f;
-    const int gc = g < n ? g : 0;  // lanes beyond n alias entry 0 (never used): no branch around loads
-    const float qinv = inject ? 0.f : 1.0f / a.q[b];
-    if constexpr (GRAM) {
-        // input: dM | W1 | XX (NP x NP each); lane (r0, c0 ..) takes its elements of each and the
-        // mirrored elements of W1, so that every sum below runs down a column:
-        //   dHpost[c] = sum_r Hpre[r] W1[c][r] / q        A1[c] = sum_r Hpost[r] W1[r][c]
-        //   A2[c] = sum_r Hpre[r] XX[r][c]                s1 = sum_c Hpost[c] (sum_r Hpre[r] W1[c][r])
-        // The column results are handed to lanes 0 .. n-1 through LDS (same wave: no barrier).
-        float w1[SK::EPL], w1t[SK::EPL], xx[SK::EPL];
-#pragma unroll
-        for (int e = 0; e < SK::EPL; e++) w1[e] = w1t[e] = xx[e] = 0.f;
-        for (int p = 0; p < a.parts; p++) {
-            const float *rp = raw + (size_t)p * K;
-            float t0[SK::EPL], t1[SK::EPL], t2[SK::EPL];
-            load_vec<float, SK::EPL>(rp + r0 * NP + c0, t0);
-            load_vec<float, SK::EPL>(rp + NP * NP + r0 * NP + c0, t1);
-            load_vec<float, SK::EPL>(rp + 2 * NP * NP + r0 * NP + c0, t2);
-#pragma unroll
-            for (int e = 0; e < SK::EPL; e++) {
-                dMe[e] += t0[e]; w1[e] += t1[e]; xx[e] += t2[e];
-                w1t[e] += rp[NP * NP + (c0 + e) * NP + r0];
-            }
-        }
-        const float hpre_r = r0 < n ? a.Hpre[(size_t)b * n + r0] : 0.f;
-        const float hpost_r = r0 < n ? a.Hpost[(size_t)b * n + r0] : 0.f;
-        // with an injected f, W1 = dy [f; 0; ...]^T and dHpost is its column 0
-        const float sel = inject ? (r0 == 0 ? 1.f : 0.f) : hpre_r;
-        float *xch = sc + SK::scaling_floats(a.T) + (tid / SK::kGroup) * 3 * NP;
-#pragma unroll
-        for (int e = 0; e < SK::EPL; e++) {
-            const float x0 = SK::col_allreduce(sel * w1t[e]);
-            const float x1 = SK::col_allreduce(hpost_r * w1[e]);
-            const float x2 = SK::col_allreduce(hpre_r * xx[e]);
-            if (r0 == 0) { xch[c0 + e] = x0; xch[NP + c0 + e] = x1; xch[2 * NP + c0 + e] = x2; }
-        }
-        const float hw = xch[gc];
-        if (inject) {
-            tpost = hw;
-        } else {
-            tpost = hw * qinv;
-            tA1 = xch[NP + gc];
-            tA2 = xch[2 * NP + gc];
-            s1 = SK::group_allreduce(g < n ? a.Hpost[(size_t)b * n + gc] * hw : 0.f);
-        }
-    } else {
-        for (int p = 0; p < a.parts; p++) {
-            const float *rp = raw + (size_t)p * K;
-#pragma unroll
-            for (int e = 0; e < SK::EPL; e++) dMe[e] += rp[r0 * NP + c0 + e];
-            tpost += rp[NP * NP + gc]; tA1 += rp[NP * NP + NP + gc]; tA2 += rp[NP * NP + 2 * NP + gc];
-            s1 += rp[K - 1];
-        }
-    }
-    const float *Pb = a.P + (size_t)b * D;
-    const float al0 = a.alpha[0], al1 = a.alpha[1], al2 = a.alpha[2];
-    const float rinv = 1.0f / a.r[b];
-    float pres[SK::EPL], bres[SK::EPL];
-#pragma unroll
-    for (int e = 0; e < SK::EPL; e++) {
-        const bool ok = r0 < n && c0 + e < n;
-        pres[e] = ok ? Pb[2 * n + r0 * n + c0 + e] : 0.f;
-        bres[e] = ok ? a.b_res[r0 * n + c0 + e] : 0.f;
-    }
-    float hp = 0.f, ho = 0.f, ppre = 0.f, ppost = 0.f;
-    if (g < n) { hp = a.Hpre[(size_t)b * n + g]; ho = a.Hpost[(size_t)b * n + g]; ppre = Pb[g]; ppost = Pb[n + g]; }
-
-    if (g == 0) a.out.s1[b] = s1;
-    float *dt = a.out.dt + (size_t)b * (D + 3);
-    const DPWriter dpw{a.out, b, a.B, a.DP};
-    float S0 = 0.f, S1 = 0.f, S2 = 0.f;  // sum_d dt_d p_d per alpha group
-    if (g < n) {
-        const float dHpost = tpost;
-        const float dHpre = inject ? 0.f : tA1 * qinv - s1 * tA2 * qinv * qinv * qinv / (float)C;
-        const float dtp = dHpre * hp * (1.0f - hp);
-        const float dto = dHpost * ho * (1.0f - 0.5f * ho);
-        dt[g] = dtp; dt[n + g] = dto;
-        dpw.put(g, dtp * al0 * rinv); dpw.put(n + g, dto * al1 * rinv);
-        S0 = dtp * ppre; S1 = dto * ppost;
-    }
-    float E[SK::EPL], m[SK::EPL], d[SK::EPL];
-#pragma unroll
-    for (int e = 0; e < SK::EPL; e++) {
-        const bool ok = r0 < n && c0 + e < n;
-        E[e] = ok ? expf(al2 * pres[e] + bres[e]) : 0.f;
-        m[e] = E[e];
-        d[e] = ok ? dMe[e] : 0.f;
-    }
-    SK::template forward<PRECISE>(m, g, n, a.T, a.eps, sc, tid);
-    SK::template backward<PRECISE>(d, m, a.T, sc, tid);
-#pragma unroll
-    for (int e = 0; e < SK::EPL; e++) {
-        const int c = c0 + e;
-        if (r0 < n && c < n) {
-            const int di = 2 * n + r0 * n + c;
-            const float dtr = d[e] * E[e];
-            dt[di] = dtr;
-            dpw.put(di, dtr * al2 * rinv);
-            S2 += dtr * pres[e];
-        }
-    }
-    S0 = SK::group_allreduce(S0); S1 = SK::group_allreduce(S1); S2 = SK::group_allreduce(S2);
-    if (g == 0) {
-        dt[D] = S0; dt[D + 1] = S1; dt[D + 2] = S2;
-        a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv / (float)(n * C);
-    }
-    dpw.pad(D, g, SK::kGroup);
+    CB cb;
+    cb.prefetch(a, b, g);
+    cb.run(a, b, g, tid, a.raw + (size_t)b * a.parts * CB::K, a.parts, sc,
+           sc + SK::scaling_floats(a.T) + (tid / SK::kGroup) * CB::kXch);
 }
 
 // =============================================================================================
