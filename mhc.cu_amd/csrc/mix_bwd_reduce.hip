@@ -406,16 +406,28 @@ __device__ __forceinline__ f32x4_t mfma4(bf16x4_t a, bf16x4_t b, f32x4_t c) {
     return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a, b, c, 0, 0, 0);
 }
 
-template <int NP, int WMODE>
+// FUSED (one column part per sample): the first lanes of wave 0 go on with the sample's coefficient
+// backward (CoefBwdSmall) as soon as the sums are complete, its other inputs requested at the start;
+// with several workgroups per CU the serial Sinkhorn chain of one runs under the loads of the others,
+// and the launch of the coefficient kernel is saved.
+template <int NP, int WMODE, bool FUSED>
 __global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
     static_assert(NP == 4 || NP == 8, "stream groups of four");
+    using SK = SkSmall<NP>;
+    using CB = CoefBwdSmall<NP, false, true>;
     constexpr int NB = NP / 4;            // stream groups
     constexpr int U = NP == 4 ? 2 : 1;    // steps of a wave in flight
     constexpr int K = 3 * NP * NP;
     constexpr bool inject = WMODE == kGramInject;
     __shared__ float slot_s[K * 16];  // one slot per 16-lane row of the workgroup
+    __shared__ float tot_s[FUSED ? K : 1];
+    extern __shared__ float sc[];     // FUSED: Sinkhorn denominators, SK::scaling_floats(T), then CB::kXch
     const int b = blockIdx.x, part = blockIdx.y, n = a.n, C = a.C;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    CB cb;
+    if constexpr (FUSED) {
+        if (tid < SK::kGroup) cb.prefetch(a, b, tid);
+    }
     const int blk = lane >> 2, i = lane & 3;
     const int nsteps = (C + 127) / 128, spp = (nsteps + a.parts - 1) / a.parts;
     const int s_begin = part * spp, s_end = min(nsteps, s_begin + spp);
@@ -530,7 +542,12 @@ __global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
         float v = 0.f;
 #pragma unroll
         for (int sl = 0; sl < 16; sl++) v += slot_s[tid * 16 + sl];
-        a.raw[((size_t)b * a.parts + part) * K + tid] = v;
+        if constexpr (FUSED) tot_s[tid] = v;
+        else a.raw[((size_t)b * a.parts + part) * K + tid] = v;
+    }
+    if constexpr (FUSED) {
+        __syncthreads();
+        if (tid < SK::kGroup) cb.run(a, b, tid, tid, tot_s, 1, sc, sc + SK::scaling_floats(a.T));
     }
 }
 
@@ -995,17 +1012,35 @@ static bool gram_small_supported(const BwdReduceArgs &a) { return a.raw != nullp
 // Column parts of gram_small_kernel: never more than bwd_reduce_parts(), which sizes `raw`.
 static int gram_small_parts(int B, int C) { return C >= 1024 && B < 1024 ? 2 : 1; }
 
+// One launch (channel sums, then the coefficient backward at the tail of every workgroup) unless the
+// Sinkhorn state would take the LDS that keeps several workgroups per CU resident, or the batch is
+// too small to do without column parts.
+static bool gram_small_fused(const BwdReduceArgs &a) {
+    return a.T <= 32 && (a.B >= 128 || a.C <= 2048);
+}
+
+template <int NP, bool FUSED>
+static hipError_t launch_gram_small_kernel(const BwdReduceArgs &a, size_t smem, hipStream_t stream) {
+    const dim3 grid(a.B, a.parts);
+    if (a.f_inject) gram_small_kernel<NP, kGramInject, FUSED><<<grid, 256, smem, stream>>>(a);
+    else if (a.w_bf16) gram_small_kernel<NP, kGramWBf16, FUSED><<<grid, 256, smem, stream>>>(a);
+    else gram_small_kernel<NP, kGramWF32, FUSED><<<grid, 256, smem, stream>>>(a);
+    return hipGetLastError();
+}
+
 template <int NP>
 static hipError_t launch_gram_small(BwdReduceArgs a, hipStream_t stream) {
-    a.parts = gram_small_parts(a.B, a.C);
-    const dim3 grid(a.B, a.parts);
-    if (a.f_inject) gram_small_kernel<NP, kGramInject><<<grid, 256, 0, stream>>>(a);
-    else if (a.w_bf16) gram_small_kernel<NP, kGramWBf16><<<grid, 256, 0, stream>>>(a);
-    else gram_small_kernel<NP, kGramWF32><<<grid, 256, 0, stream>>>(a);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
     using SK = SkSmall<NP>;
-    const size_t smem = sizeof(float) * (SK::scaling_floats(a.T) + SK::kPerWave * 3 * NP);  // + the column results
+    using CB = CoefBwdSmall<NP, false, true>;
+    if (gram_small_fused(a)) {
+        a.parts = 1;
+        const size_t smem = sizeof(float) * (SK::scaling_floats(a.T) + CB::kXch);  // at most 16 KB + 96 B
+        return launch_gram_small_kernel<NP, true>(a, smem, stream);
+    }
+    a.parts = gram_small_parts(a.B, a.C);
+    hipError_t e = launch_gram_small_kernel<NP, false>(a, 0, stream);
+    if (e != hipSuccess) return e;
+    const size_t smem = sizeof(float) * (SK::scaling_floats(a.T) + SK::kPerWave * CB::kXch);
     e = allow_dynamic_lds(&coef_bwd_small_kernel<NP, false, true>, smem);
     if (e != hipSuccess) return e;
     coef_bwd_small_kernel<NP, false, true><<<(a.B + SK::kPerWave - 1) / SK::kPerWave, 64, smem, stream>>>(a);
