@@ -35,6 +35,20 @@ def _t(a):
     return torch.from_numpy(np.asarray(a))
 
 
+def _alpha_as_vector(g, like=None):
+    """The three alpha gradients are one float[3] output of the backward entry point
+    (mhc_layer_bwd_dynamic's dalpha) and are compared as that vector, like every other gradient
+    tensor: each is a single sum over batch and projection rows whose terms can cancel, and a
+    cancelled one (seen: 0.08 next to 62) is then measured against the scale of its siblings
+    instead of its own - plain float32 PyTorch misses such a value by 1e-4 of itself as well."""
+    g = dict(g)
+    like = g if like is None else like   # with an injected f the oracle has no alpha_pre entry
+    keys = [k for k in ("alpha_pre", "alpha_post", "alpha_res") if k in like]
+    if keys:
+        g["alpha"] = torch.stack([torch.as_tensor(g.pop(k)).reshape(()).double() for k in keys])
+    return g
+
+
 # ------------------------------------------------------------------------------------------------
 # golden vectors written from the reference's own naive layers
 # ------------------------------------------------------------------------------------------------
@@ -111,12 +125,14 @@ def test_dynamic_fp32_vs_oracle(B, n, C, inject):
     y_ref, g_ref = nm.mhc_dynamic_fwd_bwd(x, p, dy, T, eps, f_inject=f, dtype=torch.float64)
     y, g = hip_dynamic(x, p, dy, T, eps, f_inject=f)
     _check(y, y_ref, "fp32", "y")
+    assert set(g_ref) <= set(g), f"missing gradients {set(g_ref) - set(g)}"
+    if n > 1:
+        g, g_ref = _alpha_as_vector(g, g_ref), _alpha_as_vector(g_ref)
     for k, ref in g_ref.items():
-        assert k in g, f"missing gradient {k}"
         if n == 1 and k in ("phi_pre", "b_pre", "alpha_pre"):
             # one stream: f = RMSNorm(H_pre x) w does not depend on H_pre except through eps, so
-            # the true gradient is O(eps) and a relative comparison is meaningless
-            assert float(g[k].abs().max()) < 1e-4
+            # the true gradient is O(eps) (times the batch) and a relative comparison is meaningless
+            assert float((g[k].double() - torch.as_tensor(ref).double()).abs().max()) < 1e-4
             continue
         _check(g[k], ref, "fp32", "d" + k)
 
@@ -201,7 +217,7 @@ def test_bf16_small_n_coefficient_gradients_are_tight(B, n, C, inject, w_dtype):
         if inject and k in ("b_pre", "alpha_pre"):
             continue  # an injected f does not depend on H_pre
         if n == 1 and k in ("b_pre", "alpha_pre"):
-            assert float(g[k].abs().max()) < 1e-4  # O(eps), see test_dynamic_fp32_vs_oracle
+            assert float((g[k].double() - g_ref[k].double()).abs().max()) < 1e-4  # O(eps), see test_dynamic_fp32_vs_oracle
             continue
         e = rel_err(g[k], g_ref[k])
         assert e <= 2e-4, f"d{k}: normalised err {e:.3e}"
@@ -317,13 +333,17 @@ def test_random_shapes_vs_oracle(B, n, C, T, dyn, bf16, inject):
         y_ref, g_ref = nm.mhc_static_fwd_bwd(x, p, dy, T, eps, f_inject=f, dtype=ref_dtype)
         y, g = hip_static(x, p, dy, T, eps, f_inject=f, act_dtype=act, out_dtype=act, w_dtype=act)
     _check(y, y_ref, tier, "y")
+    assert set(g_ref) <= set(g), f"missing gradients {set(g_ref) - set(g)}"
+    if n > 1 and C > 1:
+        g, g_ref = _alpha_as_vector(g, g_ref), _alpha_as_vector(g_ref)
     for k, ref in g_ref.items():
-        assert k in g, f"missing gradient {k}"
-        tiny = ("phi_pre", "b_pre", "alpha_pre", "H_pre") + (("phi_res", "b_res", "alpha_res", "H_res") if T > 0 else ())
-        if n == 1 and k in tiny:
+        tiny = ("phi_pre", "b_pre", "alpha_pre", "H_pre") + (("phi_res", "b_res", "alpha_res", "H_res") if T > 0 and n == 1 else ())
+        # one channel: the inner RMSNorm maps the aggregate to its sign, so f does not depend on H_pre
+        # either (except through eps)
+        if (n == 1 or (C == 1 and not inject)) and k in tiny:
             # one stream: f does not depend on H_pre except through eps, and the 1 x 1 Sinkhorn output
             # (after at least one iteration) is 1 / (1 + O(eps)) whatever its logit, so these gradients are O(eps) (bf16: rounding
             # noise of that size) and a relative comparison is meaningless
-            assert float(g[k].abs().max()) < (1e-2 if bf16 else 1e-4), k
+            assert float((g[k].double() - torch.as_tensor(ref).double()).abs().max()) < (1e-2 if bf16 else 1e-4), k
             continue
         _check(g[k], ref, tier, "d" + k)
