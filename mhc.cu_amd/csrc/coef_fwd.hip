@@ -115,16 +115,19 @@ template <int NP, bool PRECISE> __global__ __launch_bounds__(256) void coef_fwd_
     if (dyn) {
         const float *pb = a.Ppart + (size_t)b * a.DP;
         constexpr int KB = MD > 2 ? 24 : 32;  // splits per round: up to 120 / 64 loads in flight per thread
+        // per-lane offsets once, the split's row as a uniform base: one address computation per
+        // load instead of a select and a 64-bit multiply-add each
+        int dm[MD];
+#pragma unroll
+        for (int m = 0; m < MD; m++) dm[m] = tid + 256 * m < D ? tid + 256 * m : 0;
         for (int k0 = 0; k0 < a.KS; k0 += KB) {
             float tv[MD][KB];
 #pragma unroll
-            for (int m = 0; m < MD; m++)
+            for (int q = 0; q < KB; q++) {
+                const float *row = pb + (size_t)(k0 + q < a.KS ? k0 + q : 0) * pstride;  // uniform
 #pragma unroll
-                for (int q = 0; q < KB; q++) {
-                    const int d = tid + 256 * m;
-                    const bool ok = d < D && k0 + q < a.KS;
-                    tv[m][q] = pb[ok ? (size_t)(k0 + q) * pstride + d : 0];
-                }
+                for (int m = 0; m < MD; m++) tv[m][q] = row[dm[m]];
+            }
 #pragma unroll
             for (int m = 0; m < MD; m++)
 #pragma unroll
