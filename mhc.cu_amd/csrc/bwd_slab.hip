@@ -16,6 +16,8 @@
 // of all streams, which finishes dx on the VALU and stores 16 bytes per stream.
 // Per tile: two barriers, x and dy read once from HBM, dx written once; no atomics.
 #include "launchers.h"
+
+#include <type_traits>
 #include "mhc_common.h"
 #include "phase_profiler.h"
 
@@ -23,6 +25,9 @@ namespace mhc {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 constexpr int kSlabCW = 64;                 // channels per slab
 constexpr int kSlabNS = 4;                  // streams (padded)
@@ -85,8 +90,32 @@ template <> struct Raw8<float> {
     }
 };
 
+// Four fp32 coefficients as two bf16x4 MFMA operands: the rounded values and their remainders.
+struct CoefRow {
+    bf16x4_t hi, lo;
+    __device__ __forceinline__ void set(float c0, float c1, float c2, float c3) {
+        const uint32_t h0 = pack_bf16x2(c0, c1), h1 = pack_bf16x2(c2, c3);
+        const uint32_t l0 = pack_bf16x2(c0 - bf16lo_to_f32(h0), c1 - bf16hi_to_f32(h0));
+        const uint32_t l1 = pack_bf16x2(c2 - bf16lo_to_f32(h1), c3 - bf16hi_to_f32(h1));
+        hi = __builtin_bit_cast(bf16x4_t, make_uint2(h0, h1));
+        lo = __builtin_bit_cast(bf16x4_t, make_uint2(l0, l1));
+    }
+};
+__device__ __forceinline__ f32x4_t mfma4(bf16x4_t a, bf16x4_t b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a, b, c, 0, 0, 0);
+}
+// The four streams of one channel as a bf16x4 operand, from the word of each stream that holds the
+// channel pair: the low halves (even channel) or the high halves (odd channel).
+template <bool ODD>
+__device__ __forceinline__ bf16x4_t streams_of_channel(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+    constexpr uint32_t sel = ODD ? 0x07060302u : 0x05040100u;
+    return __builtin_bit_cast(bf16x4_t, make_uint2(__builtin_amdgcn_perm(w1, w0, sel), __builtin_amdgcn_perm(w3, w2, sel)));
+}
+
 template <typename TG>
 __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
+    // bf16 dy: the per-sample 4x4 mixing of phase C runs on v_mfma_f32_4x4x4_16b_bf16 (below)
+    constexpr bool kMixMfma = std::is_same<TG, bf16_t>::value;
     extern __shared__ float smem_f[];
     float *dxf_s = smem_f;                                                  // [32][LDF] fp32
     bf16_t *x_s = reinterpret_cast<bf16_t *>(dxf_s + 32 * kSlabLDF);         // [32][LDX] bf16
@@ -182,7 +211,11 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
 
 
     MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 0, pclk);
-    for (int sb = b_begin; sb < b_end; sb += 32) {
+    // One tile: `cur` holds its data (requested a whole tile earlier); the next tile's loads go to
+    // `nxt` right behind this tile's small operand loads and have the three phases to arrive.  The
+    // loop alternates the two register sets instead of copying one into the other (a copy waits for
+    // the loads it copies).
+    auto process_tile = [&](int sb, TileRegs &cur, TileRegs &nxt) {
         const int b = sb + bl;
         const bool bok = b < b_end && cok;
         // MFMA operands that come straight from global memory: dP^T hi/lo (rows d) and dP (rows b);
@@ -200,20 +233,28 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
         // this thread's sample coefficients for phase C: asked for here so that they arrive behind
         // the barriers and the matrix-core phase (slots beyond the split alias sample 0, streams
         // >= n alias stream 0; both are discarded below)
-        float hpre[kSlabNS], hpost[kSlabNS], Mr[kSlabNS][kSlabNS], cxv, qv = 1.f, s1v = 0.f;
+        // (matrix-core mixing: a lane only needs column lane & 3 of M)
+        constexpr int MC = kMixMfma ? 1 : kSlabNS;
+        const int jq = tid & 3;
+        float hpre[kSlabNS], hpost[kSlabNS], Mr[kSlabNS][MC], cxv, qv = 1.f, s1v = 0.f;
         {
-            const size_t bc = bok ? b : 0;
+            // by sample only, whatever the lane's channel chunk: in the matrix-core mixing the four
+            // lanes of a block supply each other's coefficient rows
+            const size_t bc = b < b_end ? b : 0;
 #pragma unroll
             for (int i = 0; i < kSlabNS; i++) {
                 hpre[i] = a.Hpre[bc * n + (i < n ? i : 0)];
                 hpost[i] = a.Hpost[bc * n + (i < n ? i : 0)];
 #pragma unroll
-                for (int j = 0; j < kSlabNS; j++)
-                    Mr[i][j] = a.M[bc * n * n + ((i < n && j < n) ? i * n + j : 0)];
+                for (int j = 0; j < MC; j++) {
+                    const int jj = kMixMfma ? jq : j;
+                    Mr[i][j] = a.M[bc * n * n + ((i < n && jj < n) ? i * n + jj : 0)];
+                }
             }
             cxv = a.cx[bc];
             if (!inject) { qv = a.q[bc]; s1v = a.s1[bc]; }
         }
+        if (sb + 32 < b_end) load_tile(sb + 32, nxt);
         // x tile -> LDS
 #pragma unroll
         for (int j = 0; j < kSlabNS; j++)
@@ -259,9 +300,101 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
         __syncthreads();
         MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 2, pclk);
 
-        // ---- prefetch the next tile, then phase C: finish dx on the VALU ---------------------------
-        const bool more = sb + 32 < b_end;
-        if (more) load_tile(sb + 32, nxt);
+        // ---- phase C: finish dx ------------------------------------------------------------------
+        if constexpr (kMixMfma) {
+            // One v_mfma_f32_4x4x4_16b_bf16 is 16 independent 4x4x4 products; a block is four
+            // consecutive lanes, here four channel chunks of ONE sample.  With B = the four streams of
+            // a lane's channel (column = lane) and A = a coefficient matrix of the sample (row r from
+            // lane r of the block), lane l receives column l: the four output streams of its own channel.
+            //   D1 = G (M^T dy) + X (-(Hpre Hpre^T k2 + cx I) x)        rows: dx streams (without the
+            //   D2 = [Hpost; 0; 0; 0] dy + [0; Hpre; 0; 0] x             projection and da terms)
+            //                                                            rows 0, 1: df and the aggregate a
+            // Coefficients enter as bf16 value + remainder (two instructions each).  Every lane runs
+            // the instructions (lanes beyond the split or the channel range compute on aliased data
+            // that is never stored).
+            float qinv = 0.f, k2 = 0.f;
+            if (!inject) {
+                qinv = 1.0f / qv;
+                k2 = s1v * qinv * qinv * qinv / (float)C;
+            }
+#pragma unroll
+            for (int i = 0; i < kSlabNS; i++)
+                if (i >= n) { hpre[i] = 0.f; hpost[i] = 0.f; }
+            float mcol[kSlabNS], xrow[kSlabNS];
+            const float hq = jq == 0 ? hpre[0] : (jq == 1 ? hpre[1] : (jq == 2 ? hpre[2] : hpre[3]));  // Hpre[lane & 3]
+#pragma unroll
+            for (int i = 0; i < kSlabNS; i++) {
+                mcol[i] = (i < n && jq < n) ? Mr[i][0] : 0.f;
+                xrow[i] = -(hq * hpre[i] * k2 + (i == jq ? cxv : 0.f));
+            }
+            CoefRow cg, cxr, cdf, caa;
+            cg.set(mcol[0], mcol[1], mcol[2], mcol[3]);
+            cxr.set(xrow[0], xrow[1], xrow[2], xrow[3]);
+            const bool r0 = jq == 0, r1 = jq == 1;
+            cdf.set(r0 ? hpost[0] : 0.f, r0 ? hpost[1] : 0.f, r0 ? hpost[2] : 0.f, r0 ? hpost[3] : 0.f);
+            caa.set(r1 ? hpre[0] : 0.f, r1 ? hpre[1] : 0.f, r1 ? hpre[2] : 0.f, r1 ? hpre[3] : 0.f);
+            const uint32_t gw[kSlabNS][4] = {{cur.gr[0].r.x, cur.gr[0].r.y, cur.gr[0].r.z, cur.gr[0].r.w},
+                                             {cur.gr[1].r.x, cur.gr[1].r.y, cur.gr[1].r.z, cur.gr[1].r.w},
+                                             {cur.gr[2].r.x, cur.gr[2].r.y, cur.gr[2].r.z, cur.gr[2].r.w},
+                                             {cur.gr[3].r.x, cur.gr[3].r.y, cur.gr[3].r.z, cur.gr[3].r.w}};
+            const uint32_t xw[kSlabNS][4] = {{cur.xr[0].x, cur.xr[0].y, cur.xr[0].z, cur.xr[0].w},
+                                             {cur.xr[1].x, cur.xr[1].y, cur.xr[1].z, cur.xr[1].w},
+                                             {cur.xr[2].x, cur.xr[2].y, cur.xr[2].z, cur.xr[2].w},
+                                             {cur.xr[3].x, cur.xr[3].y, cur.xr[3].z, cur.xr[3].w}};
+            float dfv[8];
+            uint32_t dxw[kSlabNS][2];  // packed dx of the first half, stored with the second (16 bytes per stream)
+#pragma unroll
+            for (int h = 0; h < 2; h++) {  // two halves of four channels keep the accumulators small
+                f32x4_t d1[4], d2[4];
+                bf16x4_t bg[4], bx[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int p = 2 * h + (v >> 1);  // word of the channel pair
+                    if (v & 1) {
+                        bg[v] = streams_of_channel<true>(gw[0][p], gw[1][p], gw[2][p], gw[3][p]);
+                        bx[v] = streams_of_channel<true>(xw[0][p], xw[1][p], xw[2][p], xw[3][p]);
+                    } else {
+                        bg[v] = streams_of_channel<false>(gw[0][p], gw[1][p], gw[2][p], gw[3][p]);
+                        bx[v] = streams_of_channel<false>(xw[0][p], xw[1][p], xw[2][p], xw[3][p]);
+                    }
+                }
+                const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int v = 0; v < 4; v++) { d1[v] = mfma4(cg.hi, bg[v], zero); d2[v] = mfma4(cdf.hi, bg[v], zero); }
+#pragma unroll
+                for (int v = 0; v < 4; v++) { d1[v] = mfma4(cg.lo, bg[v], d1[v]); d2[v] = mfma4(cdf.lo, bg[v], d2[v]); }
+#pragma unroll
+                for (int v = 0; v < 4; v++) { d1[v] = mfma4(cxr.hi, bx[v], d1[v]); d2[v] = mfma4(caa.hi, bx[v], d2[v]); }
+#pragma unroll
+                for (int v = 0; v < 4; v++) { d1[v] = mfma4(cxr.lo, bx[v], d1[v]); d2[v] = mfma4(caa.lo, bx[v], d2[v]); }
+                float dw4[4];  // df * w / q per channel: the da term of dx is Hpre[j] times this
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const float s_df = d2[v][0], s_a = d2[v][1];
+                    dfv[4 * h + v] = s_df;
+                    dw4[v] = s_df * wv[4 * h + v] * qinv;
+                    usum[4 * h + v] += bok ? s_df * s_a * qinv : 0.f;
+                }
+                if (bok) {
+#pragma unroll
+                    for (int j = 0; j < kSlabNS; j++) {
+                        if (j < n) {
+                            const float4 p0 = *reinterpret_cast<const float4 *>(dxf_s + (size_t)bl * kSlabLDF + j * kSlabCW + ch * 8 + 4 * h);
+                            const float out[4] = {p0.x + d1[0][j] + hpre[j] * dw4[0], p0.y + d1[1][j] + hpre[j] * dw4[1],
+                                                  p0.z + d1[2][j] + hpre[j] * dw4[2], p0.w + d1[3][j] + hpre[j] * dw4[3]};
+                            if (h == 0) {
+                                dxw[j][0] = pack_bf16x2(out[0], out[1]);
+                                dxw[j][1] = pack_bf16x2(out[2], out[3]);
+                            } else {
+                                st16<true>(a.dx + (size_t)b * nC + (size_t)j * C + cth, dxw[j][0], dxw[j][1],
+                                           pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3]));
+                            }
+                        }
+                    }
+                }
+            }
+            if (bok && inject && a.df) store_vec<bf16_t, 8>(a.df + (size_t)b * C + cth, dfv);
+        } else
         if (bok) {
             float qinv = 0.f, k2 = 0.f;
 #pragma unroll
@@ -327,8 +460,11 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
         }
         // no barrier needed here: the next tile's x_s writes come after barrier 2 of this tile (all
         // fragment reads done) and its dxf_s writes come after its own barrier 1 (all phase C done)
-        if (more) cur = nxt;
         MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 3, pclk);
+    };
+    for (int sb = b_begin; sb < b_end; sb += 64) {
+        process_tile(sb, cur, nxt);
+        if (sb + 32 < b_end) process_tile(sb + 32, nxt, cur);
     }
 
     // ---- outputs of the split -----------------------------------------------------------------------
