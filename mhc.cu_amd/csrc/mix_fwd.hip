@@ -124,9 +124,10 @@ __global__ __launch_bounds__(256) void mix_fwd_kernel(MixFwdArgs a) {
 // Fused layer forward for n <= 8: coefficients + mix in one launch, x read from HBM exactly once.
 //
 // Every workgroup first issues the loads of its sample's whole [n, C] tile (kept in registers),
-// then 16 lanes of wave 0 turn the projection partial sums (dynamic H) or the shared logits
-// (static H) into H_pre, H_post and M - the Sinkhorn chain runs while the x loads are in
-// flight - and finally all threads aggregate, normalise and mix out of registers.
+// then the first lanes of wave 0 (16 for a 4x4 matrix, all 64 for 8x8) turn the projection partial
+// sums (dynamic H) or the shared logits (static H) into H_pre, H_post and M - the Sinkhorn chain
+// runs while the x loads are in flight - and finally all threads aggregate, normalise and mix out
+// of registers.
 // Replaces fused_h_activations + sinkhorn_knopp_forward_batched + stream_aggregate +
 // rmsnorm_forward_with_rms + stream_distribute_mix_add of the reference
 // (bindings.cu:449-477) by one kernel.
