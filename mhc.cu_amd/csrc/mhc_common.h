@@ -241,6 +241,19 @@ template <int NT> __device__ __forceinline__ float block_allreduce_sum(float v, 
     return total;
 }
 
+// The same for a workgroup of `nwaves` whole waves known only at run time.
+__device__ __forceinline__ float block_allreduce_sum(float v, float *red, int nwaves) {
+    v = wave_allreduce_sum(v);
+    if (nwaves == 1) return v;
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();  // previous readers of red are done
+    if ((threadIdx.x & (kWave - 1)) == 0) red[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int i = 0; i < nwaves; i++) total += red[i];
+    return total;
+}
+
 __device__ __forceinline__ float sigmoidf_acc(float t) { return 1.0f / (1.0f + expf(-t)); }
 
 // v_rcp_f32: 1 ulp, one instruction (an IEEE division costs ~10 dependent instructions, which

@@ -151,6 +151,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
     __shared__ float coef_s[NP * NP + 2 * NP];  // M | Hpre | Hpost
     __shared__ float red[4];
     const int b = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x;
+    const int nt = blockDim.x;  // whole waves, as few as hold the sample's chunks (256 for 8x8: the four waves share the split sums)
     const TX *__restrict__ xb = static_cast<const TX *>(a.x) + (size_t)b * n * C;
     TY *__restrict__ yb = static_cast<TY *>(a.y) + (size_t)b * n * C;
     const bool inject = a.f_inject != nullptr;
@@ -206,7 +207,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
     auto issue_tile = [&]() {
 #pragma unroll
         for (int k = 0; k < CPT; k++) {
-            const int ch = tid + k * 256;
+            const int ch = tid + k * nt;
             const TX *xc = xb + (size_t)(ch < nch ? ch : 0) * V;
 #pragma unroll
             for (int i = 0; i < NP; i++) xr[k][i].load(xc + (size_t)(i < n ? i : 0) * C);
@@ -214,7 +215,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
         if (inject) {
 #pragma unroll
             for (int k = 0; k < CPT; k++) {
-                const int ch = tid + k * 256;
+                const int ch = tid + k * nt;
                 fr[k].load(static_cast<const TX *>(a.f_inject) + (size_t)b * C + (size_t)(ch < nch ? ch : 0) * V);
             }
         }
@@ -333,7 +334,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
         float ssq = 0.f;
 #pragma unroll
         for (int k = 0; k < CPT; k++) {
-            const bool live = tid + k * 256 < nch;  // chunks beyond C alias chunk 0: not counted
+            const bool live = tid + k * nt < nch;  // chunks beyond C alias chunk 0: not counted
             float s_a[V];
 #pragma unroll
             for (int v = 0; v < V; v++) s_a[v] = 0.f;
@@ -350,7 +351,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
                 ssq += live ? s_a[v] * s_a[v] : 0.f;
             }
         }
-        ssq = block_allreduce_sum<256>(ssq, red);
+        ssq = block_allreduce_sum(ssq, red, nt / kWave);
         const float q = sqrtf(ssq / (float)C + a.eps);
         qinv = 1.0f / q;
         if (tid == 0 && a.q) a.q[b] = q;
@@ -362,7 +363,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
     // ---- 4. mix + distribute -------------------------------------------------------------------
 #pragma unroll
     for (int k = 0; k < CPT; k++) {
-        const int ch = tid + k * 256;
+        const int ch = tid + k * nt;
         if (ch < nch) {
             const int c = ch * V;
             float f[V];
@@ -416,9 +417,13 @@ static bool launch_fused_small(const LayerFwdArgs &a, hipStream_t stream, hipErr
     if (a.C % V != 0) return false;
     const int nch = a.C / V;
     const int cpt = (nch + 255) / 256;
-    if (cpt == 1) layer_fwd_small_kernel<TX, TY, NP, V, 1><<<a.B, 256, 0, stream>>>(a);
-    else if (cpt == 2) layer_fwd_small_kernel<TX, TY, NP, V, 2><<<a.B, 256, 0, stream>>>(a);
-    else if (cpt <= 4 && NP == 4) layer_fwd_small_kernel<TX, TY, 4, V, 4><<<a.B, 256, 0, stream>>>(a);
+    // as few whole waves as hold the chunks: a thread without a chunk of its own still runs the loads
+    // and the arithmetic on an aliased one (320 chunks on 2 x 256 slots would waste 37 % of both)
+    const int per = cpt == 3 ? 4 : cpt;  // chunks per thread of the instantiation that runs
+    const int nt = NP == 8 ? 256 : round_up((nch + per - 1) / per, kWave);
+    if (cpt == 1) layer_fwd_small_kernel<TX, TY, NP, V, 1><<<a.B, nt, 0, stream>>>(a);
+    else if (cpt == 2) layer_fwd_small_kernel<TX, TY, NP, V, 2><<<a.B, nt, 0, stream>>>(a);
+    else if (cpt <= 4 && NP == 4) layer_fwd_small_kernel<TX, TY, 4, V, 4><<<a.B, nt, 0, stream>>>(a);
     else return false;
     *err = hipGetLastError();
     return true;
