@@ -12,6 +12,7 @@
 //   proj_fwd_generic_kernel any dtype / any C: fp32 FMA, exact products (the fp32 parity tier).
 #include "launchers.h"
 #include "mhc_common.h"
+#include "phase_profiler.h"
 
 namespace mhc {
 
@@ -87,6 +88,10 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
     const int set = (blockIdx.x >> 3) / tiles_s;
     const int st = (blockIdx.x >> 3) % tiles_s, ks = (blockIdx.x & 7) + 8 * set;
     if (ks >= KS) return;  // the whole workgroup, before any barrier
+    const int pwg = blockIdx.y * gridDim.x + blockIdx.x;
+    (void)pwg;
+    MHC_PHASE_ZERO(kPhaseProjFwd, pwg);
+    MHC_PHASE_BEGIN(pclk);
     const int row = lane & 31, kh = lane >> 5;
     const int b = st * 32 + row;
     const int dbase = blockIdx.y * NT * 32;
@@ -151,8 +156,10 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
     float ssq = 0.f;
 
     if (kbeg < kend) fetch(kbeg);
+    MHC_PHASE_ADD(kPhaseProjFwd, pwg, 0, pclk);
     for (int k0 = kbeg; k0 < kend; k0 += 64) {
         park();
+        MHC_PHASE_ADD(kPhaseProjFwd, pwg, 1, pclk);
         if (k0 + 64 < kend) fetch(k0 + 64);  // in flight while this chunk is multiplied
 #pragma unroll
         for (int u = 0; u < 4; u++) {
@@ -173,6 +180,7 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
                 }
             }
         }
+        MHC_PHASE_ADD(kPhaseProjFwd, pwg, 2, pclk);
     }
     __syncthreads();  // every wave is done with its chunk tile: the memory becomes the cross-wave buffer
     ssq = xor32_add(ssq);  // both K halves of the row
@@ -212,6 +220,7 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
         }
         if (blockIdx.y == 0 && kh == 0 && bvalid) ssqpart[(size_t)ks * B + b] = ssq;
     }
+    MHC_PHASE_ADD(kPhaseProjFwd, pwg, 3, pclk);
 }
 
 // --------------------------------------------------------------------------------------------

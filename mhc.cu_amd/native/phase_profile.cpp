@@ -100,6 +100,12 @@ int main(int argc, char **argv) {
     summary("fused forward kernel, one workgroup per sample", 0, std::min(B, 4096),
             {"issue loads (early half: tile too)", "coefficient inputs arrive", "activations + Sinkhorn", "tile request (late half), barrier", "tile arrives, aggregate, RMS",
              "mix, stores issued"}, true);
+    {
+        const int tiles = (B + 31) / 32;
+        summary("narrow projection kernel, one workgroup per (32 samples, K slab), wave 0 of each", 3, std::min(tiles * 16, 4096),
+                {"start, first chunk requested", "waits for chunks, parks (all chunks)", "fragments, matrix cores (all chunks)",
+                 "cross-wave sum, partial stores"}, false);
+    }
     if (n > 4) {
         summary("projection backward kernel, one workgroup per 32 columns of x_flat", 2, std::min((int)(nC / 32), 4096),
                 {"prologue (phi slab, first x block requested)", "operands requested, x block parked (all blocks)",
