@@ -55,9 +55,6 @@ struct DPWriter {
     int b, B, DP;
     __device__ __forceinline__ void put(int d, float v) const {
         o.dP[(size_t)b * DP + d] = v;
-#ifdef MHC_EXP_NO_DPW
-        return;
-#endif
         if (o.dPb) {
             const bf16_t h = f32_to_bf16(v);
             const size_t plane = (size_t)DP * o.BP;
