@@ -192,11 +192,13 @@ int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype
                                           st));
         return MHC_OK;
     }
+    // n > 8 in the bf16 tier: the coefficient launch also forms the stream aggregate and its RMS
+    const bool agg = !f_inject && ws.agg && coef_fwd_aggregates(n, C, x_dtype);
     MHC_LAUNCH(launch_coef_fwd(ws.Ppart, ws.ssqpart, KS, padded_D(n), alpha, bias, bias + n,
                                bias + 2 * n, H_pre, H_post, M, P, r, B, n, n * C, iters, eps,
-                               x_dtype == kF32, st));
+                               x_dtype == kF32, agg ? x : nullptr, ws.agg, q, st));
     MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, H_pre, H_post, M, n, q,
-                              ws.agg, B, n, C, eps, st));
+                              ws.agg, B, n, C, eps, agg, st));
     return MHC_OK;
 }
 
@@ -300,9 +302,9 @@ int mhc_layer_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
     float *m = M ? M : ws.M, *qq = q ? q : ws.q;
     MHC_LAUNCH(launch_coef_fwd(nullptr, nullptr, 0, 0, nullptr, H_pre_logits, H_post_logits,
                                H_res_logits, hp, ho, m, nullptr, nullptr, 1, n, n * C, iters, eps,
-                               x_dtype == kF32, st));
+                               x_dtype == kF32, nullptr, nullptr, nullptr, st));
     MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, hp, ho, m, 0, qq,
-                              n > 8 ? ws.agg : nullptr, B, n, C, eps, st));
+                              n > 8 ? ws.agg : nullptr, B, n, C, eps, false, st));
     return MHC_OK;
 }
 

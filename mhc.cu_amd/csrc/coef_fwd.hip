@@ -21,6 +21,10 @@ struct CoefArgs {
     float *P, *r;             // [B,D], [B]  (dynamic only)
     int B, n, nC, T;
     float eps;
+    // n > 8, bf16 x, one 16-byte chunk of every stream per thread (C <= 2048): the kernel also forms the
+    // stream aggregate a = Hpre^T x (fp32 [B, C]) and its RMS q, from loads that fly under the Sinkhorn chain
+    const bf16_t *x_agg;
+    float *a_ws, *q;
 };
 
 // eight loads in flight per round (a plain loop would pay one memory latency per split)
@@ -81,8 +85,11 @@ template <int NP> __global__ __launch_bounds__(64) void coef_fwd_small_kernel(Co
 // One workgroup (4 waves) per sample.  All 256 threads finish the split-K sums (D = n^2 + 2n
 // logits, KS partial sums each, eight loads in flight per thread), then run Sinkhorn with the
 // matrix spread over their registers (SkWg).
-template <int NP, bool PRECISE> __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
+template <int NP, bool PRECISE, bool AGG = false>
+__global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     using SK = SkWg<NP>;
+    __shared__ float hp_s[AGG ? 32 : 1];
+    __shared__ float red_s[4];
     extern __shared__ __align__(16) float lds[];
     float *lg = lds;                       // [NP*NP + 2*NP] logits: pre | post | res (row-major n x n)
     float *sk_s = lg + NP * NP + 2 * NP;   // SK::lds_floats(T)
@@ -156,8 +163,22 @@ template <int NP, bool PRECISE> __global__ __launch_bounds__(256) void coef_fwd_
     }
     __syncthreads();
     if (tid < n) {
-        a.Hpre[b * n + tid] = sigmoidf_acc(lg[tid]);
+        const float hp = sigmoidf_acc(lg[tid]);
+        a.Hpre[b * n + tid] = hp;
         a.Hpost[b * n + tid] = 2.0f * sigmoidf_acc(lg[n + tid]);
+        if constexpr (AGG) hp_s[tid] = hp;
+    } else if (AGG && tid < 32) {
+        hp_s[tid] = 0.f;
+    }
+    // AGG: this thread's chunk of every stream is requested now and consumed behind the Sinkhorn
+    // chain (whose barriers also publish hp_s); streams >= n alias stream 0 and meet Hpre = 0
+    constexpr int NS = AGG ? NP : 1;
+    RawVec<bf16_t, 8> xr[NS];
+    const int C = a.nC / n, nch = C / 8;
+    if constexpr (AGG) {
+        const bf16_t *xb = a.x_agg + (size_t)b * a.nC + (size_t)(tid < nch ? tid : 0) * 8;
+#pragma unroll
+        for (int i = 0; i < NS; i++) xr[i].load(xb + (size_t)(i < n ? i : 0) * C);
     }
     const int r0 = SK::row(tid), c0 = SK::col0(tid);
     float E[SK::EPL], u, v[SK::EPL];
@@ -168,14 +189,37 @@ template <int NP, bool PRECISE> __global__ __launch_bounds__(256) void coef_fwd_
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         if (r0 < n && c0 + e < n) a.M[(size_t)b * n * n + r0 * n + c0 + e] = u * E[e] * v[e];
+    if constexpr (AGG) {
+        __syncthreads();  // hp_s (with zero iterations the Sinkhorn step has no barrier of its own)
+        float acc[8], ssq = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) acc[k] = 0.f;
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            float xv[8];
+            xr[i].get(xv);
+            const float hp = hp_s[i];
+#pragma unroll
+            for (int k = 0; k < 8; k++) acc[k] += hp * xv[k];
+        }
+        if (tid < nch) {
+            store_vec<float, 8>(a.a_ws + (size_t)b * C + tid * 8, acc);
+#pragma unroll
+            for (int k = 0; k < 8; k++) ssq += acc[k] * acc[k];
+        }
+        ssq = block_allreduce_sum<256>(ssq, red_s);
+        if (tid == 0) a.q[b] = sqrtf(ssq / (float)C + a.eps);
+    }
 }
 
 hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int DP,
                            const float *alpha, const float *b_pre, const float *b_post,
                            const float *b_res, float *Hpre, float *Hpost, float *M, float *P,
                            float *r, int B, int n, int nC, int T, float eps, bool precise,
-                           hipStream_t stream) {
-    CoefArgs a{Ppart, ssqpart, KS, DP, alpha, b_pre, b_post, b_res, Hpre, Hpost, M, P, r, B, n, nC, T, eps};
+                           const void *x_agg, float *a_ws, float *q, hipStream_t stream) {
+    CoefArgs a{Ppart, ssqpart, KS, DP, alpha, b_pre, b_post, b_res, Hpre, Hpost, M, P, r, B, n, nC, T, eps,
+               static_cast<const bf16_t *>(x_agg), a_ws, q};
+    const bool agg = x_agg != nullptr;  // the caller has checked coef_fwd_aggregates()
     if (n <= 4)
         coef_fwd_small_kernel<4><<<(B + 3) / 4, 64, 0, stream>>>(a);
     else if (n <= 8)
@@ -185,17 +229,31 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
         hipError_t e = precise ? allow_dynamic_lds(&coef_fwd_lds_kernel<16, true>, smem)
                                : allow_dynamic_lds(&coef_fwd_lds_kernel<16, false>, smem);
         if (e != hipSuccess) return e;
-        if (precise) coef_fwd_lds_kernel<16, true><<<B, 256, smem, stream>>>(a);
+        if (agg) {
+            e = allow_dynamic_lds(&coef_fwd_lds_kernel<16, false, true>, smem);
+            if (e != hipSuccess) return e;
+            coef_fwd_lds_kernel<16, false, true><<<B, 256, smem, stream>>>(a);
+        } else if (precise) coef_fwd_lds_kernel<16, true><<<B, 256, smem, stream>>>(a);
         else coef_fwd_lds_kernel<16, false><<<B, 256, smem, stream>>>(a);
     } else {
         const size_t smem = sizeof(float) * (32 * 32 + 64 + SkWg<32>::lds_floats(T));
         hipError_t e = precise ? allow_dynamic_lds(&coef_fwd_lds_kernel<32, true>, smem)
                                : allow_dynamic_lds(&coef_fwd_lds_kernel<32, false>, smem);
         if (e != hipSuccess) return e;
-        if (precise) coef_fwd_lds_kernel<32, true><<<B, 256, smem, stream>>>(a);
+        if (agg) {
+            e = allow_dynamic_lds(&coef_fwd_lds_kernel<32, false, true>, smem);
+            if (e != hipSuccess) return e;
+            coef_fwd_lds_kernel<32, false, true><<<B, 256, smem, stream>>>(a);
+        } else if (precise) coef_fwd_lds_kernel<32, true><<<B, 256, smem, stream>>>(a);
         else coef_fwd_lds_kernel<32, false><<<B, 256, smem, stream>>>(a);
     }
     return hipGetLastError();
+}
+
+// Whether launch_coef_fwd can also produce the stream aggregate and its RMS for this shape (dynamic
+// H, n > 8, bf16 x, one 16-byte chunk per thread and stream).
+bool coef_fwd_aggregates(int n, int C, int x_dtype) {
+    return n > 8 && x_dtype == kBF16 && C % 8 == 0 && C / 8 <= 256;
 }
 
 }  // namespace mhc

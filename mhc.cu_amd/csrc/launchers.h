@@ -42,7 +42,11 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
                            const float *alpha, const float *b_pre, const float *b_post,
                            const float *b_res, float *Hpre, float *Hpost, float *M, float *P,
                            float *r, int B, int n, int nC, int T, float eps, bool precise,
-                           hipStream_t stream);
+                           const void *x_agg, float *a_ws, float *q, hipStream_t stream);
+// x_agg != nullptr (only where coef_fwd_aggregates() holds): the launch also writes the stream
+// aggregate a = Hpre^T x (a_ws, fp32 [B, C]) and its RMS q, which launch_mix_fwd then takes as given
+// (have_agg).
+bool coef_fwd_aggregates(int n, int C, int x_dtype);
 // precise: IEEE divisions in the n > 8 Sinkhorn (fp32 parity tier); otherwise v_rcp_f32
 
 // y = M x + Hpost (x) f, f = RMSNorm(Hpre . x) * w or f_inject.  hstride = n (per-sample
@@ -50,7 +54,7 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
 hipError_t launch_mix_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
                           const void *f_inject, void *y, int y_dtype, const float *Hpre,
                           const float *Hpost, const float *M, int hstride, float *q, float *a_ws,
-                          int B, int n, int C, float eps, hipStream_t stream);
+                          int B, int n, int C, float eps, bool have_agg, hipStream_t stream);
 // a_ws: scratch of B * C floats, needed (with q) by the matrix-core path, see mix_fwd_large_supported
 bool mix_fwd_large_supported(int n, int C, int x_dtype);
 

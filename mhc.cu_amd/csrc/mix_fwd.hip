@@ -624,8 +624,8 @@ __global__ __launch_bounds__(256) void mix_fwd_large_kernel(MixLargeArgs a) {
     }
 }
 
-static hipError_t launch_large_mfma(const MixLargeArgs &a, int y_dtype, hipStream_t stream) {
-    if (!a.f_inject) {
+static hipError_t launch_large_mfma(const MixLargeArgs &a, int y_dtype, bool have_agg, hipStream_t stream) {
+    if (!a.f_inject && !have_agg) {
         agg_large_kernel<<<a.B, 256, 0, stream>>>(a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -669,11 +669,11 @@ static hipError_t launch_t(const MixFwdArgs &a, hipStream_t stream) {
 hipError_t launch_mix_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
                           const void *f_inject, void *y, int y_dtype, const float *Hpre,
                           const float *Hpost, const float *M, int hstride, float *q, float *a_ws,
-                          int B, int n, int C, float eps, hipStream_t stream) {
+                          int B, int n, int C, float eps, bool have_agg, hipStream_t stream) {
     if (mix_fwd_large_supported(n, C, x_dtype) && (f_inject || (a_ws && q))) {
         MixLargeArgs la{static_cast<const bf16_t *>(x), w, static_cast<const bf16_t *>(f_inject), y, Hpre, Hpost,
                         M, q, a_ws, hstride, w_dtype == kBF16, B, n, C, eps};
-        return launch_large_mfma(la, y_dtype, stream);
+        return launch_large_mfma(la, y_dtype, have_agg, stream);
     }
     MixFwdArgs a{x, w, f_inject, y, Hpre, Hpost, M, q, hstride, w_dtype == kBF16, B, n, C, eps};
     if (x_dtype == kF32 && y_dtype == kF32) return launch_t<float, float>(a, stream);
