@@ -265,6 +265,8 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
     int r0, c0, gc;
     bool inject, mv;
     float qinv, rinv, al0, al1, al2, pres, bres, hp, ho, ppre, ppost, hpre_r, hpost_r;
+    float E, m_fin;  // exp(logit) and the final Sinkhorn iterate of this lane's element (forward_recompute)
+    float dMe, s_a, s_b, s_c, s_d;  // this lane's channel sums (fetch_sums): GRAM w1, w1t, xx | else dHpost, A1, A2, s1
 
     __device__ __forceinline__ void prefetch(const BwdReduceArgs &a, int b, int g) {
         const int n = a.n, D = n * n + 2 * n;
@@ -284,26 +286,44 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
         hpost_r = a.Hpost[(size_t)b * n + (r0 < n ? r0 : 0)];
     }
 
-    // g: lane within the group; lane: lane within the wave (indexes the denominators in sc);
-    // xch: kXch floats of LDS private to the group
-    __device__ __forceinline__ void run(const BwdReduceArgs &a, int b, int g, int lane, const float *sums,
-                                        int parts, float *sc, float *xch) {
+    // The Sinkhorn forward recompute, which keeps the denominators of every iteration in sc: it needs
+    // none of the channel sums, so a caller that produces them itself can run it while they are
+    // still on their way.  g: lane within the group; lane: lane within the wave (indexes sc).
+    __device__ __forceinline__ void forward_recompute(const BwdReduceArgs &a, int g, int lane, float *sc) {
+        E = mv ? expf(al2 * pres + bres) : 0.f;
+        float m[1] = {E};
+        SK::template forward<PRECISE>(m, g, a.n, a.T, a.eps, sc, lane);
+        m_fin = m[0];
+    }
+
+    // This lane's entries of the channel sums, summed over the column parts.
+    __device__ __forceinline__ void fetch_sums(const float *sums, int parts) {
+        dMe = s_a = s_b = s_c = s_d = 0.f;
+        for (int p = 0; p < parts; p++) {
+            const float *rp = sums + (size_t)p * K;
+            dMe += rp[r0 * NP + c0];
+            if constexpr (GRAM) {
+                s_a += rp[NP * NP + r0 * NP + c0];
+                s_b += rp[NP * NP + c0 * NP + r0];
+                s_c += rp[2 * NP * NP + r0 * NP + c0];
+            } else {
+                s_a += rp[NP * NP + gc]; s_b += rp[NP * NP + NP + gc]; s_c += rp[NP * NP + 2 * NP + gc];
+                s_d += rp[K - 1];
+            }
+        }
+    }
+
+    // after fetch_sums() and forward_recompute(); xch: kXch floats of LDS private to the group
+    __device__ __forceinline__ void run(const BwdReduceArgs &a, int b, int g, int lane, float *sc, float *xch) {
         const int n = a.n, C = a.C, D = n * n + 2 * n;
-        float dMe = 0.f, tpost = 0.f, tA1 = 0.f, tA2 = 0.f, s1 = 0.f;
+        float tpost = 0.f, tA1 = 0.f, tA2 = 0.f, s1 = 0.f;
         if constexpr (GRAM) {
             // lane (r0, c0) takes its element of each matrix and the mirrored element of W1, so that
             // every sum below runs down a column:
             //   dHpost[c] = sum_r Hpre[r] W1[c][r] / q        A1[c] = sum_r Hpost[r] W1[r][c]
             //   A2[c] = sum_r Hpre[r] XX[r][c]                s1 = sum_c Hpost[c] (sum_r Hpre[r] W1[c][r])
             // The column results are handed to lanes 0 .. n-1 through LDS (same wave: no barrier).
-            float w1 = 0.f, w1t = 0.f, xx = 0.f;
-            for (int p = 0; p < parts; p++) {
-                const float *rp = sums + (size_t)p * K;
-                dMe += rp[r0 * NP + c0];
-                w1 += rp[NP * NP + r0 * NP + c0];
-                w1t += rp[NP * NP + c0 * NP + r0];
-                xx += rp[2 * NP * NP + r0 * NP + c0];
-            }
+            const float w1 = s_a, w1t = s_b, xx = s_c;
             const float hr = r0 < n ? hpre_r : 0.f, hor = r0 < n ? hpost_r : 0.f;
             // with an injected f, W1 = dy [f; 0; ...]^T and dHpost is its column 0
             const float sel = inject ? (r0 == 0 ? 1.f : 0.f) : hr;
@@ -321,12 +341,7 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
                 s1 = SK::group_allreduce(g < n ? ho * hw : 0.f);
             }
         } else {
-            for (int p = 0; p < parts; p++) {
-                const float *rp = sums + (size_t)p * K;
-                dMe += rp[r0 * NP + c0];
-                tpost += rp[NP * NP + gc]; tA1 += rp[NP * NP + NP + gc]; tA2 += rp[NP * NP + 2 * NP + gc];
-                s1 += rp[K - 1];
-            }
+            tpost = s_a; tA1 = s_b; tA2 = s_c; s1 = s_d;
         }
         if (g == 0) a.out.s1[b] = s1;
         float *dt = a.out.dt + (size_t)b * (D + 3);
@@ -341,9 +356,7 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
             dpw.put(g, dtp * al0 * rinv); dpw.put(n + g, dto * al1 * rinv);
             S0 = dtp * ppre; S1 = dto * ppost;
         }
-        const float E = mv ? expf(al2 * pres + bres) : 0.f;
-        float m[1] = {E}, d[1] = {mv ? dMe : 0.f};
-        SK::template forward<PRECISE>(m, g, n, a.T, a.eps, sc, lane);
+        float m[1] = {m_fin}, d[1] = {mv ? dMe : 0.f};
         SK::template backward<PRECISE>(d, m, a.T, sc, lane);
         if (mv) {
             const int di = 2 * n + r0 * n + c0;
@@ -374,8 +387,9 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
     if (b >= a.B) return;  // whole groups leave together; the reductions never cross groups
     CB cb;
     cb.prefetch(a, b, g);
-    cb.run(a, b, g, tid, a.raw + (size_t)b * a.parts * CB::K, a.parts, sc,
-           sc + SK::scaling_floats(a.T) + (tid / SK::kGroup) * CB::kXch);
+    cb.fetch_sums(a.raw + (size_t)b * a.parts * CB::K, a.parts);  // requested before the chain, used after it
+    cb.forward_recompute(a, g, tid, sc);
+    cb.run(a, b, g, tid, sc, sc + SK::scaling_floats(a.T) + (tid / SK::kGroup) * CB::kXch);
 }
 
 // =============================================================================================
@@ -423,7 +437,12 @@ __global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     CB cb;
     if constexpr (FUSED) {
-        if (tid < SK::kGroup) cb.prefetch(a, b, tid);
+        // the Sinkhorn forward recompute needs none of the sums: it runs here, on the first lanes of
+        // wave 0, while the other waves already stream (and not at the tail of the workgroup)
+        if (tid < SK::kGroup) {
+            cb.prefetch(a, b, tid);
+            cb.forward_recompute(a, tid, tid, sc);
+        }
     }
     const int blk = lane >> 2, i = lane & 3;
     const int nsteps = (C + 127) / 128, spp = (nsteps + a.parts - 1) / a.parts;
@@ -544,7 +563,10 @@ __global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
     }
     if constexpr (FUSED) {
         __syncthreads();
-        if (tid < SK::kGroup) cb.run(a, b, tid, tid, tot_s, 1, sc, sc + SK::scaling_floats(a.T));
+        if (tid < SK::kGroup) {
+            cb.fetch_sums(tot_s, 1);
+            cb.run(a, b, tid, tid, sc, sc + SK::scaling_floats(a.T));
+        }
     }
 }
 
