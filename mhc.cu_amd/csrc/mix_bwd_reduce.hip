@@ -15,6 +15,7 @@
 // n > 8 computes three 32x32 Gram matrices per sample on the matrix cores (operands loaded from
 // global memory in MFMA layout) from which all the sums above follow.
 #include "launchers.h"
+#include "phase_profiler.h"
 #include "sinkhorn_device.h"
 
 namespace mhc {
@@ -435,6 +436,10 @@ __global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
     extern __shared__ float sc[];     // FUSED: Sinkhorn denominators, SK::scaling_floats(T), then CB::kXch
     const int b = blockIdx.x, part = blockIdx.y, n = a.n, C = a.C;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int pwg = blockIdx.y * gridDim.x + blockIdx.x;
+    (void)pwg;
+    MHC_PHASE_ZERO(kPhaseGramSmall, pwg);
+    MHC_PHASE_BEGIN(pclk);
     CB cb;
     if constexpr (FUSED) {
         // the Sinkhorn forward recompute needs none of the sums: it runs here, on the first lanes of
@@ -465,15 +470,20 @@ __global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
         for (int I = 0; I < NB; I++)
 #pragma unroll
             for (int J = 0; J < NB; J++) acc[m][I][J] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    MHC_PHASE_ADD(kPhaseGramSmall, pwg, 0, pclk);
 
-    for (int s0 = s_begin + wave; s0 < s_end; s0 += 4 * U) {
+    // FUSED: wave 0 is busy with the forward recompute while the others stream, so the steps are
+    // shared by waves 1 .. 3 only
+    constexpr int SW = FUSED ? 3 : 4;  // streaming waves
+    const int sw = FUSED ? wave - 1 : wave;
+    for (int s0 = sw >= 0 ? s_begin + sw : s_end; s0 < s_end; s0 += SW * U) {
         uint4 gr[U][NB], xr[U][NB], fr[U];
         RawVec<bf16_t, 8> wb[U];
         RawVec<float, 8> wf[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int c = (s0 + 4 * u) * 128 + blk * 8;
-            const bool in = s0 + 4 * u < s_end && c < C;  // C % 8 == 0: a chunk is inside or outside
+            const int c = (s0 + SW * u) * 128 + blk * 8;
+            const bool in = s0 + SW * u < s_end && c < C;  // C % 8 == 0: a chunk is inside or outside
             const int cc = in ? c : 0;
 #pragma unroll
             for (int I = 0; I < NB; I++) {
@@ -536,6 +546,7 @@ __global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
         }
     }
 
+    MHC_PHASE_ADD(kPhaseGramSmall, pwg, 1, pclk);
     // Lane (block, j) holds column j of its block's products, register = row.  Sum over the four
     // blocks of a 16-lane row with DPP, one LDS slot per row, then K threads finish.
     const int slot = tid >> 4;
@@ -563,10 +574,12 @@ __global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
     }
     if constexpr (FUSED) {
         __syncthreads();
+        MHC_PHASE_ADD(kPhaseGramSmall, pwg, 2, pclk);
         if (tid < SK::kGroup) {
             cb.fetch_sums(tot_s, 1);
             cb.run(a, b, tid, tid, sc, sc + SK::scaling_floats(a.T));
         }
+        MHC_PHASE_ADD(kPhaseGramSmall, pwg, 3, pclk);
     }
 }
 

@@ -106,6 +106,9 @@ int main(int argc, char **argv) {
                 {"start, first chunk requested", "waits for chunks, parks (all chunks)", "fragments, matrix cores (all chunks)",
                  "cross-wave sum, partial stores"}, false);
     }
+    summary("channel sums + coefficient backward kernel, one workgroup per sample", 4, std::min(B, 4096),
+            {"start: coefficient inputs, Sinkhorn forward recompute (wave 0)", "streaming loop (wave 0's steps)",
+             "workgroup sums", "coefficient backward (Sinkhorn reverse sweep, dP stores)"}, false);
     if (n > 4) {
         summary("projection backward kernel, one workgroup per 32 columns of x_flat", 2, std::min((int)(nC / 32), 4096),
                 {"prologue (phi slab, first x block requested)", "operands requested, x block parked (all blocks)",
