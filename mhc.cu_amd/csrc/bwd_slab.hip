@@ -481,6 +481,7 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
             }
         }
     }
+    MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 4, pclk);
     __syncthreads();  // everyone is done with dxf_s; reuse it for the two small reductions
     if (!inject) {
         // dw summands: sum over the 32 sample slots that share a channel chunk
@@ -507,7 +508,7 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
             a.dt_part[(size_t)blockIdx.y * (D + 3) + tid] = s;
         }
     }
-    MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 4, pclk);
+    MHC_PHASE_ADD(kPhaseBwdSlab, pwg, 5, pclk);
 }
 
 bool bwd_slab_supported(int x_dtype, int y_dtype, int phi_dtype, int n, int C) {

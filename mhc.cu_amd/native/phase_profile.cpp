@@ -118,6 +118,6 @@ int main(int argc, char **argv) {
     const int slabs = (C + 63) / 64;
     summary("slab backward kernel, one workgroup per (64 channels, batch split)", 1, std::min(slabs * 4, 4096),
             {"prologue (phi slab, first loads)", "tile loads, LDS, barrier (all tiles)", "matrix cores, barrier (all tiles)",
-             "coefficients, VALU, stores (all)", "epilogue (partials)"}, false);
+             "coefficients, mixing, stores (all)", "epilogue: dphi partial stores", "epilogue: dw / dbias partial sums"}, false);
     return 0;
 }
