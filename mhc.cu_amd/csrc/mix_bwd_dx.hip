@@ -9,6 +9,7 @@
 // Also writes df (kernel-level view) and u[b,c] = df a / q, the per-sample summand of dw.
 #include "launchers.h"
 #include "mhc_common.h"
+#include "phase_profiler.h"
 
 namespace mhc {
 
@@ -31,6 +32,10 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
     extern __shared__ float smem[];
     float *M_s = smem;  // [NP*NP] (NP >= 16 only)
     const int grp = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x, nt = blockDim.x;
+    const int pwg = blockIdx.y * gridDim.x + blockIdx.x;
+    (void)pwg;
+    MHC_PHASE_ZERO(kPhaseDxSmall, pwg);
+    MHC_PHASE_BEGIN(pclk);
     const int b_first = grp * a.spg, b_last = min(a.B, b_first + a.spg);
     const bool inject = a.f_inject != nullptr;
     const int D = n * n + 2 * n, nC = n * C;
@@ -45,7 +50,11 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
     }
     // grid.y workgroups share the channels of a sample group
     const int nch = C / V;
-    for (int ch = blockIdx.y * nt + tid; ch < nch; ch += nt * gridDim.y) {
+    // The loop runs for whole workgroups (all lanes take part in staging M); a lane without a chunk of
+    // its own works on chunk 0 and stores nothing.
+    for (int ch0 = blockIdx.y * nt; ch0 < nch; ch0 += nt * gridDim.y) {
+      const bool live = ch0 + tid < nch;
+      const int ch = live ? ch0 + tid : 0;
       const int c = ch * V;
       float usum[V];
 #pragma unroll
@@ -57,23 +66,17 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
         const float *__restrict__ Hpre = a.Hpre + (size_t)b * a.hstride;
         const float *__restrict__ Hpost = a.Hpost + (size_t)b * a.hstride;
         const float *__restrict__ M = a.M + (size_t)b * a.hstride * n;
-        const float qinv = inject ? 0.f : 1.0f / a.q[b];
-        const float k2 = inject ? 0.f : a.s1[b] * qinv * qinv * qinv / (float)C;
-        const float cx = a.cx ? a.cx[b] : 0.f;
-        float hpre[NP], hpost[NP];
-#pragma unroll
-        for (int i = 0; i < NP; i++) {
-            hpre[i] = i < n ? Hpre[i] : 0.f;
-            hpost[i] = i < n ? Hpost[i] : 0.f;
-        }
-        // streams >= n alias stream 0 (no branch around the loads, so all of them are in flight
-        // together); they only ever meet zero coefficients
-        float gv[NP][V], xv[NP][V];
+        // The bulk loads come first and nothing is computed from the sample's coefficients until they
+        // are all requested (a division on q here would make the wave wait for the coefficient round
+        // trip before it asks for its data).  Streams >= n alias stream 0 (no branch around the loads,
+        // so all of them are in flight together); they only ever meet zero coefficients.
+        RawVec<TG, V> graw[NP];
+        RawVec<TX, V> xraw[NP];
 #pragma unroll
         for (int i = 0; i < NP; i++) {
             const size_t so = (size_t)(i < n ? i : 0) * C + c;
-            load_vec<TG, V>(gb + so, gv[i]);
-            load_vec<TX, V>(xb + so, xv[i]);
+            graw[i].load(gb + so);
+            xraw[i].load(xb + so);
         }
         // dx_in may alias dx, so the compiler cannot move its loads above the stores of earlier
         // rows: request all rows here (every thread reads exactly the elements it later writes)
@@ -83,6 +86,32 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
             for (int j = 0; j < NP; j++)
                 prev[j].load(static_cast<const TX *>(a.dx_in) + ((size_t)b * n + (j < n ? j : 0)) * C + c);
         }
+        // the sample's coefficients.  n <= 8 (one wave per workgroup): M goes through LDS, one load per
+        // lane instead of one uniform load per use inside the mixing loops; the wave's own LDS
+        // accesses complete in order, so no barrier is involved
+        float hpre[NP], hpost[NP];
+#pragma unroll
+        for (int i = 0; i < NP; i++) {
+            hpre[i] = Hpre[i < n ? i : 0];
+            hpost[i] = Hpost[i < n ? i : 0];
+        }
+        if constexpr (NP < 16) {
+            const int mi = tid / NP, mj = tid % NP;
+            const bool mok = mi < n && mj < n;
+            const float mval = M[mok ? mi * n + mj : 0];
+            if (tid < NP * NP) M_s[tid] = mok ? mval : 0.f;
+        }
+        const float qraw = inject ? 1.0f : a.q[b], s1raw = inject ? 0.f : a.s1[b];
+        const float cx = a.cx ? a.cx[b] : 0.f;
+#pragma unroll
+        for (int i = 0; i < NP; i++)
+            if (i >= n) { hpre[i] = 0.f; hpost[i] = 0.f; }
+        const float qinv = inject ? 0.f : 1.0f / qraw;
+        const float k2 = inject ? 0.f : s1raw * qinv * qinv * qinv / (float)C;
+        float gv[NP][V], xv[NP][V];
+#pragma unroll
+        for (int i = 0; i < NP; i++) { graw[i].get(gv[i]); xraw[i].get(xv[i]); }
+        MHC_PHASE_ADD(kPhaseDxSmall, pwg, 0, pclk);
         float da[V], dfv[V], uv[V];
 #pragma unroll
         for (int v = 0; v < V; v++) {
@@ -98,11 +127,12 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
             }
         }
         if (inject) {
-            if (a.df) store_vec<TX, V>(static_cast<TX *>(a.df) + (size_t)b * C + c, dfv);
+            if (a.df && live) store_vec<TX, V>(static_cast<TX *>(a.df) + (size_t)b * C + c, dfv);
         } else {
 #pragma unroll
             for (int v = 0; v < V; v++) usum[v] += uv[v];
         }
+        MHC_PHASE_ADD(kPhaseDxSmall, pwg, 1, pclk);
 #pragma unroll
         for (int j = 0; j < NP; j++) {
             if (j < n) {
@@ -111,9 +141,7 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
                 for (int v = 0; v < V; v++) out[v] = hpre[j] * da[v] - cx * xv[j][v];
 #pragma unroll
                 for (int i = 0; i < NP; i++) {
-                    float mij;
-                    if constexpr (NP >= 16) mij = M_s[i * NP + j];
-                    else mij = (i < n) ? M[i * n + j] : 0.f;
+                    const float mij = M_s[i * NP + j];
 #pragma unroll
                     for (int v = 0; v < V; v++) out[v] += mij * gv[i][v];
                 }
@@ -136,11 +164,12 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
 #pragma unroll
                     for (int v = 0; v < V; v++) out[v] += pv[v];
                 }
-                store_vec<TX, V, true>(dxb + (size_t)j * C + c, out);
+                if (live) store_vec<TX, V, true>(dxb + (size_t)j * C + c, out);
             }
         }
       }
-      if (!inject && a.u) store_vec<float, V>(a.u + (size_t)grp * C + c, usum);
+      MHC_PHASE_ADD(kPhaseDxSmall, pwg, 2, pclk);
+      if (!inject && a.u && live) store_vec<float, V>(a.u + (size_t)grp * C + c, usum);
     }
     // per-group sums of the logit gradients (feeds dbias / dalpha)
     if (a.dtpart && blockIdx.y == 0) {
@@ -150,6 +179,7 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
             a.dtpart[(size_t)grp * (D + 3) + col] = acc;
         }
     }
+    MHC_PHASE_ADD(kPhaseDxSmall, pwg, 3, pclk);
 }
 
 // =============================================================================================
@@ -354,7 +384,7 @@ static hipError_t launch_one(const BwdDxArgs &a, hipStream_t stream) {
         nt = 64;
         ny = (nch + 63) / 64;
     }
-    const size_t smem = sizeof(float) * (NP >= 16 ? NP * NP : 1);
+    const size_t smem = sizeof(float) * NP * NP;
     mix_bwd_dx_kernel<TG, TX, NP, V><<<dim3(groups_of(a), ny), nt, smem, stream>>>(a);
     return hipGetLastError();
 }

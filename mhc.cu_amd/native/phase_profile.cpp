@@ -110,6 +110,8 @@ int main(int argc, char **argv) {
             {"start: coefficient inputs, Sinkhorn forward recompute (wave 0)", "streaming loop (wave 0's steps)",
              "workgroup sums", "coefficient backward (Sinkhorn reverse sweep, dP stores)"}, false);
     if (n > 4) {
+        summary("dx kernel (generic, one wave per workgroup)", 5, std::min(B * ((C / 4 + 63) / 64), 4096),
+                {"start: coefficients and all loads requested", "data arrives, df / a / da", "mixing, dx stores issued", "dw / dt partial sums"}, false);
         summary("projection backward kernel, one workgroup per 32 columns of x_flat", 2, std::min((int)(nC / 32), 4096),
                 {"prologue (phi slab, first x block requested)", "operands requested, x block parked (all blocks)",
                  "fragments, dphi on the matrix cores (all)", "dxflat on the matrix cores, stores (all)", "dphi stores"}, false);
