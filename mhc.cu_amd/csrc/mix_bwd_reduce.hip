@@ -104,7 +104,9 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
     const float *__restrict__ Hpre = a.Hpre + (size_t)b * a.hstride;
     const float *__restrict__ Hpost = a.Hpost + (size_t)b * a.hstride;
     const bool inject = a.f_inject != nullptr;
-    const float qinv = inject ? 0.f : 1.0f / a.q[b];
+    // q is only requested here: a division in front of the loop would make the wave wait for this
+    // round trip before it asks for its data; 1/q is applied to the sums behind the loop instead
+    const float qraw = inject ? 1.0f : a.q[b];
 
     float hpre[NP], hpost[NP];
 #pragma unroll
@@ -142,7 +144,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
                 dfw[v] = 0.f;
             } else {
                 const float wv = load_w_(a.w, a.w_bf16, c + v);
-                fv[v] = s_a * qinv * wv;
+                fv[v] = s_a * wv;  // f * q
                 dfw[v] = s_df * wv;
             }
             acc[K - 1] += dfw[v] * s_a;
@@ -162,6 +164,11 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
         }
     }
 
+    const float qinv = inject ? 0.f : 1.0f / qraw;
+    if (!inject) {
+#pragma unroll
+        for (int i = 0; i < NP; i++) acc[NP * NP + i] *= qinv;  // dHpost was summed against f * q
+    }
     // workgroup sum: DPP within each 16-lane row, one LDS slot per row, then K lanes finish
     const int slot = tid >> 4, nslots = nt >> 4;
 #pragma unroll
