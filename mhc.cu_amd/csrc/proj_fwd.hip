@@ -74,6 +74,7 @@ __global__ __launch_bounds__(256) void proj_fwd_generic_kernel(const TX *__restr
 // full set of sample tiles), so that all sample tiles of a slab run on one XCD and the slab of phi
 // is fetched from memory once instead of once per XCD.  Ids whose slab is beyond KS do nothing.
 // --------------------------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 constexpr int kNarrowPitch = 72;  // LDS row of a 64-element chunk: 128 data bytes + 16 pad (bf16 elements)
 
 template <int NT>
@@ -121,17 +122,34 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
         }
     }
     uint32_t xq[4][4], pq[NT][4][4];  // scalar words: whole-uint4 array elements can end up in scratch
+    // Rows beyond B (x) or D (phi) alias row 0: what they produce is finite and is either not stored
+    // (samples >= B) or zeroed at the store (projection rows >= D), so only the K tail of the last
+    // slab needs a mask - a uniform test per chunk instead of four selects per load (the kernel is
+    // bound by VALU issue, not by memory, with four waves per SIMD).
     auto fetch = [&](int k0) {
         const int k = k0 + seg * 8;
+        if (k0 + 64 <= kend) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(xrow[j] + k);
+                xq[j][0] = v.x; xq[j][1] = v.y; xq[j][2] = v.z; xq[j][3] = v.w;
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const uint4 p = *reinterpret_cast<const uint4 *>(prow[t][j] + k);
+                    pq[t][j][0] = p.x; pq[t][j][1] = p.y; pq[t][j][2] = p.z; pq[t][j][3] = p.w;
+                }
+            }
+            return;
+        }
         const bool kv = k < kend;  // kend and k are multiples of 8
         const int off = kv ? k : 0;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(xrow[j] + off), kv && xval[j]);
+            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(xrow[j] + off), kv);
             xq[j][0] = v.x; xq[j][1] = v.y; xq[j][2] = v.z; xq[j][3] = v.w;
 #pragma unroll
             for (int t = 0; t < NT; t++) {
-                const uint4 p = load16_masked(reinterpret_cast<const uint4 *>(prow[t][j] + off), kv && pval[t][j]);
+                const uint4 p = load16_masked(reinterpret_cast<const uint4 *>(prow[t][j] + off), kv);
                 pq[t][j][0] = p.x; pq[t][j][1] = p.y; pq[t][j][2] = p.z; pq[t][j][3] = p.w;
             }
         }
@@ -171,12 +189,12 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
                 const uint4 bv = *reinterpret_cast<const uint4 *>(cb + (size_t)(32 + t * 32 + row) * kNarrowPitch + u * 16 + kh * 8);
                 acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(bf16x8_t, bv), acc[t], 0, 0, 0);
             }
-            if (blockIdx.y == 0) {
+            if (blockIdx.y == 0) {  // sum of squares: v_dot2c_f32_bf16, two elements per instruction
                 const uint32_t w4[4] = {av.x, av.y, av.z, av.w};
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const float lo = bf16lo_to_f32(w4[i]), hi = bf16hi_to_f32(w4[i]);
-                    ssq += lo * lo + hi * hi;
+                    const bf16x2_t pr = __builtin_bit_cast(bf16x2_t, w4[i]);
+                    ssq = __builtin_amdgcn_fdot2_f32_bf16(pr, pr, ssq, false);
                 }
             }
         }
@@ -215,7 +233,7 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int bs = st * 32 + 8 * (i >> 2) + 4 * kh + (i & 3);
-                if (bs < B && d < DP) out[(size_t)bs * DP + d] = acc[t][i];
+                if (bs < B && d < DP) out[(size_t)bs * DP + d] = d < D ? acc[t][i] : 0.f;  // padded rows stay zero
             }
         }
         if (blockIdx.y == 0 && kh == 0 && bvalid) ssqpart[(size_t)ks * B + b] = ssq;
