@@ -26,9 +26,6 @@ namespace mhc {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
-typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
-
 constexpr int kSlabCW = 64;                 // channels per slab
 constexpr int kSlabNS = 4;                  // streams (padded)
 constexpr int kSlabKW = kSlabNS * kSlabCW;  // x_flat columns per slab tile row
@@ -89,28 +86,6 @@ template <> struct Raw8<float> {
         v[0] = r0.x; v[1] = r0.y; v[2] = r0.z; v[3] = r0.w; v[4] = r1.x; v[5] = r1.y; v[6] = r1.z; v[7] = r1.w;
     }
 };
-
-// Four fp32 coefficients as two bf16x4 MFMA operands: the rounded values and their remainders.
-struct CoefRow {
-    bf16x4_t hi, lo;
-    __device__ __forceinline__ void set(float c0, float c1, float c2, float c3) {
-        const uint32_t h0 = pack_bf16x2(c0, c1), h1 = pack_bf16x2(c2, c3);
-        const uint32_t l0 = pack_bf16x2(c0 - bf16lo_to_f32(h0), c1 - bf16hi_to_f32(h0));
-        const uint32_t l1 = pack_bf16x2(c2 - bf16lo_to_f32(h1), c3 - bf16hi_to_f32(h1));
-        hi = __builtin_bit_cast(bf16x4_t, make_uint2(h0, h1));
-        lo = __builtin_bit_cast(bf16x4_t, make_uint2(l0, l1));
-    }
-};
-__device__ __forceinline__ f32x4_t mfma4(bf16x4_t a, bf16x4_t b, f32x4_t c) {
-    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a, b, c, 0, 0, 0);
-}
-// The four streams of one channel as a bf16x4 operand, from the word of each stream that holds the
-// channel pair: the low halves (even channel) or the high halves (odd channel).
-template <bool ODD>
-__device__ __forceinline__ bf16x4_t streams_of_channel(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
-    constexpr uint32_t sel = ODD ? 0x07060302u : 0x05040100u;
-    return __builtin_bit_cast(bf16x4_t, make_uint2(__builtin_amdgcn_perm(w1, w0, sel), __builtin_amdgcn_perm(w3, w2, sel)));
-}
 
 template <typename TG>
 __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {

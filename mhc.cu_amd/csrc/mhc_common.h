@@ -184,6 +184,39 @@ __device__ __forceinline__ uint4 load16_masked(const uint4 *p, bool ok) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// v_mfma_f32_4x4x4_16b_bf16: 16 independent 4x4x4 products per instruction.  Block = four
+// consecutive lanes; lane r of a block supplies row r of A (four bf16 along k) and column r of B,
+// and receives column r of the product (register = row).
+// ---------------------------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+__device__ __forceinline__ bf16x4_t bf16x4_of(uint32_t w0, uint32_t w1) {
+    return __builtin_bit_cast(bf16x4_t, make_uint2(w0, w1));
+}
+__device__ __forceinline__ f32x4_t mfma4(bf16x4_t a, bf16x4_t b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a, b, c, 0, 0, 0);
+}
+// Four fp32 coefficients as two bf16x4 operands: the rounded values and their remainders.
+struct CoefRow {
+    bf16x4_t hi, lo;
+    __device__ __forceinline__ void set(float c0, float c1, float c2, float c3) {
+        const uint32_t h0 = pack_bf16x2(c0, c1), h1 = pack_bf16x2(c2, c3);
+        const uint32_t l0 = pack_bf16x2(c0 - bf16lo_to_f32(h0), c1 - bf16hi_to_f32(h0));
+        const uint32_t l1 = pack_bf16x2(c2 - bf16lo_to_f32(h1), c3 - bf16hi_to_f32(h1));
+        hi = bf16x4_of(h0, h1);
+        lo = bf16x4_of(l0, l1);
+    }
+};
+// The four streams of one channel as a bf16x4 operand, from the word of each stream that holds the
+// channel pair: the low halves (even channel) or the high halves (odd channel).
+template <bool ODD>
+__device__ __forceinline__ bf16x4_t streams_of_channel(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+    constexpr uint32_t sel = ODD ? 0x07060302u : 0x05040100u;
+    return bf16x4_of(__builtin_amdgcn_perm(w1, w0, sel), __builtin_amdgcn_perm(w3, w2, sel));
+}
+
+// ---------------------------------------------------------------------------------------------
 // Cross-lane primitives
 // ---------------------------------------------------------------------------------------------
 // DPP controls (GFX9 encoding): quad_perm = 8-bit selector, row_ror:n = 0x120 + n

@@ -414,16 +414,7 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
 // With an injected f, W1 = dy [f; 0; ...]^T (its column 0 is dHpost) and XX is not needed.
 // Output: raw[b][part][m][i][j] (NP x NP each), m = dM | W1 | XX.
 // =============================================================================================
-typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 enum { kGramInject = 0, kGramWBf16 = 1, kGramWF32 = 2 };
-
-__device__ __forceinline__ bf16x4_t bf16x4_of(uint32_t w0, uint32_t w1) {
-    return __builtin_bit_cast(bf16x4_t, make_uint2(w0, w1));
-}
-__device__ __forceinline__ f32x4_t mfma4(bf16x4_t a, bf16x4_t b, f32x4_t c) {
-    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a, b, c, 0, 0, 0);
-}
 
 // FUSED (one column part per sample): the first lanes of wave 0 go on with the sample's coefficient
 // backward (CoefBwdSmall) as soon as the sums are complete, its other inputs requested at the start;

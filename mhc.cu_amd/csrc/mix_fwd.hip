@@ -145,7 +145,7 @@ struct LayerFwdArgs {
 constexpr int kFwdStaggerMinB = 512;  // two or more workgroups per CU
 
 template <typename TX, typename TY, int NP, int V, int CPT>
-__global__ __launch_bounds__(256, (CPT == 2 && NP == 4 && !std::is_same<TX, float>::value) ? 5 : 1)
+__global__ __launch_bounds__(256, (CPT == 2 && NP == 4 && !std::is_same<TX, float>::value) ? 4 : 1)
 void layer_fwd_small_kernel(LayerFwdArgs a) {
     using SK = SkSmall<NP>;
     __shared__ float coef_s[NP * NP + 2 * NP];  // M | Hpre | Hpost
@@ -315,93 +315,190 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
         for (int j = 0; j < NP; j++) Mr[i][j] = coef_s[i * NP + j];
     }
 
-    // ---- 3. aggregate + RMS ------------------------------------------------------------------
-    // The tile stays in registers as raw words; LEAN (two chunks per thread) widens a stream at
-    // the point of use instead of holding the fp32 copy of the whole tile, which keeps the
-    // kernel under 96 registers, i.e. five workgroups per CU (1280 samples then fit in one round
-    // of the grid); the extra conversions are cheaper than a second round.
-    constexpr bool LEAN = CPT >= 2 && NP <= 4 && !std::is_same<TX, float>::value;
-    float xv[LEAN ? 1 : CPT][NP][V];
-    if constexpr (!LEAN) {
+    // bf16 x, n <= 4: the per-sample 4x4 products of steps 3 and 4 run on v_mfma_f32_4x4x4_16b_bf16
+    // (a block = four consecutive lanes, all of the same sample here): the B column of a lane is the
+    // four streams of one of its channels (two v_perm_b32), the A rows are the sample's coefficients
+    // (bf16 value + remainder), the lane receives the four output streams of its own channel.  With
+    // the products on the VALU this kernel is bound by VALU issue once several workgroups share a CU.
+    constexpr bool kMixMfma = std::is_same<TX, bf16_t>::value && NP == 4 && V == 8;
+    if constexpr (kMixMfma) {
+        const int jq = tid & 3;
+        CoefRow cm, ca;  // row jq of M; [Hpre; 0; 0; 0]
+        cm.set(coef_s[jq * NP + 0], coef_s[jq * NP + 1], coef_s[jq * NP + 2], coef_s[jq * NP + 3]);
+        const bool r0 = jq == 0;
+        ca.set(r0 ? hpre[0] : 0.f, r0 ? hpre[1] : 0.f, r0 ? hpre[2] : 0.f, r0 ? hpre[3] : 0.f);
+        const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+        // B operands of a chunk: channel v = 2p + odd, p = word of the channel pair
+        auto channel = [&](int k, int v) {
+            const int p = v >> 1;
+            return (v & 1) ? streams_of_channel<true>(xr[k][0].w[p], xr[k][1].w[p], xr[k][2].w[p], xr[k][3].w[p])
+                           : streams_of_channel<false>(xr[k][0].w[p], xr[k][1].w[p], xr[k][2].w[p], xr[k][3].w[p]);
+        };
+        // ---- 3. aggregate + RMS ----------------------------------------------------------------
+        // (four channels at a time keep the accumulators small; the aggregate is formed again in
+        // step 4 instead of being kept across the barrier: 8 cheap instructions per half chunk)
+        float qinv = 1.0f;
+        if (!inject) {
+            float ssq = 0.f;
 #pragma unroll
-        for (int k = 0; k < CPT; k++)
+            for (int k = 0; k < CPT; k++) {
+                const bool live = tid + k * nt < nch;  // chunks beyond C alias chunk 0: not counted
 #pragma unroll
-            for (int i = 0; i < NP; i++) xr[k][i].get(xv[k][i]);  // streams >= n meet zero coefficients
-    }
-    float av[LEAN ? 1 : CPT][V];  // LEAN recomputes the aggregate in step 4 instead of keeping it
-    float qinv = 1.0f;
-    if (!inject) {
-        float ssq = 0.f;
+                for (int h = 0; h < 2; h++) {
+                    f32x4_t d[4];
+#pragma unroll
+                    for (int v = 0; v < 4; v++) d[v] = mfma4(ca.hi, channel(k, 4 * h + v), zero);
+#pragma unroll
+                    for (int v = 0; v < 4; v++) d[v] = mfma4(ca.lo, channel(k, 4 * h + v), d[v]);
+#pragma unroll
+                    for (int v = 0; v < 4; v++) ssq += live ? d[v][0] * d[v][0] : 0.f;
+                }
+            }
+            ssq = block_allreduce_sum(ssq, red, nt / kWave);
+            const float q = sqrtf(ssq / (float)C + a.eps);
+            qinv = 1.0f / q;
+            if (tid == 0 && a.q) a.q[b] = q;
+        } else if (tid == 0 && a.q) {
+            a.q[b] = 1.0f;
+        }
+        MHC_PHASE(kPhaseFwdFused, b, 5);
+        // ---- 4. mix + distribute -----------------------------------------------------------------
 #pragma unroll
         for (int k = 0; k < CPT; k++) {
-            const bool live = tid + k * nt < nch;  // chunks beyond C alias chunk 0: not counted
-            float s_a[V];
-#pragma unroll
-            for (int v = 0; v < V; v++) s_a[v] = 0.f;
-#pragma unroll
-            for (int i = 0; i < NP; i++) {
-                float t[V];
-                if constexpr (LEAN) xr[k][i].get(t);
-#pragma unroll
-                for (int v = 0; v < V; v++) s_a[v] += hpre[i] * (LEAN ? t[v] : xv[LEAN ? 0 : k][i][v]);
-            }
-#pragma unroll
-            for (int v = 0; v < V; v++) {
-                if constexpr (!LEAN) av[k][v] = s_a[v];
-                ssq += live ? s_a[v] * s_a[v] : 0.f;
-            }
-        }
-        ssq = block_allreduce_sum(ssq, red, nt / kWave);
-        const float q = sqrtf(ssq / (float)C + a.eps);
-        qinv = 1.0f / q;
-        if (tid == 0 && a.q) a.q[b] = q;
-    } else if (tid == 0 && a.q) {
-        a.q[b] = 1.0f;
-    }
-
-    MHC_PHASE(kPhaseFwdFused, b, 5);
-    // ---- 4. mix + distribute -------------------------------------------------------------------
-#pragma unroll
-    for (int k = 0; k < CPT; k++) {
-        const int ch = tid + k * nt;
-        if (ch < nch) {
-            const int c = ch * V;
+            const int ch = tid + k * nt;
+            const int c = (ch < nch ? ch : 0) * V;
             float f[V];
             if (inject) {
                 fr[k].get(f);
             } else {
-                if constexpr (LEAN) {
+                if (a.w_bf16) load_vec<bf16_t, V>(static_cast<const bf16_t *>(a.w) + c, f);
+                else load_vec<float, V>(static_cast<const float *>(a.w) + c, f);
+            }
+            uint32_t yw[NP][2];  // packed first half (bf16 output), stored with the second
+            float yf[NP][4];     // first half (fp32 output)
 #pragma unroll
-                    for (int v = 0; v < V; v++) f[v] = 0.f;
+            for (int h = 0; h < 2; h++) {
+                f32x4_t d[4], da[4];
+                bf16x4_t bx[4];
 #pragma unroll
-                    for (int i = 0; i < NP; i++) {
-                        float t[V];
-                        xr[k][i].get(t);
+                for (int v = 0; v < 4; v++) bx[v] = channel(k, 4 * h + v);
 #pragma unroll
-                        for (int v = 0; v < V; v++) f[v] += hpre[i] * t[v];
+                for (int v = 0; v < 4; v++) { d[v] = mfma4(cm.hi, bx[v], zero); da[v] = mfma4(ca.hi, bx[v], zero); }
+#pragma unroll
+                for (int v = 0; v < 4; v++) { d[v] = mfma4(cm.lo, bx[v], d[v]); da[v] = mfma4(ca.lo, bx[v], da[v]); }
+                float fh[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++) fh[v] = inject ? f[4 * h + v] : da[v][0] * qinv * f[4 * h + v];
+#pragma unroll
+                for (int i = 0; i < NP; i++) {
+                    const float o0 = d[0][i] + hpost[i] * fh[0], o1 = d[1][i] + hpost[i] * fh[1];
+                    const float o2 = d[2][i] + hpost[i] * fh[2], o3 = d[3][i] + hpost[i] * fh[3];
+                    if constexpr (std::is_same<TY, bf16_t>::value) {
+                        if (h == 0) {
+                            yw[i][0] = pack_bf16x2(o0, o1); yw[i][1] = pack_bf16x2(o2, o3);
+                        } else if (i < n && ch < nch) {
+                            st16<true>(yb + (size_t)i * C + c, yw[i][0], yw[i][1], pack_bf16x2(o0, o1), pack_bf16x2(o2, o3));
+                        }
+                    } else {
+                        if (h == 0) {
+                            yf[i][0] = o0; yf[i][1] = o1; yf[i][2] = o2; yf[i][3] = o3;
+                        } else if (i < n && ch < nch) {
+                            const float out[V] = {yf[i][0], yf[i][1], yf[i][2], yf[i][3], o0, o1, o2, o3};
+                            store_vec<TY, V, true>(yb + (size_t)i * C + c, out);
+                        }
                     }
-#pragma unroll
-                    for (int v = 0; v < V; v++) f[v] = f[v] * qinv * load_w(a.w, a.w_bf16, c + v);
-                } else {
-#pragma unroll
-                    for (int v = 0; v < V; v++) f[v] = av[k][v] * qinv * load_w(a.w, a.w_bf16, c + v);
                 }
             }
+        }
+    } else {
+        // ---- 3. aggregate + RMS ------------------------------------------------------------------
+        // (VALU path: fp32 x, n > 4, or rows not a multiple of 8.)  The tile stays in registers as raw
+        // words; LEAN (two chunks per thread) widens a stream at the point of use instead of holding
+        // the fp32 copy of the whole tile, which keeps the register count down; the extra
+        // conversions are cheaper than a second round of the grid.
+        constexpr bool LEAN = CPT >= 2 && NP <= 4 && !std::is_same<TX, float>::value;
+        float xv[LEAN ? 1 : CPT][NP][V];
+        if constexpr (!LEAN) {
 #pragma unroll
-            for (int i = 0; i < NP; i++) {
-                if (i < n) {
-                    float out[V];
+            for (int k = 0; k < CPT; k++)
 #pragma unroll
-                    for (int v = 0; v < V; v++) out[v] = hpost[i] * f[v];
+                for (int i = 0; i < NP; i++) xr[k][i].get(xv[k][i]);  // streams >= n meet zero coefficients
+        }
+        float av[LEAN ? 1 : CPT][V];  // LEAN recomputes the aggregate in step 4 instead of keeping it
+        float qinv = 1.0f;
+        if (!inject) {
+            float ssq = 0.f;
 #pragma unroll
-                    for (int j = 0; j < NP; j++) {
-                        float t[V];
-                        if constexpr (LEAN) xr[k][j].get(t);
-                        const float mij = LEAN ? coef_s[i * NP + j] : Mr[i][j];
+            for (int k = 0; k < CPT; k++) {
+                const bool live = tid + k * nt < nch;  // chunks beyond C alias chunk 0: not counted
+                float s_a[V];
 #pragma unroll
-                        for (int v = 0; v < V; v++) out[v] += mij * (LEAN ? t[v] : xv[LEAN ? 0 : k][j][v]);
+                for (int v = 0; v < V; v++) s_a[v] = 0.f;
+#pragma unroll
+                for (int i = 0; i < NP; i++) {
+                    float t[V];
+                    if constexpr (LEAN) xr[k][i].get(t);
+#pragma unroll
+                    for (int v = 0; v < V; v++) s_a[v] += hpre[i] * (LEAN ? t[v] : xv[LEAN ? 0 : k][i][v]);
+                }
+#pragma unroll
+                for (int v = 0; v < V; v++) {
+                    if constexpr (!LEAN) av[k][v] = s_a[v];
+                    ssq += live ? s_a[v] * s_a[v] : 0.f;
+                }
+            }
+            ssq = block_allreduce_sum(ssq, red, nt / kWave);
+            const float q = sqrtf(ssq / (float)C + a.eps);
+            qinv = 1.0f / q;
+            if (tid == 0 && a.q) a.q[b] = q;
+        } else if (tid == 0 && a.q) {
+            a.q[b] = 1.0f;
+        }
+
+        MHC_PHASE(kPhaseFwdFused, b, 5);
+        // ---- 4. mix + distribute -------------------------------------------------------------------
+#pragma unroll
+        for (int k = 0; k < CPT; k++) {
+            const int ch = tid + k * nt;
+            if (ch < nch) {
+                const int c = ch * V;
+                float f[V];
+                if (inject) {
+                    fr[k].get(f);
+                } else {
+                    if constexpr (LEAN) {
+#pragma unroll
+                        for (int v = 0; v < V; v++) f[v] = 0.f;
+#pragma unroll
+                        for (int i = 0; i < NP; i++) {
+                            float t[V];
+                            xr[k][i].get(t);
+#pragma unroll
+                            for (int v = 0; v < V; v++) f[v] += hpre[i] * t[v];
+                        }
+#pragma unroll
+                        for (int v = 0; v < V; v++) f[v] = f[v] * qinv * load_w(a.w, a.w_bf16, c + v);
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < V; v++) f[v] = av[k][v] * qinv * load_w(a.w, a.w_bf16, c + v);
                     }
-                    store_vec<TY, V, true>(yb + (size_t)i * C + c, out);
+                }
+#pragma unroll
+                for (int i = 0; i < NP; i++) {
+                    if (i < n) {
+                        float out[V];
+#pragma unroll
+                        for (int v = 0; v < V; v++) out[v] = hpost[i] * f[v];
+#pragma unroll
+                        for (int j = 0; j < NP; j++) {
+                            float t[V];
+                            if constexpr (LEAN) xr[k][j].get(t);
+                            const float mij = LEAN ? coef_s[i * NP + j] : Mr[i][j];
+#pragma unroll
+                            for (int v = 0; v < V; v++) out[v] += mij * (LEAN ? t[v] : xv[LEAN ? 0 : k][j][v]);
+                        }
+                        store_vec<TY, V, true>(yb + (size_t)i * C + c, out);
+                    }
                 }
             }
         }
