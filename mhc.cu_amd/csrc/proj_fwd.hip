@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
                                                             float *__restrict__ ssqpart, int B,
                                                             int D, int DP, int nC, int tiles_s, int KS,
                                                             int sub /* K per wave, multiple of 64 */) {
-    extern __shared__ __align__(16) float lds[];  // per wave [(1 + NT) * 32][pitch] bf16; later [3][NT*16 + 1][64] fp32
+    extern __shared__ __align__(16) float lds[];  // per wave [(1 + NT) * 32][pitch] bf16; later [4][NT*16 + 1][64] fp32
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int set = (blockIdx.x >> 3) / tiles_s;
     const int st = (blockIdx.x >> 3) % tiles_s, ks = (blockIdx.x & 7) + 8 * set;
@@ -203,10 +203,11 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
     __syncthreads();  // every wave is done with its chunk tile: the memory becomes the cross-wave buffer
     ssq = xor32_add(ssq);  // both K halves of the row
 
-    // cross-wave sum: waves 1..3 park their tiles in LDS, wave 0 adds and writes
+    // cross-wave sum: every wave parks its tiles in LDS, then wave w adds and writes accumulator
+    // registers 4w .. 4w+3 of every tile (rows 8w + 4 kh .. +3 of the 32 x 32 tile), wave 0 also x^2
     constexpr int R = NT * 16 + 1;
-    if (wave > 0) {
-        float *dst = lds + (size_t)(wave - 1) * R * 64;
+    {
+        float *dst = lds + (size_t)wave * R * 64;
 #pragma unroll
         for (int t = 0; t < NT; t++)
 #pragma unroll
@@ -214,29 +215,27 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
         dst[(R - 1) * 64 + lane] = ssq;
     }
     __syncthreads();
-    if (wave == 0) {
+    // accumulator layout of the 32x32 tile: lane -> column (lane & 31),
+    // register i -> row 8 * (i / 4) + 4 * (lane / 32) + (i % 4)
+    float *out = Ppart + (size_t)ks * B * DP;
 #pragma unroll
-        for (int w = 0; w < 3; w++) {
-            const float *src = lds + (size_t)w * R * 64;
+    for (int t = 0; t < NT; t++) {
+        const int d = dbase + t * 32 + row;
 #pragma unroll
-            for (int t = 0; t < NT; t++)
+        for (int q = 0; q < 4; q++) {
+            const int i = 4 * wave + q;
+            float v = 0.f;
 #pragma unroll
-                for (int i = 0; i < 16; i++) acc[t][i] += src[(t * 16 + i) * 64 + lane];
-            ssq += src[(R - 1) * 64 + lane];
+            for (int w = 0; w < 4; w++) v += lds[((size_t)w * R + t * 16 + i) * 64 + lane];
+            const int bs = st * 32 + 8 * wave + 4 * kh + q;
+            if (bs < B && d < DP) out[(size_t)bs * DP + d] = d < D ? v : 0.f;  // padded rows stay zero
         }
-        // accumulator layout of the 32x32 tile: lane -> column (lane & 31),
-        // register i -> row 8 * (i / 4) + 4 * (lane / 32) + (i % 4)
-        float *out = Ppart + (size_t)ks * B * DP;
+    }
+    if (wave == 0 && blockIdx.y == 0 && kh == 0 && bvalid) {
+        float v = 0.f;
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const int d = dbase + t * 32 + row;
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int bs = st * 32 + 8 * (i >> 2) + 4 * kh + (i & 3);
-                if (bs < B && d < DP) out[(size_t)bs * DP + d] = d < D ? acc[t][i] : 0.f;  // padded rows stay zero
-            }
-        }
-        if (blockIdx.y == 0 && kh == 0 && bvalid) ssqpart[(size_t)ks * B + b] = ssq;
+        for (int w = 0; w < 4; w++) v += lds[((size_t)w * R + R - 1) * 64 + lane];
+        ssqpart[(size_t)ks * B + b] = v;
     }
     MHC_PHASE_ADD(kPhaseProjFwd, pwg, 3, pclk);
 }
@@ -488,7 +487,7 @@ static hipError_t launch_mfma(const void *x, const void *phi, float *Ppart, floa
     const int sub = round_up((nC + KS * 4 - 1) / (KS * 4), 64);  // whole 128-byte lines per lane pair
     dim3 grid(tiles_s * round_up(KS, 8), groups);
     const size_t smem_chunks = sizeof(bf16_t) * 4 * (1 + NT) * 32 * kNarrowPitch;
-    const size_t smem_sum = sizeof(float) * 3 * (NT * 16 + 1) * 64;
+    const size_t smem_sum = sizeof(float) * 4 * (NT * 16 + 1) * 64;
     const size_t smem = smem_chunks > smem_sum ? smem_chunks : smem_sum;
     if (hipError_t e = allow_dynamic_lds(&proj_fwd_mfma_kernel<NT>, smem); e != hipSuccess) return e;
     proj_fwd_mfma_kernel<NT><<<grid, 256, smem, stream>>>(static_cast<const bf16_t *>(x),
