@@ -421,12 +421,12 @@ enum { kGramInject = 0, kGramWBf16 = 1, kGramWF32 = 2 };
 // with several workgroups per CU the serial Sinkhorn chain of one runs under the loads of the others,
 // and the launch of the coefficient kernel is saved.
 template <int NP, int WMODE, bool FUSED>
-__global__ __launch_bounds__(256) void gram_small_kernel(BwdReduceArgs a) {
+__global__ __launch_bounds__(256, NP == 4 ? 4 : 1) void gram_small_kernel(BwdReduceArgs a) {
     static_assert(NP == 4 || NP == 8, "stream groups of four");
     using SK = SkSmall<NP>;
     using CB = CoefBwdSmall<NP, false, true>;
     constexpr int NB = NP / 4;            // stream groups
-    constexpr int U = NP == 4 ? 2 : 1;    // steps of a wave in flight
+    constexpr int U = 2;                  // steps of a wave in flight
     constexpr int K = 3 * NP * NP;
     constexpr bool inject = WMODE == kGramInject;
     __shared__ float slot_s[K * 16];  // one slot per 16-lane row of the workgroup
