@@ -315,28 +315,53 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
         for (int j = 0; j < NP; j++) Mr[i][j] = coef_s[i * NP + j];
     }
 
-    // bf16 x, n <= 4: the per-sample 4x4 products of steps 3 and 4 run on v_mfma_f32_4x4x4_16b_bf16
-    // (a block = four consecutive lanes, all of the same sample here): the B column of a lane is the
-    // four streams of one of its channels (two v_perm_b32), the A rows are the sample's coefficients
-    // (bf16 value + remainder), the lane receives the four output streams of its own channel.  With
-    // the products on the VALU this kernel is bound by VALU issue once several workgroups share a CU.
-    constexpr bool kMixMfma = std::is_same<TX, bf16_t>::value && NP == 4 && V == 8;
+    // bf16 x: the per-sample n x n products of steps 3 and 4 run on v_mfma_f32_4x4x4_16b_bf16 (a block
+    // = four consecutive lanes, all of the same sample here): the B column of a lane is four streams
+    // of one of its channels (two v_perm_b32), the A rows are the sample's coefficients (bf16 value
+    // + remainder), the lane receives four output streams of its own channel; for n > 4 the streams
+    // form two groups of four and M is 2 x 2 such blocks.  With the products on the VALU this kernel
+    // is bound by VALU issue once several workgroups share a CU.
+    constexpr bool kMixMfma = std::is_same<TX, bf16_t>::value && V == 8;
     if constexpr (kMixMfma) {
+        constexpr int NB = NP / 4;  // stream groups
         const int jq = tid & 3;
-        CoefRow cm, ca;  // row jq of M; [Hpre; 0; 0; 0]
-        cm.set(coef_s[jq * NP + 0], coef_s[jq * NP + 1], coef_s[jq * NP + 2], coef_s[jq * NP + 3]);
+        CoefRow cm[NB][NB], ca[NB];  // rows 4J + jq of M, columns 4I ..; [Hpre; 0; 0; 0]
         const bool r0 = jq == 0;
-        ca.set(r0 ? hpre[0] : 0.f, r0 ? hpre[1] : 0.f, r0 ? hpre[2] : 0.f, r0 ? hpre[3] : 0.f);
+#pragma unroll
+        for (int I = 0; I < NB; I++) {
+#pragma unroll
+            for (int J = 0; J < NB; J++) {
+                const float *mr = coef_s + (4 * J + jq) * NP + 4 * I;
+                cm[J][I].set(mr[0], mr[1], mr[2], mr[3]);
+            }
+            ca[I].set(r0 ? hpre[4 * I] : 0.f, r0 ? hpre[4 * I + 1] : 0.f, r0 ? hpre[4 * I + 2] : 0.f,
+                      r0 ? hpre[4 * I + 3] : 0.f);
+        }
         const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
-        // B operands of a chunk: channel v = 2p + odd, p = word of the channel pair
-        auto channel = [&](int k, int v) {
+        // B operand: streams 4I .. 4I+3 of channel v = 2p + odd of chunk k, p = word of the channel pair
+        auto channel = [&](int k, int v, int I) {
             const int p = v >> 1;
-            return (v & 1) ? streams_of_channel<true>(xr[k][0].w[p], xr[k][1].w[p], xr[k][2].w[p], xr[k][3].w[p])
-                           : streams_of_channel<false>(xr[k][0].w[p], xr[k][1].w[p], xr[k][2].w[p], xr[k][3].w[p]);
+            const uint32_t w0 = xr[k][4 * I].w[p], w1 = xr[k][4 * I + 1].w[p], w2 = xr[k][4 * I + 2].w[p],
+                           w3 = xr[k][4 * I + 3].w[p];
+            return (v & 1) ? streams_of_channel<true>(w0, w1, w2, w3) : streams_of_channel<false>(w0, w1, w2, w3);
+        };
+        // aggregate of four channels: register 0 of da[v]
+        auto aggregate4 = [&](const bf16x4_t (&bx)[NB][4], f32x4_t (&da)[4]) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) da[v] = mfma4(ca[0].hi, bx[0][v], zero);
+#pragma unroll
+            for (int v = 0; v < 4; v++) da[v] = mfma4(ca[0].lo, bx[0][v], da[v]);
+#pragma unroll
+            for (int I = 1; I < NB; I++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) da[v] = mfma4(ca[I].hi, bx[I][v], da[v]);
+#pragma unroll
+                for (int v = 0; v < 4; v++) da[v] = mfma4(ca[I].lo, bx[I][v], da[v]);
+            }
         };
         // ---- 3. aggregate + RMS ----------------------------------------------------------------
         // (four channels at a time keep the accumulators small; the aggregate is formed again in
-        // step 4 instead of being kept across the barrier: 8 cheap instructions per half chunk)
+        // step 4 instead of being kept across the barrier: a few cheap instructions per half chunk)
         float qinv = 1.0f;
         if (!inject) {
             float ssq = 0.f;
@@ -345,13 +370,15 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
                 const bool live = tid + k * nt < nch;  // chunks beyond C alias chunk 0: not counted
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
-                    f32x4_t d[4];
+                    bf16x4_t bx[NB][4];
 #pragma unroll
-                    for (int v = 0; v < 4; v++) d[v] = mfma4(ca.hi, channel(k, 4 * h + v), zero);
+                    for (int I = 0; I < NB; I++)
 #pragma unroll
-                    for (int v = 0; v < 4; v++) d[v] = mfma4(ca.lo, channel(k, 4 * h + v), d[v]);
+                        for (int v = 0; v < 4; v++) bx[I][v] = channel(k, 4 * h + v, I);
+                    f32x4_t da[4];
+                    aggregate4(bx, da);
 #pragma unroll
-                    for (int v = 0; v < 4; v++) ssq += live ? d[v][0] * d[v][0] : 0.f;
+                    for (int v = 0; v < 4; v++) ssq += live ? da[v][0] * da[v][0] : 0.f;
                 }
             }
             ssq = block_allreduce_sum(ssq, red, nt / kWave);
@@ -378,21 +405,40 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             float yf[NP][4];     // first half (fp32 output)
 #pragma unroll
             for (int h = 0; h < 2; h++) {
-                f32x4_t d[4], da[4];
-                bf16x4_t bx[4];
+                bf16x4_t bx[NB][4];
 #pragma unroll
-                for (int v = 0; v < 4; v++) bx[v] = channel(k, 4 * h + v);
+                for (int I = 0; I < NB; I++)
 #pragma unroll
-                for (int v = 0; v < 4; v++) { d[v] = mfma4(cm.hi, bx[v], zero); da[v] = mfma4(ca.hi, bx[v], zero); }
+                    for (int v = 0; v < 4; v++) bx[I][v] = channel(k, 4 * h + v, I);
+                f32x4_t d[NB][4], da[4];
 #pragma unroll
-                for (int v = 0; v < 4; v++) { d[v] = mfma4(cm.lo, bx[v], d[v]); da[v] = mfma4(ca.lo, bx[v], da[v]); }
+                for (int J = 0; J < NB; J++) {
+#pragma unroll
+                    for (int v = 0; v < 4; v++) d[J][v] = mfma4(cm[J][0].hi, bx[0][v], zero);
+#pragma unroll
+                    for (int v = 0; v < 4; v++) d[J][v] = mfma4(cm[J][0].lo, bx[0][v], d[J][v]);
+#pragma unroll
+                    for (int I = 1; I < NB; I++) {
+#pragma unroll
+                        for (int v = 0; v < 4; v++) d[J][v] = mfma4(cm[J][I].hi, bx[I][v], d[J][v]);
+#pragma unroll
+                        for (int v = 0; v < 4; v++) d[J][v] = mfma4(cm[J][I].lo, bx[I][v], d[J][v]);
+                    }
+                }
                 float fh[4];
+                if (inject) {
 #pragma unroll
-                for (int v = 0; v < 4; v++) fh[v] = inject ? f[4 * h + v] : da[v][0] * qinv * f[4 * h + v];
+                    for (int v = 0; v < 4; v++) fh[v] = f[4 * h + v];
+                } else {
+                    aggregate4(bx, da);
+#pragma unroll
+                    for (int v = 0; v < 4; v++) fh[v] = da[v][0] * qinv * f[4 * h + v];
+                }
 #pragma unroll
                 for (int i = 0; i < NP; i++) {
-                    const float o0 = d[0][i] + hpost[i] * fh[0], o1 = d[1][i] + hpost[i] * fh[1];
-                    const float o2 = d[2][i] + hpost[i] * fh[2], o3 = d[3][i] + hpost[i] * fh[3];
+                    const int J = i >> 2, r = i & 3;
+                    const float o0 = d[J][0][r] + hpost[i] * fh[0], o1 = d[J][1][r] + hpost[i] * fh[1];
+                    const float o2 = d[J][2][r] + hpost[i] * fh[2], o3 = d[J][3][r] + hpost[i] * fh[3];
                     if constexpr (std::is_same<TY, bf16_t>::value) {
                         if (h == 0) {
                             yw[i][0] = pack_bf16x2(o0, o1); yw[i][1] = pack_bf16x2(o2, o3);
