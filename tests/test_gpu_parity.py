@@ -178,7 +178,9 @@ def test_largest_iteration_counts(B, n, C, T, dyn):
                                    # splits), a row too long for the fused forward kernel, odd expansion rates
                                    (4100, 4, 64), (2, 4, 8200), (3, 17, 24), (2, 31, 40), (600, 8, 64),
                                    # wide projection with batch splits and many sample blocks per split
-                                   (4000, 20, 32)])
+                                   (4000, 20, 32),
+                                   # two chunks per thread in the fused forward with 8 x 8 coefficients
+                                   (3, 8, 2568), (2, 5, 4096)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_dynamic_bf16_vs_oracle(B, n, C, out_dtype):
     x, dy, _, p = nm.make_dynamic_inputs(B, n, C, bf16_round=True)
@@ -231,7 +233,8 @@ def test_bf16_small_n_coefficient_gradients_are_tight(B, n, C, inject, w_dtype):
         assert e <= 2e-4, f"d{k}: normalised err {e:.3e}"
 
 
-@pytest.mark.parametrize("B,n,C", [(16, 4, 256), (8, 8, 128), (4, 16, 64), (3, 32, 72), (5, 32, 1040)])
+@pytest.mark.parametrize("B,n,C", [(16, 4, 256), (8, 8, 128), (4, 16, 64), (3, 32, 72), (5, 32, 1040),
+                                   (5, 4, 2568), (3, 7, 2176)])
 @pytest.mark.parametrize("inject", [False, True])
 def test_static_bf16_vs_oracle(B, n, C, inject):
     """Static H with bf16 activations: the shared-coefficient mode of the bf16 kernels."""
