@@ -20,8 +20,8 @@ BF16_RTOL, BF16_ATOL = 2e-2, 1e-2
 
 
 def _check(got, ref, tier, what, ref32=None):
-    """ref32 (fp32 tier, alpha gradients only): the same quantity from the oracle evaluated in plain
-    float32 PyTorch.  Where that evaluation itself misses the float64 value by more than a third of the
+    """ref32 (fp32 tier; gradients that are one sum over the batch with mixed signs: dalpha and the
+    static coefficient gradients): the same quantity from the oracle evaluated in plain float32 PyTorch.  Where that evaluation itself misses the float64 value by more than a third of the
     bar (a sum over batch and projection rows with mixed signs: 1.3e-5 at the headline shape), three
     times its deviation is the bar."""
     ref = torch.as_tensor(ref).double()
@@ -320,7 +320,13 @@ def _random_cases(count, seed):
     return cases
 
 
-@pytest.mark.parametrize("B,n,C,T,dyn,bf16,inject", _random_cases(40, seed=2024))
+# two cases kept from wider sweeps: a static Sinkhorn gradient that plain float32 PyTorch misses by
+# 7.5e-5, and a single-channel layer with 32 streams
+_KEPT_CASES = [(260, 2, 100, 20, False, False, False), (1, 32, 1, 1, True, False, False),
+               (3, 32, 1, 1, True, False, False)]
+
+
+@pytest.mark.parametrize("B,n,C,T,dyn,bf16,inject", _random_cases(40, seed=2024) + _KEPT_CASES)
 def test_random_shapes_vs_oracle(B, n, C, T, dyn, bf16, inject):
     """Seeded sweep over shapes, iteration counts (0 and 1 included), both coefficient modes, both
     precision tiers and both views, against the oracle."""
@@ -347,6 +353,8 @@ def test_random_shapes_vs_oracle(B, n, C, T, dyn, bf16, inject):
                            w_dtype=act)
     else:
         y_ref, g_ref = nm.mhc_static_fwd_bwd(x, p, dy, T, eps, f_inject=f, dtype=ref_dtype)
+        if not bf16:
+            g_ref32 = nm.mhc_static_fwd_bwd(x, p, dy, T, eps, f_inject=f, dtype=torch.float32)[1]
         y, g = hip_static(x, p, dy, T, eps, f_inject=f, act_dtype=act, out_dtype=act, w_dtype=act)
     _check(y, y_ref, tier, "y")
     assert set(g_ref) <= set(g), f"missing gradients {set(g_ref) - set(g)}"
@@ -365,4 +373,14 @@ def test_random_shapes_vs_oracle(B, n, C, T, dyn, bf16, inject):
             # noise of that size) and a relative comparison is meaningless
             assert float((g[k].double() - torch.as_tensor(ref).double()).abs().max()) < (1e-2 if bf16 else 1e-4), k
             continue
-        _check(g[k], ref, tier, "d" + k, ref32=g_ref32[k] if (g_ref32 is not None and k == "alpha") else None)
+        if C == 1 and not inject and not bf16 and k == "x":
+            # one channel: the backward of the inner RMSNorm is the difference of two terms that are
+            # equal up to eps / q^2, and the kernels rebuild the aggregate in two launches with
+            # different summation orders, so the difference carries their rounding (seen: 4.6e-5 of
+            # |dx| with 32 streams); a hidden size of 1 is a degenerate layer
+            assert rel_err(torch.as_tensor(g[k]).double().cpu(), torch.as_tensor(ref).double()) <= 2e-4, k
+            continue
+        # batch sums with mixed signs (dalpha; the static coefficient gradients): measured against
+        # what plain float32 PyTorch achieves on them when that is worse than the bar
+        summed = k in ("alpha", "H_res", "H_pre", "H_post")
+        _check(g[k], ref, tier, "d" + k, ref32=g_ref32[k] if (g_ref32 is not None and summed) else None)
