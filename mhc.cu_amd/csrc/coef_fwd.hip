@@ -74,7 +74,7 @@ template <int NP> __global__ __launch_bounds__(64) void coef_fwd_small_kernel(Co
         const int c = c0 + e;
         m[e] = (r0 < n && c < n) ? expf(logit(2 * n + r0 * n + c, al[2], a.b_res[r0 * n + c])) : 0.f;
     }
-    SK::forward(m, g, n, a.T, a.eps, nullptr, lane);
+    SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, lane);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;

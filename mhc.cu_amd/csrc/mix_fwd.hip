@@ -297,7 +297,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             } else {
                 m[0] = 0.f;
             }
-            SK::forward(m, g, n, a.T, a.eps, nullptr, tid);
+            SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, tid);
             coef_s[r0 * NP + c0] = m[0];
             if (wr && a.M && mv) a.M[ms + r0 * n + c0] = m[0];
         }

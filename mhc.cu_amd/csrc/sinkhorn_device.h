@@ -55,11 +55,12 @@ template <int NP> struct SkSmall {
     __device__ static __forceinline__ float group_allreduce(float v) { return col_allreduce(row_allreduce(v)); }
 
     // m: in = exp(logits) (0 outside n x n), out = final iterate.
-    // sc != nullptr: keep, per iteration t and lane, the row denominator and per element the column
-    // denominator:  sc[(t * kRec + k) * 64 + lane], k = 0: rho | 1..EPL: s
+    // RECORD: keep, per iteration t and lane, the row denominator and per element the column
+    // denominator:  sc[(t * kRec + k) * 64 + lane], k = 0: rho | 1..EPL: s  (a compile-time switch:
+    // a test of the pointer stays in the loop as two branches per iteration)
     // PRECISE selects IEEE divisions (fp32 parity tier) instead of v_rcp_f32.
     static constexpr int kRec = 1 + EPL;
-    template <bool PRECISE = false>
+    template <bool PRECISE = false, bool RECORD = true>
     __device__ static __forceinline__ void forward(float (&m)[EPL], int g, int n, int T, float eps,
                                                    float *sc, int lane) {
         // rows and columns beyond n hold zeros: their denominator is made 1 (not eps, which may be
@@ -74,12 +75,12 @@ template <int NP> struct SkSmall {
             for (int e = 0; e < EPL; e++) rs += m[e];
             rs = row_allreduce(rs) + eps_r;
             const float rinv = PRECISE ? 1.0f / rs : fast_rcp(rs);
-            if (sc) sc[(t * kRec) * kWave + lane] = rs;
+            if constexpr (RECORD) sc[(t * kRec) * kWave + lane] = rs;
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
                 m[e] = PRECISE ? m[e] / rs : m[e] * rinv;
                 const float cs = col_allreduce(m[e]) + eps_c[e];
-                if (sc) sc[(t * kRec + 1 + e) * kWave + lane] = cs;
+                if constexpr (RECORD) sc[(t * kRec + 1 + e) * kWave + lane] = cs;
                 m[e] = PRECISE ? m[e] / cs : m[e] * fast_rcp(cs);
             }
         }
@@ -91,25 +92,40 @@ template <int NP> struct SkSmall {
     template <bool PRECISE = false>
     __device__ static __forceinline__ void backward(float (&d)[EPL], float (&m)[EPL], int T,
                                                     const float *sc, int lane) {
-        for (int t = T - 1; t >= 0; t--) {
-            const float rs = sc[(t * kRec) * kWave + lane];
-            const float rinv = PRECISE ? 0.f : fast_rcp(rs);
-            float rdot = 0.f;
-            float dR[EPL];
-#pragma unroll
-            for (int e = 0; e < EPL; e++) {
-                const float cs = sc[(t * kRec + 1 + e) * kWave + lane];
-                const float cdot = col_allreduce(d[e] * m[e]);
-                dR[e] = PRECISE ? (d[e] - cdot) / cs : (d[e] - cdot) * fast_rcp(cs);
-                m[e] *= cs;  // R_t
-                rdot += dR[e] * m[e];
-            }
-            rdot = row_allreduce(rdot);
-#pragma unroll
-            for (int e = 0; e < EPL; e++) {
-                d[e] = PRECISE ? (dR[e] - rdot) / rs : (dR[e] - rdot) * rinv;
-                m[e] *= rs;  // Out_{t-1}
-            }
+        static_assert(EPL == 1, "one element per lane");
+        // The denominators of an iteration are requested one iteration ahead of their use (two
+        // register pairs, alternating), so that the LDS round trip stays off the dependent chain.
+        auto fetch = [&](int t, float &rs, float &cs) {
+            t = t < 0 ? 0 : t;
+            rs = sc[(t * kRec) * kWave + lane];
+            cs = sc[(t * kRec + 1) * kWave + lane];
+        };
+        auto step = [&](float rs, float cs) {
+            const float cdot = col_allreduce(d[0] * m[0]);
+            const float dR = PRECISE ? (d[0] - cdot) / cs : (d[0] - cdot) * fast_rcp(cs);
+            m[0] *= cs;  // R_t
+            const float rdot = row_allreduce(dR * m[0]);
+            d[0] = PRECISE ? (dR - rdot) / rs : (dR - rdot) * fast_rcp(rs);
+            m[0] *= rs;  // Out_{t-1}
+        };
+        float rs0, cs0, rs1, cs1;
+        int t = T - 1;
+        fetch(t, rs0, cs0);
+        if (T & 1) {  // an odd count: one step ahead of the pairs
+            step(rs0, cs0);
+            fetch(--t, rs0, cs0);
+        }
+        // (the scheduling barriers keep the reciprocals of the values in flight, which do not depend
+        // on the chain, from being moved up into the step before and dragging the wait with them)
+        for (; t >= 1; t -= 2) {
+            fetch(t - 1, rs1, cs1);
+            __builtin_amdgcn_sched_barrier(0);
+            step(rs0, cs0);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(t - 2, rs0, cs0);
+            __builtin_amdgcn_sched_barrier(0);
+            step(rs1, cs1);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
     __host__ __device__ static constexpr int scaling_floats(int T) { return T * kRec * kWave; }
