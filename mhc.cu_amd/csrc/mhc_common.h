@@ -289,6 +289,12 @@ __device__ __forceinline__ float block_allreduce_sum(float v, float *red, int nw
 
 __device__ __forceinline__ float sigmoidf_acc(float t) { return 1.0f / (1.0f + expf(-t)); }
 
+// bf16 tier: exp and sigmoid on the hardware's exp2 and reciprocal (1 ulp each, a handful of
+// instructions; the library versions are ~15 and ~30 dependent instructions, which shows on the
+// serial coefficient step that every workgroup runs before it can mix its tile).
+__device__ __forceinline__ float exp_fast(float t) { return __builtin_amdgcn_exp2f(t * 1.44269504088896341f); }
+__device__ __forceinline__ float sigmoid_fast(float t) { return __builtin_amdgcn_rcpf(1.0f + exp_fast(-t)); }
+
 // v_rcp_f32: 1 ulp, one instruction (an IEEE division costs ~10 dependent instructions, which
 // matters on the serial Sinkhorn chain).
 __device__ __forceinline__ float fast_rcp(float v) { return __builtin_amdgcn_rcpf(v); }

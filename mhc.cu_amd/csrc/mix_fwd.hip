@@ -267,10 +267,13 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
     if (tid < 64) {
         MHC_PHASE(kPhaseFwdFused, b, 2);
         if (tid < SK::kGroup) {
+            // bf16 tier: hardware exp2 / reciprocal / square root (1 ulp) instead of the library routines
+            constexpr bool kFast = !std::is_same<TX, float>::value;
             float rinv = 0.f;
             if (dyn) {
-                const float r = sqrtf(ssq / (float)(n * C) + a.eps);
-                rinv = 1.0f / r;
+                const float ms = ssq * (1.0f / (float)(n * C)) + a.eps;
+                const float r = kFast ? __builtin_amdgcn_sqrtf(ms) : sqrtf(ssq / (float)(n * C) + a.eps);
+                rinv = kFast ? fast_rcp(r) : 1.0f / r;
                 if (g == 0) a.r[b] = r;
             }
             const bool wr = dyn || b == 0;  // static coefficients are written once
@@ -279,7 +282,10 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
                 const bool pre = g < n;
                 const int gi = pre ? g : g - n;
                 const float p = pvec * rinv;
-                const float h = pre ? sigmoidf_acc(al0 * p + bvec) : 2.0f * sigmoidf_acc(al1 * p + bvec);
+                // one sigmoid for both kinds of lane (two would run one after the other)
+                const float z = (pre ? al0 : al1) * p + bvec;
+                const float sg = kFast ? sigmoid_fast(z) : sigmoidf_acc(z);
+                const float h = pre ? sg : 2.0f * sg;
                 coef_s[NP * NP + (pre ? 0 : NP) + gi] = h;
                 float *dst = pre ? a.Hpre : a.Hpost;
                 if (wr && dst) dst[hs + gi] = h;
@@ -293,7 +299,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             if (mv) {
                 const float p = pe * rinv;
                 if (dyn) a.P[(size_t)b * D + 2 * n + r0 * n + c0] = p;
-                m[0] = expf(al2 * p + bres);
+                m[0] = kFast ? exp_fast(al2 * p + bres) : expf(al2 * p + bres);
             } else {
                 m[0] = 0.f;
             }
