@@ -272,7 +272,7 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
 
     int r0, c0, gc;
     bool inject, mv;
-    float qinv, rinv, al0, al1, al2, pres, bres, hp, ho, ppre, ppost, hpre_r, hpost_r;
+    float qinv, rinv, inv_c, inv_nc, al0, al1, al2, pres, bres, hp, ho, ppre, ppost, hpre_r, hpost_r;
     float E, m_fin;  // exp(logit) and the final Sinkhorn iterate of this lane's element (forward_recompute)
     float dMe, s_a, s_b, s_c, s_d;  // this lane's channel sums (fetch_sums): GRAM w1, w1t, xx | else dHpost, A1, A2, s1
 
@@ -282,10 +282,12 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
         gc = g < n ? g : 0;  // lanes beyond n alias entry 0 (never used): no branch around loads
         mv = r0 < n && c0 < n;
         inject = a.f_inject != nullptr;
-        qinv = inject ? 0.f : 1.0f / a.q[b];
+        // PRECISE keeps IEEE divisions; otherwise v_rcp_f32 / v_exp_f32 (1 ulp) keep the step short
+        qinv = inject ? 0.f : (PRECISE ? 1.0f / a.q[b] : fast_rcp(a.q[b]));
+        inv_c = 1.0f / (float)a.C; inv_nc = 1.0f / (float)(n * a.C);
         const float *Pb = a.P + (size_t)b * D;
         al0 = a.alpha[0]; al1 = a.alpha[1]; al2 = a.alpha[2];
-        rinv = 1.0f / a.r[b];
+        rinv = PRECISE ? 1.0f / a.r[b] : fast_rcp(a.r[b]);
         pres = Pb[mv ? 2 * n + r0 * n + c0 : 0];
         bres = a.b_res[mv ? r0 * n + c0 : 0];
         hp = a.Hpre[(size_t)b * n + gc]; ho = a.Hpost[(size_t)b * n + gc];
@@ -298,7 +300,7 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
     // none of the channel sums, so a caller that produces them itself can run it while they are
     // still on their way.  g: lane within the group; lane: lane within the wave (indexes sc).
     __device__ __forceinline__ void forward_recompute(const BwdReduceArgs &a, int g, int lane, float *sc) {
-        E = mv ? expf(al2 * pres + bres) : 0.f;
+        E = mv ? (PRECISE ? expf(al2 * pres + bres) : exp_fast(al2 * pres + bres)) : 0.f;
         float m[1] = {E};
         SK::template forward<PRECISE>(m, g, a.n, a.T, a.eps, sc, lane);
         m_fin = m[0];
@@ -323,7 +325,7 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
 
     // after fetch_sums() and forward_recompute(); xch: kXch floats of LDS private to the group
     __device__ __forceinline__ void run(const BwdReduceArgs &a, int b, int g, int lane, float *sc, float *xch) {
-        const int n = a.n, C = a.C, D = n * n + 2 * n;
+        const int n = a.n, D = n * n + 2 * n;
         float tpost = 0.f, tA1 = 0.f, tA2 = 0.f, s1 = 0.f;
         if constexpr (GRAM) {
             // lane (r0, c0) takes its element of each matrix and the mirrored element of W1, so that
@@ -357,7 +359,7 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
         float S0 = 0.f, S1 = 0.f, S2 = 0.f;  // sum_d dt_d p_d per alpha group
         if (g < n) {
             const float dHpost = tpost;
-            const float dHpre = inject ? 0.f : tA1 * qinv - s1 * tA2 * qinv * qinv * qinv / (float)C;
+            const float dHpre = inject ? 0.f : tA1 * qinv - s1 * tA2 * qinv * qinv * qinv * inv_c;
             const float dtp = dHpre * hp * (1.0f - hp);
             const float dto = dHpost * ho * (1.0f - 0.5f * ho);
             dt[g] = dtp; dt[n + g] = dto;
@@ -376,7 +378,7 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
         S0 = SK::group_allreduce(S0); S1 = SK::group_allreduce(S1); S2 = SK::group_allreduce(S2);
         if (g == 0) {
             dt[D] = S0; dt[D + 1] = S1; dt[D + 2] = S2;
-            a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv / (float)(n * C);
+            a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv * inv_nc;
         }
         dpw.pad(D, g, SK::kGroup);
     }
