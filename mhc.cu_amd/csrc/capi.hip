@@ -34,6 +34,7 @@ int check_shape(int B, int n, int C, int iters) {
     if (n < 1 || n > MHC_MAX_N) return MHC_ERR_BAD_N;
     if (B < 1 || C < 1 || iters < 0 || iters > max_layer_sinkhorn_iters(n)) return MHC_ERR_BAD_SHAPE;
     if ((long long)B * n * C > (1ll << 40)) return MHC_ERR_BAD_SHAPE;
+    if (n > 8 && B > 65535) return MHC_ERR_BAD_SHAPE;  // the n > 8 kernels index samples by blockIdx.y
     return MHC_OK;
 }
 
