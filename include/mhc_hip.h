@@ -42,6 +42,7 @@ extern "C" {
 
 #define MHC_ABI_VERSION 1
 #define MHC_MAX_N 32
+#define MHC_MAX_C 32768 /* largest hidden size C of the layer entry points (a [C] float row is kept in LDS) */
 
 enum mhc_dtype { MHC_F32 = 0, MHC_BF16 = 1 };
 
@@ -49,7 +50,7 @@ enum mhc_status {
     MHC_OK = 0,
     MHC_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
     MHC_ERR_BAD_N = 2,          /* expansion rate outside 1..MHC_MAX_N */
-    MHC_ERR_BAD_SHAPE = 3,      /* B, C or iters not positive / too large (n > 8: B <= 65535) */
+    MHC_ERR_BAD_SHAPE = 3,      /* B, C or iters not positive / too large (C <= MHC_MAX_C; n > 8: B <= 65535) */
     MHC_ERR_BAD_DTYPE = 4,      /* unknown or unsupported dtype combination */
     MHC_ERR_MISALIGNED = 5,     /* a tensor base pointer is not 16-byte aligned */
     MHC_ERR_WORKSPACE = 6,      /* workspace NULL, misaligned or too small */

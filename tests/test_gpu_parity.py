@@ -324,6 +324,11 @@ def _random_cases(count, seed):
 # 7.5e-5, and a single-channel layer with 32 streams
 _KEPT_CASES = [(260, 2, 100, 20, False, False, False), (1, 32, 1, 1, True, False, False),
                (3, 32, 1, 1, True, False, False)]
+# long rows, up to the largest accepted hidden size (a wider sweep over C = 8192 .. 32768, n = 1 .. 32, both
+# tiers and both coefficient modes passed as well)
+_KEPT_CASES += [(3, 4, 32768, 20, True, True, False), (2, 32, 32768, 20, True, True, False),
+                (3, 8, 20000, 20, True, True, False), (33, 1, 32768, 20, False, False, False),
+                (3, 9, 16384, 20, True, False, False), (3, 4, 12296, 20, False, True, False)]
 
 
 @pytest.mark.parametrize("B,n,C,T,dyn,bf16,inject", _random_cases(40, seed=2024) + _KEPT_CASES)
@@ -361,8 +366,6 @@ def test_random_shapes_vs_oracle(B, n, C, T, dyn, bf16, inject):
     if n > 1 and C > 1:
         g, g_ref = _alpha_as_vector(g, g_ref), _alpha_as_vector(g_ref)
         g_ref32 = None if g_ref32 is None else _alpha_as_vector(g_ref32)
-    else:
-        g_ref32 = None
     for k, ref in g_ref.items():
         tiny = ("phi_pre", "b_pre", "alpha_pre", "H_pre") + (("phi_res", "b_res", "alpha_res", "H_res") if T > 0 and n == 1 else ())
         # one channel: the inner RMSNorm maps the aggregate to its sign, so f does not depend on H_pre
@@ -371,7 +374,9 @@ def test_random_shapes_vs_oracle(B, n, C, T, dyn, bf16, inject):
             # one stream: f does not depend on H_pre except through eps, and the 1 x 1 Sinkhorn output
             # (after at least one iteration) is 1 / (1 + O(eps)) whatever its logit, so these gradients are O(eps) (bf16: rounding
             # noise of that size) and a relative comparison is meaningless
-            assert float((g[k].double() - torch.as_tensor(ref).double()).abs().max()) < (1e-2 if bf16 else 1e-4), k
+            # (their rounding noise grows with the row length: plain float32 PyTorch is 1.5e-4 off at C = 32768)
+            bar = 1e-2 if bf16 else 1e-4 * max(1.0, C / 1024)
+            assert float((g[k].double() - torch.as_tensor(ref).double()).abs().max()) < bar, k
             continue
         if C == 1 and not inject and not bf16 and k == "x":
             # one channel: the backward of the inner RMSNorm is the difference of two terms that are
@@ -382,5 +387,5 @@ def test_random_shapes_vs_oracle(B, n, C, T, dyn, bf16, inject):
             continue
         # batch sums with mixed signs (dalpha; the static coefficient gradients): measured against
         # what plain float32 PyTorch achieves on them when that is worse than the bar
-        summed = k in ("alpha", "H_res", "H_pre", "H_post")
+        summed = k.startswith("alpha") or k in ("H_res", "H_pre", "H_post")
         _check(g[k], ref, tier, "d" + k, ref32=g_ref32[k] if (g_ref32 is not None and summed) else None)
