@@ -12,6 +12,12 @@ constexpr int kSkMax = 128;
 // Iterate = diag(u) inp diag(v); a half step only updates u or v.  One workgroup per matrix;
 // the matrix itself stays in global memory (L2 resident), u / v / sums live in LDS.
 // scal (optional, backward): [batch][T][2][kSkMax] divisors (-1 where the division was skipped).
+// A rows x cols matrix with rows != cols has row sums near cols / rows after every column step, so
+// the plain scalings would grow like (rows / cols)^t and (cols / rows)^t and leave float32 after a
+// few dozen iterations (128 x 3: 25).  The stored u therefore carries an extra factor kappa^t and the
+// stored v the factor kappa^-t, kappa = cols / rows: every row step multiplies u by kappa on top of
+// its division and every column step finds its sums multiplied by kappa.  The product u v, the
+// recorded divisors and the eps test are those of the plain iteration; kappa = 1 for square input.
 __global__ __launch_bounds__(256) void sinkhorn_plain_fwd_kernel(const float *__restrict__ inp,
                                                                  float *__restrict__ out, int rows,
                                                                  int cols, int T, float eps,
@@ -21,6 +27,7 @@ __global__ __launch_bounds__(256) void sinkhorn_plain_fwd_kernel(const float *__
     const float *A = inp + (size_t)blockIdx.x * rows * cols;
     float *sc = scal ? scal + (size_t)blockIdx.x * T * 2 * kSkMax : nullptr;
     if (tid < kSkMax) { u[tid] = 1.f; v[tid] = 1.f; }
+    const float kappa = (float)cols / (float)rows, kappa_inv = (float)rows / (float)cols;
     __syncthreads();
     for (int t = 0; t < T; t++) {
         // rows: two threads per row
@@ -33,7 +40,7 @@ __global__ __launch_bounds__(256) void sinkhorn_plain_fwd_kernel(const float *__
             if (r < rows && h == 0) {
                 const float sum = u[r] * acc;
                 const bool doit = sum > eps;
-                if (doit) u[r] /= sum;
+                u[r] = doit ? u[r] / sum * kappa : u[r] * kappa;
                 if (sc) sc[(t * 2) * kSkMax + r] = doit ? sum : -1.0f;  // negative = skipped
             }
         }
@@ -48,9 +55,10 @@ __global__ __launch_bounds__(256) void sinkhorn_plain_fwd_kernel(const float *__
             if (h == 1) half_sum[c] = acc;
             __syncthreads();
             if (h == 0 && c < cols) {
-                const float sum = v[c] * (acc + half_sum[c]);
+                const float scaled = v[c] * (acc + half_sum[c]);  // kappa x the column sum
+                const float sum = scaled * kappa_inv;
                 const bool doit = sum > eps;
-                if (doit) v[c] /= sum;
+                v[c] = doit ? v[c] / scaled : v[c] * kappa_inv;
                 if (sc) sc[(t * 2 + 1) * kSkMax + c] = doit ? sum : -1.0f;
             }
         }
@@ -74,11 +82,13 @@ __global__ __launch_bounds__(256) void sinkhorn_plain_bwd_kernel(const float *__
     const float *G = grad + (size_t)blockIdx.x * rows * cols;
     float *dO = d_inp + (size_t)blockIdx.x * rows * cols;
     const float *sc = scal + (size_t)blockIdx.x * T * 2 * kSkMax;
+    // u and v carry kappa^t and kappa^-t like the forward kernel's (see there)
+    const float kappa = (float)cols / (float)rows, kappa_inv = (float)rows / (float)cols;
     if (tid < kSkMax) {
         float uu = 1.f, vv = 1.f;
         for (int t = 0; t < T; t++) {
-            uu /= fabsf(sc[(t * 2) * kSkMax + tid]);  // entries beyond rows/cols are masked below
-            vv /= fabsf(sc[(t * 2 + 1) * kSkMax + tid]);
+            uu = uu / fabsf(sc[(t * 2) * kSkMax + tid]) * kappa;  // entries beyond rows/cols are masked below
+            vv = vv / fabsf(sc[(t * 2 + 1) * kSkMax + tid]) * kappa_inv;
         }
         u[tid] = tid < rows ? uu : 0.f;
         v[tid] = tid < cols ? vv : 0.f;
@@ -113,8 +123,8 @@ __global__ __launch_bounds__(256) void sinkhorn_plain_bwd_kernel(const float *__
             dO[e] = ((dO[e] - cdot[c]) / fabsf(s[c]) - rdot[r]) / fabsf(rho[r]);
         }
         __syncthreads();
-        if (tid < rows) u[tid] *= fabsf(rho[tid]);
-        if (tid < cols) v[tid] *= fabsf(s[tid]);
+        if (tid < rows) u[tid] *= fabsf(rho[tid]) * kappa_inv;
+        if (tid < cols) v[tid] *= fabsf(s[tid]) * kappa;
         __syncthreads();
     }
 }

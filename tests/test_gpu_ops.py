@@ -20,7 +20,9 @@ def test_sinkhorn_knopp_doubly_stochastic():
 
 
 @pytest.mark.parametrize("shape,iters", [((32, 32), 10), ((64, 64), 20), ((4, 4), 20), ((5, 9), 7),
-                                         ((3, 16, 16), 10), ((128, 128), 5), ((2, 8, 8), 20)])
+                                         ((3, 16, 16), 10), ((128, 128), 5), ((2, 8, 8), 20),
+                                         ((70000, 4, 4), 20), ((3000, 32, 32), 3), ((7, 128, 3), 1024),
+                                         ((4, 3, 100), 200), ((2, 64, 128), 60)])
 def test_sinkhorn_knopp_forward_backward_vs_oracle(shape, iters):
     from mhc import sinkhorn_knopp
     g = torch.Generator().manual_seed(1)
@@ -45,7 +47,7 @@ def test_sinkhorn_knopp_stability_and_zero_rows():
     assert torch.equal(sinkhorn_knopp(z, num_iters=3), z)   # thresholded division: no 0/0
 
 
-@pytest.mark.parametrize("rows,C", [(8, 128), (128, 4096), (16, 64), (5, 100)])
+@pytest.mark.parametrize("rows,C", [(8, 128), (128, 4096), (16, 64), (5, 100), (3, 100000), (70000, 64), (1, 1)])
 def test_rmsnorm_forward_backward_vs_oracle(rows, C):
     """bf16 operator as in the reference (test_rmsnorm.cu tolerance 1e-2, backward 2e-2)."""
     from mhc import rmsnorm
