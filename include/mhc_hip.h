@@ -147,7 +147,8 @@ MHC_API int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtyp
 MHC_API int mhc_sinkhorn_knopp_fwd(const float *inp, float *out, int batch, int rows, int cols, int iters,
                            float eps, void *stream);
 
-/* Exact gradient of the call above w.r.t. inp (recomputes the iterates from inp). */
+/* Exact gradient of the call above w.r.t. inp (recomputes the iterates from inp).  float32 round-off
+ * relative to float64 grows by about 1e-7 per iteration (1e-5 at 100, 1e-4 at the limit of 1024). */
 MHC_API int mhc_sinkhorn_knopp_bwd(const float *grad_out, const float *inp, float *d_inp, int batch,
                            int rows, int cols, int iters, float eps, void *workspace,
                            size_t workspace_bytes, void *stream);
