@@ -171,3 +171,34 @@ def test_derived_parameter_caches_never_serve_a_different_tensor():
         assert rel_err(y, ref) < 1e-5
         outs.append(y)
     assert (outs[0] - outs[1]).abs().max() > 1e-4
+
+
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_layer_unusual_inputs(dynamic):
+    """Half and double inputs are widened like the reference's .float() (gradients come back in the
+    input's dtype), views that are not contiguous are accepted, and a graph kept alive can be
+    differentiated twice with the same result."""
+    from mhc import MHCLayer
+    B, n, C = 5, 4, 96
+    torch.manual_seed(3)
+    layer = MHCLayer(hidden_dim=C, expansion_rate=n, use_dynamic_h=dynamic).cuda()
+    base = torch.randn(B, n, C, device="cuda")
+    y0 = layer(base)
+    for dt in (torch.float16, torch.float64):
+        x = base.to(dt).requires_grad_(True)
+        y = layer(x)
+        assert y.dtype == torch.float32
+        y.sum().backward()
+        assert x.grad.dtype == dt and x.grad.shape == x.shape
+        assert rel_err(y, layer(x.detach().float())) < 1e-6
+    xt = base.transpose(0, 1).contiguous().transpose(0, 1)   # same values, strides of [n, B, C]
+    assert not xt.is_contiguous()
+    assert torch.equal(layer(xt), y0)
+    x = base.clone().requires_grad_(True)
+    y = layer(x)
+    g1, = torch.autograd.grad(y, x, torch.ones_like(y), retain_graph=True)
+    g2, = torch.autograd.grad(y, x, torch.ones_like(y))
+    assert torch.equal(g1, g2)
+    layer.eval()
+    with torch.no_grad():
+        assert rel_err(layer(base), y0) < 1e-6   # inference path: same numbers, nothing saved
