@@ -143,8 +143,10 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     }
     float rinv = 0.f;
     if (dyn) {
-        const float r = sqrtf(wave_allreduce_sum(ssq_l) / (float)a.nC + a.eps);
-        rinv = 1.0f / r;
+        // PRECISE keeps the library routines; otherwise v_sqrt_f32 / v_rcp_f32 / v_exp_f32 (1 ulp)
+        const float ms = wave_allreduce_sum(ssq_l) / (float)a.nC + a.eps;
+        const float r = PRECISE ? sqrtf(ms) : __builtin_amdgcn_sqrtf(ms);
+        rinv = PRECISE ? 1.0f / r : fast_rcp(r);
         if (tid == 0) a.r[b] = r;
     }
 #pragma unroll
@@ -163,9 +165,9 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     }
     __syncthreads();
     if (tid < n) {
-        const float hp = sigmoidf_acc(lg[tid]);
+        const float hp = PRECISE ? sigmoidf_acc(lg[tid]) : sigmoid_fast(lg[tid]);
         a.Hpre[b * n + tid] = hp;
-        a.Hpost[b * n + tid] = 2.0f * sigmoidf_acc(lg[n + tid]);
+        a.Hpost[b * n + tid] = 2.0f * (PRECISE ? sigmoidf_acc(lg[n + tid]) : sigmoid_fast(lg[n + tid]));
         if constexpr (AGG) hp_s[tid] = hp;
     } else if (AGG && tid < 32) {
         hp_s[tid] = 0.f;
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     float E[SK::EPL], u, v[SK::EPL];
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
-        E[e] = (r0 < n && c0 + e < n) ? expf(lg[2 * n + r0 * n + c0 + e]) : 0.f;
+        E[e] = (r0 < n && c0 + e < n) ? (PRECISE ? expf(lg[2 * n + r0 * n + c0 + e]) : exp_fast(lg[2 * n + r0 * n + c0 + e])) : 0.f;
     SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)

@@ -880,7 +880,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
     const int b = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x, lane = tid & 63;
     const bool w0 = tid < 64;
     const bool inject = a.f_inject != nullptr;
-    const float qinv = inject ? 0.f : 1.0f / a.q[b];
+    const float qinv = inject ? 0.f : (PRECISE ? 1.0f / a.q[b] : fast_rcp(a.q[b]));
     if (tid < 32) {
         hp_s[tid] = tid < n ? a.Hpre[(size_t)b * a.hstride + tid] : 0.f;
         ho_s[tid] = tid < n ? a.Hpost[(size_t)b * a.hstride + tid] : 0.f;
@@ -894,7 +894,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
     float al0 = 0.f, al1 = 0.f, al2 = 0.f, rinv = 0.f;
     if (dyn) {
         al0 = a.alpha[0]; al1 = a.alpha[1]; al2 = a.alpha[2];
-        rinv = 1.0f / a.r[b];
+        rinv = PRECISE ? 1.0f / a.r[b] : fast_rcp(a.r[b]);
     }
     float pres[SK::EPL], bres[SK::EPL];
 #pragma unroll
@@ -920,7 +920,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         for (int e = 0; e < SK::EPL; e++) {
             const bool ok = r0 < n && c0 + e < n;
             pres[e] = ok ? pres[e] : 0.f;
-            E[e] = ok ? expf(al2 * pres[e] + bres[e]) : 0.f;
+            E[e] = ok ? (PRECISE ? expf(al2 * pres[e] + bres[e]) : exp_fast(al2 * pres[e] + bres[e])) : 0.f;
         }
         SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
     }
