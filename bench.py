@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # WRITE_SIZE summed over the step's kernels and scaled by what the same counters read for
 # `--copy-calibration` (a 64 MiB copy).  Filled from the committed counter summaries; None where
 # no counter run exists for the configuration.
-MEASURED_TRAFFIC_BYTES = {"c1": 13275965, "c2": 42677762, "c3": 248310104, "c4": 75947976, "c5": 549146397}
+MEASURED_TRAFFIC_BYTES = {"c1": 13275949, "c2": 42677933, "c3": 248312520, "c4": 75948103, "c5": 549083493}
 
 CONFIGS = {
     "c1": dict(kind="static", B=320, n=4, C=1280, dtype="f32", bwd=False),
