@@ -54,7 +54,8 @@ enum mhc_status {
     MHC_ERR_BAD_DTYPE = 4,      /* unknown or unsupported dtype combination */
     MHC_ERR_MISALIGNED = 5,     /* a tensor base pointer is not 16-byte aligned */
     MHC_ERR_WORKSPACE = 6,      /* workspace NULL, misaligned or too small */
-    MHC_ERR_LAUNCH = 7          /* the HIP runtime refused a kernel launch */
+    MHC_ERR_LAUNCH = 7,         /* the HIP runtime refused a kernel launch */
+    MHC_ERR_SCRATCH_LIMIT = 8   /* the shape needs more than MHC_STATIC_SCRATCH_BYTES of scratch */
 };
 
 /* Version of this header the library was built from (== MHC_ABI_VERSION). */
@@ -107,6 +108,29 @@ MHC_API int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, in
                           const float *q, void *dx, void *df, float *dw, float *dphi,
                           float *dbias, float *dalpha, int B, int n, int C, int iters, float eps,
                           void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * mhc_layer_fwd_dynamic for callers that cannot allocate device memory or pass a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Same arguments and results as mhc_layer_fwd_dynamic minus the
+ * workspace: the scratch is a device array of MHC_STATIC_SCRATCH_BYTES inside the library (held by
+ * every GPU the library runs on until the process ends).  The call allocates nothing.  Shapes whose
+ * scratch need (mhc_layer_fwd_dynamic_scratch_bytes) exceeds the array return
+ * MHC_ERR_SCRATCH_LIMIT before any launch.  All calls on one GPU share that GPU's array: calls that
+ * overlap on one GPU (different streams or threads) race; order them on one stream.
+ * mhc_static_scratch_init looks up the array's address for the current device (the first call on a
+ * device does the same); call it once per device before capturing a graph.
+ */
+#define MHC_STATIC_SCRATCH_BYTES (32u << 20)
+MHC_API size_t mhc_static_scratch_capacity(void);
+MHC_API size_t mhc_layer_fwd_dynamic_scratch_bytes(int B, int n, int C);
+MHC_API int mhc_static_scratch_init(void);
+MHC_API int mhc_layer_fwd_dynamic_static_scratch(const void *x, int x_dtype, const void *w, int w_dtype,
+                                         const void *phi, int phi_dtype, const float *bias,
+                                         const float *alpha, const void *f_inject, void *y, int y_dtype,
+                                         float *H_pre, float *H_post, float *M, float *P, float *r,
+                                         float *q, int B, int n, int C, int iters, float eps,
+                                         void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Static-H layer.  Replaces mhc_cuda.mhc_layer_fwd / mhc_layer_fwd_inference / mhc_layer_bwd

@@ -1,12 +1,16 @@
 // C ABI of libmhc_hip.so (declared in include/mhc_hip.h): argument validation, workspace
 // carving and the launch sequence of each entry point.  No allocation, no synchronisation,
-// no global state; every call only enqueues kernels on the caller's stream.
+// no global state; every call only enqueues kernels on the caller's stream.  The one exception
+// is mhc_layer_fwd_dynamic_static_scratch at the end of this file, whose scratch memory is a
+// device array owned by the library.
 #include "../../include/mhc_hip.h"
 
 #include "launchers.h"
 #include "phase_profiler.h"
 
 #include <stdint.h>
+
+#include <mutex>
 
 using namespace mhc;
 
@@ -156,6 +160,8 @@ const char *mhc_status_string(int status) {
         case MHC_ERR_MISALIGNED: return "tensor base pointer is not 16-byte aligned";
         case MHC_ERR_WORKSPACE: return "workspace NULL, not 256-byte aligned or too small";
         case MHC_ERR_LAUNCH: return "HIP kernel launch failed";
+        case MHC_ERR_SCRATCH_LIMIT:
+            return "shape needs more scratch than the library's static array holds (mhc_static_scratch_capacity)";
         default: return "unknown status";
     }
 }
@@ -410,6 +416,71 @@ int mhc_rmsnorm_bwd(const void *grad_out, const void *inp, int dtype, const void
     MHC_LAUNCH(launch_rmsnorm_bwd(grad_out, inp, dtype, w, w_dtype, rms, d_inp, u, rows, C, st));
     MHC_LAUNCH(launch_colsum(u, rows, C, C, d_w, part, st));
     return MHC_OK;
+}
+
+}  // extern "C"
+
+// ===============================================================================================
+// Dynamic forward for callers that cannot allocate (HIP graph capture, serving loops, harnesses
+// that forbid hipMalloc): the scratch of the split-K projection lives in a device array of this
+// library instead of a caller workspace.  Every GPU holds its own copy of the array at its own
+// address; the address is looked up once per device and only that pointer is handed to kernels
+// (the array's name is a host-side stand-in, not a device address).
+// ===============================================================================================
+static __device__ __align__(256) unsigned char scratch[MHC_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` per device, nullptr until looked up
+
+int static_scratch_pointer(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MHC_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return MHC_ERR_LAUNCH;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return MHC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t mhc_static_scratch_capacity(void) { return MHC_STATIC_SCRATCH_BYTES; }
+
+size_t mhc_layer_fwd_dynamic_scratch_bytes(int B, int n, int C) {
+    if (check_shape(B, n, C, 0) != MHC_OK) return 0;
+    return carve_dyn_fwd(nullptr, B, n, C).bytes;
+}
+
+int mhc_static_scratch_init(void) {
+    void *p = nullptr;
+    return static_scratch_pointer(&p);
+}
+
+int mhc_layer_fwd_dynamic_static_scratch(const void *x, int x_dtype, const void *w, int w_dtype,
+                                         const void *phi, int phi_dtype, const float *bias,
+                                         const float *alpha, const void *f_inject, void *y, int y_dtype,
+                                         float *H_pre, float *H_post, float *M, float *P, float *r,
+                                         float *q, int B, int n, int C, int iters, float eps,
+                                         void *stream) {
+    if (int s = check_shape(B, n, C, iters)) return s;
+    // every byte the kernels touch lies below `need`; nothing has to start at zero (the projection
+    // writes each partial sum that the coefficient step reads), so the contents left by the last call
+    // are simply overwritten
+    const size_t need = carve_dyn_fwd(nullptr, B, n, C).bytes;
+    if (need > MHC_STATIC_SCRATCH_BYTES) return MHC_ERR_SCRATCH_LIMIT;
+    void *ptr = nullptr;
+    if (int s = static_scratch_pointer(&ptr)) return s;
+    return mhc_layer_fwd_dynamic(x, x_dtype, w, w_dtype, phi, phi_dtype, bias, alpha, f_inject, y, y_dtype,
+                                 H_pre, H_post, M, P, r, q, B, n, C, iters, eps, ptr,
+                                 MHC_STATIC_SCRATCH_BYTES, stream);
 }
 
 }  // extern "C"

@@ -31,11 +31,11 @@ def test_status_strings():
     from mhc import _lib
 
     seen = set()
-    for code in range(0, 8):
+    for code in range(0, 9):
         s = _lib.lib.mhc_status_string(code).decode()
         assert s and s != "unknown status"
         seen.add(s)
-    assert len(seen) == 8
+    assert len(seen) == 9
     assert _lib.lib.mhc_status_string(99).decode() == "unknown status"
 
 
@@ -85,6 +85,26 @@ def test_argument_validation_happens_before_any_launch():
     assert fwd() == 6                                  # MHC_ERR_WORKSPACE (none given)
     assert L.mhc_sinkhorn_knopp_fwd(a16, a16, 1, 129, 4, 3, 1e-8, None) == 3
     assert L.mhc_rmsnorm_fwd(None, 0, a16, 0, a16, None, 1, 8, 1e-5, None) == 1
+
+
+def test_static_scratch_entry_point_checks_its_limit_before_any_launch():
+    """The entry point that allocates nothing refuses shapes beyond its static array up front."""
+    from mhc import _lib
+
+    L = _lib.lib
+    cap = L.mhc_static_scratch_capacity()
+    assert cap == 32 << 20
+    assert 0 < L.mhc_layer_fwd_dynamic_scratch_bytes(320, 4, 1280) <= cap
+    assert L.mhc_layer_fwd_dynamic_scratch_bytes(8, 33, 64) == 0
+    big = (4096, 32, 1280)  # 37 MiB of split-K partial sums
+    assert L.mhc_layer_fwd_dynamic_scratch_bytes(*big) > cap
+    P = ctypes.c_void_p
+    buf = (ctypes.c_char * 4096)()
+    a16 = P((ctypes.addressof(buf) + 255) // 256 * 256)
+    call = lambda B, n, C: L.mhc_layer_fwd_dynamic_static_scratch(
+        a16, 1, a16, 1, a16, 1, a16, a16, None, a16, 1, a16, a16, a16, a16, a16, a16, B, n, C, 20, 1e-6, None)
+    assert call(*big) == 8          # MHC_ERR_SCRATCH_LIMIT
+    assert call(0, 4, 64) == 3      # shape checks come first
 
 
 def test_python_surface_matches_reference_names():
