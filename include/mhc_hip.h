@@ -110,6 +110,18 @@ MHC_API int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, in
                           void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Gathers the parameters as mhc.MHCLayer stores them (src/python/mhc/layer.py:44-54: phi_pre,
+ * phi_post [n, nC], phi_res [n*n, nC] in src_dtype; b_pre, b_post [n], b_res [n, n] fp32; the three
+ * alpha scalars, fp32, on the device) into phi [D, nC] (phi_dtype), bias [D] and alpha [3] as the two
+ * calls above take them, in one launch.  Replaces the torch.cat(...).bfloat16() and the three
+ * .item() host synchronisations of every reference forward call (src/python/mhc/ops.py:172-188).
+ */
+MHC_API int mhc_pack_dynamic_params(const void *phi_pre, const void *phi_post, const void *phi_res, int src_dtype,
+                            const float *b_pre, const float *b_post, const float *b_res,
+                            const float *alpha_pre, const float *alpha_post, const float *alpha_res,
+                            void *phi, int phi_dtype, float *bias, float *alpha, int n, int C, void *stream);
+
+/*
  * mhc_layer_fwd_dynamic for callers that cannot allocate device memory or pass a workspace: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference.  Same arguments and results as mhc_layer_fwd_dynamic minus the

@@ -1,6 +1,6 @@
 """Builds libmhc_hip.so (hand-written HIP kernels + C ABI) for gfx950 with hipcc.
 
-    python mhc.cu_amd/build.py [--jobs N] [--profile]
+    python mhc.cu_amd/build.py [--jobs N] [--profile] [--no-ext]
 
 hipcc cross-compiles for gfx950 without a GPU.  The library lands in mhc.cu_amd/mhc/ next to
 the Python package that loads it; object files go to mhc.cu_amd/build/.
@@ -18,8 +18,8 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "mhc", "libmhc_hip.so")
 
-SOURCES = ["capi.hip", "proj_fwd.hip", "gemm_f32.hip", "proj_bwd.hip", "proj_bwd_large.hip", "bwd_slab.hip", "coef_fwd.hip", "mix_fwd.hip", "mix_bwd_reduce.hip",
-           "mix_bwd_dx.hip", "param_grads.hip", "ops.hip"]
+SOURCES = ["capi.hip", "proj_fwd.hip", "gemm_f32.hip", "proj_bwd.hip", "proj_bwd_large.hip", "bwd_slab.hip", "coef_fwd.hip", "mix_fwd.hip", "layer_fwd_onepass.hip", "mix_bwd_reduce.hip",
+           "mix_bwd_dx.hip", "param_grads.hip", "pack_params.hip", "ops.hip"]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are not trusted on this hardware pool.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -65,9 +65,50 @@ def build(jobs: int = 8, verbose: bool = True, profile: bool = False):
     return lib
 
 
+EXT_SRC = os.path.join(HERE, "torch_ext", "mhc_torch_ext.cpp")
+EXT_NAME = "mhc_torch_ext"
+
+
+def ext_path():
+    import sysconfig
+    return os.path.join(HERE, "mhc", EXT_NAME + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+
+
+def build_torch_ext(verbose: bool = True):
+    """Compiles the PyTorch-ROCm extension (torch_ext/mhc_torch_ext.cpp: host C++ only, it calls the
+    C ABI of libmhc_hip.so) with g++ against the installed torch headers and links it next to the
+    library.  Needs libmhc_hip.so (build() above)."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    os.makedirs(OBJ, exist_ok=True)
+    obj = os.path.join(OBJ, EXT_NAME + ".o")
+    inc = [f"-I{p}" for p in ce.include_paths()] + [f"-I{sysconfig.get_paths()['include']}", "-I/opt/rocm/include"]
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    cxx = os.environ.get("CXX", "g++")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", f"-DTORCH_EXTENSION_NAME={EXT_NAME}",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", "-DUSE_ROCM=1", "-D__HIP_PLATFORM_AMD__=1", "-DHIPBLAS_V2",
+           f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-Wno-deprecated-declarations", *inc, "-c", EXT_SRC, "-o", obj]
+    subprocess.check_call(cmd)
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    out = ext_path()
+    cmd = [cxx, "-shared", obj, "-o", out, f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
+           "-ltorch_python", f"-L{os.path.join(HERE, 'mhc')}", "-lmhc_hip", "-Wl,-rpath,$ORIGIN",
+           f"-Wl,-rpath,{tlib}"]
+    subprocess.check_call(cmd)
+    if verbose:
+        print("built", out)
+    return out
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
     ap.add_argument("--profile", action="store_true", help="build libmhc_hip_profile.so (in-kernel phase profiler)")
+    ap.add_argument("--no-ext", action="store_true", help="skip the PyTorch extension (about a minute of g++)")
     a = ap.parse_args()
     build(a.jobs, profile=a.profile)
+    if not a.profile and not a.no_ext:
+        build_torch_ext()

@@ -7,12 +7,17 @@
 
 #include "launchers.h"
 #include "phase_profiler.h"
+#include "tuning.h"
 
 #include <stdint.h>
 
 #include <mutex>
 
 using namespace mhc;
+
+namespace mhc {
+int g_tuning[kTuneCount];
+}
 
 namespace {
 
@@ -147,6 +152,13 @@ __attribute__((visibility("default"))) int mhc_phase_read(int kernel, unsigned l
 
 int mhc_abi_version(void) { return MHC_ABI_VERSION; }
 
+// Experiment hook (csrc/tuning.h), deliberately absent from the public header.
+__attribute__((visibility("default"))) int mhc_tuning_set(int key, int value) {
+    if (key < 0 || key >= kTuneCount) return -1;
+    g_tuning[key] = value;
+    return 0;
+}
+
 int mhc_max_sinkhorn_iters(int n) { return (n < 1 || n > MHC_MAX_N) ? 0 : max_layer_sinkhorn_iters(n); }
 
 const char *mhc_status_string(int status) {
@@ -192,6 +204,12 @@ int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype
     const DynFwdWs ws = carve_dyn_fwd(workspace, B, n, C);
     if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (layer_fwd_onepass_supported(x_dtype, phi_dtype, B, n, C)) {
+        // projection, coefficients and mix in one launch; x crosses HBM once
+        MHC_LAUNCH(launch_layer_fwd_onepass(x, w, w_dtype, f_inject, y, y_dtype, phi, alpha, bias, H_pre, H_post,
+                                            M, P, r, q, B, n, C, iters, eps, st));
+        return MHC_OK;
+    }
     const int KS = proj_fwd_ksplit(x_dtype, phi_dtype, B, n, C);
     MHC_LAUNCH(launch_proj_fwd(x, x_dtype, phi, phi_dtype, ws.Ppart, ws.ssqpart, KS, B, n, C, st));
     if (layer_fwd_fused_supported(n, C, x_dtype)) {
@@ -272,6 +290,22 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     }
     MHC_LAUNCH(launch_finalize(ws.u, groups, C, f_inject ? nullptr : dw, ws.dtpart, groups, D, dbias,
                                dalpha, ws.dphi_part, S, (size_t)D * n * C, dphi, st));
+    return MHC_OK;
+}
+
+int mhc_pack_dynamic_params(const void *phi_pre, const void *phi_post, const void *phi_res, int src_dtype,
+                            const float *b_pre, const float *b_post, const float *b_res,
+                            const float *alpha_pre, const float *alpha_post, const float *alpha_res,
+                            void *phi, int phi_dtype, float *bias, float *alpha, int n, int C, void *stream) {
+    if (n < 1 || n > MHC_MAX_N) return MHC_ERR_BAD_N;
+    if (C < 1 || C > MHC_MAX_C) return MHC_ERR_BAD_SHAPE;
+    if (!phi_pre || !phi_post || !phi_res || !b_pre || !b_post || !b_res || !alpha_pre || !alpha_post ||
+        !alpha_res || !phi || !bias || !alpha)
+        return MHC_ERR_NULL_POINTER;
+    if (!valid_dtype(src_dtype) || !valid_dtype(phi_dtype)) return MHC_ERR_BAD_DTYPE;
+    MHC_LAUNCH(launch_pack_params(phi_pre, phi_post, phi_res, src_dtype, b_pre, b_post, b_res, alpha_pre,
+                                  alpha_post, alpha_res, phi, phi_dtype, bias, alpha, n, C,
+                                  static_cast<hipStream_t>(stream)));
     return MHC_OK;
 }
 

@@ -69,6 +69,14 @@ hipError_t launch_layer_fwd_fused(const void *x, int x_dtype, const void *w, int
                                   float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
                                   int B, int n, int C, int T, float eps, hipStream_t stream);
 
+// Whole dynamic-H forward in one launch (bf16 x and phi, n <= 4, n*C % 64 == 0): projection,
+// coefficients and mix with the samples' rows resident in LDS.  bias = [pre | post | res].
+bool layer_fwd_onepass_supported(int x_dtype, int phi_dtype, int B, int n, int C);
+hipError_t launch_layer_fwd_onepass(const void *x, const void *w, int w_dtype, const void *f_inject, void *y,
+                                    int y_dtype, const void *phi, const float *alpha, const float *bias,
+                                    float *Hpre, float *Hpost, float *M, float *P, float *r, float *q, int B,
+                                    int n, int C, int T, float eps, hipStream_t stream);
+
 // fp32 matrix-core GEMMs of the exact float32 tier (wide projections): see gemm_f32.hip.
 bool gemm_f32_supported(int x_dtype, int phi_dtype, int n, int C);
 int gemm_f32_proj_ksplit(int B, int n, int C, int max_splits);
@@ -166,6 +174,14 @@ hipError_t launch_colsum_split(const float *in, int rows, int cols, int ld, floa
 hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const float *Hpost,
                                   const float *H_res_logits, float *dH_pre, float *dH_post,
                                   float *dH_res, int n, int T, float eps, hipStream_t stream);
+
+// phi [D, nC] (out_dtype) = rows [pre | post | res] of the three parameter matrices (src_dtype),
+// bias [D] and alpha [3] likewise, in one launch.
+hipError_t launch_pack_params(const void *phi_pre, const void *phi_post, const void *phi_res, int src_dtype,
+                              const float *b_pre, const float *b_post, const float *b_res,
+                              const float *alpha_pre, const float *alpha_post, const float *alpha_res,
+                              void *phi_out, int out_dtype, float *bias, float *alpha, int n, int C,
+                              hipStream_t stream);
 
 // ---- stand-alone operators -------------------------------------------------------------------
 hipError_t launch_sinkhorn_plain_fwd(const float *inp, float *out, int batch, int rows, int cols,

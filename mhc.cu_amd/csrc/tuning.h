@@ -1,0 +1,24 @@
+// Launch-heuristic overrides for experiments (host side only).  Every knob defaults to 0 = "use
+// the built-in heuristic"; mhc_tuning_set (exported, but not part of the public header) changes
+// one for the whole process.  Not thread-safe and not meant for production callers: the public
+// entry points behave identically with all knobs at 0.
+#pragma once
+
+namespace mhc {
+
+enum TuneKey {
+    kTuneOnepassOff = 0,    // one-launch forward: 0 = by cost model, 1 = never, 2 = whenever the shape allows
+    kTuneOnepassG = 1,      // samples per workgroup of the one-launch forward
+    kTuneOnepassWaves = 2,  // waves per workgroup of the one-launch forward (4..8)
+    kTuneSlabSplits = 3,    // batch splits of the slab backward
+    kTuneSpare0 = 4,
+    kTuneSpare1 = 5,
+    kTuneSpare2 = 6,
+    kTuneSpare3 = 7,
+    kTuneCount = 8
+};
+
+extern int g_tuning[kTuneCount];
+inline int tuning_get(int key) { return g_tuning[key]; }
+
+}  // namespace mhc

@@ -38,6 +38,7 @@ _SIGNATURES = {
                                       _P, _I, _I, _I, _I, _F, _P, _Z, _P]),
     "mhc_layer_bwd_dynamic": (c_int, [_P, _I, _P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P,
                                       _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _P, _Z, _P]),
+    "mhc_pack_dynamic_params": (c_int, [_P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P]),
     "mhc_static_scratch_capacity": (_Z, []),
     "mhc_layer_fwd_dynamic_scratch_bytes": (_Z, [_I, _I, _I]),
     "mhc_static_scratch_init": (c_int, []),

@@ -20,6 +20,7 @@
 #include "../../include/mhc_hip.h"
 
 extern "C" int mhc_phase_read(int kernel, unsigned long long *host, int workgroups);
+extern "C" int mhc_tuning_set(int key, int value);  // experiment hook of the library (csrc/tuning.h)
 
 #define HIP_OK(e) do { hipError_t _e = (e); if (_e != hipSuccess) { fprintf(stderr, "HIP error %s at line %d\n", hipGetErrorString(_e), __LINE__); exit(1); } } while (0)
 #define MHC_OK_(e) do { int _s = (e); if (_s != MHC_OK) { fprintf(stderr, "mhc error %d (%s) at line %d\n", _s, mhc_status_string(_s), __LINE__); exit(1); } } while (0)
@@ -76,6 +77,7 @@ int main(int argc, char **argv) {
         if (is("--batch") && i + 1 < argc) B = atoi(argv[++i]);
         else if (is("--hidden") && i + 1 < argc) C = atoi(argv[++i]);
         else if (is("--expansion") && i + 1 < argc) n = atoi(argv[++i]);
+        else if (is("--tune") && i + 2 < argc) { mhc_tuning_set(atoi(argv[i + 1]), atoi(argv[i + 2])); i += 2; }
         else { fprintf(stderr, "unknown argument %s\n", argv[i]); return 2; }
     }
     if (n > 8 || C % 8) { fprintf(stderr, "the instrumented kernels serve n <= 8 with C %% 8 == 0\n"); return 2; }
@@ -97,6 +99,12 @@ int main(int argc, char **argv) {
         HIP_OK(hipDeviceSynchronize());
     }
     printf("phase profile: dynamic H, bf16, B=%d C=%d n=%d (last of 3 warm calls)\n", B, C, n);
+    if (n <= 4 && (n * C) % 64 == 0) {
+        const int G = std::min(16, std::max(1, (B + 255) / 256));
+        summary("one-launch forward kernel, one workgroup per G samples (wave 0 of each)", 6, std::min((B + G - 1) / G, 4096),
+                {"phase A: stream x and phi, project", "wait for the other waves", "activations",
+                 "Sinkhorn (wave 0) while the other waves aggregate", "RMS", "mix pass, stores issued"}, true);
+    }
     summary("fused forward kernel, one workgroup per sample", 0, std::min(B, 4096),
             {"issue loads (early half: tile too)", "coefficient inputs arrive", "activations + Sinkhorn", "tile request (late half), barrier", "tile arrives, aggregate, RMS",
              "mix, stores issued"}, true);

@@ -136,41 +136,59 @@ def test_phi_cache_follows_parameter_updates():
     assert (y0 - y1).abs().max() > 1e-4
 
 
-def test_derived_parameter_caches_never_serve_a_different_tensor():
-    """phi / bias / alpha caches: hit for the same unchanged parameters, miss after an in-place update
-    of the small parameters, and miss for new tensors that reuse the addresses of freed ones."""
+@pytest.mark.parametrize("cache", [False, True])
+def test_parameter_updates_always_reach_the_kernels(cache):
+    """The gathered copy of phi / bias / alpha is rebuilt on every call by default, so any way of
+    writing a parameter is seen (also through `.data`, which does not bump the version counter); with
+    the opt-in cache, in-place updates that bump the counter and new tensors at reused addresses are."""
     import gc
     from mhc import MHCLayer, ops
     B, n, C = 4, 4, 64
     x = torch.randn(B, n, C, device="cuda")
-
-    layer = MHCLayer(hidden_dim=C, expansion_rate=n, alpha_init=1.0).cuda()
-    layer(x)
-    cached = ops._phi_concat(layer.phi_pre, layer.phi_post, layer.phi_res, torch.float32)
-    assert cached is ops._phi_concat(layer.phi_pre, layer.phi_post, layer.phi_res, torch.float32)
-    y0 = layer(x).detach().clone()
-    with torch.no_grad():
-        layer.b_res.add_(1.0, alpha=1.0).mul_(torch.linspace(-2, 2, n * n, device="cuda").reshape(n, n))
-        layer.alpha_res.mul_(-2.0)
-    assert (y0 - layer(x).detach()).abs().max() > 1e-4
-
-    # same shapes, same allocation pattern, different values: the outputs must follow the new values
-    outs = []
-    for seed in (1, 2):
-        del layer
-        gc.collect()
-        torch.manual_seed(seed)
+    ops.set_param_cache(cache)
+    try:
         layer = MHCLayer(hidden_dim=C, expansion_rate=n, alpha_init=1.0).cuda()
+        y0 = layer(x).detach().clone()
+        assert torch.equal(layer(x).detach(), y0)
         with torch.no_grad():
-            layer.b_res.normal_()
-        p = {k: getattr(layer, k).detach().float().cpu() for k in nm.DYN_PARAM_NAMES if k != "w"}
-        p["w"] = layer.rmsnorm_weight.detach().float().cpu()
-        ref, _ = nm.mhc_dynamic_fwd_bwd(x.cpu(), p, torch.ones(B, n, C), layer.sinkhorn_iters, layer.eps,
-                                        dtype=torch.float64)
-        y = layer(x).detach().cpu()
-        assert rel_err(y, ref) < 1e-5
-        outs.append(y)
-    assert (outs[0] - outs[1]).abs().max() > 1e-4
+            layer.b_res.add_(1.0, alpha=1.0).mul_(torch.linspace(-2, 2, n * n, device="cuda").reshape(n, n))
+            layer.alpha_res.mul_(-2.0)
+        y1 = layer(x).detach().clone()
+        assert (y0 - y1).abs().max() > 1e-4
+        if not cache:
+            layer.phi_res.data.copy_(torch.randn_like(layer.phi_res))   # version counter unchanged
+            assert (y1 - layer(x).detach()).abs().max() > 1e-4
+
+        # same shapes, same allocation pattern, different values: the outputs must follow the new values
+        outs = []
+        for seed in (1, 2):
+            del layer
+            gc.collect()
+            torch.manual_seed(seed)
+            layer = MHCLayer(hidden_dim=C, expansion_rate=n, alpha_init=1.0).cuda()
+            with torch.no_grad():
+                layer.b_res.normal_()
+            p = {k: getattr(layer, k).detach().float().cpu() for k in nm.DYN_PARAM_NAMES if k != "w"}
+            p["w"] = layer.rmsnorm_weight.detach().float().cpu()
+            ref, _ = nm.mhc_dynamic_fwd_bwd(x.cpu(), p, torch.ones(B, n, C), layer.sinkhorn_iters, layer.eps,
+                                            dtype=torch.float64)
+            y = layer(x).detach().cpu()
+            assert rel_err(y, ref) < 1e-5
+            outs.append(y)
+        assert (outs[0] - outs[1]).abs().max() > 1e-4
+    finally:
+        ops.set_param_cache(False)
+
+
+def test_misaligned_views_are_copied_not_refused():
+    """A contiguous view whose storage offset is not a multiple of 16 bytes still works."""
+    from mhc import MHCLayer
+    B, n, C = 3, 4, 64
+    layer = MHCLayer(hidden_dim=C, expansion_rate=n).cuda()
+    flat = torch.randn(B * n * C + 1, device="cuda")
+    x = flat[1:].view(B, n, C)
+    assert x.data_ptr() % 16 != 0 and x.is_contiguous()
+    assert torch.equal(layer(x), layer(x.clone()))
 
 
 @pytest.mark.parametrize("dynamic", [False, True])
