@@ -219,12 +219,42 @@ def event_time_batched(torch, fn, reps, rounds=5):
     return best
 
 
+def physical_cores():
+    """Physical cores this process may use: distinct (package, core) pairs of the CPUs in its affinity
+    mask, capped by the container's CPU quota where one is set."""
+    try:
+        allowed = sorted(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = list(range(os.cpu_count() or 1))
+    seen = set()
+    for c in allowed:
+        try:
+            with open(f"/sys/devices/system/cpu/cpu{c}/topology/core_id") as f1, \
+                    open(f"/sys/devices/system/cpu/cpu{c}/topology/physical_package_id") as f2:
+                seen.add((f2.read().strip(), f1.read().strip()))
+        except OSError:
+            seen.add(("?", str(c)))
+    cores = max(1, len(seen))
+    try:
+        with open("/sys/fs/cgroup/cpu.max") as f:
+            quota, period = f.read().split()
+        if quota != "max":
+            cores = max(1, min(cores, int(int(quota) / int(period))))
+    except (OSError, ValueError):
+        pass
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        cores = max(1, min(cores, int(env)))
+    return cores
+
+
 def cpu_baseline(step, torch, budget_s=20.0):
     """The oracle (naive PyTorch layer) on the host cores: same seeded inputs, fp32."""
     from oracle import naive_mhc as nm
 
     cfg, h = step.cfg, step.host
-    cores = torch.get_num_threads()
+    cores = physical_cores()
+    torch.set_num_threads(cores)
     f = h["f"]
 
     def run():
@@ -257,10 +287,87 @@ def cpu_baseline(step, torch, budget_s=20.0):
             break
     times.sort()
     med = times[len(times) // 2]
+    par = [l.strip() for l in torch.__config__.parallel_info().splitlines()
+           if any(k in l for k in ("ATen parallel backend", "OpenMP", "omp_get_max_threads", "MKL", "mkl_get_max_threads"))]
     return {"value": med * 1e6, "unit": "us/layer", "cores": cores, "kind": "port",
+            "threads": torch.get_num_threads(), "parallel_info": "; ".join(par)[:400],
             "sample": f"{len(times)} runs of the full {cfg['kind']} "
                       f"{'fwd+bwd' if cfg['bwd'] else 'fwd'} step at B={cfg['B']} n={cfg['n']} C={cfg['C']}, "
                       f"fp32 naive PyTorch layer, median"}
+
+
+def stream_probe(torch):
+    """Read-only / copy / write-only streaming rates of hand-written kernels (csrc/stream_probe.hip)."""
+    from mhc import _lib
+
+    fn = _lib.lib.mhc_stream_probe
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
+                   ctypes.c_void_p]
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    flush = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rows = []
+    for mib, cold in ((32, False), (32, True), (128, True), (512, True), (2048, True)):
+        nbytes = mib * 1024 * 1024
+        src = torch.empty(nbytes // 4, dtype=torch.int32, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for mode, name, moved in ((0, "read", nbytes), (1, "copy", 2 * nbytes), (2, "write", nbytes),
+                                  (3, "read", nbytes), (4, "copy", 2 * nbytes), (5, "write", nbytes)):
+            for blocks in (2048, 4096):
+                def run():
+                    st = fn(mode, src.data_ptr(), dst.data_ptr(), nbytes, blocks, sink.data_ptr(), stream)
+                    assert st == 0, st
+                for _ in range(3):
+                    run()
+                times = []
+                for _ in range(10):
+                    if cold:
+                        flush.fill_(1.0)  # the buffers leave the 256 MB Infinity Cache
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    run()
+                    e1.record()
+                    e1.synchronize()
+                    times.append(e0.elapsed_time(e1) * 1e-3)
+                times.sort()
+                t = times[len(times) // 2]
+                rows.append({"kernel": name, "hint": "nt" if mode < 3 else "plain", "MiB": mib,
+                             "cache": "cold" if cold else "warm", "blocks": blocks,
+                             "us": round(t * 1e6, 1), "GB/s": round(moved / t / 1e9, 1)})
+        del src, dst
+    # launch floor: a chain of dependent kernels that do nothing, eager and as one HIP graph
+    floor = {}
+    for blocks in (256, 2048):
+        def chain(k=10):
+            cur = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)  # the capture stream under capture
+            for _ in range(k):
+                assert fn(6, None, None, 0, blocks, sink.data_ptr(), cur) == 0
+        chain()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            chain()
+        for name, run in (("eager", chain), ("graph", g.replay)):
+            run()
+            best_t = float("inf")
+            for _ in range(10):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(10):
+                    run()
+                e1.record()
+                e1.synchronize()
+                best_t = min(best_t, e0.elapsed_time(e1) * 1e3 / 100)
+            floor[f"{name}_{blocks}_workgroups"] = round(best_t, 2)
+    best = {}
+    for r in rows:
+        key = (r["kernel"], r["MiB"], r["cache"])
+        if key not in best or r["GB/s"] > best[key]["GB/s"]:
+            best[key] = r
+    print(json.dumps({"stream_probe": True, "protocol": "cold: 512 MiB fill before every timed launch; warm: back to back; median of 10, "
+                      "HIP events on the launch stream", "rows": rows,
+                      "empty_kernel_us_per_launch": floor, "ceiling_GBs": {f"{k[0]}_{k[1]}MiB_{k[2]}": round(v["GB/s"], 1) for k, v in sorted(best.items())}}))
 
 
 def main():
@@ -272,6 +379,10 @@ def main():
     ap.add_argument("--view", default="L", choices=["L", "K"])
     ap.add_argument("--mode", default="graph", choices=["graph", "eager"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--stream-probe", action="store_true",
+                    help="run the library's plain streaming kernels (read-only, copy, write-only; 16-byte accesses, "
+                         "all CUs) over 128 MiB .. 2 GiB and print what this GPU delivers to each, HIP events on the "
+                         "launch stream: the measured ceiling that the memory-bound kernels are compared with")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run a plain 64 MiB device copy instead of the layer (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
@@ -287,6 +398,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if a.stream_probe:
+        stream_probe(torch)
+        return
     if a.copy_calibration:
         nbytes = 64 * 1024 * 1024
         src = torch.arange(nbytes // 4, dtype=torch.int32, device="cuda")

@@ -50,7 +50,7 @@ enum mhc_status {
     MHC_OK = 0,
     MHC_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
     MHC_ERR_BAD_N = 2,          /* expansion rate outside 1..MHC_MAX_N */
-    MHC_ERR_BAD_SHAPE = 3,      /* B, C or iters not positive / too large (C <= MHC_MAX_C; n > 8: B <= 65535) */
+    MHC_ERR_BAD_SHAPE = 3,      /* B, C or iters not positive / too large (C <= MHC_MAX_C, B * n * C <= 2^40) */
     MHC_ERR_BAD_DTYPE = 4,      /* unknown or unsupported dtype combination */
     MHC_ERR_MISALIGNED = 5,     /* a tensor base pointer is not 16-byte aligned */
     MHC_ERR_WORKSPACE = 6,      /* workspace NULL, misaligned or too small */

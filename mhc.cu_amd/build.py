@@ -19,7 +19,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "mhc", "libmhc_hip.so")
 
 SOURCES = ["capi.hip", "proj_fwd.hip", "gemm_f32.hip", "proj_bwd.hip", "proj_bwd_large.hip", "bwd_slab.hip", "coef_fwd.hip", "mix_fwd.hip", "layer_fwd_onepass.hip", "mix_bwd_reduce.hip",
-           "mix_bwd_dx.hip", "param_grads.hip", "pack_params.hip", "ops.hip"]
+           "mix_bwd_dx.hip", "param_grads.hip", "pack_params.hip", "ops.hip", "stream_probe.hip"]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are not trusted on this hardware pool.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

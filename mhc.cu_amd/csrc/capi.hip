@@ -44,7 +44,6 @@ int check_shape(int B, int n, int C, int iters) {
     if (B < 1 || C < 1 || iters < 0 || iters > max_layer_sinkhorn_iters(n)) return MHC_ERR_BAD_SHAPE;
     if ((long long)B * n * C > (1ll << 40)) return MHC_ERR_BAD_SHAPE;
     if (C > MHC_MAX_C) return MHC_ERR_BAD_SHAPE;       // the generic kernels keep a [C] float row in LDS
-    if (n > 8 && B > 65535) return MHC_ERR_BAD_SHAPE;  // the n > 8 kernels index samples by blockIdx.y
     return MHC_OK;
 }
 
@@ -167,7 +166,7 @@ const char *mhc_status_string(int status) {
         case MHC_ERR_NULL_POINTER: return "a required pointer is NULL";
         case MHC_ERR_BAD_N: return "expansion rate n must be in 1..32";
         case MHC_ERR_BAD_SHAPE:
-            return "B, C or iters out of range (C <= 32768; n > 8: B <= 65535; iters <= mhc_max_sinkhorn_iters(n))";
+            return "B, C or iters out of range (C <= 32768; B * n * C <= 2^40; iters <= mhc_max_sinkhorn_iters(n))";
         case MHC_ERR_BAD_DTYPE: return "unsupported dtype combination";
         case MHC_ERR_MISALIGNED: return "tensor base pointer is not 16-byte aligned";
         case MHC_ERR_WORKSPACE: return "workspace NULL, not 256-byte aligned or too small";

@@ -133,6 +133,12 @@ __device__ __forceinline__ void store_vec(T *__restrict__ p, const float (&v)[V]
     }
 }
 
+// 16-byte load with the streaming (non-temporal) hint.
+__device__ __forceinline__ uint4 ldg16_stream(const uint4 *p) {
+    const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+    return make_uint4(t[0], t[1], t[2], t[3]);
+}
+
 // V consecutive elements kept exactly as loaded.  No conversion instruction sits behind the load,
 // so a batch of loads stays in flight across whatever code follows (another basic block
 // included); get() widens to fp32 at the point of use.  The pointer must be dereferenceable and
@@ -157,6 +163,19 @@ template <typename T, int V> struct RawVec {
         } else {
             static_assert(kBytes == 2, "unsupported vector width");
             w[0] = *reinterpret_cast<const uint16_t *>(p);
+        }
+    }
+    // The same with the streaming hint (the `nt` bit of the load).  A cold read-only pass over
+    // 128-512 MiB runs at 4.7-4.9 TB/s with the hint and at 2.4-3.2 TB/s without it on this GPU, but the
+    // hint also keeps the data out of the 256 MB Infinity Cache: with back-to-back steps the 89 MB of
+    // phi at n = 32 are partly served from that cache, and the hinted loads made the two kernels that
+    // stream phi 15-35 % slower.  Kept for data that is truly read once.  16-byte multiples only.
+    __device__ __forceinline__ void load_stream(const T *__restrict__ p) {
+        static_assert(kBytes % 16 == 0, "streaming loads are 16-byte loads");
+#pragma unroll
+        for (int i = 0; i < kBytes / 16; i++) {
+            const uint4 t = ldg16_stream(reinterpret_cast<const uint4 *>(p) + i);
+            w[4 * i] = t.x; w[4 * i + 1] = t.y; w[4 * i + 2] = t.z; w[4 * i + 3] = t.w;
         }
     }
     __device__ __forceinline__ void get(float (&v)[V]) const {

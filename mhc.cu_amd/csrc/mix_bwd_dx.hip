@@ -174,9 +174,9 @@ __global__ __launch_bounds__(256) void mix_bwd_dx_kernel(BwdDxArgs a) {
     // per-group sums of the logit gradients (feeds dbias / dalpha)
     if (a.dtpart && blockIdx.y == 0) {
         for (int col = tid; col < D + 3; col += nt) {
-            float acc = 0.f;
-            for (int b = b_first; b < b_last; b++) acc += a.dt[(size_t)b * (D + 3) + col];
-            a.dtpart[(size_t)grp * (D + 3) + col] = acc;
+            double acc = 0.0;  // float64 like the batch sums that follow (finalize_kernel)
+            for (int b = b_first; b < b_last; b++) acc += (double)a.dt[(size_t)b * (D + 3) + col];
+            a.dtpart[(size_t)grp * (D + 3) + col] = (float)acc;
         }
     }
     MHC_PHASE_ADD(kPhaseDxSmall, pwg, 3, pclk);
@@ -237,7 +237,10 @@ __global__ __launch_bounds__(256, 5) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
     float *hp_s = reinterpret_cast<float *>(x_s + 32 * kDxlLDT);  // [32] Hpre (0 beyond n)
     float *ho_s = hp_s + 32;                                 // [32] Hpost (0 beyond n)
     static_assert(sizeof(float) * 32 * kDxlLDO <= sizeof(bf16_t) * 2 * 32 * kDxlLDT, "output tile must fit in the input tiles");
-    const int b = blockIdx.y, cb0 = blockIdx.x * kDxlCB, n = a.n, C = a.C, tid = threadIdx.x;
+    // linear workgroup id = sample * column blocks + column block (one grid dimension: no bound on B)
+    const int ncb = (a.C + kDxlCB - 1) / kDxlCB;
+    const int b = blockIdx.x / ncb, cblk = blockIdx.x % ncb;
+    const int cb0 = cblk * kDxlCB, n = a.n, C = a.C, tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6, row = lane & 31, kh = lane >> 5;
     const bool inject = a.f_inject != nullptr;
     const bf16_t *gb = static_cast<const bf16_t *>(a.dy) + (size_t)b * n * C;
@@ -357,7 +360,7 @@ __global__ __launch_bounds__(256, 5) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
         }
     }
     // per-sample "group" sums of the logit gradients (one sample per group on this path)
-    if (a.dtpart && blockIdx.x == 0) {
+    if (a.dtpart && cblk == 0) {
         const int D = n * n + 2 * n;
         for (int col = tid; col < D + 3; col += 256)
             a.dtpart[(size_t)b * (D + 3) + col] = a.dt[(size_t)b * (D + 3) + col];
@@ -366,7 +369,7 @@ __global__ __launch_bounds__(256, 5) void mix_bwd_dx_large_kernel(BwdDxArgs a) {
 
 static hipError_t launch_large_mfma(const BwdDxArgs &a, hipStream_t stream) {
     const size_t smem = sizeof(bf16_t) * 2 * 32 * kDxlLDT + sizeof(float) * 64;
-    mix_bwd_dx_large_kernel<<<dim3((a.C + kDxlCB - 1) / kDxlCB, a.B), 256, smem, stream>>>(a);
+    mix_bwd_dx_large_kernel<<<(unsigned)((a.C + kDxlCB - 1) / kDxlCB) * (unsigned)a.B, 256, smem, stream>>>(a);
     return hipGetLastError();
 }
 

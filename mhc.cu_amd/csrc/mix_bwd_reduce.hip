@@ -716,6 +716,10 @@ __global__ __launch_bounds__(256) void gram_large_kernel(BwdReduceArgs a) {
         if (wave < nchunks) fetch(wave);
         for (int chunk = wave; chunk < nchunks; chunk += 4) {
             park();
+            // the rows come back in operand layout from this wave's own tile: a wave's LDS accesses
+            // complete in order, the fence keeps the compiler from moving the reads above the writes
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
             if (chunk + 4 < nchunks) fetch(chunk + 4);
 #pragma unroll
             for (int u = 0; u < 4; u++) {

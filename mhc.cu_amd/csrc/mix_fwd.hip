@@ -672,7 +672,10 @@ __global__ __launch_bounds__(256) void mix_fwd_large_kernel(MixLargeArgs a) {
     float *o_s = reinterpret_cast<float *>(x_s + 32 * kMflLDT);  // [32][LDO]
     float *ho_s = o_s + 32 * kMflLDO;                            // [32] Hpost (0 beyond n)
     float *m_s = ho_s + 32;                                      // [32][33] M (0 beyond n x n)
-    const int b = blockIdx.y, cb0 = blockIdx.x * kMflCB, n = a.n, C = a.C, tid = threadIdx.x;
+    // linear workgroup id = sample * column blocks + column block (one grid dimension: no bound on B)
+    const int ncb = (a.C + kMflCB - 1) / kMflCB;
+    const int b = blockIdx.x / ncb, cblk = blockIdx.x % ncb;
+    const int cb0 = cblk * kMflCB, n = a.n, C = a.C, tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6, row = lane & 31, kh = lane >> 5;
     const bool inject = a.f_inject != nullptr;
     const bf16_t *xb = a.x + (size_t)b * n * C;
@@ -702,7 +705,7 @@ __global__ __launch_bounds__(256) void mix_fwd_large_kernel(MixLargeArgs a) {
         const int k = (tid & 7) * 4 + i;
         m_s[trow * 33 + k] = (trow < n && k < n) ? mraw[i] : 0.f;
     }
-    if (inject && a.q && blockIdx.x == 0 && tid == 0) a.q[b] = 1.0f;  // q is defined as 1 with an injected f
+    if (inject && a.q && cblk == 0 && tid == 0) a.q[b] = 1.0f;  // q is defined as 1 with an injected f
     // f of this lane's channel in the matrix-core phase
     const int cw = cb0 + wave * 32 + row;
     float f = 0.f;
@@ -780,7 +783,7 @@ static hipError_t launch_large_mfma(const MixLargeArgs &a, int y_dtype, bool hav
         if (e != hipSuccess) return e;
     }
     const size_t smem = sizeof(bf16_t) * 32 * kMflLDT + sizeof(float) * (32 * kMflLDO + 32 + 32 * 33);
-    const dim3 grid((a.C + kMflCB - 1) / kMflCB, a.B);
+    const unsigned grid = (unsigned)((a.C + kMflCB - 1) / kMflCB) * (unsigned)a.B;
     if (y_dtype == kBF16) mix_fwd_large_kernel<bf16_t><<<grid, 256, smem, stream>>>(a);
     else mix_fwd_large_kernel<float><<<grid, 256, smem, stream>>>(a);
     return hipGetLastError();

@@ -148,47 +148,59 @@ struct FinalizeArgs {
 };
 
 __global__ __launch_bounds__(1024) void finalize_kernel(FinalizeArgs a) {
-    __shared__ float red[16][65];
+    // Batch sums in float64: dalpha (and the static coefficient gradients) are sums of B * n^2 terms of
+    // mixed sign whose total can be a hundred times smaller than the terms; a float32 running sum then
+    // loses what the 1e-5 parity tier needs.  The terms themselves stay float32.
+    __shared__ double red[16][65];
     const int tid = threadIdx.x;
     if ((int)blockIdx.x < a.nblk_a) {
         const int cl = tid & 63, rg = tid >> 6;
         const int col = blockIdx.x * 64 + cl;
         const int ncol_u = a.dw ? a.C : 0;
         const int ncols = ncol_u + a.D + 3;
-        float acc = 0.f;
+        double acc = 0.0;
         if (col < ncols) {
             const bool is_u = col < ncol_u;
             const float *src = is_u ? a.u + col : a.dt + (col - ncol_u);
             const int ld = is_u ? a.C : a.D + 3;
             const int rows = is_u ? a.rows_u : a.rows_dt;
-            float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+            double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
             int r = rg;
             for (; r + 48 < rows; r += 64) {
-                a0 += src[(size_t)r * ld];
-                a1 += src[(size_t)(r + 16) * ld];
-                a2 += src[(size_t)(r + 32) * ld];
-                a3 += src[(size_t)(r + 48) * ld];
+                const float t0 = src[(size_t)r * ld], t1 = src[(size_t)(r + 16) * ld];
+                const float t2 = src[(size_t)(r + 32) * ld], t3 = src[(size_t)(r + 48) * ld];
+                a0 += (double)t0; a1 += (double)t1; a2 += (double)t2; a3 += (double)t3;
             }
-            for (; r < rows; r += 16) a0 += src[(size_t)r * ld];
+            for (; r < rows; r += 16) a0 += (double)src[(size_t)r * ld];
             acc = (a0 + a1) + (a2 + a3);
         }
         red[rg][cl] = acc;
         __syncthreads();
         if (rg == 0 && col < ncols) {
-            float v = 0.f;
+            double v = 0.0;
 #pragma unroll
             for (int i = 0; i < 16; i++) v += red[i][cl];
-            if (col < ncol_u) a.dw[col] = v;
-            else if (col - ncol_u < a.D) a.dbias[col - ncol_u] = v;
-            else a.dalpha[col - ncol_u - a.D] = v;
+            if (col < ncol_u) a.dw[col] = (float)v;
+            else if (col - ncol_u < a.D) a.dbias[col - ncol_u] = (float)v;
+            else a.dalpha[col - ncol_u - a.D] = (float)v;
         }
         return;
     }
     // dphi partial sums: one float per thread per 1024-column block (coalesced)
     const size_t e = (size_t)(blockIdx.x - a.nblk_a) * 1024 + tid;
     if (e < a.dphi_elems) {
+        // all copies requested together (eight per round), added in split order
         float v = 0.f;
-        for (int s = 0; s < a.S; s++) v += a.dphi_part[(size_t)s * a.dphi_elems + e];
+        for (int s0 = 0; s0 < a.S; s0 += 8) {
+            float t[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int s = s0 + u < a.S ? s0 + u : a.S - 1;
+                t[u] = __builtin_nontemporal_load(a.dphi_part + (size_t)s * a.dphi_elems + e);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) v += s0 + u < a.S ? t[u] : 0.f;
+        }
         a.dphi[e] = v;
     }
 }

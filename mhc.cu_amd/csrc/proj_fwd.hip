@@ -177,6 +177,10 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
     MHC_PHASE_ADD(kPhaseProjFwd, pwg, 0, pclk);
     for (int k0 = kbeg; k0 < kend; k0 += 64) {
         park();
+        // (a wave's LDS accesses complete in order; the fence keeps the compiler from moving the
+        // fragment reads above the writes of its own tile)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
         MHC_PHASE_ADD(kPhaseProjFwd, pwg, 1, pclk);
         if (k0 + 64 < kend) fetch(k0 + 64);  // in flight while this chunk is multiplied
 #pragma unroll

@@ -91,3 +91,36 @@ def static_backward(x, dy, w, logits, T, eps, f_inject=None):
                                           _p(dlogits))
     assert rc == 0
     return dict(x=dx, f=df, w=dw, logits=dlogits)
+
+
+def sinkhorn_plain_forward(inp, T, eps):
+    inp = _d(inp)
+    rows, cols = inp.shape
+    out = np.empty_like(inp)
+    assert lib().mhc_oracle_sinkhorn_plain_forward(_p(inp), _p(out), rows, cols, int(T), ctypes.c_double(eps)) == 0
+    return out
+
+
+def sinkhorn_plain_backward(grad_out, inp, T, eps):
+    grad_out, inp = _d(grad_out), _d(inp)
+    rows, cols = inp.shape
+    d_inp = np.empty_like(inp)
+    assert lib().mhc_oracle_sinkhorn_plain_backward(_p(grad_out), _p(inp), _p(d_inp), rows, cols, int(T),
+                                                    ctypes.c_double(eps)) == 0
+    return d_inp
+
+
+def rmsnorm_forward(inp, w, eps):
+    inp, w = _d(inp), _d(w)
+    rows, C = inp.shape
+    out, rms = np.empty_like(inp), np.empty(rows)
+    assert lib().mhc_oracle_rmsnorm_forward(_p(inp), _p(w), _p(out), _p(rms), rows, C, ctypes.c_double(eps)) == 0
+    return out, rms
+
+
+def rmsnorm_backward(grad, inp, w, rms):
+    grad, inp, w, rms = _d(grad), _d(inp), _d(w), _d(rms)
+    rows, C = inp.shape
+    d_inp, d_w = np.empty_like(inp), np.empty(C)
+    assert lib().mhc_oracle_rmsnorm_backward(_p(grad), _p(inp), _p(w), _p(rms), _p(d_inp), _p(d_w), rows, C) == 0
+    return d_inp, d_w

@@ -331,3 +331,110 @@ int mhc_oracle_static_backward(const double *x, const double *dy, const double *
     free(a); free(f); free(da); free(yb); free(rho); free(s);
     return 0;
 }
+
+/* ------------------------------------------------------------------------------------------------
+ * Stand-alone operators (loop-level restatements of the reference's own CPU references).
+ *   Sinkhorn-Knopp, threshold form: src/csrc/tests/test_sinkhorn_knopp.cu:16-47 - no exp, T x (every
+ *     row divided by its sum if the sum exceeds eps, then every column likewise), any rows x cols.
+ *     The backward is the exact reverse sweep of that recursion (a row / column that was not
+ *     divided passes its gradient through unchanged).
+ *   RMSNorm: src/csrc/tests/test_rmsnorm.cu:17-30 (forward) and
+ *     src/csrc/tests/test_rmsnorm_backward.cu:17-39 (backward from the saved rms).
+ * Pinned in tests/test_oracle_math.py: one-iteration closed forms on a non-square matrix, the
+ * PyTorch restatement, torch.nn.functional.rms_norm and central differences.
+ * ---------------------------------------------------------------------------------------------- */
+int mhc_oracle_sinkhorn_plain_forward(const double *inp, double *out, int rows, int cols, int T, double eps) {
+    memcpy(out, inp, sizeof(double) * (size_t)rows * cols);
+    for (int t = 0; t < T; t++) {
+        for (int r = 0; r < rows; r++) {
+            double s = 0.0;
+            for (int c = 0; c < cols; c++) s += out[r * cols + c];
+            if (s > eps)
+                for (int c = 0; c < cols; c++) out[r * cols + c] /= s;
+        }
+        for (int c = 0; c < cols; c++) {
+            double s = 0.0;
+            for (int r = 0; r < rows; r++) s += out[r * cols + c];
+            if (s > eps)
+                for (int r = 0; r < rows; r++) out[r * cols + c] /= s;
+        }
+    }
+    return 0;
+}
+
+int mhc_oracle_sinkhorn_plain_backward(const double *grad_out, const double *inp, double *d_inp, int rows,
+                                       int cols, int T, double eps) {
+    const size_t sz = (size_t)rows * cols;
+    /* iterates: A[t] = input of iteration t, R[t] = after the row step; sums kept per iteration */
+    double *A = (double *)malloc(sizeof(double) * sz * (size_t)(T + 1));
+    double *R = (double *)malloc(sizeof(double) * sz * (size_t)(T > 0 ? T : 1));
+    double *rs = (double *)malloc(sizeof(double) * (size_t)rows * (size_t)(T > 0 ? T : 1));
+    double *cs = (double *)malloc(sizeof(double) * (size_t)cols * (size_t)(T > 0 ? T : 1));
+    if (!A || !R || !rs || !cs) { free(A); free(R); free(rs); free(cs); return 1; }
+    memcpy(A, inp, sizeof(double) * sz);
+    for (int t = 0; t < T; t++) {
+        const double *a = A + sz * t;
+        double *rr = R + sz * t, *o = A + sz * (t + 1);
+        for (int r = 0; r < rows; r++) {
+            double s = 0.0;
+            for (int c = 0; c < cols; c++) s += a[r * cols + c];
+            rs[t * rows + r] = s;
+            for (int c = 0; c < cols; c++) rr[r * cols + c] = s > eps ? a[r * cols + c] / s : a[r * cols + c];
+        }
+        for (int c = 0; c < cols; c++) {
+            double s = 0.0;
+            for (int r = 0; r < rows; r++) s += rr[r * cols + c];
+            cs[t * cols + c] = s;
+            for (int r = 0; r < rows; r++) o[r * cols + c] = s > eps ? rr[r * cols + c] / s : rr[r * cols + c];
+        }
+    }
+    double *d = d_inp;
+    memcpy(d, grad_out, sizeof(double) * sz);
+    for (int t = T - 1; t >= 0; t--) {
+        const double *o = A + sz * (t + 1), *rr = R + sz * t;
+        for (int c = 0; c < cols; c++) {   /* o = rr / s: d_rr = (d_o - sum_k d_o o) / s */
+            const double s = cs[t * cols + c];
+            if (!(s > eps)) continue;
+            double dot = 0.0;
+            for (int r = 0; r < rows; r++) dot += d[r * cols + c] * o[r * cols + c];
+            for (int r = 0; r < rows; r++) d[r * cols + c] = (d[r * cols + c] - dot) / s;
+        }
+        for (int r = 0; r < rows; r++) {
+            const double s = rs[t * rows + r];
+            if (!(s > eps)) continue;
+            double dot = 0.0;
+            for (int c = 0; c < cols; c++) dot += d[r * cols + c] * rr[r * cols + c];
+            for (int c = 0; c < cols; c++) d[r * cols + c] = (d[r * cols + c] - dot) / s;
+        }
+    }
+    free(A); free(R); free(rs); free(cs);
+    return 0;
+}
+
+int mhc_oracle_rmsnorm_forward(const double *inp, const double *w, double *out, double *rms, int rows, int C,
+                               double eps) {
+    for (int i = 0; i < rows; i++) {
+        double ss = 0.0;
+        for (int j = 0; j < C; j++) ss += inp[(size_t)i * C + j] * inp[(size_t)i * C + j];
+        const double r = sqrt(ss / (double)C + eps);
+        if (rms) rms[i] = r;
+        for (int j = 0; j < C; j++) out[(size_t)i * C + j] = inp[(size_t)i * C + j] / r * w[j];
+    }
+    return 0;
+}
+
+int mhc_oracle_rmsnorm_backward(const double *grad, const double *inp, const double *w, const double *rms,
+                                double *d_inp, double *d_w, int rows, int C) {
+    for (int j = 0; j < C; j++) d_w[j] = 0.0;
+    for (int i = 0; i < rows; i++) {
+        const double r = rms[i], rinv = 1.0 / r;
+        double dot = 0.0;
+        for (int j = 0; j < C; j++) dot += grad[(size_t)i * C + j] * w[j] * inp[(size_t)i * C + j];
+        const double corr = dot / ((double)C * r * r);
+        for (int j = 0; j < C; j++) {
+            d_inp[(size_t)i * C + j] = grad[(size_t)i * C + j] * w[j] * rinv - inp[(size_t)i * C + j] * corr * rinv;
+            d_w[j] += grad[(size_t)i * C + j] * inp[(size_t)i * C + j] * rinv;
+        }
+    }
+    return 0;
+}

@@ -70,9 +70,9 @@ def test_argument_validation_happens_before_any_launch():
         kw.get("ws", None), kw.get("wsb", 0), None)
     assert fwd(n=0) == 2 and fwd(n=33) == 2            # MHC_ERR_BAD_N
     assert fwd(B=0) == 3                               # MHC_ERR_BAD_SHAPE
-    # n > 8 indexes samples by the second grid dimension: at most 65535 per call (n <= 8: no such bound)
     assert fwd(C=32768 + 8) == 3 and fwd(C=32768) == 6   # MHC_MAX_C
-    assert fwd(n=9, B=65536) == 3 and fwd(n=9, B=65535) == 6 and fwd(n=8, B=65536) == 6
+    # no bound on the batch beyond B * n * C <= 2^40 (samples are not tied to a 16-bit grid dimension)
+    assert fwd(n=9, B=65536) == 6 and fwd(n=32, B=1 << 20) == 6 and fwd(n=32, B=1 << 30, C=64) == 3
     # iteration counts beyond what the backward keeps in LDS are refused up front, per n
     assert [L.mhc_max_sinkhorn_iters(n) for n in (0, 1, 4, 5, 8, 9, 16, 17, 32, 33)] == \
         [0, 256, 256, 256, 256, 256, 256, 256, 256, 0]

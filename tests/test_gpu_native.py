@@ -14,6 +14,17 @@ EXE = os.path.join(HERE, "native", "test_mhc_layer")
 
 
 @pytest.mark.gpu
+def test_native_operator_parity_executable():
+    """tests/native/test_ops: mhc_sinkhorn_knopp_* and mhc_rmsnorm_* against the C oracle."""
+    exe = os.path.join(HERE, "native", "test_ops")
+    assert os.path.exists(exe), "build tests/native first (make -C tests/native)"
+    p = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    print(p.stdout[-4000:])
+    assert p.returncode == 0, p.stdout[-4000:] + p.stderr[-2000:]
+    assert "all comparisons passed" in p.stdout
+
+
+@pytest.mark.gpu
 def test_native_parity_executable():
     assert os.path.exists(EXE), "build tests/native first (make -C tests/native)"
     p = subprocess.run([EXE], capture_output=True, text=True, timeout=100)

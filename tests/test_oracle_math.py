@@ -148,3 +148,64 @@ def test_rmsnorm_backward_reference_is_autograd():
     nm.rmsnorm(x, w, 1e-5).backward(go)
     dx, dw = nm.rmsnorm_backward_ref(go, x.detach(), w.detach(), 1e-5)
     assert rel_err(dx, x.grad) < 1e-13 and rel_err(dw, w.grad) < 1e-13
+
+
+def test_plain_sinkhorn_one_iteration_closed_form_on_a_non_square_matrix():
+    """One iteration is: rows divided by their sums, THEN columns divided by the sums of that
+    result.  On a 2 x 3 matrix worked by hand the two orders give different answers, and a
+    transposed operand (columns first) fails; both restatements must give the row-then-column one."""
+    a = np.array([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]])
+    rows_first = a / a.sum(1, keepdims=True)                  # [[1/6, 1/3, 1/2], [4/15, 1/3, 2/5]]
+    want = rows_first / rows_first.sum(0, keepdims=True)
+    hand = np.array([[(1 / 6) / (1 / 6 + 4 / 15), 0.5, 0.5 / 0.9], [(4 / 15) / (1 / 6 + 4 / 15), 0.5, 0.4 / 0.9]])
+    assert np.allclose(want, hand, rtol=0, atol=1e-15)
+    cols_first = a / a.sum(0, keepdims=True)
+    cols_first = cols_first / cols_first.sum(1, keepdims=True)
+    assert np.abs(cols_first - want).max() > 1e-2             # the two orders are far apart
+    got_c = c_oracle.sinkhorn_plain_forward(a, 1, 1e-8)
+    got_t = nm.sinkhorn_knopp_plain(torch.from_numpy(a), 1, 1e-8).numpy()
+    assert np.abs(got_c - want).max() < 1e-15 and np.abs(got_t - want).max() < 1e-15
+    # after a column step every column sums to one exactly; the rows of a 2 x 3 matrix sum to 3/2
+    # in the limit (total mass = number of columns), not to one
+    far = c_oracle.sinkhorn_plain_forward(a, 200, 1e-8)
+    assert np.abs(far.sum(0) - 1).max() < 1e-14 and np.abs(far.sum(1) - 1.5).max() < 1e-12
+    # the threshold: a row whose sum does not exceed eps is left alone (no 0/0), the others are not
+    z = np.array([[0.0, 0.0, 0.0], [1.0, 1.0, 2.0]])
+    out = c_oracle.sinkhorn_plain_forward(z, 1, 1e-8)
+    assert np.array_equal(out[0], np.zeros(3)) and np.allclose(out[1], [1.0, 1.0, 1.0])
+
+
+@pytest.mark.parametrize("rows,cols,T", [(4, 4, 5), (3, 7, 4), (6, 2, 3), (5, 5, 0)])
+def test_c_oracle_plain_sinkhorn_matches_torch_and_finite_differences(rows, cols, T):
+    rng = np.random.default_rng(rows * 10 + cols)
+    inp = rng.random((rows, cols)) + 0.2
+    go = rng.standard_normal((rows, cols))
+    out_c = c_oracle.sinkhorn_plain_forward(inp, T, 1e-8)
+    t = torch.from_numpy(inp).requires_grad_(True)
+    out_t = nm.sinkhorn_knopp_plain(t, T, 1e-8)
+    assert np.abs(out_c - out_t.detach().numpy()).max() < 1e-14
+    out_t.backward(torch.from_numpy(go))
+    d_c = c_oracle.sinkhorn_plain_backward(go, inp, T, 1e-8)
+    assert np.abs(d_c - t.grad.numpy()).max() < 1e-12 * max(1.0, np.abs(d_c).max())
+    d = rng.standard_normal((rows, cols))
+    h = 1e-6
+    fd = ((c_oracle.sinkhorn_plain_forward(inp + h * d, T, 1e-8) - c_oracle.sinkhorn_plain_forward(inp - h * d, T, 1e-8))
+          * go).sum() / (2 * h)
+    assert abs(fd - (d_c * d).sum()) <= 1e-7 * max(1.0, abs(fd))
+
+
+def test_c_oracle_rmsnorm_against_the_library_routine_and_finite_differences():
+    rng = np.random.default_rng(5)
+    rows, C, eps = 5, 24, 1e-5
+    x, w, go = rng.standard_normal((rows, C)), 1 + 0.3 * rng.standard_normal(C), rng.standard_normal((rows, C))
+    out, rms = c_oracle.rmsnorm_forward(x, w, eps)
+    ref = torch.nn.functional.rms_norm(torch.from_numpy(x), (C,), torch.from_numpy(w), eps).numpy()
+    assert np.abs(out - ref).max() < 1e-14
+    assert np.abs(rms - np.sqrt((x * x).mean(1) + eps)).max() < 1e-15
+    d_x, d_w = c_oracle.rmsnorm_backward(go, x, w, rms)
+    h = 1e-6
+    for name, val, grad in (("x", x, d_x), ("w", w, d_w)):
+        d = rng.standard_normal(val.shape)
+        f = lambda v: (c_oracle.rmsnorm_forward(v if name == "x" else x, v if name == "w" else w, eps)[0] * go).sum()
+        fd = (f(val + h * d) - f(val - h * d)) / (2 * h)
+        assert abs(fd - (grad * d).sum()) <= 1e-7 * max(1.0, abs(fd)), name
