@@ -128,6 +128,7 @@ class Step:
             self.Hp, self.Ho = torch.empty((B, n), **f32), torch.empty((B, n), **f32)
             self.M, self.P = torch.empty((B, n, n), **f32), torch.empty((B, D), **f32)
             self.r = torch.empty(B, **f32)
+            self.sk = torch.empty(max(self.lib.mhc_layer_sinkhorn_state_floats(B, n, T_ITERS), 1), **f32)
             self.dphi = torch.empty((D, n * C), **f32)
             self.dbias, self.dalpha = torch.empty(D, **f32), torch.empty(3, **f32)
             nbytes = self.lib.mhc_layer_dynamic_workspace_bytes(B, n, C)
@@ -149,7 +150,8 @@ class Step:
             st = L.mhc_layer_fwd_dynamic(p(self.x), dc(self.x), p(self.w), dc(self.w), p(self.phi), dc(self.phi),
                                          p(self.bias), p(self.alpha), p(self.f), p(self.y), dc(self.y),
                                          p(self.Hp), p(self.Ho), p(self.M), p(self.P), p(self.r), p(self.q),
-                                         B, n, C, T_ITERS, EPS, p(self.ws), self.ws.numel(), self._stream())
+                                         p(self.sk), B, n, C, T_ITERS, EPS, p(self.ws), self.ws.numel(),
+                                         self._stream())
         else:
             st = L.mhc_layer_fwd(p(self.x), dc(self.x), p(self.w), dc(self.w), p(self.Hl[0]), p(self.Hl[1]),
                                  p(self.Hl[2]), p(self.f), p(self.y), dc(self.y), p(self.Hp), p(self.Ho),
@@ -164,7 +166,7 @@ class Step:
             st = L.mhc_layer_bwd_dynamic(p(self.dy), dc(self.dy), p(self.x), dc(self.x), p(self.w), dc(self.w),
                                          p(self.phi), dc(self.phi), p(self.bias), p(self.alpha), p(self.f),
                                          p(self.Hp), p(self.Ho), p(self.M), p(self.P), p(self.r), p(self.q),
-                                         p(self.dx), p(self.df), p(self.dw), p(self.dphi), p(self.dbias),
+                                         p(self.sk), p(self.dx), p(self.df), p(self.dw), p(self.dphi), p(self.dbias),
                                          p(self.dalpha), B, n, C, T_ITERS, EPS, p(self.ws), self.ws.numel(),
                                          self._stream())
         else:

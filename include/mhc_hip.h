@@ -24,6 +24,8 @@
  *   M                 [B, n, n] fp32 Sinkhorn-normalised mixing matrix (static H: [n, n])
  *   P                 [B, D] fp32   rows of RMSNorm(x_flat) @ phi^T (before alpha and bias)
  *   r, q              [B]   fp32    r = rms of x_flat, q = rms of the aggregated stream
+ *   sk_state          [B, iters, 2, NP] fp32  row and column denominators of every Sinkhorn iteration
+ *                                   (NP = n rounded up to 4, 8, 16 or 32); optional, see below
  */
 #ifndef MHC_HIP_H
 #define MHC_HIP_H
@@ -40,7 +42,7 @@ extern "C" {
 #define MHC_API
 #endif
 
-#define MHC_ABI_VERSION 1
+#define MHC_ABI_VERSION 2
 #define MHC_MAX_N 32
 #define MHC_MAX_C 32768 /* largest hidden size C of the layer entry points (a [C] float row is kept in LDS) */
 
@@ -83,29 +85,36 @@ MHC_API int mhc_max_sinkhorn_iters(int n);
 /* Scratch bytes needed by one dynamic forward or backward call of this shape. */
 MHC_API size_t mhc_layer_dynamic_workspace_bytes(int B, int n, int C);
 
+/* Floats of the optional sk_state tensor of the two calls below (0 for invalid arguments). */
+MHC_API size_t mhc_layer_sinkhorn_state_floats(int B, int n, int iters);
+
 /*
  * y = M_b x_b + H_post_b (x) f_b with per-sample coefficients computed from x.
  * f_inject == NULL: f = RMSNorm(sum_i H_pre[b,i] x[b,i,:]) * w  (the layer).
  * f_inject != NULL: f is that [B, C] tensor (kernel-level view; w is ignored, may be NULL).
  * H_pre, H_post, M, P, r, q are outputs kept for the backward call; all six are required.
+ * sk_state (may be NULL) receives the Sinkhorn denominators of every iteration: handed to the
+ * backward call it saves that call the forward recompute of the iterations (the reference's backward
+ * kernel re-runs the forward as well, src/csrc/kernels/sinkhorn_knopp.cuh:587-690).
  */
 MHC_API int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype,
                           const void *phi, int phi_dtype, const float *bias, const float *alpha,
                           const void *f_inject, void *y, int y_dtype, float *H_pre, float *H_post,
-                          float *M, float *P, float *r, float *q, int B, int n, int C, int iters,
-                          float eps, void *workspace, size_t workspace_bytes, void *stream);
+                          float *M, float *P, float *r, float *q, float *sk_state, int B, int n, int C,
+                          int iters, float eps, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Gradients of the call above for upstream gradient dy (dtype y_dtype).
  * dx has x's dtype.  df (x's dtype) is written only when f_inject != NULL and df != NULL;
  * dw [C] fp32 is written only when f_inject == NULL.  dphi [D, nC], dbias [D], dalpha [3] fp32.
  * Every output is fully overwritten (no pre-zeroing needed); sums are order-deterministic.
+ * sk_state: the tensor written by the forward call, or NULL (the iterations are then recomputed).
  */
 MHC_API int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtype, const void *w,
                           int w_dtype, const void *phi, int phi_dtype, const float *bias,
                           const float *alpha, const void *f_inject, const float *H_pre,
                           const float *H_post, const float *M, const float *P, const float *r,
-                          const float *q, void *dx, void *df, float *dw, float *dphi,
+                          const float *q, const float *sk_state, void *dx, void *df, float *dw, float *dphi,
                           float *dbias, float *dalpha, int B, int n, int C, int iters, float eps,
                           void *workspace, size_t workspace_bytes, void *stream);
 
@@ -141,7 +150,7 @@ MHC_API int mhc_layer_fwd_dynamic_static_scratch(const void *x, int x_dtype, con
                                          const void *phi, int phi_dtype, const float *bias,
                                          const float *alpha, const void *f_inject, void *y, int y_dtype,
                                          float *H_pre, float *H_post, float *M, float *P, float *r,
-                                         float *q, int B, int n, int C, int iters, float eps,
+                                         float *q, float *sk_state, int B, int n, int C, int iters, float eps,
                                          void *stream);
 
 /* ------------------------------------------------------------------------------------------

@@ -187,11 +187,16 @@ size_t mhc_layer_dynamic_workspace_bytes(int B, int n, int C) {
     return f > b ? f : b;
 }
 
+size_t mhc_layer_sinkhorn_state_floats(int B, int n, int iters) {
+    if (n < 1 || n > MHC_MAX_N || B < 1 || iters < 0) return 0;
+    return (size_t)B * iters * 2 * sinkhorn_state_np(n);
+}
+
 int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype, const void *phi,
                           int phi_dtype, const float *bias, const float *alpha,
                           const void *f_inject, void *y, int y_dtype, float *H_pre, float *H_post,
-                          float *M, float *P, float *r, float *q, int B, int n, int C, int iters,
-                          float eps, void *workspace, size_t workspace_bytes, void *stream) {
+                          float *M, float *P, float *r, float *q, float *sk_state, int B, int n, int C,
+                          int iters, float eps, void *workspace, size_t workspace_bytes, void *stream) {
     if (int s = check_shape(B, n, C, iters)) return s;
     if (!x || !phi || !bias || !alpha || !y || !H_pre || !H_post || !M || !P || !r || !q)
         return MHC_ERR_NULL_POINTER;
@@ -206,7 +211,7 @@ int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype
     if (layer_fwd_onepass_supported(x_dtype, phi_dtype, B, n, C)) {
         // projection, coefficients and mix in one launch; x crosses HBM once
         MHC_LAUNCH(launch_layer_fwd_onepass(x, w, w_dtype, f_inject, y, y_dtype, phi, alpha, bias, H_pre, H_post,
-                                            M, P, r, q, B, n, C, iters, eps, st));
+                                            M, P, r, q, sk_state, B, n, C, iters, eps, st));
         return MHC_OK;
     }
     const int KS = proj_fwd_ksplit(x_dtype, phi_dtype, B, n, C);
@@ -214,15 +219,15 @@ int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype
     if (layer_fwd_fused_supported(n, C, x_dtype)) {
         MHC_LAUNCH(launch_layer_fwd_fused(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, ws.Ppart,
                                           ws.ssqpart, KS, padded_D(n), alpha, bias, bias + n,
-                                          bias + 2 * n, H_pre, H_post, M, P, r, q, B, n, C, iters, eps,
-                                          st));
+                                          bias + 2 * n, H_pre, H_post, M, P, r, q, sk_state, B, n, C, iters,
+                                          eps, st));
         return MHC_OK;
     }
     // n > 8 in the bf16 tier: the coefficient launch also forms the stream aggregate and its RMS
     const bool agg = !f_inject && ws.agg && coef_fwd_aggregates(n, C, x_dtype);
     MHC_LAUNCH(launch_coef_fwd(ws.Ppart, ws.ssqpart, KS, padded_D(n), alpha, bias, bias + n,
                                bias + 2 * n, H_pre, H_post, M, P, r, B, n, n * C, iters, eps,
-                               x_dtype == kF32, agg ? x : nullptr, ws.agg, q, st));
+                               x_dtype == kF32, agg ? x : nullptr, ws.agg, q, sk_state, st));
     MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, H_pre, H_post, M, n, q,
                               ws.agg, B, n, C, eps, agg, st));
     return MHC_OK;
@@ -232,7 +237,7 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
                           int w_dtype, const void *phi, int phi_dtype, const float *bias,
                           const float *alpha, const void *f_inject, const float *H_pre,
                           const float *H_post, const float *M, const float *P, const float *r,
-                          const float *q, void *dx, void *df, float *dw, float *dphi,
+                          const float *q, const float *sk_state, void *dx, void *df, float *dw, float *dphi,
                           float *dbias, float *dalpha, int B, int n, int C, int iters, float eps,
                           void *workspace, size_t workspace_bytes, void *stream) {
     if (int s = check_shape(B, n, C, iters)) return s;
@@ -252,7 +257,8 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     const bool mfma = proj_bwd_mfma_supported(x_dtype, phi_dtype, C);
     BwdCoefOut out{ws.dt, ws.dP, ws.cx, ws.s1, nullptr, mfma ? ws.dPb : nullptr, ws.dPT, ws.BP};
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
-                                     n, q, P, r, alpha, bias + 2 * n, out, ws.raw, B, n, C, iters, eps, st));
+                                     n, q, P, r, alpha, bias + 2 * n, sk_state, out, ws.raw, B, n, C, iters, eps,
+                                     st));
     if (mfma && bwd_slab_supported(x_dtype, y_dtype, phi_dtype, n, C)) {
         // n <= 4: one slab kernel finishes dx and produces every batch-split partial sum
         const int S = bwd_slab_batch_splits(B, n, C);
@@ -333,7 +339,8 @@ int mhc_layer_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
         // one launch; every workgroup derives the shared coefficients itself, none need storing
         MHC_LAUNCH(launch_layer_fwd_fused(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, nullptr, nullptr,
                                           0, 0, nullptr, H_pre_logits, H_post_logits, H_res_logits,
-                                          H_pre, H_post, M, nullptr, nullptr, q, B, n, C, iters, eps, st));
+                                          H_pre, H_post, M, nullptr, nullptr, q, nullptr, B, n, C, iters, eps,
+                                          st));
         return MHC_OK;
     }
     const StaFwdWs ws = carve_sta_fwd(workspace, B, n, C);
@@ -344,7 +351,7 @@ int mhc_layer_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
     float *m = M ? M : ws.M, *qq = q ? q : ws.q;
     MHC_LAUNCH(launch_coef_fwd(nullptr, nullptr, 0, 0, nullptr, H_pre_logits, H_post_logits,
                                H_res_logits, hp, ho, m, nullptr, nullptr, 1, n, n * C, iters, eps,
-                               x_dtype == kF32, nullptr, nullptr, nullptr, st));
+                               x_dtype == kF32, nullptr, nullptr, nullptr, nullptr, st));
     MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, hp, ho, m, 0, qq,
                               n > 8 ? ws.agg : nullptr, B, n, C, eps, false, st));
     return MHC_OK;
@@ -371,8 +378,8 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
     const int D = n * n + 2 * n;
     BwdCoefOut out{nullptr, nullptr, nullptr, ws.s1, ws.red, nullptr, nullptr, 0};
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
-                                     0, q, nullptr, nullptr, nullptr, nullptr, out, n > 8 ? ws.raw : nullptr, B, n, C,
-                                     iters, eps, st));
+                                     0, q, nullptr, nullptr, nullptr, nullptr, nullptr, out, n > 8 ? ws.raw : nullptr,
+                                     B, n, C, iters, eps, st));
     MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, 0,
                                  q, ws.s1, nullptr, nullptr, 0, nullptr, 0, nullptr, dx, df, ws.u, nullptr,
                                  nullptr, 1, B, n, C, st));
@@ -501,7 +508,7 @@ int mhc_layer_fwd_dynamic_static_scratch(const void *x, int x_dtype, const void 
                                          const void *phi, int phi_dtype, const float *bias,
                                          const float *alpha, const void *f_inject, void *y, int y_dtype,
                                          float *H_pre, float *H_post, float *M, float *P, float *r,
-                                         float *q, int B, int n, int C, int iters, float eps,
+                                         float *q, float *sk_state, int B, int n, int C, int iters, float eps,
                                          void *stream) {
     if (int s = check_shape(B, n, C, iters)) return s;
     // every byte the kernels touch lies below `need`; nothing has to start at zero (the projection
@@ -512,7 +519,7 @@ int mhc_layer_fwd_dynamic_static_scratch(const void *x, int x_dtype, const void 
     void *ptr = nullptr;
     if (int s = static_scratch_pointer(&ptr)) return s;
     return mhc_layer_fwd_dynamic(x, x_dtype, w, w_dtype, phi, phi_dtype, bias, alpha, f_inject, y, y_dtype,
-                                 H_pre, H_post, M, P, r, q, B, n, C, iters, eps, ptr,
+                                 H_pre, H_post, M, P, r, q, sk_state, B, n, C, iters, eps, ptr,
                                  MHC_STATIC_SCRATCH_BYTES, stream);
 }
 

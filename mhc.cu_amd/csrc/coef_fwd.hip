@@ -25,6 +25,8 @@ struct CoefArgs {
     // stream aggregate a = Hpre^T x (fp32 [B, C]) and its RMS q, from loads that fly under the Sinkhorn chain
     const bf16_t *x_agg;
     float *a_ws, *q;
+    float *sk_state;  // dynamic: [B][T][2][NP] Sinkhorn denominators kept for the backward, or nullptr
+    bool precise;     // fp32 tier: IEEE divisions in the iterations whose denominators are kept
 };
 
 // eight loads in flight per round (a plain loop would pay one memory latency per split)
@@ -74,7 +76,14 @@ template <int NP> __global__ __launch_bounds__(64) void coef_fwd_small_kernel(Co
         const int c = c0 + e;
         m[e] = (r0 < n && c < n) ? expf(logit(2 * n + r0 * n + c, al[2], a.b_res[r0 * n + c])) : 0.f;
     }
-    SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, lane);
+    // The backward call rebuilds the iterates by undoing the scalings with the kept denominators
+    // (m * s * rho).  After v_rcp_f32 that product is off by the same fraction of an ulp in every
+    // iteration once the denominators have converged, which adds up over hundreds of iterations:
+    // the fp32 tier divides.
+    float *st = a.sk_state ? a.sk_state + (size_t)b * SK::state_floats(a.T) : nullptr;
+    if (st && a.precise) SK::template forward_save<true>(m, g, n, a.T, a.eps, st);
+    else if (st) SK::template forward_save<false>(m, g, n, a.T, a.eps, st);
+    else SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, lane);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;
@@ -191,6 +200,7 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         if (r0 < n && c0 + e < n) a.M[(size_t)b * n * n + r0 * n + c0 + e] = u * E[e] * v[e];
+    if (a.sk_state) SK::save_state(sk_s, a.T, a.sk_state + (size_t)b * SK::state_floats(a.T), tid);
     if constexpr (AGG) {
         __syncthreads();  // hp_s (with zero iterations the Sinkhorn step has no barrier of its own)
         float acc[8], ssq = 0.f;
@@ -218,9 +228,9 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
                            const float *alpha, const float *b_pre, const float *b_post,
                            const float *b_res, float *Hpre, float *Hpost, float *M, float *P,
                            float *r, int B, int n, int nC, int T, float eps, bool precise,
-                           const void *x_agg, float *a_ws, float *q, hipStream_t stream) {
+                           const void *x_agg, float *a_ws, float *q, float *sk_state, hipStream_t stream) {
     CoefArgs a{Ppart, ssqpart, KS, DP, alpha, b_pre, b_post, b_res, Hpre, Hpost, M, P, r, B, n, nC, T, eps,
-               static_cast<const bf16_t *>(x_agg), a_ws, q};
+               static_cast<const bf16_t *>(x_agg), a_ws, q, sk_state, precise};
     const bool agg = x_agg != nullptr;  // the caller has checked coef_fwd_aggregates()
     if (n <= 4)
         coef_fwd_small_kernel<4><<<(B + 3) / 4, 64, 0, stream>>>(a);

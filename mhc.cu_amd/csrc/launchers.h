@@ -42,7 +42,11 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
                            const float *alpha, const float *b_pre, const float *b_post,
                            const float *b_res, float *Hpre, float *Hpost, float *M, float *P,
                            float *r, int B, int n, int nC, int T, float eps, bool precise,
-                           const void *x_agg, float *a_ws, float *q, hipStream_t stream);
+                           const void *x_agg, float *a_ws, float *q, float *sk_state, hipStream_t stream);
+// sk_state (dynamic H, optional): [B][T][2][NP] floats, NP = sinkhorn_state_np(n): the row and column
+// denominators of every Sinkhorn iteration, kept for the backward call (which otherwise recomputes
+// the forward iterations to get them).
+inline int sinkhorn_state_np(int n) { return n <= 4 ? 4 : (n <= 8 ? 8 : (n <= 16 ? 16 : 32)); }
 // x_agg != nullptr (only where coef_fwd_aggregates() holds): the launch also writes the stream
 // aggregate a = Hpre^T x (a_ws, fp32 [B, C]) and its RMS q, which launch_mix_fwd then takes as given
 // (have_agg).
@@ -67,15 +71,15 @@ hipError_t launch_layer_fwd_fused(const void *x, int x_dtype, const void *w, int
                                   const float *ssqpart, int KS, int DP, const float *alpha,
                                   const float *b_pre, const float *b_post, const float *b_res,
                                   float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
-                                  int B, int n, int C, int T, float eps, hipStream_t stream);
+                                  float *sk_state, int B, int n, int C, int T, float eps, hipStream_t stream);
 
 // Whole dynamic-H forward in one launch (bf16 x and phi, n <= 4, n*C % 64 == 0): projection,
 // coefficients and mix with the samples' rows resident in LDS.  bias = [pre | post | res].
 bool layer_fwd_onepass_supported(int x_dtype, int phi_dtype, int B, int n, int C);
 hipError_t launch_layer_fwd_onepass(const void *x, const void *w, int w_dtype, const void *f_inject, void *y,
                                     int y_dtype, const void *phi, const float *alpha, const float *bias,
-                                    float *Hpre, float *Hpost, float *M, float *P, float *r, float *q, int B,
-                                    int n, int C, int T, float eps, hipStream_t stream);
+                                    float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
+                                    float *sk_state, int B, int n, int C, int T, float eps, hipStream_t stream);
 
 // fp32 matrix-core GEMMs of the exact float32 tier (wide projections): see gemm_f32.hip.
 bool gemm_f32_supported(int x_dtype, int phi_dtype, int n, int C);
@@ -106,8 +110,8 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
                                  const void *w, int w_dtype, const void *f_inject,
                                  const float *Hpre, const float *Hpost, const float *M, int hstride,
                                  const float *q, const float *P, const float *r, const float *alpha,
-                                 const float *b_res, BwdCoefOut out, float *raw, int B, int n, int C,
-                                 int T, float eps, hipStream_t stream);
+                                 const float *b_res, const float *sk_state, BwdCoefOut out, float *raw, int B,
+                                 int n, int C, int T, float eps, hipStream_t stream);
 // raw (optional, dynamic H, n <= 8): scratch of B * bwd_reduce_parts() * (NP*NP + 3*NP + 1) floats;
 // when given, the channel sums and the coefficient backward run as two launches.
 int bwd_reduce_parts(int B, int n, int C);

@@ -38,6 +38,7 @@ struct OnePassArgs {
     float *Hpre, *Hpost, *M, *P, *r, *q;
     int w_bf16, B, n, C, T, G;
     float eps;
+    float *sk_state;  // [B][T][2][NP] Sinkhorn denominators kept for the backward, or nullptr
 };
 
 constexpr int kOpMaxG = 16;      // samples per workgroup: the columns of one 16-wide tile
@@ -350,7 +351,9 @@ __global__ __launch_bounds__(512) void layer_fwd_onepass_kernel(OnePassArgs a) {
         }
     };
     if (coef_wave) {
-        SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, lane);
+        // (samples beyond the group write the state of the last valid one again: same values)
+        if (a.sk_state) SK::template forward_save<false>(m, g, n, a.T, a.eps, a.sk_state + (size_t)(b0 + sc) * SK::state_floats(a.T));
+        else SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, lane);
         if (sv && mv) a.M[(size_t)(b0 + sc) * n * n + r0 * n + c0] = m[0];
         // row r0 of M as an A row (bf16 value + remainder): the quad that holds the row sees all of it
         const float m0 = dpp_mov<kDppQuadBcast0>(m[0]), m1 = dpp_mov<kDppQuadBcast1>(m[0]);
@@ -461,14 +464,14 @@ bool layer_fwd_onepass_supported(int x_dtype, int phi_dtype, int B, int n, int C
 
 hipError_t launch_layer_fwd_onepass(const void *x, const void *w, int w_dtype, const void *f_inject, void *y,
                                     int y_dtype, const void *phi, const float *alpha, const float *bias,
-                                    float *Hpre, float *Hpost, float *M, float *P, float *r, float *q, int B,
-                                    int n, int C, int T, float eps, hipStream_t stream) {
+                                    float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
+                                    float *sk_state, int B, int n, int C, int T, float eps, hipStream_t stream) {
     const int G = onepass_group(B, n, C);
     int NW = tuning_get(kTuneOnepassWaves);
     if (NW < 4 || NW > 8) NW = 8;
     OnePassArgs a{static_cast<const bf16_t *>(x), w, static_cast<const bf16_t *>(f_inject), y,
                   static_cast<const bf16_t *>(phi), alpha, bias, Hpre, Hpost, M, P, r, q,
-                  w_dtype == kBF16, B, n, C, T, G, eps};
+                  w_dtype == kBF16, B, n, C, T, G, eps, sk_state};
     const size_t smem = OnePassLds(G, n * C, round_up(C / 8, 4), NW).total;
     const int grid = (B + G - 1) / G;
     hipError_t e = hipSuccess;

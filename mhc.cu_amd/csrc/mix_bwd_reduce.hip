@@ -26,6 +26,7 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 struct BwdReduceArgs {
     const void *dy, *x, *w, *f_inject;
     const float *Hpre, *Hpost, *M, *q, *P, *r, *alpha, *b_res;
+    const float *sk_state;  // dynamic: Sinkhorn denominators saved by the forward ([B][T][2][NP]) or nullptr
     BwdCoefOut out;
     int hstride, w_bf16, B, n, C, T, DP;
     float eps;
@@ -299,8 +300,15 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
     // The Sinkhorn forward recompute, which keeps the denominators of every iteration in sc: it needs
     // none of the channel sums, so a caller that produces them itself can run it while they are
     // still on their way.  g: lane within the group; lane: lane within the wave (indexes sc).
-    __device__ __forceinline__ void forward_recompute(const BwdReduceArgs &a, int g, int lane, float *sc) {
+    // With the denominators saved by the forward call there is nothing to iterate: they are copied
+    // into sc and the final iterate is the saved M.
+    __device__ __forceinline__ void forward_recompute(const BwdReduceArgs &a, int b, int g, int lane, float *sc) {
         E = mv ? (PRECISE ? expf(al2 * pres + bres) : exp_fast(al2 * pres + bres)) : 0.f;
+        if (a.sk_state) {
+            m_fin = mv ? a.M[(size_t)b * a.n * a.n + r0 * a.n + c0] : 0.f;
+            SK::load_state(a.sk_state + (size_t)b * SK::state_floats(a.T), g, a.T, sc, lane);
+            return;
+        }
         float m[1] = {E};
         SK::template forward<PRECISE>(m, g, a.n, a.T, a.eps, sc, lane);
         m_fin = m[0];
@@ -398,7 +406,7 @@ __global__ __launch_bounds__(64) void coef_bwd_small_kernel(BwdReduceArgs a) {
     CB cb;
     cb.prefetch(a, b, g);
     cb.fetch_sums(a.raw + (size_t)b * a.parts * CB::K, a.parts);  // requested before the chain, used after it
-    cb.forward_recompute(a, g, tid, sc);
+    cb.forward_recompute(a, b, g, tid, sc);
     cb.run(a, b, g, tid, sc, sc + SK::scaling_floats(a.T) + (tid / SK::kGroup) * CB::kXch);
 }
 
@@ -446,7 +454,7 @@ __global__ __launch_bounds__(256, NP == 4 ? 4 : 1) void gram_small_kernel(BwdRed
         // wave 0, while the other waves already stream (and not at the tail of the workgroup)
         if (tid < SK::kGroup) {
             cb.prefetch(a, b, tid);
-            cb.forward_recompute(a, tid, tid, sc);
+            cb.forward_recompute(a, b, tid, tid, sc);
         }
     }
     const int blk = lane >> 2, i = lane & 3;
@@ -926,7 +934,8 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
             pres[e] = ok ? pres[e] : 0.f;
             E[e] = ok ? (PRECISE ? expf(al2 * pres[e] + bres[e]) : exp_fast(al2 * pres[e] + bres[e])) : 0.f;
         }
-        SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
+        if (a.sk_state) SK::template load_state<PRECISE>(a.sk_state + (size_t)b * SK::state_floats(a.T), u, v, a.T, sk_s, tid);
+        else SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
     }
     {
         float acc[EPT];
@@ -1175,13 +1184,13 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
                                  const void *w, int w_dtype, const void *f_inject,
                                  const float *Hpre, const float *Hpost, const float *M, int hstride,
                                  const float *q, const float *P, const float *r, const float *alpha,
-                                 const float *b_res, BwdCoefOut out, float *raw, int B, int n, int C,
-                                 int T, float eps, hipStream_t stream) {
+                                 const float *b_res, const float *sk_state, BwdCoefOut out, float *raw, int B,
+                                 int n, int C, int T, float eps, hipStream_t stream) {
     // n <= 8, dynamic H: channel sums per (sample, column part), coefficient backward as a second
     // small launch (static H: everything in the per-sample workgroup).  n > 8: always two launches.
     if (n > 8 && raw == nullptr) return hipErrorInvalidValue;
     const bool split = raw != nullptr && (n > 8 || hstride != 0);
-    BwdReduceArgs a{dy, x, w, f_inject, Hpre, Hpost, M, q, P, r, alpha, b_res, out,
+    BwdReduceArgs a{dy, x, w, f_inject, Hpre, Hpost, M, q, P, r, alpha, b_res, sk_state, out,
                     hstride, w_dtype == kBF16, B, n, C, T, padded_D(n), eps,
                     split ? raw : nullptr, split ? bwd_reduce_parts(B, n, C) : 1};
     if (n <= 8) {

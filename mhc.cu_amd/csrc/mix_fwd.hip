@@ -140,6 +140,7 @@ struct LayerFwdArgs {
     float *Hpre, *Hpost, *M, *P, *r, *q;  // outputs (static: shared [n], [n], [n,n]; may be null)
     int KS, DP, w_bf16, B, n, C, T;
     float eps;
+    float *sk_state;  // dynamic: [B][T][2][NP] Sinkhorn denominators kept for the backward, or nullptr
 };
 
 constexpr int kFwdStaggerMinB = 512;  // two or more workgroups per CU
@@ -303,7 +304,10 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             } else {
                 m[0] = 0.f;
             }
-            SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, tid);
+            // kept denominators: the fp32 tier divides, so that the backward call can undo the
+            // scalings (m * s * rho) without a bias that grows with the iteration count
+            if (dyn && a.sk_state) SK::template forward_save<!kFast>(m, g, n, a.T, a.eps, a.sk_state + (size_t)b * SK::state_floats(a.T));
+            else SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, tid);
             coef_s[r0 * NP + c0] = m[0];
             if (wr && a.M && mv) a.M[ms + r0 * n + c0] = m[0];
         }
@@ -591,9 +595,9 @@ hipError_t launch_layer_fwd_fused(const void *x, int x_dtype, const void *w, int
                                   const float *ssqpart, int KS, int DP, const float *alpha,
                                   const float *b_pre, const float *b_post, const float *b_res,
                                   float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
-                                  int B, int n, int C, int T, float eps, hipStream_t stream) {
+                                  float *sk_state, int B, int n, int C, int T, float eps, hipStream_t stream) {
     LayerFwdArgs a{x, w, f_inject, y, Ppart, ssqpart, alpha, b_pre, b_post, b_res, Hpre, Hpost, M, P, r, q,
-                   KS, DP, w_dtype == kBF16, B, n, C, T, eps};
+                   KS, DP, w_dtype == kBF16, B, n, C, T, eps, sk_state};
     hipError_t err = hipErrorInvalidValue;
     bool ok = false;
 #define MHC_FUSED(TX, TY)                                                        \

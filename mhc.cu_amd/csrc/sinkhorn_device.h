@@ -86,6 +86,46 @@ template <int NP> struct SkSmall {
         }
     }
 
+    // The same forward, keeping the denominators of every iteration in GLOBAL memory for the backward
+    // call: st[(t * 2 + 0) * NP + row] = rho_t[row], st[(t * 2 + 1) * NP + col] = s_t[col] (every lane
+    // of a row / column writes the same value).  2 T NP floats per matrix.
+    template <bool PRECISE = false>
+    __device__ static __forceinline__ void forward_save(float (&m)[EPL], int g, int n, int T, float eps, float *st) {
+        static_assert(EPL == 1, "one element per lane");
+        const int r = row(g), c = col0(g);
+        const float eps_r = r < n ? eps : 1.0f, eps_c = c < n ? eps : 1.0f;
+        for (int t = 0; t < T; t++) {
+            const float rs = row_allreduce(m[0]) + eps_r;
+            st[(t * 2) * NP + r] = rs;
+            m[0] = PRECISE ? m[0] / rs : m[0] * fast_rcp(rs);
+            const float cs = col_allreduce(m[0]) + eps_c;
+            st[(t * 2 + 1) * NP + c] = cs;
+            m[0] = PRECISE ? m[0] / cs : m[0] * fast_rcp(cs);
+        }
+    }
+    // Denominators saved by forward_save() -> the per-lane LDS layout that backward() reads.  All
+    // loads are independent (four iterations requested at a time).
+    __device__ static __forceinline__ void load_state(const float *st, int g, int T, float *sc, int lane) {
+        const int r = row(g), c = col0(g);
+        for (int t0 = 0; t0 < T; t0 += 4) {
+            float rs[4], cs[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int t = t0 + u < T ? t0 + u : T - 1;
+                rs[u] = st[(t * 2) * NP + r];
+                cs[u] = st[(t * 2 + 1) * NP + c];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (t0 + u < T) {
+                    sc[((t0 + u) * kRec) * kWave + lane] = rs[u];
+                    sc[((t0 + u) * kRec + 1) * kWave + lane] = cs[u];
+                }
+            }
+        }
+    }
+    __host__ __device__ static constexpr int state_floats(int T) { return 2 * T * NP; }
+
     // d: in = dL/dM, out = dL/dE.  m: the final iterate from forward (destroyed).  The reverse
     // sweep rebuilds the iterates it needs by undoing the scalings with the saved denominators
     // (Out_t = m, R_t = Out_t s_t, Out_{t-1} = R_t rho_t) instead of reading stored copies.
@@ -246,6 +286,44 @@ template <int NP> struct SkWg {
             ld_vec(vb + b0, v);
         }
     }
+
+    // Copies the denominators that forward() left in LDS to global memory for the backward call:
+    // st[(t * 2 + 0) * NP + a] = rho_t[a], st[(t * 2 + 1) * NP + a] = s_t[a].  Every thread calls it.
+    __device__ static __forceinline__ void save_state(const float *lds, int T, float *st, int tid) {
+        const float *rho = lds + kTile + 2 * NP, *s = rho + T * NP;
+        for (int e = tid; e < T * NP; e += 256) {
+            const int t = e / NP, a = e % NP;
+            st[(t * 2) * NP + a] = rho[e];
+            st[(t * 2 + 1) * NP + a] = s[e];
+        }
+    }
+    // The inverse: puts saved denominators where backward() expects them and rebuilds the final
+    // scalings u, v with the recurrence of forward() (u <- u / rho_t, v <- v / s_t), so that
+    // backward() can follow without the forward recompute.  Every thread calls it; ends on a barrier.
+    template <bool PRECISE = true>
+    __device__ static __forceinline__ void load_state(const float *st, float &u, float (&v)[EPL], int T, float *lds,
+                                                      int tid) {
+        float *rho = lds + kTile + 2 * NP, *s = rho + T * NP;
+        for (int e = tid; e < T * NP; e += 256) {
+            const int t = e / NP, a = e % NP;
+            rho[e] = st[(t * 2) * NP + a];
+            s[e] = st[(t * 2 + 1) * NP + a];
+        }
+        __syncthreads();
+        const int a = row(tid), b0 = col0(tid);
+        u = 1.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) v[e] = 1.0f;
+        for (int t = 0; t < T; t++) {
+            const float rr = rho[t * NP + a];
+            u = PRECISE ? u / rr : u * fast_rcp(rr);
+            float sc[EPL];
+            ld_vec(s + t * NP + b0, sc);
+#pragma unroll
+            for (int e = 0; e < EPL; e++) v[e] = PRECISE ? v[e] / sc[e] : v[e] * fast_rcp(sc[e]);
+        }
+    }
+    __host__ __device__ static constexpr int state_floats(int T) { return 2 * T * NP; }
 
     // d: in = dL/dM, out = dL/dE.  E, u, v, LDS contents: as left by forward() (u and v are
     // destroyed).

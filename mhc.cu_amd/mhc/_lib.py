@@ -18,7 +18,7 @@ LIB_PATH = os.environ.get("MHC_HIP_LIBRARY") or os.path.join(_HERE, "libmhc_hip.
 
 MHC_F32, MHC_BF16 = 0, 1
 MHC_MAX_N = 32
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(
@@ -34,16 +34,17 @@ _SIGNATURES = {
     "mhc_status_string": (c_char_p, [_I]),
     "mhc_max_sinkhorn_iters": (c_int, [_I]),
     "mhc_layer_dynamic_workspace_bytes": (_Z, [_I, _I, _I]),
+    "mhc_layer_sinkhorn_state_floats": (_Z, [_I, _I, _I]),
     "mhc_layer_fwd_dynamic": (c_int, [_P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P,
-                                      _P, _I, _I, _I, _I, _F, _P, _Z, _P]),
+                                      _P, _P, _I, _I, _I, _I, _F, _P, _Z, _P]),
     "mhc_layer_bwd_dynamic": (c_int, [_P, _I, _P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P,
-                                      _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _P, _Z, _P]),
+                                      _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _P, _Z, _P]),
     "mhc_pack_dynamic_params": (c_int, [_P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P]),
     "mhc_static_scratch_capacity": (_Z, []),
     "mhc_layer_fwd_dynamic_scratch_bytes": (_Z, [_I, _I, _I]),
     "mhc_static_scratch_init": (c_int, []),
     "mhc_layer_fwd_dynamic_static_scratch": (c_int, [_P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P,
-                                                     _P, _P, _P, _I, _I, _I, _I, _F, _P]),
+                                                     _P, _P, _P, _P, _I, _I, _I, _I, _F, _P]),
     "mhc_layer_static_workspace_bytes": (_Z, [_I, _I, _I]),
     "mhc_layer_fwd": (c_int, [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I,
                               _F, _P, _Z, _P]),

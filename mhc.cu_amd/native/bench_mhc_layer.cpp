@@ -89,6 +89,7 @@ static void run_config(int B, int C, int n, int T, bool dynamic, bool bf16, int 
     upload(w, std::vector<float>(C, 1.f), bf16);
     DeviceBuf Hp((dynamic ? B : 1) * n * 4), Ho((dynamic ? B : 1) * n * 4), M((dynamic ? B : 1) * n * n * 4);
     DeviceBuf q(B * 4), r(B * 4), P(B * D * 4);
+    DeviceBuf sk(std::max<size_t>(mhc_layer_sinkhorn_state_floats(B, n, T), 4) * 4);
     DeviceBuf phi(dynamic ? D * nC * es : 16), dphi(dynamic ? D * nC * 4 : 16), bias(D * 4), dbias(D * 4);
     DeviceBuf alpha(16), dalpha(16), logits(D * 4), dlogits(D * 4);
     if (dynamic) {
@@ -108,7 +109,7 @@ static void run_config(int B, int C, int n, int T, bool dynamic, bool bf16, int 
         if (dynamic)
             MHC_OK_(mhc_layer_fwd_dynamic(x.p, act, w.p, act, phi.p, act, (float *)bias.p, (float *)alpha.p, nullptr,
                                           y.p, act, (float *)Hp.p, (float *)Ho.p, (float *)M.p, (float *)P.p,
-                                          (float *)r.p, (float *)q.p, B, n, C, T, eps, ws.p, wsb, nullptr));
+                                          (float *)r.p, (float *)q.p, (float *)sk.p, B, n, C, T, eps, ws.p, wsb, nullptr));
         else
             MHC_OK_(mhc_layer_fwd(x.p, act, w.p, act, lg, lg + n, lg + 2 * n, nullptr, y.p, act, (float *)Hp.p,
                                   (float *)Ho.p, (float *)M.p, (float *)q.p, B, n, C, T, eps, ws.p, wsb, nullptr));
@@ -117,7 +118,7 @@ static void run_config(int B, int C, int n, int T, bool dynamic, bool bf16, int 
         if (dynamic)
             MHC_OK_(mhc_layer_bwd_dynamic(dy.p, act, x.p, act, w.p, act, phi.p, act, (float *)bias.p, (float *)alpha.p,
                                           nullptr, (float *)Hp.p, (float *)Ho.p, (float *)M.p, (float *)P.p,
-                                          (float *)r.p, (float *)q.p, dx.p, nullptr, (float *)dw.p, (float *)dphi.p,
+                                          (float *)r.p, (float *)q.p, (float *)sk.p, dx.p, nullptr, (float *)dw.p, (float *)dphi.p,
                                           (float *)dbias.p, (float *)dalpha.p, B, n, C, T, eps, ws.p, wsb, nullptr));
         else
             MHC_OK_(mhc_layer_bwd(dy.p, act, x.p, act, w.p, act, lg, lg + n, lg + 2 * n, nullptr, (float *)Hp.p,

@@ -89,13 +89,14 @@ int main(int argc, char **argv) {
     float *bias = dev_f32(D, 0.f), *alpha = dev_f32(3, 0.01f), *Hp = dev_f32((size_t)B * n, 0.f), *Ho = dev_f32((size_t)B * n, 0.f),
           *M = dev_f32((size_t)B * n * n, 0.f), *P = dev_f32(B * D, 0.f), *r = dev_f32(B, 0.f), *q = dev_f32(B, 0.f),
           *dw = dev_f32(C, 0.f), *dphi = dev_f32(D * nC, 0.f), *dbias = dev_f32(D, 0.f), *dalpha = dev_f32(3, 0.f);
+    float *sk = dev_f32(mhc_layer_sinkhorn_state_floats(B, n, T), 0.f);
     const size_t wsb = mhc_layer_dynamic_workspace_bytes(B, n, C);
     void *ws; HIP_OK(hipMalloc(&ws, wsb + 256));
     for (int it = 0; it < 3; it++) {
         MHC_OK_(mhc_layer_fwd_dynamic(x, MHC_BF16, w, MHC_BF16, phi, MHC_BF16, bias, alpha, nullptr, y, MHC_BF16, Hp, Ho, M, P, r,
-                                      q, B, n, C, T, 1e-6f, ws, wsb, nullptr));
+                                      q, sk, B, n, C, T, 1e-6f, ws, wsb, nullptr));
         MHC_OK_(mhc_layer_bwd_dynamic(dy, MHC_BF16, x, MHC_BF16, w, MHC_BF16, phi, MHC_BF16, bias, alpha, nullptr, Hp, Ho, M, P, r, q,
-                                      dx, nullptr, dw, dphi, dbias, dalpha, B, n, C, T, 1e-6f, ws, wsb, nullptr));
+                                      sk, dx, nullptr, dw, dphi, dbias, dalpha, B, n, C, T, 1e-6f, ws, wsb, nullptr));
         HIP_OK(hipDeviceSynchronize());
     }
     printf("phase profile: dynamic H, bf16, B=%d C=%d n=%d (last of 3 warm calls)\n", B, C, n);

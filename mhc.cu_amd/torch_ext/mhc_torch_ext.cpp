@@ -172,26 +172,30 @@ Packed pack_params(const Tensor &phi_pre, const Tensor &phi_post, const Tensor &
 // dynamic-H layer (reference ops.py:154-417, bindings.cu:405-542)
 // ---------------------------------------------------------------------------------------------
 struct DynFwdOut {
-    Tensor y, small;  // small = fp32 [B * (2n + n*n + D + 2)]: Hpre | Hpost | M | P | r | q
+    Tensor y, small;  // small = fp32: Hpre | Hpost | M | P | r | q | Sinkhorn state, B * (2n + n*n + D + 2) + state floats
 };
 
 struct SmallViews {
-    float *Hp, *Ho, *M, *P, *r, *q;
+    float *Hp, *Ho, *M, *P, *r, *q, *sk;
+    static int64_t coef_floats(int B, int n) { return (int64_t)B * (2 * n + n * n + (n * n + 2 * n) + 2); }
     SmallViews(const Tensor &small, int B, int n) {
         const int D = n * n + 2 * n;
         float *b = small.data_ptr<float>();
         Hp = b; Ho = Hp + (size_t)B * n; M = Ho + (size_t)B * n; P = M + (size_t)B * n * n;
         r = P + (size_t)B * D; q = r + B;
+        sk = small.numel() > coef_floats(B, n) ? q + B : nullptr;  // present when the forward ran under autograd
     }
 };
 
 DynFwdOut dyn_forward(const Tensor &x, const OptTensor &w, const Packed &pk, const OptTensor &f_inject,
-                      at::ScalarType out_dtype, int iters, double eps) {
+                      at::ScalarType out_dtype, int iters, double eps, bool for_backward) {
     const int B = x.size(0), n = x.size(1), C = x.size(2), D = n * n + 2 * n;
     c10::DeviceGuard guard(x.device());
     DynFwdOut o;
     o.y = at::empty({B, n, C}, x.options().dtype(out_dtype));
-    o.small = at::empty({(int64_t)B * (2 * n + n * n + D + 2)}, x.options().dtype(at::kFloat));
+    // the Sinkhorn denominators are only worth writing when a backward call will read them
+    const int64_t state = for_backward ? (int64_t)mhc_layer_sinkhorn_state_floats(B, n, iters) : 0;
+    o.small = at::empty({SmallViews::coef_floats(B, n) + state}, x.options().dtype(at::kFloat));
     SmallViews v(o.small, B, n);
     const size_t need = mhc_layer_dynamic_workspace_bytes(B, n, C);
     Tensor ws = workspace(x, need);
@@ -200,8 +204,8 @@ DynFwdOut dyn_forward(const Tensor &x, const OptTensor &w, const Packed &pk, con
     float *ba = pk.ba.data_ptr<float>();
     check("mhc_layer_fwd_dynamic",
           mhc_layer_fwd_dynamic(ptr(x), dt(x), ptr(wt), wt.defined() ? dt(wt) : 0, ptr(pk.phi), dt(pk.phi), ba, ba + D,
-                                ptr(ft), ptr(o.y), dt(o.y), v.Hp, v.Ho, v.M, v.P, v.r, v.q, B, n, C, iters, (float)eps,
-                                ws.data_ptr(), (size_t)ws.numel(), stream_of(x)));
+                                ptr(ft), ptr(o.y), dt(o.y), v.Hp, v.Ho, v.M, v.P, v.r, v.q, v.sk, B, n, C, iters,
+                                (float)eps, ws.data_ptr(), (size_t)ws.numel(), stream_of(x)));
     return o;
 }
 
@@ -210,7 +214,7 @@ struct MHCDynamicFn : public torch::autograd::Function<MHCDynamicFn> {
                           const Tensor &phi_post, const Tensor &phi_res, const Tensor &alpha_pre,
                           const Tensor &alpha_post, const Tensor &alpha_res, const Tensor &b_pre, const Tensor &b_post,
                           const Tensor &b_res, int64_t iters, double eps, c10::optional<at::ScalarType> out_dtype,
-                          const OptTensor &f_in) {
+                          const OptTensor &f_in, bool grad_mode) {
         TORCH_CHECK(x_in.dim() == 3, "mhc: x must be [B, n, C]");
         const Tensor x = act(is_act_dtype(x_in) ? x_in : x_in.to(at::kFloat));
         const int n = x.size(1), C = x.size(2);
@@ -219,7 +223,7 @@ struct MHCDynamicFn : public torch::autograd::Function<MHCDynamicFn> {
         if (f_in.has_value() && f_in->defined()) f = act(f_in->to(x.scalar_type()));
         const Packed pk = pack_params(phi_pre, phi_post, phi_res, alpha_pre, alpha_post, alpha_res, b_pre, b_post, b_res,
                                       n, C, x.scalar_type());
-        DynFwdOut o = dyn_forward(x, w, pk, f, out_dtype.value_or(at::kFloat), (int)iters, eps);
+        DynFwdOut o = dyn_forward(x, w, pk, f, out_dtype.value_or(at::kFloat), (int)iters, eps, grad_mode);
         ctx->save_for_backward({x, w.has_value() ? *w : Tensor(), pk.phi, pk.ba, f.has_value() ? *f : Tensor(), o.small});
         ctx->saved_data["iters"] = iters;
         ctx->saved_data["eps"] = eps;
@@ -255,7 +259,7 @@ struct MHCDynamicFn : public torch::autograd::Function<MHCDynamicFn> {
         float *bap = ba.data_ptr<float>();
         check("mhc_layer_bwd_dynamic",
               mhc_layer_bwd_dynamic(ptr(dy), dt(dy), ptr(x), dt(x), ptr(w), w.defined() ? dt(w) : 0, ptr(phi), dt(phi), bap,
-                                    bap + D, ptr(f), v.Hp, v.Ho, v.M, v.P, v.r, v.q, ptr(dx), ptr(df),
+                                    bap + D, ptr(f), v.Hp, v.Ho, v.M, v.P, v.r, v.q, v.sk, ptr(dx), ptr(df),
                                     dw.defined() ? dw.data_ptr<float>() : nullptr, dphi.data_ptr<float>(),
                                     dba.data_ptr<float>(), dba.data_ptr<float>() + D, B, n, C, iters, (float)eps,
                                     ws.data_ptr(), (size_t)ws.numel(), stream_of(x)));
@@ -267,7 +271,7 @@ struct MHCDynamicFn : public torch::autograd::Function<MHCDynamicFn> {
         const auto ad = ctx->saved_data["alpha_dtypes"].toIntVector();
         const auto bd = ctx->saved_data["b_dtypes"].toIntVector();
         const auto brs = ctx->saved_data["b_res_shape"].toIntVector();
-        variable_list out(15);
+        variable_list out(16);
         out[0] = to(dx, ctx->saved_data["x_dtype"].toInt());
         out[1] = (dw.defined() && w.defined()) ? to(dw, ctx->saved_data["w_dtype"].toInt()) : Tensor();
         out[2] = to(dphi.narrow(0, 0, n), pd[0]);
@@ -469,7 +473,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
              const Tensor &b_post, const Tensor &b_res, int64_t iters, double eps, c10::optional<at::ScalarType> out_dtype,
              const OptTensor &f_inject) {
               return MHCDynamicFn::apply(x, w, phi_pre, phi_post, phi_res, alpha_pre, alpha_post, alpha_res, b_pre, b_post,
-                                         b_res, iters, eps, out_dtype, f_inject);
+                                         b_res, iters, eps, out_dtype, f_inject, at::GradMode::is_enabled());
           },
           "mhc_layer_fwd_dynamic / mhc_layer_bwd_dynamic with autograd (reference bindings.cu:405-542)");
     m.def("mhc_layer_static",

@@ -84,18 +84,24 @@ static void test_dynamic(int B, int n, int C, int T) {
     float *y_ = dev_alloc((size_t)B * nC), *Hp_ = dev_alloc(B * n), *Ho_ = dev_alloc(B * n), *M_ = dev_alloc((size_t)B * n * n),
           *P_ = dev_alloc((size_t)B * D), *r_ = dev_alloc(B), *q_ = dev_alloc(B), *gx = dev_alloc((size_t)B * nC),
           *gw = dev_alloc(C), *gphi = dev_alloc((size_t)D * nC), *gb = dev_alloc(D), *ga = dev_alloc(3);
+    float *sk_ = dev_alloc(std::max<size_t>(mhc_layer_sinkhorn_state_floats(B, n, T), 1));
     const size_t wsb = mhc_layer_dynamic_workspace_bytes(B, n, C);
     void *ws; HIP_OK(hipMalloc(&ws, wsb + 256));
     MHC_OK_(mhc_layer_fwd_dynamic(dx_, MHC_F32, dw_, MHC_F32, dphi_, MHC_F32, dbias_, dalpha_, nullptr, y_, MHC_F32, Hp_,
-                                  Ho_, M_, P_, r_, q_, B, n, C, T, (float)eps, ws, wsb, nullptr));
-    MHC_OK_(mhc_layer_bwd_dynamic(ddy, MHC_F32, dx_, MHC_F32, dw_, MHC_F32, dphi_, MHC_F32, dbias_, dalpha_, nullptr, Hp_,
-                                  Ho_, M_, P_, r_, q_, gx, nullptr, gw, gphi, gb, ga, B, n, C, T, (float)eps, ws, wsb,
-                                  nullptr));
+                                  Ho_, M_, P_, r_, q_, sk_, B, n, C, T, (float)eps, ws, wsb, nullptr));
     HIP_OK(hipDeviceSynchronize());
     compare("y", y_, y); compare("H_pre", Hp_, Hp); compare("H_post", Ho_, Ho); compare("M", M_, M);
-    compare("dx", gx, dx); compare("dw", gw, dw); compare("dphi", gphi, dphi); compare("dbias", gb, dbias);
-    compare("dalpha", ga, dalpha);
-    for (float *p : {dx_, ddy, dw_, dphi_, dbias_, dalpha_, y_, Hp_, Ho_, M_, P_, r_, q_, gx, gw, gphi, gb, ga}) (void)hipFree(p);
+    // the backward once from the saved Sinkhorn denominators, once recomputing the iterations
+    for (const float *state : {(const float *)sk_, (const float *)nullptr}) {
+        printf("    backward %s\n", state ? "from the saved Sinkhorn state" : "recomputing the Sinkhorn iterations");
+        MHC_OK_(mhc_layer_bwd_dynamic(ddy, MHC_F32, dx_, MHC_F32, dw_, MHC_F32, dphi_, MHC_F32, dbias_, dalpha_, nullptr,
+                                      Hp_, Ho_, M_, P_, r_, q_, state, gx, nullptr, gw, gphi, gb, ga, B, n, C, T,
+                                      (float)eps, ws, wsb, nullptr));
+        HIP_OK(hipDeviceSynchronize());
+        compare("dx", gx, dx); compare("dw", gw, dw); compare("dphi", gphi, dphi); compare("dbias", gb, dbias);
+        compare("dalpha", ga, dalpha);
+    }
+    for (float *p : {dx_, ddy, dw_, dphi_, dbias_, dalpha_, y_, Hp_, Ho_, M_, P_, r_, q_, sk_, gx, gw, gphi, gb, ga}) (void)hipFree(p);
     (void)hipFree(ws);
 }
 

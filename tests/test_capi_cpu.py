@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(_lib.lib, name), f"{name} declared in mhc_hip.h but not exported"
         assert name in _lib._SIGNATURES, f"{name} has no ctypes signature in the binding"
-    assert _lib.lib.mhc_abi_version() == 1
+    assert _lib.lib.mhc_abi_version() == 2
 
 
 def test_status_strings():
@@ -66,8 +66,8 @@ def test_argument_validation_happens_before_any_launch():
     odd = P(a16.value + 4)
     fwd = lambda **kw: L.mhc_layer_fwd_dynamic(
         kw.get("x", a16), kw.get("xd", 0), a16, 0, a16, 0, a16, a16, None, kw.get("y", a16), kw.get("yd", 0),
-        a16, a16, a16, a16, a16, a16, kw.get("B", 2), kw.get("n", 4), kw.get("C", 8), kw.get("T", 20), 1e-6,
-        kw.get("ws", None), kw.get("wsb", 0), None)
+        a16, a16, a16, a16, a16, a16, kw.get("sk", None), kw.get("B", 2), kw.get("n", 4), kw.get("C", 8),
+        kw.get("T", 20), 1e-6, kw.get("ws", None), kw.get("wsb", 0), None)
     assert fwd(n=0) == 2 and fwd(n=33) == 2            # MHC_ERR_BAD_N
     assert fwd(B=0) == 3                               # MHC_ERR_BAD_SHAPE
     assert fwd(C=32768 + 8) == 3 and fwd(C=32768) == 6   # MHC_MAX_C
@@ -83,6 +83,10 @@ def test_argument_validation_happens_before_any_launch():
     assert fwd(xd=0, yd=1) == 4                        # fp32 in / bf16 out is not offered
     assert fwd(x=odd) == 5                             # MHC_ERR_MISALIGNED
     assert fwd() == 6                                  # MHC_ERR_WORKSPACE (none given)
+    # [B, iters, 2, NP] floats with NP = n rounded up to 4, 8, 16 or 32
+    state = L.mhc_layer_sinkhorn_state_floats
+    assert [state(3, n, 20) for n in (1, 4, 5, 8, 9, 16, 17, 32)] == [3 * 20 * 2 * k for k in (4, 4, 8, 8, 16, 16, 32, 32)]
+    assert state(3, 33, 20) == 0 and state(0, 4, 20) == 0 and state(3, 4, 0) == 0
     assert L.mhc_sinkhorn_knopp_fwd(a16, a16, 1, 129, 4, 3, 1e-8, None) == 3
     assert L.mhc_rmsnorm_fwd(None, 0, a16, 0, a16, None, 1, 8, 1e-5, None) == 1
 
@@ -102,7 +106,7 @@ def test_static_scratch_entry_point_checks_its_limit_before_any_launch():
     buf = (ctypes.c_char * 4096)()
     a16 = P((ctypes.addressof(buf) + 255) // 256 * 256)
     call = lambda B, n, C: L.mhc_layer_fwd_dynamic_static_scratch(
-        a16, 1, a16, 1, a16, 1, a16, a16, None, a16, 1, a16, a16, a16, a16, a16, a16, B, n, C, 20, 1e-6, None)
+        a16, 1, a16, 1, a16, 1, a16, a16, None, a16, 1, a16, a16, a16, a16, a16, a16, None, B, n, C, 20, 1e-6, None)
     assert call(*big) == 8          # MHC_ERR_SCRATCH_LIMIT
     assert call(0, 4, 64) == 3      # shape checks come first
 

@@ -40,7 +40,8 @@ def _forward(B, n, C, x, w, phi, bias, alpha, f, out_dtype, T, eps):
     f32 = dict(dtype=torch.float32, device="cuda")
     out = dict(y=torch.empty(B, n, C, dtype=out_dtype, device="cuda"), Hp=torch.empty(B, n, **f32),
                Ho=torch.empty(B, n, **f32), M=torch.empty(B, n, n, **f32), P=torch.empty(B, D, **f32),
-               r=torch.empty(B, **f32), q=torch.empty(B, **f32))
+               r=torch.empty(B, **f32), q=torch.empty(B, **f32),
+               sk=torch.empty(lib.mhc_layer_sinkhorn_state_floats(B, n, T), **f32))
     for t in out.values():
         t.fill_(float("nan"))
     ws = torch.empty(lib.mhc_layer_dynamic_workspace_bytes(B, n, C), dtype=torch.uint8, device="cuda")
@@ -48,7 +49,7 @@ def _forward(B, n, C, x, w, phi, bias, alpha, f, out_dtype, T, eps):
           lib.mhc_layer_fwd_dynamic(ptr(x), dtype_code(x), ptr(w), dtype_code(w), ptr(phi), dtype_code(phi),
                                     ptr(bias), ptr(alpha), ptr(f), ptr(out["y"]), dtype_code(out["y"]),
                                     ptr(out["Hp"]), ptr(out["Ho"]), ptr(out["M"]), ptr(out["P"]), ptr(out["r"]),
-                                    ptr(out["q"]), B, n, C, T, eps, ptr(ws), ws.numel(), _lib.stream_ptr(x.device)))
+                                    ptr(out["q"]), ptr(out["sk"]), B, n, C, T, eps, ptr(ws), ws.numel(), _lib.stream_ptr(x.device)))
     torch.cuda.synchronize()
     return {k: v.float().cpu() for k, v in out.items()}
 
@@ -92,6 +93,10 @@ def test_onepass_forward(B, n, C, G, waves, inject, out_dtype):
     _tune(K_WAVES, waves)
     one = _forward(B, n, C, x, w, phi, bias, alpha, f, out_dtype, T, eps)
 
+    # rows and columns n..NP-1 of the saved Sinkhorn denominators are padding nobody reads
+    NP = one["sk"].numel() // (B * T * 2)
+    for o in (one, two):
+        o["sk"] = o["sk"].reshape(B, T, 2, NP)[..., :n]
     for k, v in one.items():
         assert torch.isfinite(v).all(), k
     e = rel_err(one["y"], y_ref)
@@ -99,7 +104,7 @@ def test_onepass_forward(B, n, C, G, waves, inject, out_dtype):
     bad = (one["y"] - y_ref).abs() > 2e-2 * y_ref.abs() + 1e-2
     assert not bad.any()
     # same arithmetic up to summation order: the fp32 tensors saved for the backward agree closely
-    for k in ("Hp", "Ho", "M", "P", "r", "q"):
+    for k in ("Hp", "Ho", "M", "P", "r", "q", "sk"):
         e = rel_err(one[k], two[k])
         assert e <= 2e-5, f"{k} vs two-launch path: {e:.3e}"
     e = rel_err(one["y"], two["y"])

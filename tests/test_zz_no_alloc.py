@@ -28,12 +28,12 @@ def _run(entry, B, n, C, dtype, seed, T=20, eps=1e-6):
     f32 = dict(dtype=torch.float32, device="cuda")
     out = dict(y=torch.empty_like(x), Hp=torch.empty(B, n, **f32), Ho=torch.empty(B, n, **f32),
                M=torch.empty(B, n, n, **f32), P=torch.empty(B, D, **f32), r=torch.empty(B, **f32),
-               q=torch.empty(B, **f32))
+               q=torch.empty(B, **f32), sk=torch.empty(lib.mhc_layer_sinkhorn_state_floats(B, n, T), **f32))
     for t in out.values():
         t.fill_(float("nan"))
     common = (ptr(x), dtype_code(x), ptr(w), dtype_code(w), ptr(phi), dtype_code(phi), ptr(bias), ptr(alpha),
               None, ptr(out["y"]), dtype_code(out["y"]), ptr(out["Hp"]), ptr(out["Ho"]), ptr(out["M"]),
-              ptr(out["P"]), ptr(out["r"]), ptr(out["q"]), B, n, C, T, eps)
+              ptr(out["P"]), ptr(out["r"]), ptr(out["q"]), ptr(out["sk"]), B, n, C, T, eps)
     st = _lib.stream_ptr(x.device)
     if entry == "static_scratch":
         check("mhc_layer_fwd_dynamic_static_scratch", lib.mhc_layer_fwd_dynamic_static_scratch(*common, st))
@@ -42,6 +42,8 @@ def _run(entry, B, n, C, dtype, seed, T=20, eps=1e-6):
         ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
         check("mhc_layer_fwd_dynamic", lib.mhc_layer_fwd_dynamic(*common, ptr(ws), ws.numel(), st))
     torch.cuda.synchronize()
+    NP = out["sk"].numel() // (B * T * 2)  # rows and columns n..NP-1 of the saved state are padding
+    out["sk"] = out["sk"].reshape(B, T, 2, NP)[..., :n]
     return {k: v.float().cpu() for k, v in out.items()}
 
 
@@ -69,5 +71,5 @@ def test_static_scratch_refuses_shapes_beyond_its_array():
     from mhc._lib import ptr
     st = lib.mhc_layer_fwd_dynamic_static_scratch(ptr(x), 1, ptr(w), 1, ptr(phi), 1, ptr(bias), ptr(alpha), None,
                                                   ptr(x), 1, ptr(bias), ptr(bias), ptr(bias), ptr(bias),
-                                                  ptr(bias), ptr(bias), B, n, C, 20, 1e-6, None)
+                                                  ptr(bias), ptr(bias), None, B, n, C, 20, 1e-6, None)
     assert st == 8
