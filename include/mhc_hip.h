@@ -24,8 +24,9 @@
  *   M                 [B, n, n] fp32 Sinkhorn-normalised mixing matrix (static H: [n, n])
  *   P                 [B, D] fp32   rows of RMSNorm(x_flat) @ phi^T (before alpha and bias)
  *   r, q              [B]   fp32    r = rms of x_flat, q = rms of the aggregated stream
- *   sk_state          [B, iters, 2, NP] fp32  row and column denominators of every Sinkhorn iteration
- *                                   (NP = n rounded up to 4, 8, 16 or 32); optional, see below
+ *   sk_state          [B, iters + 1, 2, NP] fp32  row and column denominators of every Sinkhorn
+ *                                   iteration, then one slot the library keeps for itself (NP = n rounded
+ *                                   up to 4, 8, 16 or 32); optional, see below
  */
 #ifndef MHC_HIP_H
 #define MHC_HIP_H

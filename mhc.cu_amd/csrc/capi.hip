@@ -189,7 +189,7 @@ size_t mhc_layer_dynamic_workspace_bytes(int B, int n, int C) {
 
 size_t mhc_layer_sinkhorn_state_floats(int B, int n, int iters) {
     if (n < 1 || n > MHC_MAX_N || B < 1 || iters < 0) return 0;
-    return (size_t)B * iters * 2 * sinkhorn_state_np(n);
+    return (size_t)B * (iters + 1) * 2 * sinkhorn_state_np(n);
 }
 
 int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype, const void *phi,

@@ -5,6 +5,7 @@
 // (reference src/csrc/include/utils.cuh:50-126) and sinkhorn_knopp_forward_batched /
 // sinkhorn_knopp_forward_fused_exp (src/csrc/kernels/sinkhorn_knopp.cuh:986-1046, :461-519).
 #include "launchers.h"
+#include "phase_profiler.h"
 #include "sinkhorn_device.h"
 
 namespace mhc {
@@ -25,7 +26,7 @@ struct CoefArgs {
     // stream aggregate a = Hpre^T x (fp32 [B, C]) and its RMS q, from loads that fly under the Sinkhorn chain
     const bf16_t *x_agg;
     float *a_ws, *q;
-    float *sk_state;  // dynamic: [B][T][2][NP] Sinkhorn denominators kept for the backward, or nullptr
+    float *sk_state;  // dynamic: [B][T + 1][2][NP] Sinkhorn denominators kept for the backward, or nullptr
     bool precise;     // fp32 tier: IEEE divisions in the iterations whose denominators are kept
 };
 
@@ -106,6 +107,7 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     const int b = blockIdx.x;
     const int n = a.n, D = n * n + 2 * n;
     const bool dyn = a.Ppart != nullptr;
+    MHC_PHASE(kPhaseCoefFwdWide, b, 0);
     float al[3] = {0.f, 0.f, 0.f};
     // every wave fetches the split sums of x^2 itself (lane = split, KS <= 64): one load in flight
     // together with the partial dot products below instead of a chain of its own
@@ -117,69 +119,49 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
         al[0] = a.alpha[0]; al[1] = a.alpha[1]; al[2] = a.alpha[2];
     }
     const size_t pstride = (size_t)a.B * a.DP;
-    // logits d = tid + 256 m; the partial sums of all of a thread's logits are fetched together,
-    // all splits of a round at once (out-of-range slots alias element 0 and are discarded)
-    constexpr int MD = (NP * NP + 2 * NP + 255) / 256;
-    float psum[MD], bias[MD];
+    // Logits in fours: thread owns the 16-byte columns c4 = tid + 256 m of a partial row (DP / 4 of
+    // them: the rows are padded with zeros up to DP).  All splits of a column are requested at once;
+    // a wave whose columns lie beyond the row skips the round (the wave index is uniform).
+    constexpr int M4 = (NP * NP + 2 * NP + 1023) / 1024;
+    const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
+    float psum[M4][4], bias[M4][4];
 #pragma unroll
-    for (int m = 0; m < MD; m++) {
-        psum[m] = 0.f;
-        const int d = tid + 256 * m < D ? tid + 256 * m : 0;
-        const int grp = alpha_group(d, n);
-        bias[m] = *(grp == 0 ? a.b_pre + d : (grp == 1 ? a.b_post + (d - n) : a.b_res + (d - 2 * n)));
-    }
-    if (dyn) {
-        const float *pb = a.Ppart + (size_t)b * a.DP;
-        constexpr int KB = MD > 2 ? 24 : 32;  // splits per round: up to 120 / 64 loads in flight per thread
-        // per-lane offsets once, the split's row as a uniform base: one address computation per
-        // load instead of a select and a 64-bit multiply-add each
-        int dm[MD];
+    for (int m = 0; m < M4; m++)
 #pragma unroll
-        for (int m = 0; m < MD; m++) dm[m] = tid + 256 * m < D ? tid + 256 * m : 0;
-        for (int k0 = 0; k0 < a.KS; k0 += KB) {
-            float tv[MD][KB];
-#pragma unroll
-            for (int q = 0; q < KB; q++) {
-                const float *row = pb + (size_t)(k0 + q < a.KS ? k0 + q : 0) * pstride;  // uniform
-#pragma unroll
-                for (int m = 0; m < MD; m++) tv[m][q] = row[dm[m]];
-            }
-#pragma unroll
-            for (int m = 0; m < MD; m++)
-#pragma unroll
-                for (int q = 0; q < KB; q++) psum[m] += (tid + 256 * m < D && k0 + q < a.KS) ? tv[m][q] : 0.f;
-        }
-    }
-    float rinv = 0.f;
-    if (dyn) {
-        // PRECISE keeps the library routines; otherwise v_sqrt_f32 / v_rcp_f32 / v_exp_f32 (1 ulp)
-        const float ms = wave_allreduce_sum(ssq_l) / (float)a.nC + a.eps;
-        const float r = PRECISE ? sqrtf(ms) : __builtin_amdgcn_sqrtf(ms);
-        rinv = PRECISE ? 1.0f / r : fast_rcp(r);
-        if (tid == 0) a.r[b] = r;
-    }
-#pragma unroll
-    for (int m = 0; m < MD; m++) {
-        const int d = tid + 256 * m;
-        if (d < D) {
+        for (int j = 0; j < 4; j++) {
+            psum[m][j] = 0.f;
+            const int d0 = 4 * (tid + 256 * m) + j;
+            const int d = d0 < D ? d0 : 0;
             const int grp = alpha_group(d, n);
-            float t = bias[m];
-            if (dyn) {
-                const float p = psum[m] * rinv;
-                a.P[(size_t)b * D + d] = p;
-                t = al[grp] * p + bias[m];
-            }
-            lg[d] = t;
+            bias[m][j] = *(grp == 0 ? a.b_pre + d : (grp == 1 ? a.b_post + (d - n) : a.b_res + (d - 2 * n)));
         }
-    }
-    __syncthreads();
-    if (tid < n) {
-        const float hp = PRECISE ? sigmoidf_acc(lg[tid]) : sigmoid_fast(lg[tid]);
-        a.Hpre[b * n + tid] = hp;
-        a.Hpost[b * n + tid] = 2.0f * (PRECISE ? sigmoidf_acc(lg[n + tid]) : sigmoid_fast(lg[n + tid]));
-        if constexpr (AGG) hp_s[tid] = hp;
-    } else if (AGG && tid < 32) {
-        hp_s[tid] = 0.f;
+    if (dyn) {
+        const float4 *pb = reinterpret_cast<const float4 *>(a.Ppart + (size_t)b * a.DP);
+        const int q4 = a.DP / 4;
+        constexpr int KB = 24;  // splits per round: at most 48 loads in flight per thread
+        int cm[M4];
+#pragma unroll
+        for (int m = 0; m < M4; m++) cm[m] = tid + 256 * m < q4 ? tid + 256 * m : 0;
+        for (int k0 = 0; k0 < a.KS; k0 += KB) {
+            float4 tv[M4][KB];
+#pragma unroll
+            for (int m = 0; m < M4; m++) {
+                if (256 * m + 64 * wave_u >= q4) continue;
+#pragma unroll
+                for (int q = 0; q < KB; q++)
+                    tv[m][q] = pb[(size_t)(k0 + q < a.KS ? k0 + q : 0) * (pstride / 4) + cm[m]];
+            }
+#pragma unroll
+            for (int m = 0; m < M4; m++) {
+                if (256 * m + 64 * wave_u >= q4) continue;
+#pragma unroll
+                for (int q = 0; q < KB; q++) {
+                    const bool ok = k0 + q < a.KS;
+                    psum[m][0] += ok ? tv[m][q].x : 0.f; psum[m][1] += ok ? tv[m][q].y : 0.f;
+                    psum[m][2] += ok ? tv[m][q].z : 0.f; psum[m][3] += ok ? tv[m][q].w : 0.f;
+                }
+            }
+        }
     }
     // AGG: this thread's chunk of every stream is requested now and consumed behind the Sinkhorn
     // chain (whose barriers also publish hp_s); streams >= n alias stream 0 and meet Hpre = 0
@@ -191,16 +173,53 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
 #pragma unroll
         for (int i = 0; i < NS; i++) xr[i].load(xb + (size_t)(i < n ? i : 0) * C);
     }
+    MHC_PHASE(kPhaseCoefFwdWide, b, 1);
+    float rinv = 0.f;
+    if (dyn) {
+        // PRECISE keeps the library routines; otherwise v_sqrt_f32 / v_rcp_f32 / v_exp_f32 (1 ulp)
+        const float ms = wave_allreduce_sum(ssq_l) / (float)a.nC + a.eps;
+        const float r = PRECISE ? sqrtf(ms) : __builtin_amdgcn_sqrtf(ms);
+        rinv = PRECISE ? 1.0f / r : fast_rcp(r);
+        if (tid == 0) a.r[b] = r;
+    }
+#pragma unroll
+    for (int m = 0; m < M4; m++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int d = 4 * (tid + 256 * m) + j;
+            if (d < D) {
+                const int grp = alpha_group(d, n);
+                float t = bias[m][j];
+                if (dyn) {
+                    const float p = psum[m][j] * rinv;
+                    a.P[(size_t)b * D + d] = p;
+                    t = al[grp] * p + bias[m][j];
+                }
+                lg[d] = t;
+            }
+        }
+    __syncthreads();
+    if (tid < n) {
+        const float hp = PRECISE ? sigmoidf_acc(lg[tid]) : sigmoid_fast(lg[tid]);
+        a.Hpre[b * n + tid] = hp;
+        a.Hpost[b * n + tid] = 2.0f * (PRECISE ? sigmoidf_acc(lg[n + tid]) : sigmoid_fast(lg[n + tid]));
+        if constexpr (AGG) hp_s[tid] = hp;
+    } else if (AGG && tid < 32) {
+        hp_s[tid] = 0.f;
+    }
     const int r0 = SK::row(tid), c0 = SK::col0(tid);
     float E[SK::EPL], u, v[SK::EPL];
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         E[e] = (r0 < n && c0 + e < n) ? (PRECISE ? expf(lg[2 * n + r0 * n + c0 + e]) : exp_fast(lg[2 * n + r0 * n + c0 + e])) : 0.f;
+    MHC_PHASE(kPhaseCoefFwdWide, b, 2);
     SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
+    MHC_PHASE(kPhaseCoefFwdWide, b, 3);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
         if (r0 < n && c0 + e < n) a.M[(size_t)b * n * n + r0 * n + c0 + e] = u * E[e] * v[e];
-    if (a.sk_state) SK::save_state(sk_s, a.T, a.sk_state + (size_t)b * SK::state_floats(a.T), tid);
+    if (a.sk_state) SK::save_state(sk_s, a.T, a.sk_state + (size_t)b * SK::state_floats(a.T), tid, u, v);
+    MHC_PHASE(kPhaseCoefFwdWide, b, 4);
     if constexpr (AGG) {
         __syncthreads();  // hp_s (with zero iterations the Sinkhorn step has no barrier of its own)
         float acc[8], ssq = 0.f;
@@ -222,6 +241,7 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
         ssq = block_allreduce_sum<256>(ssq, red_s);
         if (tid == 0) a.q[b] = sqrtf(ssq / (float)C + a.eps);
     }
+    MHC_PHASE(kPhaseCoefFwdWide, b, 5);
 }
 
 hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int DP,

@@ -43,9 +43,9 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
                            const float *b_res, float *Hpre, float *Hpost, float *M, float *P,
                            float *r, int B, int n, int nC, int T, float eps, bool precise,
                            const void *x_agg, float *a_ws, float *q, float *sk_state, hipStream_t stream);
-// sk_state (dynamic H, optional): [B][T][2][NP] floats, NP = sinkhorn_state_np(n): the row and column
-// denominators of every Sinkhorn iteration, kept for the backward call (which otherwise recomputes
-// the forward iterations to get them).
+// sk_state (dynamic H, optional): [B][T + 1][2][NP] floats, NP = sinkhorn_state_np(n): the row and column
+// denominators of every Sinkhorn iteration and, in slot T for n > 8, the final row and column scalings,
+// kept for the backward call (which otherwise recomputes the forward iterations to get them).
 inline int sinkhorn_state_np(int n) { return n <= 4 ? 4 : (n <= 8 ? 8 : (n <= 16 ? 16 : 32)); }
 // x_agg != nullptr (only where coef_fwd_aggregates() holds): the launch also writes the stream
 // aggregate a = Hpre^T x (a_ws, fp32 [B, C]) and its RMS q, which launch_mix_fwd then takes as given

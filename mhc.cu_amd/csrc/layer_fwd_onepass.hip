@@ -38,7 +38,7 @@ struct OnePassArgs {
     float *Hpre, *Hpost, *M, *P, *r, *q;
     int w_bf16, B, n, C, T, G;
     float eps;
-    float *sk_state;  // [B][T][2][NP] Sinkhorn denominators kept for the backward, or nullptr
+    float *sk_state;  // [B][T + 1][2][NP] Sinkhorn denominators kept for the backward, or nullptr
 };
 
 constexpr int kOpMaxG = 16;      // samples per workgroup: the columns of one 16-wide tile

@@ -26,7 +26,7 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 struct BwdReduceArgs {
     const void *dy, *x, *w, *f_inject;
     const float *Hpre, *Hpost, *M, *q, *P, *r, *alpha, *b_res;
-    const float *sk_state;  // dynamic: Sinkhorn denominators saved by the forward ([B][T][2][NP]) or nullptr
+    const float *sk_state;  // dynamic: Sinkhorn denominators saved by the forward ([B][T + 1][2][NP]) or nullptr
     BwdCoefOut out;
     int hstride, w_bf16, B, n, C, T, DP;
     float eps;
@@ -892,6 +892,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
     const int b = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x, lane = tid & 63;
     const bool w0 = tid < 64;
     const bool inject = a.f_inject != nullptr;
+    MHC_PHASE(kPhaseCoefBwdWide, b, 0);
     const float qinv = inject ? 0.f : (PRECISE ? 1.0f / a.q[b] : fast_rcp(a.q[b]));
     if (tid < 32) {
         hp_s[tid] = tid < n ? a.Hpre[(size_t)b * a.hstride + tid] : 0.f;
@@ -934,9 +935,10 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
             pres[e] = ok ? pres[e] : 0.f;
             E[e] = ok ? (PRECISE ? expf(al2 * pres[e] + bres[e]) : exp_fast(al2 * pres[e] + bres[e])) : 0.f;
         }
-        if (a.sk_state) SK::template load_state<PRECISE>(a.sk_state + (size_t)b * SK::state_floats(a.T), u, v, a.T, sk_s, tid);
+        if (a.sk_state) SK::load_state(a.sk_state + (size_t)b * SK::state_floats(a.T), u, v, a.T, sk_s, tid);
         else SK::template forward<PRECISE>(E, u, v, n, a.T, a.eps, sk_s, tid);
     }
+    MHC_PHASE(kPhaseCoefBwdWide, b, 1);
     {
         float acc[EPT];
 #pragma unroll
@@ -968,28 +970,37 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         }
     }
     __syncthreads();
-    if (tid < 32) {          // A1[j], A2[j]
-        float a1 = 0.f, a2 = 0.f;
-#pragma unroll 8
-        for (int k = 0; k < 32; k++) { a1 += ho_s[k] * W_s[k * 33 + tid]; a2 += hp_s[k] * X_s[k * 33 + tid]; }
-        vec_s[32 + tid] = a1; vec_s[64 + tid] = a2;
-    } else if (tid < 64) {   // dHpost[i]
-        const int i = tid - 32;
-        float dh = 0.f;
-        if (inject) {
-            dh = W_s[i * 33];
-        } else {
-#pragma unroll 8
-            for (int j = 0; j < 32; j++) dh += hp_s[j] * W_s[i * 33 + j];
-            dh *= qinv;
+    MHC_PHASE(kPhaseCoefBwdWide, b, 2);
+    {
+        // dHpost[i] = sum_j Hpre[j] W1[i][j] / q,  A1[i] = sum_j Hpost[j] W1[j][i],  A2[i] = sum_j Hpre[j] XX[j][i]:
+        // thread (i, seg) = (tid / 8, tid % 8) adds four terms of each, the 8 lanes of i finish the sums
+        const int i = tid >> 3, seg = tid & 7;
+        float dh = 0.f, a1 = 0.f, a2 = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int j = seg * 4 + k;
+            const float hpj = hp_s[j], hoj = ho_s[j];
+            dh += hpj * W_s[i * 33 + j];
+            a1 += hoj * W_s[j * 33 + i];
+            a2 += hpj * X_s[j * 33 + i];
         }
-        vec_s[i] = dh;
+        auto sum8 = [](float x) {
+            x += dpp_mov<kDppQuadXor1>(x);
+            x += dpp_mov<kDppQuadXor2>(x);
+            x += dpp_mov<kDppRowHalfMirror>(x);  // lane i <-> 7 - i: the other quad of the 8 lanes
+            return x;
+        };
+        dh = sum8(dh); a1 = sum8(a1); a2 = sum8(a2);
+        if (seg == 0) {
+            vec_s[i] = inject ? W_s[i * 33] : dh * qinv;
+            vec_s[32 + i] = a1;
+            vec_s[64 + i] = a2;
+        }
     }
     __syncthreads();
     float s1 = 0.f;
-    if (!inject) {
-#pragma unroll 8
-        for (int i = 0; i < 32; i++) s1 += ho_s[i] * vec_s[i];
+    if (!inject) {  // every wave on its own: lanes 0 .. 31 hold one term each
+        s1 = wave_allreduce_sum(lane < 32 ? ho_s[lane] * vec_s[lane] : 0.f);
         s1 = s1 / qinv;  // vec_s holds W1 Hpre / q
     }
 
@@ -1018,6 +1029,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         dpw.put(lane, dtp * al0 * rinv); dpw.put(n + lane, dto * al1 * rinv);
         S0 = dtp * Pb[lane]; S1 = dto * Pb[n + lane];
     }
+    MHC_PHASE(kPhaseCoefBwdWide, b, 3);
     // exact Sinkhorn backward (the forward recompute ran above), the matrix spread over all 256 threads
     float d[SK::EPL];
 #pragma unroll
@@ -1026,6 +1038,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         d[e] = (r0 < n && c < n) ? M_s[r0 * 33 + c] : 0.f;
     }
     SK::template backward<PRECISE>(E, d, u, v, a.T, sk_s, tid);
+    MHC_PHASE(kPhaseCoefBwdWide, b, 4);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {
         const int c = c0 + e;
@@ -1046,6 +1059,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         }
     }
     dpw.pad(D, tid, 256);
+    MHC_PHASE(kPhaseCoefBwdWide, b, 5);
 }
 
 // =============================================================================================

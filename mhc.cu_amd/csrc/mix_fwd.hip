@@ -140,7 +140,7 @@ struct LayerFwdArgs {
     float *Hpre, *Hpost, *M, *P, *r, *q;  // outputs (static: shared [n], [n], [n,n]; may be null)
     int KS, DP, w_bf16, B, n, C, T;
     float eps;
-    float *sk_state;  // dynamic: [B][T][2][NP] Sinkhorn denominators kept for the backward, or nullptr
+    float *sk_state;  // dynamic: [B][T + 1][2][NP] Sinkhorn denominators kept for the backward, or nullptr
 };
 
 constexpr int kFwdStaggerMinB = 512;  // two or more workgroups per CU

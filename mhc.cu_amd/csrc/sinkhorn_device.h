@@ -124,7 +124,8 @@ template <int NP> struct SkSmall {
             }
         }
     }
-    __host__ __device__ static constexpr int state_floats(int T) { return 2 * T * NP; }
+    // one footprint for every layout: [T + 1][2][NP] (slot T is used by SkWg only)
+    __host__ __device__ static constexpr int state_floats(int T) { return 2 * (T + 1) * NP; }
 
     // d: in = dL/dM, out = dL/dE.  m: the final iterate from forward (destroyed).  The reverse
     // sweep rebuilds the iterates it needs by undoing the scalings with the saved denominators
@@ -287,43 +288,52 @@ template <int NP> struct SkWg {
         }
     }
 
-    // Copies the denominators that forward() left in LDS to global memory for the backward call:
-    // st[(t * 2 + 0) * NP + a] = rho_t[a], st[(t * 2 + 1) * NP + a] = s_t[a].  Every thread calls it.
-    __device__ static __forceinline__ void save_state(const float *lds, int T, float *st, int tid) {
+    // Copies what forward() left behind to global memory for the backward call:
+    // st[(t * 2 + 0) * NP + a] = rho_t[a], st[(t * 2 + 1) * NP + a] = s_t[a] for t < T, and in slot T
+    // the final scalings u[a], v[a] (which the reverse sweep starts from).  Every thread calls it.
+    __device__ static __forceinline__ void save_state(const float *lds, int T, float *st, int tid, float u,
+                                                      const float (&v)[EPL]) {
         const float *rho = lds + kTile + 2 * NP, *s = rho + T * NP;
         for (int e = tid; e < T * NP; e += 256) {
             const int t = e / NP, a = e % NP;
             st[(t * 2) * NP + a] = rho[e];
             st[(t * 2 + 1) * NP + a] = s[e];
         }
+        if (tid % LPR == 0) st[2 * T * NP + row(tid)] = u;
+        if (tid < LPR) {
+#pragma unroll
+            for (int e = 0; e < EPL; e++) st[(2 * T + 1) * NP + col0(tid) + e] = v[e];
+        }
     }
-    // The inverse: puts saved denominators where backward() expects them and rebuilds the final
-    // scalings u, v with the recurrence of forward() (u <- u / rho_t, v <- v / s_t), so that
-    // backward() can follow without the forward recompute.  Every thread calls it; ends on a barrier.
-    template <bool PRECISE = true>
+    // The inverse: puts the saved denominators where backward() expects them and hands back the final
+    // scalings, so that backward() can follow without the forward recompute.  All loads are requested
+    // before the first is used.  Every thread calls it; ends on a barrier.
     __device__ static __forceinline__ void load_state(const float *st, float &u, float (&v)[EPL], int T, float *lds,
                                                       int tid) {
         float *rho = lds + kTile + 2 * NP, *s = rho + T * NP;
-        for (int e = tid; e < T * NP; e += 256) {
-            const int t = e / NP, a = e % NP;
-            rho[e] = st[(t * 2) * NP + a];
-            s[e] = st[(t * 2 + 1) * NP + a];
+        const int total = 2 * T * NP;  // [t][rho | s][a]
+        u = st[total + row(tid)];
+#pragma unroll
+        for (int e = 0; e < EPL; e++) v[e] = st[total + NP + col0(tid) + e];
+        for (int e0 = 0; e0 < total; e0 += 256 * 8) {
+            float tv[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const int e = e0 + tid + 256 * k;
+                tv[k] = st[e < total ? e : 0];
+            }
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const int e = e0 + tid + 256 * k;
+                if (e < total) {
+                    const int t = e / (2 * NP), a = e % NP;
+                    ((e / NP) & 1 ? s : rho)[t * NP + a] = tv[k];
+                }
+            }
         }
         __syncthreads();
-        const int a = row(tid), b0 = col0(tid);
-        u = 1.0f;
-#pragma unroll
-        for (int e = 0; e < EPL; e++) v[e] = 1.0f;
-        for (int t = 0; t < T; t++) {
-            const float rr = rho[t * NP + a];
-            u = PRECISE ? u / rr : u * fast_rcp(rr);
-            float sc[EPL];
-            ld_vec(s + t * NP + b0, sc);
-#pragma unroll
-            for (int e = 0; e < EPL; e++) v[e] = PRECISE ? v[e] / sc[e] : v[e] * fast_rcp(sc[e]);
-        }
     }
-    __host__ __device__ static constexpr int state_floats(int T) { return 2 * T * NP; }
+    __host__ __device__ static constexpr int state_floats(int T) { return 2 * (T + 1) * NP; }
 
     // d: in = dL/dM, out = dL/dE.  E, u, v, LDS contents: as left by forward() (u and v are
     // destroyed).

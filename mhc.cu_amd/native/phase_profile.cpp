@@ -1,7 +1,8 @@
 // Prints the in-kernel phase timeline of the fused forward kernel and of the slab backward kernel.
 //
-//   phase_profile [--batch B] [--hidden C] [--expansion n]          (n <= 8, C % 8 == 0, bf16;
-//                                                                    n > 4: projection backward instead of the slab kernel)
+//   phase_profile [--batch B] [--hidden C] [--expansion n]          (C % 8 == 0, bf16;
+//                                                                    n > 4: projection backward instead of the slab kernel;
+//                                                                    n > 8: the two coefficient kernels only)
 //
 // Links libmhc_hip_profile.so (python mhc.cu_amd/build.py --profile), the build of the library with
 // csrc/phase_profiler.h compiled in.  Counterpart of the reference's HostProfiler::print_summary
@@ -80,7 +81,7 @@ int main(int argc, char **argv) {
         else if (is("--tune") && i + 2 < argc) { mhc_tuning_set(atoi(argv[i + 1]), atoi(argv[i + 2])); i += 2; }
         else { fprintf(stderr, "unknown argument %s\n", argv[i]); return 2; }
     }
-    if (n > 8 || C % 8) { fprintf(stderr, "the instrumented kernels serve n <= 8 with C %% 8 == 0\n"); return 2; }
+    if (n > 32 || C % 8) { fprintf(stderr, "the instrumented kernels serve n <= 32 with C %% 8 == 0\n"); return 2; }
     const size_t BnC = (size_t)B * n * C, nC = (size_t)n * C, D = (size_t)n * n + 2 * n;
     std::mt19937 g(0);
     void *x = dev_bf16(BnC, 1.f, g), *dy = dev_bf16(BnC, 1.f, g), *phi = dev_bf16(D * nC, 0.02f, g), *w = dev_bf16(C, 0.f, g);
@@ -100,6 +101,15 @@ int main(int argc, char **argv) {
         HIP_OK(hipDeviceSynchronize());
     }
     printf("phase profile: dynamic H, bf16, B=%d C=%d n=%d (last of 3 warm calls)\n", B, C, n);
+    if (n > 8) {
+        summary("coefficient forward kernel (n > 8), one workgroup per sample", 7, std::min(B, 4096),
+                {"split-K partial sums of the projection arrive", "logits, activations, stream tile requested",
+                 "Sinkhorn iterations", "M and Sinkhorn state stores issued", "stream tile arrives, aggregate, RMS"}, true);
+        summary("coefficient backward kernel (n > 8), one workgroup per sample", 8, std::min(B, 4096),
+                {"inputs requested, Sinkhorn state loaded (or recomputed)", "Gram parts arrive, summed, parked",
+                 "dHpre / dHpost / s1", "Sinkhorn reverse sweep", "dt / dP stores issued"}, true);
+        return 0;
+    }
     if (n <= 4 && (n * C) % 64 == 0) {
         const int G = std::min(16, std::max(1, (B + 255) / 256));
         summary("one-launch forward kernel, one workgroup per G samples (wave 0 of each)", 6, std::min((B + G - 1) / G, 4096),

@@ -83,10 +83,10 @@ def test_argument_validation_happens_before_any_launch():
     assert fwd(xd=0, yd=1) == 4                        # fp32 in / bf16 out is not offered
     assert fwd(x=odd) == 5                             # MHC_ERR_MISALIGNED
     assert fwd() == 6                                  # MHC_ERR_WORKSPACE (none given)
-    # [B, iters, 2, NP] floats with NP = n rounded up to 4, 8, 16 or 32
+    # [B, iters + 1, 2, NP] floats with NP = n rounded up to 4, 8, 16 or 32
     state = L.mhc_layer_sinkhorn_state_floats
-    assert [state(3, n, 20) for n in (1, 4, 5, 8, 9, 16, 17, 32)] == [3 * 20 * 2 * k for k in (4, 4, 8, 8, 16, 16, 32, 32)]
-    assert state(3, 33, 20) == 0 and state(0, 4, 20) == 0 and state(3, 4, 0) == 0
+    assert [state(3, n, 20) for n in (1, 4, 5, 8, 9, 16, 17, 32)] == [3 * 21 * 2 * k for k in (4, 4, 8, 8, 16, 16, 32, 32)]
+    assert state(3, 33, 20) == 0 and state(0, 4, 20) == 0 and state(3, 4, 0) == 3 * 2 * 4 and state(3, 4, -1) == 0
     assert L.mhc_sinkhorn_knopp_fwd(a16, a16, 1, 129, 4, 3, 1e-8, None) == 3
     assert L.mhc_rmsnorm_fwd(None, 0, a16, 0, a16, None, 1, 8, 1e-5, None) == 1
 

@@ -94,9 +94,9 @@ def test_onepass_forward(B, n, C, G, waves, inject, out_dtype):
     one = _forward(B, n, C, x, w, phi, bias, alpha, f, out_dtype, T, eps)
 
     # rows and columns n..NP-1 of the saved Sinkhorn denominators are padding nobody reads
-    NP = one["sk"].numel() // (B * T * 2)
+    NP = one["sk"].numel() // (B * (T + 1) * 2)
     for o in (one, two):
-        o["sk"] = o["sk"].reshape(B, T, 2, NP)[..., :n]
+        o["sk"] = o["sk"].reshape(B, T + 1, 2, NP)[:, :T, :, :n]
     for k, v in one.items():
         assert torch.isfinite(v).all(), k
     e = rel_err(one["y"], y_ref)

@@ -52,8 +52,8 @@ def _fwd_bwd(B, n, C, dtype, T, eps, seed, with_state):
     out = {k: v.float().cpu() for k, v in out.items()}
     out["M"], out["y"] = M.cpu(), y.float().cpu()
     if with_state and T > 0:
-        NP = sk.numel() // (B * T * 2)
-        out["sk"] = sk.reshape(B, T, 2, NP)[..., :n].cpu()
+        NP = sk.numel() // (B * (T + 1) * 2)
+        out["sk"] = sk.reshape(B, T + 1, 2, NP)[:, :T, :, :n].cpu()
         out["P"] = P.cpu()  # rows of RMSNorm(x_flat) @ phi^T: the logits are alpha * P + b
         out["b_res"], out["alpha_res"] = p["b_res"], float(p["alpha_res"])
     return out

@@ -42,8 +42,8 @@ def _run(entry, B, n, C, dtype, seed, T=20, eps=1e-6):
         ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
         check("mhc_layer_fwd_dynamic", lib.mhc_layer_fwd_dynamic(*common, ptr(ws), ws.numel(), st))
     torch.cuda.synchronize()
-    NP = out["sk"].numel() // (B * T * 2)  # rows and columns n..NP-1 of the saved state are padding
-    out["sk"] = out["sk"].reshape(B, T, 2, NP)[..., :n]
+    NP = out["sk"].numel() // (B * (T + 1) * 2)  # rows and columns n..NP-1 of the saved state are padding
+    out["sk"] = out["sk"].reshape(B, T + 1, 2, NP)[:, :T, :, :n]
     return {k: v.float().cpu() for k, v in out.items()}
 
 
