@@ -20,6 +20,13 @@
 
 namespace mhc {
 
+// a * b + c with the product rounded before the sum (the compiler fuses the plain expression)
+__device__ __forceinline__ float mul_add_unfused(float a, float b, float c) {
+#pragma clang fp contract(off)
+    const float t = a * b;
+    return t + c;
+}
+
 // =============================================================================================
 // SkSmall
 // =============================================================================================
@@ -185,9 +192,10 @@ template <int NP> struct SkSmall {
 // (DPP, v_permlane*_swap) and then across the 4 waves through a double-buffered LDS slot (one
 // barrier per iteration; keeping a transposed copy of the gradient as well needs two barriers and
 // measured 50 % slower); the scalings are unwound with the saved denominators (u *= rho, v *= s)
-// instead of storing iterates.  Measured against float64 the round-off of the backward grows by
-// about 2e-8 per iteration (5e-7 at the usual 20); the accepted iteration counts keep it below
-// 1e-5.  Every thread of the workgroup must call forward/backward; `lds` must be 16-byte aligned.
+// instead of storing iterates.  Against float64 the backward stays at ~2e-7 for every iteration count
+// once the forward's denominators are computed without a fused multiply-add (see forward()); with it
+// the error grew by ~2e-8 per iteration.  Every thread of the workgroup must call forward/backward;
+// `lds` must be 16-byte aligned.
 // =============================================================================================
 template <int NP> struct SkWg {
     static_assert(NP == 16 || NP == 32, "SkWg handles 16x16 and 32x32 tiles");
@@ -271,7 +279,11 @@ template <int NP> struct SkWg {
 #pragma unroll
             for (int e = 0; e < EPL; e++) p += E[e] * v[e];
             p = seg_allreduce(p);
-            const float rr = live ? u * p + eps : 1.0f;
+            // fp32 tier: product and sum rounded separately.  With a fused multiply-add the converged
+            // denominators settle one ulp off 1 on some rows and columns (u and v keep drifting against
+            // each other), and the reverse sweep, which divides by them in every iteration, drifts away
+            // from the float64 result by ~2e-8 per iteration; rounded separately they settle at exactly 1.
+            const float rr = live ? (PRECISE ? mul_add_unfused(u, p, eps) : u * p + eps) : 1.0f;
             u = PRECISE ? u / rr : u * fast_rcp(rr);
             if (head) { rho[t * NP + a] = rr; ub[a] = u; }
             __syncthreads();
@@ -280,7 +292,7 @@ template <int NP> struct SkWg {
 #pragma unroll
             for (int e = 0; e < EPL; e++) q += ET[e] * uc[e];
             q = seg_allreduce(q);
-            const float sc = live ? vc * q + eps : 1.0f;
+            const float sc = live ? (PRECISE ? mul_add_unfused(vc, q, eps) : vc * q + eps) : 1.0f;
             vc = PRECISE ? vc / sc : vc * fast_rcp(sc);
             if (head) { s[t * NP + a] = sc; vb[a] = vc; }
             __syncthreads();

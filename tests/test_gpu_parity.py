@@ -137,6 +137,22 @@ def test_dynamic_fp32_vs_oracle(B, n, C, inject):
         _check(g[k], ref, "fp32", "d" + k)
 
 
+@pytest.mark.parametrize("n", [16, 32])
+def test_sinkhorn_backward_round_off_does_not_grow_with_the_iteration_count(n):
+    """n > 8, fp32: the gradient of the Sinkhorn logits stays at a few 1e-7 of the float64 oracle from
+    20 to 256 iterations (it grew by ~2e-8 per iteration while the forward formed its denominators
+    with a fused multiply-add; tests/test_sinkhorn_roundoff_model.py holds the CPU model)."""
+    B, C, eps = 2, 8, 1e-6
+    for T in (20, 256):
+        x, dy, f, p = nm.make_dynamic_inputs(B, n, C, with_f=False)
+        p = _rand_params(p, n, C)
+        _, g_ref = nm.mhc_dynamic_fwd_bwd(x, p, dy, T, eps, dtype=torch.float64)
+        _, g = hip_dynamic(x, p, dy, T, eps)
+        for k in ("b_res", "phi_res"):
+            e = rel_err(g[k], g_ref[k])
+            assert e <= 1e-6, f"d{k} at T={T}: rel err {e:.3e}"
+
+
 @pytest.mark.parametrize("B,n,C,T", [(2, 4, 16, 256), (3, 8, 16, 256), (2, 5, 16, 256), (2, 16, 8, 256), (2, 32, 8, 256),
                                      (3, 8, 64, 60)])
 @pytest.mark.parametrize("dyn", [True, False])
