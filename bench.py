@@ -31,9 +31,24 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes of one step (all launches, graph-less run), from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE summed over the step's kernels and scaled by what the same counters read for
-# `--copy-calibration` (a 64 MiB copy).  Filled from the committed counter summaries; None where
-# no counter run exists for the configuration.
-MEASURED_TRAFFIC_BYTES = {"c1": 13275949, "c2": 42677933, "c3": 248312520, "c4": 75948103, "c5": 549083493}
+# `--copy-calibration` (a 64 MiB copy).  Filled from the committed counter summary
+# (profiles/hbm_traffic_counters.txt); `commit` is the revision of the kernels the counters ran on.
+MEASURED_TRAFFIC = {
+    "commit": "e3e99d6",
+    "bytes": {"c1": 13275949, "c2": 42677933, "c3": 248312520, "c4": 75948103, "c5": 549083493},
+}
+
+# The kernel with the largest share of a step's device time, from the committed kernel-trace summaries
+# (profiles/layer_step_<config>.txt): average duration per dispatch and the HBM bytes the algorithm
+# needs that kernel to move (its own inputs and outputs once; for the split projections the partial
+# sums are not counted).
+PROFILED_DOMINANT = {
+    "c1": dict(kernel="layer_fwd_small_kernel<float,float,4,4,2>", us=6.71, bytes=2 * 4 * 320 * 4 * 1280),
+    "c2": dict(kernel="bwd_slab_kernel<bf16>", us=10.22, bytes=3 * 2 * 320 * 4 * 1280 + 2 * 24 * 5120 + 4 * 24 * 5120),
+    "c3": dict(kernel="bwd_slab_kernel<bf16>", us=25.32, bytes=3 * 2 * 1280 * 4 * 2560 + 2 * 24 * 10240 + 4 * 24 * 10240),
+    "c4": dict(kernel="proj_bwd_mfma_kernel<1,1,true>", us=11.81, bytes=2 * 2 * 256 * 8 * 1280 + 2 * 80 * 10240 + 4 * 80 * 10240),
+    "c5": dict(kernel="dphi_large_kernel<9,true>", us=36.23, bytes=2 * 128 * 40960 + 4 * 1088 * 40960),
+}
 
 CONFIGS = {
     "c1": dict(kind="static", B=320, n=4, C=1280, dtype="f32", bwd=False),
@@ -61,6 +76,15 @@ def algorithmic_bytes(cfg, view):
     if cfg["bwd"]:
         bwd = s * (2 * BnC + fvec) + phi + s * (BnC + fvec) + 2 * phi  # dphi fp32 = 2x bf16 phi bytes
     return fwd, bwd
+
+
+def dominant_kernel(config):
+    """roofline.dominant: the step's largest kernel as profiled (not re-timed here: HIP events see whole
+    entry points, not the launches inside them)."""
+    d = dict(PROFILED_DOMINANT[config])
+    d["frac"] = d["bytes"] / (d["us"] * 1e-6) / 1e9 / HBM_PEAK_GBS
+    d["source"] = f"profiles/layer_step_{config}.txt"
+    return d
 
 
 def synthetic_inputs(torch, cfg, with_f):
@@ -479,7 +503,9 @@ def main():
                    "view": a.view, "launch": mode, "cache": "warm (back-to-back steps)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.config) if a.view == "L" else None,
+                     "traffic": MEASURED_TRAFFIC["bytes"].get(a.config) if a.view == "L" else None,
+                     "traffic_commit": MEASURED_TRAFFIC["commit"],
+                     "dominant": dominant_kernel(a.config),
                      "kernel": "whole step (all launches of one forward+backward)",
                      "algorithmic_bytes": alg, "device_us": dev_step,
                      "fwd": {"algorithmic_bytes": fwd_b, "device_us": dev_fwd,

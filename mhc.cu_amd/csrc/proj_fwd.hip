@@ -255,8 +255,9 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
 //   P chunks of global loads are in flight per thread (register FIFO) ahead of the chunk being
 //   multiplied; LDS is double-buffered, one barrier per chunk.
 // Workgroups that read the same K slab sit on the same XCD (workgroup id modulo 8 selects the
-// XCD): the slab of x is pulled into that L2 once and the other row groups hit it there.
-// grid.x = 8 * groups * sample_groups * ceil(KS / 8)
+// XCD, every XCD takes the same number of consecutive work items): the slab of x is pulled into that
+// L2 once and the other row groups hit it there.
+// grid.x = groups * sample_groups * KS rounded up to a multiple of 8
 // --------------------------------------------------------------------------------------------
 constexpr int kWideLd = 72;  // LDS row stride in bf16 elements: 128 data bytes + 16 pad
 
@@ -276,11 +277,15 @@ __global__ __launch_bounds__(256) void proj_fwd_wide_kernel(const bf16_t *__rest
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = lane & 31, kh = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int group = slot % groups;
-    const int sg = (slot / groups) % sgroups;
-    const int ks = (slot / (groups * sgroups)) * 8 + xcd;
-    if (ks >= KS) return;  // whole workgroup, before any barrier
+    // work item = (K slab, sample group, row group), rows fastest.  Workgroup ids go round the 8 XCDs,
+    // so XCD j takes the contiguous items [j * per_xcd, (j + 1) * per_xcd): the same number on every
+    // XCD, and the items that share a slab of x sit on one XCD (two where a slab straddles the border).
+    const int items = groups * sgroups * KS, per_xcd = (items + 7) >> 3;
+    const int item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || item >= items) return;  // whole workgroup, before any barrier
+    const int group = item % groups;
+    const int sg = (item / groups) % sgroups;
+    const int ks = item / (groups * sgroups);
     const int nch_all = (nC + 63) / 64;
     const int cbeg = ks * cpk, cend = min(cbeg + cpk, nch_all);
     const bool want_ssq = group == 0;
@@ -412,7 +417,7 @@ static hipError_t launch_wide(const void *x, const void *phi, float *Ppart, floa
     const int groups = (DP + NT * 64 - 1) / (NT * 64);
     const int nch_all = (nC + 63) / 64;
     const int cpk = (nch_all + KS - 1) / KS;
-    const int grid = 8 * groups * sgroups * ((KS + 7) / 8);
+    const int grid = 8 * ((groups * sgroups * KS + 7) / 8);
     const size_t smem = sizeof(bf16_t) * 2 * (128 + NT * 64) * kWideLd;
     if (smem > 64 * 1024) {  // above the default dynamic-LDS limit (the CU has 160 KB)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&proj_fwd_wide_kernel<NT, P>),
@@ -445,11 +450,11 @@ int proj_fwd_ksplit(int x_dtype, int phi_dtype, int B, int n, int C) {
     const int nC = n * C, DP = padded_D(n);
     if (use_wide(n, C)) {
         // ~1.6 workgroups per CU; a slab is at least 8 chunks; the partial sums (written here, read
-        // by the coefficient kernel) stay below ~1/4 of the bytes streamed
+        // by the coefficient kernel) stay below ~0.3 of the bytes streamed
         const int wgs = ((DP + 63) / 64) * ((B + 127) / 128);
         int ks = (410 + wgs / 2) / wgs;
         const int cap_chunks = nC / 64 / 8;
-        const int cap_bytes = (int)(0.25 * (2.0 * B * nC + 2.0 * DP * nC) / (8.0 * B * DP));
+        const int cap_bytes = (int)(0.28 * (2.0 * B * nC + 2.0 * DP * nC) / (8.0 * B * DP));
         if (ks > cap_chunks) ks = cap_chunks;
         if (ks > cap_bytes) ks = cap_bytes;
         if (ks > 64) ks = 64;
@@ -504,7 +509,7 @@ hipError_t launch_proj_fwd(const void *x, int x_dtype, const void *phi, int phi_
                            float *ssqpart, int KS, int B, int n, int C, hipStream_t stream) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
     if (use_mfma(x_dtype, phi_dtype, C)) {
-        if (use_wide(n, C)) return launch_wide<1, 4>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
+        if (use_wide(n, C)) return launch_wide<1, 2>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
         switch (mfma_nt(n)) {
             case 1: return launch_mfma<1>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
             case 2: return launch_mfma<2>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
