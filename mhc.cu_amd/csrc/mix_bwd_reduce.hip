@@ -303,12 +303,15 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
     // With the denominators saved by the forward call there is nothing to iterate: they are copied
     // into sc and the final iterate is the saved M.
     __device__ __forceinline__ void forward_recompute(const BwdReduceArgs &a, int b, int g, int lane, float *sc) {
-        E = mv ? (PRECISE ? expf(al2 * pres + bres) : exp_fast(al2 * pres + bres)) : 0.f;
         if (a.sk_state) {
-            m_fin = mv ? a.M[(size_t)b * a.n * a.n + r0 * a.n + c0] : 0.f;
+            // every load is requested before the first value (of prefetch() too) is used
+            m_fin = a.M[(size_t)b * a.n * a.n + (mv ? r0 * a.n + c0 : 0)];
             SK::load_state(a.sk_state + (size_t)b * SK::state_floats(a.T), g, a.T, sc, lane);
+            m_fin = mv ? m_fin : 0.f;
+            E = mv ? (PRECISE ? expf(al2 * pres + bres) : exp_fast(al2 * pres + bres)) : 0.f;
             return;
         }
+        E = mv ? (PRECISE ? expf(al2 * pres + bres) : exp_fast(al2 * pres + bres)) : 0.f;
         float m[1] = {E};
         SK::template forward<PRECISE>(m, g, a.n, a.T, a.eps, sc, lane);
         m_fin = m[0];

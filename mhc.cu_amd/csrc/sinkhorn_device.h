@@ -110,20 +110,21 @@ template <int NP> struct SkSmall {
             m[0] = PRECISE ? m[0] / cs : m[0] * fast_rcp(cs);
         }
     }
-    // Denominators saved by forward_save() -> the per-lane LDS layout that backward() reads.  All
-    // loads are independent (four iterations requested at a time).
+    // Denominators saved by forward_save() -> the per-lane LDS layout that backward() reads.  The
+    // loads of 24 iterations are requested together (one round trip for the usual 20).
     __device__ static __forceinline__ void load_state(const float *st, int g, int T, float *sc, int lane) {
-        const int r = row(g), c = col0(g);
-        for (int t0 = 0; t0 < T; t0 += 4) {
-            float rs[4], cs[4];
+        constexpr int kBatch = 24;
+        const float *pr = st + row(g), *pc = st + NP + col0(g);
+        for (int t0 = 0; t0 < T; t0 += kBatch) {
+            float rs[kBatch], cs[kBatch];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < kBatch; u++) {
                 const int t = t0 + u < T ? t0 + u : T - 1;
-                rs[u] = st[(t * 2) * NP + r];
-                cs[u] = st[(t * 2 + 1) * NP + c];
+                rs[u] = pr[t * 2 * NP];
+                cs[u] = pc[t * 2 * NP];
             }
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < kBatch; u++) {
                 if (t0 + u < T) {
                     sc[((t0 + u) * kRec) * kWave + lane] = rs[u];
                     sc[((t0 + u) * kRec + 1) * kWave + lane] = cs[u];
