@@ -34,8 +34,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # `--copy-calibration` (a 64 MiB copy).  Filled from the committed counter summary
 # (profiles/hbm_traffic_counters.txt); `commit` is the revision of the kernels the counters ran on.
 MEASURED_TRAFFIC = {
-    "commit": "dbac070",
-    "bytes": {"c1": 13291309, "c2": 43334100, "c3": 251469873, "c4": 76867411, "c5": 552458822},
+    "commit": "94cbad5",
+    "bytes": {"c1": 13291309, "c2": 39837120, "c3": 251469873, "c4": 76867411, "c5": 552458822},
 }
 
 # The kernel with the largest share of a step's device time, from the committed kernel-trace summaries
@@ -44,7 +44,7 @@ MEASURED_TRAFFIC = {
 # sums are not counted).
 PROFILED_DOMINANT = {
     "c1": dict(kernel="layer_fwd_small_kernel<float,float,4,4,2>", us=6.60, bytes=2 * 4 * 320 * 4 * 1280),
-    "c2": dict(kernel="bwd_slab_kernel<bf16>", us=10.11, bytes=3 * 2 * 320 * 4 * 1280 + 2 * 24 * 5120 + 4 * 24 * 5120),
+    "c2": dict(kernel="layer_fwd_onepass_kernel<bf16,1>", us=12.25, bytes=2 * 2 * 320 * 4 * 1280 + 2 * 24 * 5120),
     "c3": dict(kernel="bwd_slab_kernel<bf16>", us=25.21, bytes=3 * 2 * 1280 * 4 * 2560 + 2 * 24 * 10240 + 4 * 24 * 10240),
     "c4": dict(kernel="proj_bwd_mfma_kernel<1,1,true>", us=11.74, bytes=2 * 2 * 256 * 8 * 1280 + 2 * 80 * 10240 + 4 * 80 * 10240),
     "c5": dict(kernel="dphi_large_kernel<9,true>", us=36.34, bytes=2 * 128 * 40960 + 4 * 1088 * 40960),
