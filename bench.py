@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # `--copy-calibration` (a 64 MiB copy).  Filled from the committed counter summary
 # (profiles/hbm_traffic_counters.txt); `commit` is the revision of the kernels the counters ran on.
 MEASURED_TRAFFIC = {
-    "commit": "94cbad5",
+    "commit": "42466cc",
     "bytes": {"c1": 13291309, "c2": 39837120, "c3": 251469873, "c4": 76867411, "c5": 552458822},
 }
 
