@@ -57,10 +57,15 @@ class RMSNormFunction:
 
 
 def sinkhorn_knopp(inp, num_iters=20, eps=1e-8):
+    """Sinkhorn-Knopp normalisation of a [rows, cols] or [batch, rows, cols] matrix with an exact
+    backward (reference ops.py:13-32).  Limits of the HIP operator: rows, cols <= 128 and
+    num_iters <= 1024; beyond them the call raises MHCError (bad shape)."""
     return _ext.sinkhorn_knopp(inp.float(), int(num_iters), float(eps))
 
 
 def rmsnorm(inp, weight, eps=1e-5):
+    """RMSNorm over the last dimension in bfloat16 with float32 accumulation (reference
+    ops.py:35-52); any number of rows, row length limited by device memory only."""
     return _ext.rmsnorm(inp.bfloat16(), weight.bfloat16(), float(eps))
 
 
