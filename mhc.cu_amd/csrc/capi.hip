@@ -58,6 +58,61 @@ int ws_check(void *ws, size_t have, size_t need) {
         if ((expr) != hipSuccess) return MHC_ERR_LAUNCH; \
     } while (0)
 
+// ---- second stream for launches that share no output with their neighbours --------------------
+// Per device a pool of non-blocking streams (default priority) with two events each, created by
+// the first call that is not inside a stream capture (or by mhc_device_init) and kept until the
+// process ends.  A caller stream is bound to one pool entry on first use and keeps it, so callers
+// on different streams never share a side stream; binding creates nothing and is therefore allowed
+// inside a capture.  fork() makes the side stream wait for everything enqueued on the caller's
+// stream so far; join() makes the caller's stream wait for the side stream.  Both are plain event
+// record / wait pairs, which a stream capture records as graph edges.  Without a pool (first call
+// of the process already inside a capture) or with every entry bound, the call runs unforked.
+struct SideStream { hipStream_t main, s; hipEvent_t fork, join; bool bound; };
+constexpr int kSideDevices = 16, kSidePool = 8;
+std::mutex g_side_mutex;
+SideStream g_side[kSideDevices][kSidePool];
+bool g_side_ready[kSideDevices];
+
+bool side_pool_create(int dev, hipStream_t probe, bool have_probe) {  // caller holds g_side_mutex
+    if (g_side_ready[dev]) return true;
+    if (have_probe) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(probe, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) return false;
+    }
+    for (int i = 0; i < kSidePool; i++) {
+        SideStream &e = g_side[dev][i];
+        if (hipStreamCreateWithFlags(&e.s, hipStreamNonBlocking) != hipSuccess ||
+            hipEventCreateWithFlags(&e.fork, hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&e.join, hipEventDisableTiming) != hipSuccess)
+            return false;  // what was created stays unused; the calls run unforked
+        e.bound = false;
+    }
+    g_side_ready[dev] = true;
+    return true;
+}
+
+SideStream *side_stream(hipStream_t main) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSideDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_side_mutex);
+    if (!side_pool_create(dev, main, true)) return nullptr;
+    for (int i = 0; i < kSidePool; i++)
+        if (g_side[dev][i].bound && g_side[dev][i].main == main) return &g_side[dev][i];
+    for (int i = 0; i < kSidePool; i++)
+        if (!g_side[dev][i].bound) {
+            g_side[dev][i].bound = true;
+            g_side[dev][i].main = main;
+            return &g_side[dev][i];
+        }
+    return nullptr;
+}
+bool side_fork(SideStream *ss) {
+    return hipEventRecord(ss->fork, ss->main) == hipSuccess && hipStreamWaitEvent(ss->s, ss->fork, 0) == hipSuccess;
+}
+bool side_join(SideStream *ss) {
+    return hipEventRecord(ss->join, ss->s) == hipSuccess && hipStreamWaitEvent(ss->main, ss->join, 0) == hipSuccess;
+}
+
 // ---- dynamic workspace layout ----------------------------------------------------------------
 struct DynFwdWs { float *Ppart, *ssqpart, *agg; size_t bytes; };
 struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *raw, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
@@ -275,10 +330,17 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     if (mfma) {
         // matrix cores: dphi and the projection term of dx (written into dx, then completed in place)
         S = proj_bwd_batch_splits(B, n, C);
-        MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st));
+        // Wide projection: dphi = dP^T x (a writer of 4 D nC bytes) shares no output with dP phi and
+        // the dx kernel that follows it (readers), so it runs on a second stream beside them and
+        // joins before the batch sums.
+        SideStream *ss = proj_bwd_is_wide(n) && tuning_get(kTuneNoFork) == 0 ? side_stream(st) : nullptr;
+        if (ss && !side_fork(ss)) return MHC_ERR_LAUNCH;
+        MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st,
+                                        ss ? ss->s : st));
         MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, ws.dt,
                                      ws.dtpart, spg, B, n, C, st));
+        if (ss && !side_join(ss)) return MHC_ERR_LAUNCH;
     } else if (gemm_f32_supported(x_dtype, phi_dtype, n, C)) {
         // exact float32 tier, wide projection: both products on the fp32 matrix cores; the projection
         // term of dx is written into dx and completed in place
@@ -502,6 +564,16 @@ size_t mhc_layer_fwd_dynamic_scratch_bytes(int B, int n, int C) {
 int mhc_static_scratch_init(void) {
     void *p = nullptr;
     return static_scratch_pointer(&p);
+}
+
+int mhc_device_init(void) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0) return MHC_ERR_LAUNCH;
+    if (dev < kSideDevices) {
+        std::lock_guard<std::mutex> lock(g_side_mutex);
+        if (!side_pool_create(dev, nullptr, false)) return MHC_ERR_LAUNCH;
+    }
+    return mhc_static_scratch_init();
 }
 
 int mhc_layer_fwd_dynamic_static_scratch(const void *x, int x_dtype, const void *w, int w_dtype,

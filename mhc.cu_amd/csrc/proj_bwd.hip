@@ -257,6 +257,9 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
 // --------------------------------------------------------------------------------------------
 // shape selection
 // --------------------------------------------------------------------------------------------
+// more than 12 row tiles of 32: the two-kernel path of launch_proj_bwd_large
+bool proj_bwd_is_wide(int n) { return padded_D(n) / 32 > 12; }
+
 bool proj_bwd_mfma_supported(int x_dtype, int phi_dtype, int C) {
     return x_dtype == kBF16 && phi_dtype == kBF16 && C % 8 == 0;
 }
@@ -300,7 +303,7 @@ static hipError_t launch_shape(const ProjBwdArgs &a, int S, hipStream_t stream) 
 
 hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,
                                 int BP, float *dphi, float *dphi_part, void *dxflat, int B, int n,
-                                int C, hipStream_t stream) {
+                                int C, hipStream_t stream, hipStream_t dphi_stream) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
     const int S = proj_bwd_batch_splits(B, n, C);
     const int NTK = proj_bwd_ntk(B, n, C);
@@ -316,7 +319,8 @@ hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb,
     // Wide projections (more than 12 row tiles) run as two GEMM kernels that share no operand.
     if (NTD <= 4) e = launch_shape<1, 1, true>(a, S, stream);
     else if (NTD <= 12) e = launch_shape<1, 3, false>(a, S, stream);
-    else e = launch_proj_bwd_large(x, phi, dPb, dPT, BP, S > 1 ? dphi_part : dphi, dxflat, S, B, n, C, stream);
+    else e = launch_proj_bwd_large(x, phi, dPb, dPT, BP, S > 1 ? dphi_part : dphi, dxflat, S, B, n, C, stream,
+                                   dphi_stream);
     return e;  // with S > 1 the caller's finalize launch sums the S partial copies
 }
 

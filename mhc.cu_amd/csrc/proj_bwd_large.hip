@@ -309,7 +309,7 @@ __global__ __launch_bounds__(256) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
 
 hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb, const void *dPT,
                                  int BP, float *dphi_out, void *dxflat, int S, int B, int n, int C,
-                                 hipStream_t stream) {
+                                 hipStream_t stream, hipStream_t dphi_stream) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
     const int nblocks = (B + kPL_SB - 1) / kPL_SB;
     const int bps = (nblocks + S - 1) / S * kPL_SB;
@@ -336,11 +336,11 @@ hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb
         a.tpw = tpw;
         e = allow_dynamic_lds(&dphi_large_kernel<9, true>, smem);
         if (e != hipSuccess) return e;
-        dphi_large_kernel<9, true><<<dim3(slabs, (NTD + tpw - 1) / tpw, S), 256, smem, stream>>>(a);
+        dphi_large_kernel<9, true><<<dim3(slabs, (NTD + tpw - 1) / tpw, S), 256, smem, dphi_stream>>>(a);
     } else {
         e = allow_dynamic_lds(&dphi_large_kernel<3, false>, smem);
         if (e != hipSuccess) return e;
-        dphi_large_kernel<3, false><<<dim3(slabs, (NTD + 2) / 3, S), 256, smem, stream>>>(a);
+        dphi_large_kernel<3, false><<<dim3(slabs, (NTD + 2) / 3, S), 256, smem, dphi_stream>>>(a);
     }
     return hipGetLastError();
 }

@@ -11,7 +11,7 @@ enum TuneKey {
     kTuneOnepassG = 1,      // samples per workgroup of the one-launch forward
     kTuneOnepassWaves = 2,  // waves per workgroup of the one-launch forward (4..8)
     kTuneSlabSplits = 3,    // batch splits of the slab backward
-    kTuneSpare0 = 4,
+    kTuneNoFork = 4,        // 1 = keep the wide projection backward on one stream
     kTuneSpare1 = 5,
     kTuneSpare2 = 6,
     kTuneSpare3 = 7,

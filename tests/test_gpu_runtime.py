@@ -48,10 +48,12 @@ def test_graph_replay_matches_eager_and_is_deterministic(B, n, C):
             assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager result"
 
 
-def test_two_streams_with_separate_workspaces():
+@pytest.mark.parametrize("shapes", [((64, 4, 512), (48, 4, 1024)), ((24, 32, 128), (16, 32, 256))])
+def test_two_streams_with_separate_workspaces(shapes):
     """Two layer calls in flight on two streams, each with its own workspace, give the results of
-    running them one after the other."""
-    a, b = _bf16_step(64, 4, 512), _bf16_step(48, 4, 1024)
+    running them one after the other.  (n = 32: the backward forks its dphi product onto a second
+    stream of the library's own, one per caller stream.)"""
+    a, b = _bf16_step(*shapes[0]), _bf16_step(*shapes[1])
     for s in (a, b):
         s.step()
     torch.cuda.synchronize()
@@ -66,6 +68,36 @@ def test_two_streams_with_separate_workspaces():
     for s, r in zip((a, b), ref):
         for got, want in zip((s.y, s.dx, s.dphi), r):
             assert torch.equal(got, want)
+
+
+def test_forked_backward_matches_the_single_stream_backward():
+    """n = 32: the backward with its dphi product on the library's second stream (the default) against
+    the same call kept on one stream (experiment hook), bit for bit, repeated so that a missing
+    fork or join edge would show as a race."""
+    import ctypes
+
+    from mhc._lib import lib
+
+    lib.mhc_tuning_set.restype = ctypes.c_int
+    lib.mhc_tuning_set.argtypes = [ctypes.c_int, ctypes.c_int]
+    st = _bf16_step(40, 32, 256)
+    grads = lambda: [t.clone() for t in (st.dx, st.dw, st.dphi, st.dbias, st.dalpha)]
+    try:
+        assert lib.mhc_tuning_set(4, 1) == 0
+        st.step()
+        torch.cuda.synchronize()
+        ref = grads()
+        assert lib.mhc_tuning_set(4, 0) == 0
+        for rep in range(10):
+            for t in (st.dx, st.dw, st.dphi, st.dbias, st.dalpha):
+                t.fill_(float("nan"))
+            st.step()
+            st.dphi.sum()  # a consumer on the caller's stream right behind the call
+            torch.cuda.synchronize()
+            for name, a, b in zip(("dx", "dw", "dphi", "dbias", "dalpha"), ref, grads()):
+                assert torch.equal(a, b), f"run {rep}: {name}"
+    finally:
+        lib.mhc_tuning_set(4, 0)
 
 
 def test_compute_dtype_casts_like_the_reference():
