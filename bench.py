@@ -456,7 +456,8 @@ def main():
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 step.step()
-            graph.replay()
+            for _ in range(max(a.warmup, 1)):  # the untimed warm-up runs what the timed region runs
+                graph.replay()
             torch.cuda.synchronize()
         except Exception as exc:  # capture is an optimisation of the launch path only
             print(f"bench.py: graph capture failed ({exc}); using eager launches", file=sys.stderr)

@@ -330,10 +330,15 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     if (mfma) {
         // matrix cores: dphi and the projection term of dx (written into dx, then completed in place)
         S = proj_bwd_batch_splits(B, n, C);
-        // Wide projection: dphi = dP^T x (a writer of 4 D nC bytes) shares no output with dP phi and
-        // the dx kernel that follows it (readers), so it runs on a second stream beside them and
-        // joins before the batch sums.
-        SideStream *ss = proj_bwd_is_wide(n) && tuning_get(kTuneNoFork) == 0 ? side_stream(st) : nullptr;
+        // dphi = dP^T x (a writer of 4 D nC bytes) shares no output with dP phi and the dx kernel that
+        // follows it (readers), so on large shapes it runs on a second stream beside them and joins
+        // before the batch sums.  Measured (graph replays): -6 % of the step at B=128 n=32 C=1280,
+        // -10 % at B=256 n=16, -7 % at B=1024 n=8; no gain at B=256 n=8, and in an eager chain the
+        // four event calls cost the host ~30 us, which only steps of 100 us and more hide: the fork
+        // is taken when the three launches move at least 64 MB.
+        const int fork_mode = tuning_get(kTuneNoFork);  // 0 = by size, 1 = never, 2 = every shape
+        const double moved = 6.0 * D * n * C + 8.0 * (double)B * n * C;
+        SideStream *ss = (fork_mode == 2 || (fork_mode == 0 && moved >= 64e6)) ? side_stream(st) : nullptr;
         if (ss && !side_fork(ss)) return MHC_ERR_LAUNCH;
         MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st,
                                         ss ? ss->s : st));

@@ -152,13 +152,13 @@ hipError_t launch_finalize(const float *u, int rows_u, int C, float *dw, const f
 // dxflat = dP phi (bf16 [B, nC]) in one pass over x and phi.  With S = proj_bwd_batch_splits() > 1
 // the S partial copies land in dphi_part and the caller's finalize launch sums them.
 bool proj_bwd_mfma_supported(int x_dtype, int phi_dtype, int C);
-// dphi_stream: the stream of the dphi product.  The two products of a wide projection share no
+// dphi_stream: the stream of the dphi product.  The two products share no operand but dP and no
 // output, so a caller may put dphi on a second stream that it has forked from `stream` and joins
-// later (proj_bwd_is_wide() tells whether the shape takes these two kernels).
+// later; with dphi_stream == stream the narrow shapes compute both in one launch.
 hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb, const void *dPT,
                                  int BP, float *dphi_out, void *dxflat, int S, int B, int n, int C,
                                  hipStream_t stream, hipStream_t dphi_stream);
-bool proj_bwd_is_wide(int n);
+
 int proj_bwd_batch_splits(int B, int n, int C);
 hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,
                                 int BP, float *dphi, float *dphi_part, void *dxflat, int B, int n,

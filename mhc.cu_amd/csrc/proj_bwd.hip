@@ -44,8 +44,14 @@ __device__ __forceinline__ bf16x8_t lds_frag_t(const bf16_t *tile, int ld, int k
     return __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
 }
 
-template <int NTK, int TPW, bool PHI_REGS>
+// WHAT: kProjBoth = both products in one pass; kProjDphi / kProjDx = one of them (they share no
+// operand but dP: dphi needs x and dP^T, dxflat needs phi and dP), for callers that run the two
+// side by side on two streams.
+enum { kProjBoth = 0, kProjDphi = 1, kProjDx = 2 };
+
+template <int NTK, int TPW, bool PHI_REGS, int WHAT = kProjBoth>
 __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
+    constexpr bool DO_DPHI = WHAT != kProjDx, DO_DX = WHAT != kProjDphi;
     constexpr int NSB = 4 / NTK;         // 32-sample tiles per block
     constexpr int KW = 32 * NTK;         // slab width
     constexpr int LD = KW + 8;           // LDS row pitch (elements), keeps 16-byte alignment
@@ -89,19 +95,23 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
     };
     using Slot0 = std::integral_constant<int, 0>;
     using Slot1 = std::integral_constant<int, 1>;
-    if (b_begin < b_end) load_x(b_begin, Slot0{});
-    if (b_begin + SBR < b_end) load_x(b_begin + SBR, Slot1{});
+    if constexpr (DO_DPHI) {
+        if (b_begin < b_end) load_x(b_begin, Slot0{});
+        if (b_begin + SBR < b_end) load_x(b_begin + SBR, Slot1{});
+    }
 
     // ---- phi slab -> LDS (rows >= D and columns >= nC read as zero) ------------------------
-    for (int ch = tid; ch < a.DP * CPR; ch += 256) {
-        const int d = ch / CPR, k = k0 + (ch % CPR) * 8;
-        const bool ok = d < a.D && k < a.nC;
-        const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * a.nC + k : 0)), ok);
-        *reinterpret_cast<uint4 *>(phi_s + (size_t)d * LD + (ch % CPR) * 8) = v;
+    if constexpr (DO_DX) {
+        for (int ch = tid; ch < a.DP * CPR; ch += 256) {
+            const int d = ch / CPR, k = k0 + (ch % CPR) * 8;
+            const bool ok = d < a.D && k < a.nC;
+            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * a.nC + k : 0)), ok);
+            *reinterpret_cast<uint4 *>(phi_s + (size_t)d * LD + (ch % CPR) * 8) = v;
+        }
+        __syncthreads();
     }
-    __syncthreads();
     bf16x8_t phif[PHI_REGS ? 2 * TPW * 4 / NTK : 1];  // fragments (nt, ks) for ks < 2*NTD
-    if constexpr (PHI_REGS) {
+    if constexpr (PHI_REGS && DO_DX) {
 #pragma unroll
         for (int ks = 0; ks < 2 * TPW * 4 / NTK; ks++)
             if (ks < 2 * NTD) phif[ks] = lds_frag_t(phi_s, LD, ks * 16, nt * 32, lane);
@@ -125,16 +135,18 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
         static_assert(!PHI_REGS || EARLY, "the dxflat operands of the phi-in-registers variant are requested early");
         uint4 ah0[EARLY ? 2 * NSB : 1], al0[EARLY ? 2 * NSB : 1], av0[PHI_REGS ? 2 * TPW * 4 / NTK : 1];
         if constexpr (EARLY) {
-            const int dt = wave / NTK;
-            const bf16_t *ap = a.dPT + frag_base(dt < NTD ? dt : 0, a.BP >> 4, sb >> 4) + lane * 8;
+            if constexpr (DO_DPHI) {
+                const int dt = wave / NTK;
+                const bf16_t *ap = a.dPT + frag_base(dt < NTD ? dt : 0, a.BP >> 4, sb >> 4) + lane * 8;
 #pragma unroll
-            for (int ks = 0; ks < 2 * NSB; ks++) {
-                const bool ok = dt < NTD && sb + ks * 16 < b_end;
-                const bf16_t *apk = ok ? ap + ks * 512 : a.dPT;
-                ah0[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk), ok);
-                al0[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk + (size_t)a.DP * a.BP), ok);
+                for (int ks = 0; ks < 2 * NSB; ks++) {
+                    const bool ok = dt < NTD && sb + ks * 16 < b_end;
+                    const bf16_t *apk = ok ? ap + ks * 512 : a.dPT;
+                    ah0[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk), ok);
+                    al0[ks] = load16_masked(reinterpret_cast<const uint4 *>(apk + (size_t)a.DP * a.BP), ok);
+                }
             }
-            if constexpr (PHI_REGS) {
+            if constexpr (PHI_REGS && DO_DX) {
                 const bool ok = bs0 < b_end && b < b_end;
                 const bf16_t *dprow = a.dPb + frag_base((ok ? bs0 : 0) >> 5, a.DP >> 4, 0) + lane * 8;  // + 512 per k-step
 #pragma unroll
@@ -144,6 +156,7 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
             }
         }
         // ---- x block -> LDS, next block requested ----------------------------------------------
+        if constexpr (DO_DPHI) {
         if (sb != b_begin) __syncthreads();  // previous block's fragment reads are done
 #pragma unroll
         for (int u = 0; u < XCH; u++) {
@@ -187,10 +200,11 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
                 }
             }
         }
+        }  // DO_DPHI
 
         MHC_PHASE_ADD(kPhaseProjBwd, pwg, 2, pclk);
         // ---- dxflat tile of this wave: samples sb + 32 bt .. +32, columns nt ------------------
-        if (bs0 < b_end) {
+        if (DO_DX && bs0 < b_end) {
             f32x16_t o;
 #pragma unroll
             for (int i = 0; i < 16; i++) o[i] = 0.f;
@@ -243,7 +257,7 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
 #pragma unroll
     for (int m = 0; m < TPW; m++) {
         const int dt = (wave + 4 * m) / NTK;
-        if (dt < NTD && k < a.nC) {
+        if (DO_DPHI && dt < NTD && k < a.nC) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int d = dt * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
@@ -257,9 +271,6 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
 // --------------------------------------------------------------------------------------------
 // shape selection
 // --------------------------------------------------------------------------------------------
-// more than 12 row tiles of 32: the two-kernel path of launch_proj_bwd_large
-bool proj_bwd_is_wide(int n) { return padded_D(n) / 32 > 12; }
-
 bool proj_bwd_mfma_supported(int x_dtype, int phi_dtype, int C) {
     return x_dtype == kBF16 && phi_dtype == kBF16 && C % 8 == 0;
 }
@@ -285,11 +296,11 @@ int proj_bwd_batch_splits(int B, int n, int C) {
     return S;
 }
 
-template <int NTK, int TPW, bool PHI_REGS>
-static hipError_t launch_shape(const ProjBwdArgs &a, int S, hipStream_t stream) {
+template <int NTK, int TPW, bool PHI_REGS, int WHAT>
+static hipError_t launch_what(const ProjBwdArgs &a, int S, hipStream_t stream) {
     constexpr int LD = 32 * NTK + 8;
     const size_t smem = sizeof(bf16_t) * (size_t)LD * (a.DP + 32 * (4 / NTK));
-    auto kern = proj_bwd_mfma_kernel<NTK, TPW, PHI_REGS>;
+    auto kern = proj_bwd_mfma_kernel<NTK, TPW, PHI_REGS, WHAT>;
     if (smem > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -299,6 +310,17 @@ static hipError_t launch_shape(const ProjBwdArgs &a, int S, hipStream_t stream) 
     dim3 grid(NTK == 1 ? round_up(slabs, 16) : slabs, S);
     kern<<<grid, 256, smem, stream>>>(a);
     return hipGetLastError();
+}
+
+// One launch for both products, or (two streams given) one launch each.  The dxflat-only launch
+// ignores the batch split of dphi: it walks all samples.
+template <int NTK, int TPW, bool PHI_REGS>
+static hipError_t launch_shape(const ProjBwdArgs &a, int S, hipStream_t stream, hipStream_t dphi_stream) {
+    if (dphi_stream == stream) return launch_what<NTK, TPW, PHI_REGS, kProjBoth>(a, S, stream);
+    ProjBwdArgs ax = a;
+    ax.b_per_split = a.B;
+    if (hipError_t e = launch_what<NTK, TPW, PHI_REGS, kProjDx>(ax, 1, stream); e != hipSuccess) return e;
+    return launch_what<NTK, TPW, PHI_REGS, kProjDphi>(a, S, dphi_stream);
 }
 
 hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,
@@ -317,8 +339,8 @@ hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb,
     hipError_t e;
     // NTK == 1: dphi tiles per wave = ceil(NTD / 4); phi fragments in registers when 2*NTD <= 8.
     // Wide projections (more than 12 row tiles) run as two GEMM kernels that share no operand.
-    if (NTD <= 4) e = launch_shape<1, 1, true>(a, S, stream);
-    else if (NTD <= 12) e = launch_shape<1, 3, false>(a, S, stream);
+    if (NTD <= 4) e = launch_shape<1, 1, true>(a, S, stream, dphi_stream);
+    else if (NTD <= 12) e = launch_shape<1, 3, false>(a, S, stream, dphi_stream);
     else e = launch_proj_bwd_large(x, phi, dPb, dPT, BP, S > 1 ? dphi_part : dphi, dxflat, S, B, n, C, stream,
                                    dphi_stream);
     return e;  // with S > 1 the caller's finalize launch sums the S partial copies

@@ -11,7 +11,7 @@ enum TuneKey {
     kTuneOnepassG = 1,      // samples per workgroup of the one-launch forward
     kTuneOnepassWaves = 2,  // waves per workgroup of the one-launch forward (4..8)
     kTuneSlabSplits = 3,    // batch splits of the slab backward
-    kTuneNoFork = 4,        // 1 = keep the wide projection backward on one stream
+    kTuneNoFork = 4,        // dphi beside the dx kernels on a second stream: 0 = by size, 1 = never, 2 = always
     kTuneSpare1 = 5,
     kTuneSpare2 = 6,
     kTuneSpare3 = 7,

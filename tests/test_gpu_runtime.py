@@ -70,24 +70,25 @@ def test_two_streams_with_separate_workspaces(shapes):
             assert torch.equal(got, want)
 
 
-def test_forked_backward_matches_the_single_stream_backward():
-    """n = 32: the backward with its dphi product on the library's second stream (the default) against
-    the same call kept on one stream (experiment hook), bit for bit, repeated so that a missing
-    fork or join edge would show as a race."""
+@pytest.mark.parametrize("B,n,C", [(40, 32, 256), (70, 8, 512), (33, 12, 256)])
+def test_forked_backward_matches_the_single_stream_backward(B, n, C):
+    """The backward with its dphi product on the library's second stream (forced for every shape
+    through the experiment hook; the default takes it for large shapes) against the same call kept
+    on one stream, bit for bit, repeated so that a missing fork or join edge would show as a race."""
     import ctypes
 
     from mhc._lib import lib
 
     lib.mhc_tuning_set.restype = ctypes.c_int
     lib.mhc_tuning_set.argtypes = [ctypes.c_int, ctypes.c_int]
-    st = _bf16_step(40, 32, 256)
+    st = _bf16_step(B, n, C)
     grads = lambda: [t.clone() for t in (st.dx, st.dw, st.dphi, st.dbias, st.dalpha)]
     try:
         assert lib.mhc_tuning_set(4, 1) == 0
         st.step()
         torch.cuda.synchronize()
         ref = grads()
-        assert lib.mhc_tuning_set(4, 0) == 0
+        assert lib.mhc_tuning_set(4, 2) == 0
         for rep in range(10):
             for t in (st.dx, st.dw, st.dphi, st.dbias, st.dalpha):
                 t.fill_(float("nan"))
@@ -96,6 +97,25 @@ def test_forked_backward_matches_the_single_stream_backward():
             torch.cuda.synchronize()
             for name, a, b in zip(("dx", "dw", "dphi", "dbias", "dalpha"), ref, grads()):
                 assert torch.equal(a, b), f"run {rep}: {name}"
+        # the same under capture: the fork and the join become edges of the graph
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            st.step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            st.step()
+        scratch = torch.zeros(1 << 20, device="cuda")
+        for rep in range(3):
+            for t in (st.dx, st.dw, st.dphi, st.dbias, st.dalpha):
+                t.fill_(float("nan"))
+            scratch.add_(1.0).sum().item()  # eager work + a host sync between replays
+            graph.replay()
+            torch.cuda.synchronize()
+            for name, a, b in zip(("dx", "dw", "dphi", "dbias", "dalpha"), ref, grads()):
+                assert torch.equal(a, b), f"replay {rep}: {name}"
     finally:
         lib.mhc_tuning_set(4, 0)
 
