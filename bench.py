@@ -2,11 +2,13 @@
 """Benchmark of the fused mHC layer path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--mode graph|eager]
+                    [--graph-steps G]
 
 A step is one forward + backward pass of the layer over one batch of synthetic, seeded input
 that is already resident in HBM, issued through the C ABI (libmhc_hip.so).  Prints ONE JSON
 line.  `value` is microseconds per step over K back-to-back steps (wall clock, synchronised on
-both sides); `roofline` prices the same step's device time (HIP events on the launch stream)
+both sides; in graph mode the K steps are K / G replays of a HIP graph that holds G steps, the
+rest as single-step replays); `roofline` prices the same step's device time (HIP events on the launch stream)
 against the algorithmic HBM bytes of the configuration; `cpu_baseline` is the naive PyTorch
 restatement of the layer (the oracle) timed on this machine's host cores.
 
@@ -404,6 +406,8 @@ def main():
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--view", default="L", choices=["L", "K"])
     ap.add_argument("--mode", default="graph", choices=["graph", "eager"])
+    ap.add_argument("--graph-steps", type=int, default=10,
+                    help="steps captured into one HIP graph (a replay costs ~5 us by itself); 1 = one step per replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--stream-probe", action="store_true",
                     help="run the library's plain streaming kernels (read-only, copy, write-only; 16-byte accesses, "
@@ -441,45 +445,71 @@ def main():
     step = Step(cfg, a.view, torch)
 
     # ---- warm-up, optional graph capture ---------------------------------------------------
+    # A HIP graph replay costs ~5 us on top of its kernels (measured: c2 37.1 us per step with one
+    # step per graph, 32.9 with five, 32.4 with ten, 32.1 with twenty; 32.5 for an eager chain that
+    # the host keeps fed), so the timed region replays a graph that holds `--graph-steps` steps, the
+    # way the layer sits among many others inside a captured model; the figure for one step per
+    # replay is reported next to it (roofline.single_step_graph_us).
     for _ in range(max(a.warmup, 1)):
         step.step()
     torch.cuda.synchronize()
-    mode, graph = a.mode, None
+    mode, graph, graph1 = a.mode, None, None
+    G = max(1, min(a.graph_steps, a.steps))
+
+    def capture(count):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step.step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(count):
+                step.step()
+        return g
+
     if mode == "graph":
         try:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                step.step()
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                step.step()
-            for _ in range(max(a.warmup, 1)):  # the untimed warm-up runs what the timed region runs
+            graph1 = capture(1)
+            graph = capture(G) if G > 1 else graph1
+            for _ in range(max(a.warmup // G, 2)):  # the untimed warm-up runs what the timed region runs
                 graph.replay()
+            graph1.replay()
             torch.cuda.synchronize()
         except Exception as exc:  # capture is an optimisation of the launch path only
             print(f"bench.py: graph capture failed ({exc}); using eager launches", file=sys.stderr)
-            mode, graph = "eager", None
-    run = graph.replay if graph is not None else step.step
+            mode, graph, graph1, G = "eager", None, None, 1
+    else:
+        G = 1
+    run1 = graph1.replay if graph1 is not None else step.step
 
     # ---- timed region: exactly K steps -------------------------------------------------------
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(a.steps):
-        run()
+    if graph is not None:
+        for _ in range(a.steps // G):
+            graph.replay()
+        for _ in range(a.steps % G):
+            graph1.replay()
+    else:
+        for _ in range(a.steps):
+            step.step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     us_per_step = wall / a.steps * 1e6
 
     # ---- device time with HIP events on the launch stream (warm and cold caches) -------------
     reps = min(max(a.steps, 20), 200)
-    dev_step = event_time_batched(torch, run, reps)
+    if graph is not None:
+        dev_step = event_time_batched(torch, graph.replay, max(reps // G, 5)) / G
+    else:
+        dev_step = event_time_batched(torch, step.step, reps)
+    dev_single = event_time_batched(torch, run1, reps) if graph1 is not None else None
     dev_fwd = event_time_batched(torch, step.forward, reps)
     dev_bwd = event_time_batched(torch, step.backward, reps) if cfg["bwd"] else 0.0
     flush = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda")
-    cold_step = trimmed_mean(event_times(torch, run, min(reps, 50), flush=flush))
+    cold_step = trimmed_mean(event_times(torch, run1, min(reps, 50), flush=flush))
     del flush
 
     fwd_b, bwd_b = algorithmic_bytes(cfg, a.view)
@@ -501,14 +531,16 @@ def main():
         "config": {"workload": f"{a.config}: {cfg['kind']}-H mHC layer "
                                f"{'fwd+bwd' if cfg['bwd'] else 'fwd'} B={cfg['B']} C={cfg['C']} n={cfg['n']} "
                                f"{cfg['dtype']} T={T_ITERS} eps={EPS}",
-                   "view": a.view, "launch": mode, "cache": "warm (back-to-back steps)"},
+                   "view": a.view,
+                   "launch": (f"graph, {G} steps per replay" if mode == "graph" else mode),
+                   "cache": "warm (back-to-back steps)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC["bytes"].get(a.config) if a.view == "L" else None,
                      "traffic_commit": MEASURED_TRAFFIC["commit"],
                      "dominant": dominant_kernel(a.config),
                      "kernel": "whole step (all launches of one forward+backward)",
-                     "algorithmic_bytes": alg, "device_us": dev_step,
+                     "algorithmic_bytes": alg, "device_us": dev_step, "single_step_graph_us": dev_single,
                      "fwd": {"algorithmic_bytes": fwd_b, "device_us": dev_fwd,
                              "achieved": fwd_b / (dev_fwd * 1e-6) / 1e9},
                      "bwd": ({"algorithmic_bytes": bwd_b, "device_us": dev_bwd,
