@@ -52,14 +52,7 @@ struct BwdSlabArgs {
 
 __device__ __forceinline__ bf16x8_t slab_frag_t(const bf16_t *tile, int k0, int col0, int lane) {
     // lane (n = lane & 31, kg = lane >> 5) gets tile[k0 + kg*8 + i][col0 + n], i = 0..7
-    const bf16_t *p = tile + (size_t)(k0 + (lane >> 5) * 8) * kSlabLDX + col0 + (lane & 31);
-    uint32_t wv[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t lo = p[(2 * i) * kSlabLDX], hi = p[(2 * i + 1) * kSlabLDX];
-        wv[i] = lo | (hi << 16);
-    }
-    return __builtin_bit_cast(bf16x8_t, make_uint4(wv[0], wv[1], wv[2], wv[3]));
+    return __builtin_bit_cast(bf16x8_t, lds_frag_tr(tile, kSlabLDX, k0, col0, lane));
 }
 
 __device__ __forceinline__ void unpack8(const uint4 &r, float (&v)[8]) {

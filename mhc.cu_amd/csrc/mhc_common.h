@@ -208,6 +208,27 @@ __device__ __forceinline__ uint4 load16_masked(const uint4 *p, bool ok) {
 // and receives column r of the product (register = row).
 // ---------------------------------------------------------------------------------------------
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
+
+// ---------------------------------------------------------------------------------------------
+// Transposed MFMA operand from a row-major [k][column] bf16 tile in LDS (pitch ld elements, a
+// multiple of 4; col0 a multiple of 4; tile 8-byte aligned): lane (n = lane & 31, kg = lane >> 5)
+// receives tile[k0 + kg*8 + i][col0 + n], i = 0..7 - the B (or A) operand of
+// v_mfma_f32_32x32x16_bf16 when the contraction index is the strided one in memory.
+// Two ds_read_b64_tr_b16: within 16 lanes, lane i receives element i % 4 of the 8 bytes addressed
+// by lanes i/4 + 4j (j = 0..3).  So lane q + 4j of a group points at row j, columns 4q .. 4q+3 of
+// a 4 x 16 block, and lane i receives column i of the block with its four rows.  Layout checked on
+// the device with an index pattern.  (Eight 2-byte reads plus four packs per operand otherwise.)
+// ---------------------------------------------------------------------------------------------
+typedef short lds_tr_v4i16 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 lds_frag_tr(const bf16_t *tile, int ld, int k0, int col0, int lane) {
+    const int g = lane >> 4, q = lane & 3, j = (lane >> 2) & 3;
+    const bf16_t *p = tile + (size_t)(k0 + (g >> 1) * 8 + j) * ld + col0 + (g & 1) * 16 + q * 4;
+    typedef __attribute__((address_space(3))) lds_tr_v4i16 *lds_ptr;
+    const lds_tr_v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p);
+    const lds_tr_v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * (size_t)ld));
+    const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+    return make_uint4(l2.x, l2.y, h2.x, h2.y);
+}
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 __device__ __forceinline__ bf16x4_t bf16x4_of(uint32_t w0, uint32_t w1) {

@@ -219,14 +219,7 @@ __device__ __forceinline__ void split_frag(const float (&v)[8], bf16x8_t &hi, bf
 // B fragment (k = stream, column = channel) from a row-major [stream][channel] bf16 tile in LDS:
 // lane (c = lane & 31, kg = lane >> 5) gets tile[k0 + kg*8 + i][col0 + c], i = 0..7
 __device__ __forceinline__ bf16x8_t dxl_frag_t(const bf16_t *tile, int k0, int col0, int lane) {
-    const bf16_t *p = tile + (size_t)(k0 + (lane >> 5) * 8) * kDxlLDT + col0 + (lane & 31);
-    uint32_t wv[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t lo = p[(2 * i) * kDxlLDT], hi = p[(2 * i + 1) * kDxlLDT];
-        wv[i] = lo | (hi << 16);
-    }
-    return __builtin_bit_cast(bf16x8_t, make_uint4(wv[0], wv[1], wv[2], wv[3]));
+    return __builtin_bit_cast(bf16x8_t, lds_frag_tr(tile, kDxlLDT, k0, col0, lane));
 }
 
 __global__ __launch_bounds__(256, 5) void mix_bwd_dx_large_kernel(BwdDxArgs a) {

@@ -747,14 +747,7 @@ __global__ __launch_bounds__(256) void mix_fwd_large_kernel(MixLargeArgs a) {
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
         // B fragment: lane (c, kg) gets x[ks*16 + kg*8 + i][c], i = 0..7
-        const bf16_t *p = x_s + (size_t)(ks * 16 + kh * 8) * kMflLDT + wave * 32 + row;
-        uint32_t wv[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t lo = p[(2 * i) * kMflLDT], hi = p[(2 * i + 1) * kMflLDT];
-            wv[i] = lo | (hi << 16);
-        }
-        const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, make_uint4(wv[0], wv[1], wv[2], wv[3]));
+        const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, lds_frag_tr(x_s, kMflLDT, ks * 16, wave * 32, lane));
         o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(mh[ks], xf, o, 0, 0, 0);
         o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ml[ks], xf, o, 0, 0, 0);
     }

@@ -34,14 +34,7 @@ struct ProjBwdArgs {
 
 // Transposed fragment: lane (n = lane & 31, kg = lane >> 5) gets tile[k0 + kg*8 + i][col0 + n], i = 0..7
 __device__ __forceinline__ bf16x8_t lds_frag_t(const bf16_t *tile, int ld, int k0, int col0, int lane) {
-    const bf16_t *p = tile + (size_t)(k0 + (lane >> 5) * 8) * ld + col0 + (lane & 31);
-    uint32_t w[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t lo = p[(2 * i) * ld], hi = p[(2 * i + 1) * ld];
-        w[i] = lo | (hi << 16);
-    }
-    return __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
+    return __builtin_bit_cast(bf16x8_t, lds_frag_tr(tile, ld, k0, col0, lane));
 }
 
 // WHAT: kProjBoth = both products in one pass; kProjDphi / kProjDx = one of them (they share no

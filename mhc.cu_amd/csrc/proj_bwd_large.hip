@@ -33,14 +33,7 @@ struct ProjBwdLargeArgs {
 
 // lane (n = lane & 31, kg = lane >> 5) gets tile[k0 + kg*8 + i][col0 + n], i = 0..7
 __device__ __forceinline__ bf16x8_t pl_frag_t(const bf16_t *tile, int k0, int col0, int lane) {
-    const bf16_t *p = tile + (size_t)(k0 + (lane >> 5) * 8) * kPL_LD + col0 + (lane & 31);
-    uint32_t w[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t lo = p[(2 * i) * kPL_LD], hi = p[(2 * i + 1) * kPL_LD];
-        w[i] = lo | (hi << 16);
-    }
-    return __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
+    return __builtin_bit_cast(bf16x8_t, lds_frag_tr(tile, kPL_LD, k0, col0, lane));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -255,14 +248,7 @@ __global__ __launch_bounds__(256) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             // B fragment: lane (col, kg) gets phi[chunk row ks*16 + kg*8 + i][wn*32 + col]
-            const bf16_t *p = buf + (size_t)(ks * 16 + kg * 8) * kDxfLD + wn * 32 + row;
-            uint32_t w[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t lo = p[(2 * i) * kDxfLD], hi = p[(2 * i + 1) * kDxfLD];
-                w[i] = lo | (hi << 16);
-            }
-            pf[ks] = __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
+            pf[ks] = __builtin_bit_cast(bf16x8_t, lds_frag_tr(buf, kDxfLD, ks * 16, wn * 32, lane));
         }
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
