@@ -409,6 +409,10 @@ def main():
     ap.add_argument("--graph-steps", type=int, default=10,
                     help="steps captured into one HIP graph (a replay costs ~5 us by itself); 1 = one step per replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--single-stream", action="store_true",
+                    help="profiling aid: keep every launch of the backward on the caller's stream (large shapes "
+                         "run one product beside the dx kernels otherwise), so that per-kernel durations in a "
+                         "trace do not overlap")
     ap.add_argument("--stream-probe", action="store_true",
                     help="run the library's plain streaming kernels (read-only, copy, write-only; 16-byte accesses, "
                          "all CUs) over 128 MiB .. 2 GiB and print what this GPU delivers to each, HIP events on the "
@@ -443,6 +447,10 @@ def main():
         return
     cfg = CONFIGS[a.config]
     step = Step(cfg, a.view, torch)
+    if a.single_stream:
+        step.lib.mhc_tuning_set.restype = ctypes.c_int
+        step.lib.mhc_tuning_set.argtypes = [ctypes.c_int, ctypes.c_int]
+        step.lib.mhc_tuning_set(4, 1)  # csrc/tuning.h: kTuneNoFork
 
     # ---- warm-up, optional graph capture ---------------------------------------------------
     # A HIP graph replay costs ~5 us on top of its kernels (measured: c2 37.1 us per step with one
