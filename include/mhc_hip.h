@@ -110,10 +110,11 @@ MHC_API int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int
  * dw [C] fp32 is written only when f_inject == NULL.  dphi [D, nC], dbias [D], dalpha [3] fp32.
  * Every output is fully overwritten (no pre-zeroing needed); sums are order-deterministic.
  * sk_state: the tensor written by the forward call, or NULL (the iterations are then recomputed).
- * On large shapes of the bf16 tier with n > 4 (the launches in question move 64 MB or more) one
- * launch of the call, dphi = dP^T x, runs on a second stream of the library's own, forked from
- * `stream` and joined again before the call's last launch: it shares no output with the launches
- * beside it.  Those streams (a pool per GPU, default priority, one bound
+ * While `stream` is being captured, on large shapes of the bf16 tier with n > 4 (the launches in
+ * question move 64 MB or more), one launch of the call, dphi = dP^T x, runs on a second stream of
+ * the library's own, forked from `stream` and joined again before the call's last launch: it
+ * shares no output with the launches beside it, and in a graph the fork and join are edges that
+ * cost nothing (in an eager chain the event calls cost more than the overlap gains).  Those streams (a pool per GPU, default priority, one bound
  * to each caller stream on first use) are created by the first call outside a stream capture or by
  * mhc_device_init and live until the process ends; the fork and join are event record / wait
  * pairs, so the call can be captured in a HIP graph like any other.

@@ -106,6 +106,12 @@ SideStream *side_stream(hipStream_t main) {
         }
     return nullptr;
 }
+void side_pool_prepare() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSideDevices) return;
+    std::lock_guard<std::mutex> lock(g_side_mutex);
+    (void)side_pool_create(dev, nullptr, false);
+}
 bool side_fork(SideStream *ss) {
     return hipEventRecord(ss->fork, ss->main) == hipSuccess && hipStreamWaitEvent(ss->s, ss->fork, 0) == hipSuccess;
 }
@@ -334,11 +340,19 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
         // follows it (readers), so on large shapes it runs on a second stream beside them and joins
         // before the batch sums.  Measured (graph replays): -6 % of the step at B=128 n=32 C=1280,
         // -10 % at B=256 n=16, -7 % at B=1024 n=8; no gain at B=256 n=8, and in an eager chain the
-        // four event calls cost the host ~30 us, which only steps of 100 us and more hide: the fork
-        // is taken when the three launches move at least 64 MB.
-        const int fork_mode = tuning_get(kTuneNoFork);  // 0 = by size, 1 = never, 2 = every shape
+        // four event calls cost the host ~30 us and each cross-stream wait a few us on the device
+        // (B=128 n=32, eager, cold caches: 134 -> 140 us for the call), while in a captured graph
+        // they are edges that cost nothing: the fork is taken when the call is being captured and
+        // the three launches move at least 64 MB.
+        const int fork_mode = tuning_get(kTuneNoFork);  // 0 = by size under capture, 1 = never, 2 = always
         const double moved = 6.0 * D * n * C + 8.0 * (double)B * n * C;
-        SideStream *ss = (fork_mode == 2 || (fork_mode == 0 && moved >= 64e6)) ? side_stream(st) : nullptr;
+        bool fork = fork_mode == 2;
+        if (fork_mode == 0 && moved >= 64e6) {
+            hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+            fork = hipStreamIsCapturing(st, &cs) == hipSuccess && cs == hipStreamCaptureStatusActive;
+            if (!fork) side_pool_prepare();  // an eager call (the warm-up before a capture) creates the pool
+        }
+        SideStream *ss = fork ? side_stream(st) : nullptr;
         if (ss && !side_fork(ss)) return MHC_ERR_LAUNCH;
         MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st,
                                         ss ? ss->s : st));
