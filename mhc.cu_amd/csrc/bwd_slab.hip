@@ -20,6 +20,7 @@
 #include <type_traits>
 #include "mhc_common.h"
 #include "phase_profiler.h"
+#include "tuning.h"
 
 namespace mhc {
 
@@ -487,6 +488,10 @@ bool bwd_slab_supported(int x_dtype, int y_dtype, int phi_dtype, int n, int C) {
 int bwd_slab_batch_splits(int B, int n, int C) {
     const int slabs = (C + kSlabCW - 1) / kSlabCW;
     const int tiles = (B + 31) / 32;
+    if (const int forced = tuning_get(kTuneSlabSplits); forced > 0) {  // experiment hook
+        const int tps = (tiles + (forced < tiles ? forced : tiles) - 1) / (forced < tiles ? forced : tiles);
+        return (tiles + tps - 1) / tps;
+    }
     int S = (512 + slabs - 1) / slabs;  // two workgroups per CU
     if (S > tiles) S = tiles;
     // the dphi partial copies (written here, read once by the finalize launch) stay below 12 MB or
