@@ -337,6 +337,9 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
     // after fetch_sums() and forward_recompute(); xch: kXch floats of LDS private to the group
     __device__ __forceinline__ void run(const BwdReduceArgs &a, int b, int g, int lane, float *sc, float *xch) {
         const int n = a.n, D = n * n + 2 * n;
+        const int pwg_r = blockIdx.y * gridDim.x + blockIdx.x;
+        (void)pwg_r;
+        MHC_PHASE_BEGIN(rclk);
         float tpost = 0.f, tA1 = 0.f, tA2 = 0.f, s1 = 0.f;
         if constexpr (GRAM) {
             // lane (r0, c0) takes its element of each matrix and the mirrored element of W1, so that
@@ -378,7 +381,9 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
             S0 = dtp * ppre; S1 = dto * ppost;
         }
         float m[1] = {m_fin}, d[1] = {mv ? dMe : 0.f};
+        if constexpr (GRAM) MHC_PHASE_ADD(kPhaseGramSmall, pwg_r, 4, rclk);
         SK::template backward<PRECISE>(d, m, a.T, sc, lane);
+        if constexpr (GRAM) MHC_PHASE_ADD(kPhaseGramSmall, pwg_r, 5, rclk);
         if (mv) {
             const int di = 2 * n + r0 * n + c0;
             const float dtr = d[0] * E;
@@ -392,6 +397,7 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
             a.out.cx[b] = (al0 * S0 + al1 * S1 + al2 * S2) * rinv * rinv * inv_nc;
         }
         dpw.pad(D, g, SK::kGroup);
+        if constexpr (GRAM) MHC_PHASE_ADD(kPhaseGramSmall, pwg_r, 6, rclk);
     }
 };
 

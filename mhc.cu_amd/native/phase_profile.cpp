@@ -54,7 +54,7 @@ static void summary(const char *title, int kernel, int wgs, const std::vector<co
         for (int i = 0; i < np; i++) {
             const double v = stamps ? (double)(t[(size_t)w * M + i + 1] - t[(size_t)w * M + i]) : (double)t[(size_t)w * M + i];
             d[i].push_back(v);
-            total += v;
+            if (names[i][0] != ' ') total += v;  // indented lines break a phase down and are not added again
         }
         life.push_back(total);
     }
@@ -126,8 +126,9 @@ int main(int argc, char **argv) {
                  "cross-wave sum, partial stores"}, false);
     }
     summary("channel sums + coefficient backward kernel, one workgroup per sample", 4, std::min(B, 4096),
-            {"start: coefficient inputs, Sinkhorn forward recompute (wave 0)", "streaming loop (wave 0's steps)",
-             "workgroup sums", "coefficient backward (Sinkhorn reverse sweep, dP stores)"}, false);
+            {"start: coefficient inputs, Sinkhorn state (wave 0)", "streaming loop (wave 0's steps)",
+             "workgroup sums", "coefficient backward (all of it: the three lines below)",
+             "  channel-sum vectors, dHpre / dHpost", "  Sinkhorn reverse sweep", "  dt / dP stores, alpha sums"}, false);
     if (n > 4) {
         summary("dx kernel (generic, one wave per workgroup)", 5, std::min(B * ((C / 4 + 63) / 64), 4096),
                 {"start: coefficients and all loads requested", "data arrives, df / a / da", "mixing, dx stores issued", "dw / dt partial sums"}, false);
