@@ -218,6 +218,9 @@ __attribute__((visibility("default"))) int mhc_tuning_set(int key, int value) {
     g_tuning[key] = value;
     return 0;
 }
+__attribute__((visibility("default"))) int mhc_tuning_get(int key) {
+    return (key < 0 || key >= kTuneCount) ? -1 : g_tuning[key];
+}
 
 int mhc_max_sinkhorn_iters(int n) { return (n < 1 || n > MHC_MAX_N) ? 0 : max_layer_sinkhorn_iters(n); }
 
@@ -354,6 +357,7 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
         }
         SideStream *ss = fork ? side_stream(st) : nullptr;
         if (ss && !side_fork(ss)) return MHC_ERR_LAUNCH;
+        if (ss) g_tuning[kTuneForkCount]++;
         MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st,
                                         ss ? ss->s : st));
         MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,

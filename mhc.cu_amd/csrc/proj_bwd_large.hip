@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
 
 // ---------------------------------------------------------------------------------------------
 // dxflat[b, k] = sum_d dP[b, d] phi[d, k]: workgroup = 128 samples x 64 columns, so a column slab
-// of phi is streamed exactly once per 128 samples.  The 4 waves form a 2 x 2 grid (two 32-sample
+// of phi is streamed exactly once per 128 samples.  The waves form a (4 / MT) x 2 grid (MT 32-sample
 // tiles x 32 columns each).  phi arrives in chunks of 64 rows x 128 contiguous bytes (8 lanes per
 // row), two chunks in flight per thread (register FIFO), is parked in a double-buffered LDS tile
 // and read back transposed (the contraction runs over d, the strided axis); the dP operand comes
@@ -190,7 +190,14 @@ constexpr int kDxfCW = 64;            // columns per workgroup
 constexpr int kDxfLD = kDxfCW + 8;    // LDS row pitch (elements)
 constexpr int kDxfDC = 64;            // phi rows per chunk
 
-__global__ __launch_bounds__(256) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
+// MT = 32-sample tiles per wave: 2 (four waves) or 1 (eight waves; one wave's MFMAs run under
+// another's LDS reads on the same SIMD: 3 us faster at B=128 n=32 C=1280 when the kernel runs alone;
+// beside the dphi kernel on the second stream the two variants measure the same).
+template <int MT>
+__global__ __launch_bounds__(512 / MT) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
+    constexpr int NTHR = 512 / MT;
+    constexpr int PH = 512 / NTHR;       // 16-byte pieces of a phi chunk per thread (64 rows x 8)
+    constexpr int PSTEP = NTHR / 8;      // rows covered by one round of the workgroup's loads
     extern __shared__ bf16_t pl_lds[];  // [2][kDxfDC][kDxfLD]; later the [128][kDxfLD] output tile
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = lane & 31, kg = lane >> 5;
@@ -200,39 +207,39 @@ __global__ __launch_bounds__(256) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
     const int tiles_all = a.BP >> 5;
     const int nchunks = (a.DP + kDxfDC - 1) / kDxfDC;
 
-    // phi piece of this thread: rows (tid >> 3) + 32 h of the chunk, 16-byte segment tid & 7.
+    // phi piece of this thread: rows (tid >> 3) + PSTEP h of the chunk, 16-byte segment tid & 7.
     // Out-of-range rows / columns alias valid memory: rows in [D, DP) meet zero dP, rows >= DP are
     // never multiplied, columns >= nC are never stored.
     const int prow = tid >> 3, pseg = tid & 7;
     const int kc = k0 + pseg * 8 < a.nC ? k0 + pseg * 8 : 0;
     // dP fragments of this wave: sample tiles st0, st0 + 1 (clamped: surplus tiles are not stored)
-    const int st0 = sg * 4 + wm * 2;
-    const bf16_t *ap[2];
+    const int st0 = sg * 4 + wm * MT;
+    const bf16_t *ap[MT];
 #pragma unroll
-    for (int m = 0; m < 2; m++)
+    for (int m = 0; m < MT; m++)
         ap[m] = a.dPb + frag_base(min(st0 + m, tiles_all - 1), a.DP >> 4, 0) + lane * 8;
 
     // register FIFO of two chunks; a slot holds 2 phi pieces and 2 x 4 dP fragments
     // (RawVec keeps the loaded words as scalars: whole-uint4 copies of an array element can end up in
     // scratch memory, and a scratch store waits for the load it parks)
-    struct Slot { RawVec<bf16_t, 8> p[2]; uint4 f[8]; };
+    struct Slot { RawVec<bf16_t, 8> p[PH]; uint4 f[4 * MT]; };
     auto issue = [&](Slot &sl, int c) {
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int d = c * kDxfDC + prow + 32 * h;
+        for (int h = 0; h < PH; h++) {
+            const int d = c * kDxfDC + prow + PSTEP * h;
             sl.p[h].load(a.phi + (size_t)(d < a.D ? d : 0) * a.nC + kc);
         }
 #pragma unroll
-        for (int m = 0; m < 2; m++)
+        for (int m = 0; m < MT; m++)
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
                 const int d0 = c * kDxfDC + ks * 16;
                 sl.f[m * 4 + ks] = *reinterpret_cast<const uint4 *>(ap[m] + (size_t)(d0 < a.DP ? d0 >> 4 : 0) * 512);
             }
     };
-    f32x16_t o[2];
+    f32x16_t o[MT];
 #pragma unroll
-    for (int m = 0; m < 2; m++)
+    for (int m = 0; m < MT; m++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o[m][i] = 0.f;
 
@@ -240,8 +247,8 @@ __global__ __launch_bounds__(256) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
     auto compute = [&](const Slot &sl, int par, int c) {
         bf16_t *buf = pl_lds + (size_t)par * kDxfDC * kDxfLD;
 #pragma unroll
-        for (int h = 0; h < 2; h++)
-            *reinterpret_cast<uint4 *>(buf + (size_t)(prow + 32 * h) * kDxfLD + pseg * 8) =
+        for (int h = 0; h < PH; h++)
+            *reinterpret_cast<uint4 *>(buf + (size_t)(prow + PSTEP * h) * kDxfLD + pseg * 8) =
                 make_uint4(sl.p[h].w[0], sl.p[h].w[1], sl.p[h].w[2], sl.p[h].w[3]);
         __syncthreads();
         bf16x8_t pf[4];
@@ -254,7 +261,7 @@ __global__ __launch_bounds__(256) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
         for (int ks = 0; ks < 4; ks++) {
             const bool live = c * kDxfDC + ks * 16 < a.DP;  // uniform; dead k-steps get a zero A operand
 #pragma unroll
-            for (int m = 0; m < 2; m++) {
+            for (int m = 0; m < MT; m++) {
                 uint4 av = sl.f[m * 4 + ks];
                 av.x = live ? av.x : 0u; av.y = live ? av.y : 0u; av.z = live ? av.z : 0u; av.w = live ? av.w : 0u;
                 o[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), pf[ks], o[m], 0, 0, 0);
@@ -278,14 +285,14 @@ __global__ __launch_bounds__(256) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
     // accumulator layout: column = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4.
     bf16_t *o_s = pl_lds;  // [128][kDxfLD]
 #pragma unroll
-    for (int m = 0; m < 2; m++)
+    for (int m = 0; m < MT; m++)
 #pragma unroll
         for (int i = 0; i < 16; i++)
-            o_s[(size_t)((wm * 2 + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3)) * kDxfLD + wn * 32 + row] = f32_to_bf16(o[m][i]);
+            o_s[(size_t)((wm * MT + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3)) * kDxfLD + wn * 32 + row] = f32_to_bf16(o[m][i]);
     __syncthreads();
 #pragma unroll
-    for (int h = 0; h < 4; h++) {
-        const int r = prow + 32 * h;
+    for (int h = 0; h < 1024 / NTHR; h++) {
+        const int r = prow + PSTEP * h;
         const int bo = sg * 128 + r;
         if (bo < a.B && k0 + pseg * 8 < a.nC)
             *reinterpret_cast<uint4 *>(a.dxflat + (size_t)bo * a.nC + k0 + pseg * 8) =
@@ -304,8 +311,8 @@ hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb
                        static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, bps, 9};
     const int slabs = (nC + kPL_KW - 1) / kPL_KW;
     const int NTD = DP / 32;
-    dxflat_wide_kernel<<<dim3((nC + kDxfCW - 1) / kDxfCW, (B + 127) / 128), 256,
-                         sizeof(bf16_t) * 128 * kDxfLD, stream>>>(a);
+    dxflat_wide_kernel<1><<<dim3((nC + kDxfCW - 1) / kDxfCW, (B + 127) / 128), 512,
+                            sizeof(bf16_t) * 128 * kDxfLD, stream>>>(a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     // the x block, later two operand tiles of 16 KB in the same memory

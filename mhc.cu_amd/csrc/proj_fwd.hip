@@ -251,7 +251,10 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
 // fraction of the L1 rate, so here both operands are fetched with row-contiguous loads (8 lanes
 // per 128-byte line), parked in LDS and read back in MFMA layout.
 //   workgroup tile: 128 samples x (NT * 64) projection rows, K chunks of 64 elements
-//   4 waves as 2 x 2: a wave owns 64 samples x NT*32 rows (2 x NT accumulator tiles)
+//   NWM x 2 waves: a wave owns 128 / NWM samples x NT*32 rows.  Eight waves (NWM = 4, one 32 x 32
+//   accumulator tile each at NT = 1) are 12 % faster than four with two tiles each: the kernel is
+//   bound by its own pipeline (global loads, LDS parking, LDS reads and MFMAs take turns behind one
+//   barrier per chunk), and two waves per SIMD let one wave's MFMAs run under the other's LDS reads.
 //   P chunks of global loads are in flight per thread (register FIFO) ahead of the chunk being
 //   multiplied; LDS is double-buffered, one barrier per chunk.
 // Workgroups that read the same K slab sit on the same XCD (workgroup id modulo 8 selects the
@@ -261,8 +264,8 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
 // --------------------------------------------------------------------------------------------
 constexpr int kWideLd = 72;  // LDS row stride in bf16 elements: 128 data bytes + 16 pad
 
-template <int NT, int P>
-__global__ __launch_bounds__(256) void proj_fwd_wide_kernel(const bf16_t *__restrict__ x,
+template <int NT, int P, int NWM = 2>
+__global__ __launch_bounds__(128 * NWM) void proj_fwd_wide_kernel(const bf16_t *__restrict__ x,
                                                             const bf16_t *__restrict__ phi,
                                                             float *__restrict__ Ppart,
                                                             float *__restrict__ ssqpart, int B,
@@ -271,8 +274,11 @@ __global__ __launch_bounds__(256) void proj_fwd_wide_kernel(const bf16_t *__rest
                                                             int cpk /* chunks per K slab */) {
     static_assert(P % 2 == 0, "buffer parity is tied to the FIFO slot");
     constexpr int R = NT * 64;   // projection rows per workgroup
-    constexpr int XJ = 4;        // 16-byte segments of the x tile per thread (128 rows x 8 / 256)
-    constexpr int PJ = R / 32;   // same for the phi tile
+    constexpr int NTHR = 128 * NWM;          // NWM x 2 waves: a wave owns 128 / NWM samples x NT*32 rows
+    constexpr int MT = 4 / NWM;              // 32-sample tiles per wave
+    constexpr int XJ = 128 * 8 / NTHR;       // 16-byte segments of the x tile per thread
+    constexpr int PJ = R * 8 / NTHR;         // same for the phi tile
+    constexpr int RSTEP = NTHR / 8;          // rows covered by one round of the workgroup's loads
     extern __shared__ __align__(16) bf16_t lds_w[];  // [2][128 + R][kWideLd]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = lane & 31, kh = lane >> 5;
@@ -296,13 +302,13 @@ __global__ __launch_bounds__(256) void proj_fwd_wide_kernel(const bf16_t *__rest
     bool xv[XJ], pv[PJ];
 #pragma unroll
     for (int j = 0; j < XJ; j++) {
-        const int b = sg * 128 + lrow + 32 * j;
+        const int b = sg * 128 + lrow + RSTEP * j;
         xv[j] = b < B;
         xg[j] = reinterpret_cast<const uint4 *>(x + (size_t)(xv[j] ? b : 0) * nC) + seg;
     }
 #pragma unroll
     for (int j = 0; j < PJ; j++) {
-        const int d = group * R + lrow + 32 * j;
+        const int d = group * R + lrow + RSTEP * j;
         pv[j] = d < D;
         pg[j] = reinterpret_cast<const uint4 *>(phi + (size_t)(pv[j] ? d : 0) * nC) + seg;
     }
@@ -317,9 +323,9 @@ __global__ __launch_bounds__(256) void proj_fwd_wide_kernel(const bf16_t *__rest
         for (int j = 0; j < XJ; j++) rg[slot_][j] = xg[j][c * 8];
     };
 
-    f32x16_t acc[2][NT];
+    f32x16_t acc[MT][NT];
 #pragma unroll
-    for (int m = 0; m < 2; m++)
+    for (int m = 0; m < MT; m++)
 #pragma unroll
         for (int t = 0; t < NT; t++)
 #pragma unroll
@@ -335,10 +341,10 @@ __global__ __launch_bounds__(256) void proj_fwd_wide_kernel(const bf16_t *__rest
         bf16_t *ps = xs + 128 * kWideLd;
 #pragma unroll
         for (int q = 0; q < XJ; q++)
-            *reinterpret_cast<uint4 *>(xs + (lrow + 32 * q) * kWideLd + seg * 8) = rg[j][q];
+            *reinterpret_cast<uint4 *>(xs + (lrow + RSTEP * q) * kWideLd + seg * 8) = rg[j][q];
 #pragma unroll
         for (int q = 0; q < PJ; q++)
-            *reinterpret_cast<uint4 *>(ps + (lrow + 32 * q) * kWideLd + seg * 8) = rg[j][XJ + q];
+            *reinterpret_cast<uint4 *>(ps + (lrow + RSTEP * q) * kWideLd + seg * 8) = rg[j][XJ + q];
         if (want_ssq) {
 #pragma unroll
             for (int q = 0; q < XJ; q++) {
@@ -354,17 +360,17 @@ __global__ __launch_bounds__(256) void proj_fwd_wide_kernel(const bf16_t *__rest
         if constexpr (decltype(prefetch)::value) issue(j, next);
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-            bf16x8_t af[2], bfr[NT];
+            bf16x8_t af[MT], bfr[NT];
 #pragma unroll
-            for (int m = 0; m < 2; m++)
+            for (int m = 0; m < MT; m++)
                 af[m] = *reinterpret_cast<const bf16x8_t *>(
-                    xs + (wm * 64 + m * 32 + row) * kWideLd + s * 16 + kh * 8);
+                    xs + (wm * 32 * MT + m * 32 + row) * kWideLd + s * 16 + kh * 8);
 #pragma unroll
             for (int t = 0; t < NT; t++)
                 bfr[t] = *reinterpret_cast<const bf16x8_t *>(
                     ps + (wn * NT * 32 + t * 32 + row) * kWideLd + s * 16 + kh * 8);
 #pragma unroll
-            for (int m = 0; m < 2; m++)
+            for (int m = 0; m < MT; m++)
 #pragma unroll
                 for (int t = 0; t < NT; t++)
                     acc[m][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[m], bfr[t], acc[m][t], 0, 0, 0);
@@ -388,13 +394,13 @@ __global__ __launch_bounds__(256) void proj_fwd_wide_kernel(const bf16_t *__rest
     // register i -> row 8 * (i / 4) + 4 * (lane / 32) + (i % 4)
     float *out = Ppart + (size_t)ks * B * DP;
 #pragma unroll
-    for (int m = 0; m < 2; m++)
+    for (int m = 0; m < MT; m++)
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             const int d = group * R + wn * NT * 32 + t * 32 + row;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int bs = sg * 128 + wm * 64 + m * 32 + 8 * (i >> 2) + 4 * kh + (i & 3);
+                const int bs = sg * 128 + wm * 32 * MT + m * 32 + 8 * (i >> 2) + 4 * kh + (i & 3);
                 if (bs < B && d < D) out[(size_t)bs * DP + d] = acc[m][t][i];
             }
         }
@@ -405,12 +411,12 @@ __global__ __launch_bounds__(256) void proj_fwd_wide_kernel(const bf16_t *__rest
             v += __shfl_xor(v, 1, kWave);
             v += __shfl_xor(v, 2, kWave);
             v += __shfl_xor(v, 4, kWave);
-            if (seg == 0 && xv[j]) ssqpart[(size_t)ks * B + sg * 128 + lrow + 32 * j] = v;
+            if (seg == 0 && xv[j]) ssqpart[(size_t)ks * B + sg * 128 + lrow + RSTEP * j] = v;
         }
     }
 }
 
-template <int NT, int P>
+template <int NT, int P, int NWM = 2>
 static hipError_t launch_wide(const void *x, const void *phi, float *Ppart, float *ssqpart, int KS,
                               int B, int D, int DP, int nC, hipStream_t stream) {
     const int sgroups = (B + 127) / 128;
@@ -420,11 +426,11 @@ static hipError_t launch_wide(const void *x, const void *phi, float *Ppart, floa
     const int grid = 8 * ((groups * sgroups * KS + 7) / 8);
     const size_t smem = sizeof(bf16_t) * 2 * (128 + NT * 64) * kWideLd;
     if (smem > 64 * 1024) {  // above the default dynamic-LDS limit (the CU has 160 KB)
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&proj_fwd_wide_kernel<NT, P>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&proj_fwd_wide_kernel<NT, P, NWM>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return e;
     }
-    proj_fwd_wide_kernel<NT, P><<<grid, 256, smem, stream>>>(
+    proj_fwd_wide_kernel<NT, P, NWM><<<grid, 128 * NWM, smem, stream>>>(
         static_cast<const bf16_t *>(x), static_cast<const bf16_t *>(phi), Ppart, ssqpart, B, D, DP,
         nC, groups, sgroups, KS, cpk);
     return hipGetLastError();
@@ -509,7 +515,7 @@ hipError_t launch_proj_fwd(const void *x, int x_dtype, const void *phi, int phi_
                            float *ssqpart, int KS, int B, int n, int C, hipStream_t stream) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
     if (use_mfma(x_dtype, phi_dtype, C)) {
-        if (use_wide(n, C)) return launch_wide<1, 2>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
+        if (use_wide(n, C)) return launch_wide<1, 2, 4>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
         switch (mfma_nt(n)) {
             case 1: return launch_mfma<1>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
             case 2: return launch_mfma<2>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);

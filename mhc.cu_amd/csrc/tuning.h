@@ -14,7 +14,7 @@ enum TuneKey {
     kTuneNoFork = 4,        // dphi beside the dx kernels on a second stream: 0 = by size, 1 = never, 2 = always
     kTuneSpare1 = 5,
     kTuneSpare2 = 6,
-    kTuneSpare3 = 7,
+    kTuneForkCount = 7,     // read-only use: backward calls that took the second stream so far (mhc_tuning_get)
     kTuneCount = 8
 };
 

@@ -116,6 +116,9 @@ def test_forked_backward_matches_the_single_stream_backward(B, n, C):
             torch.cuda.synchronize()
             for name, a, b in zip(("dx", "dw", "dphi", "dbias", "dalpha"), ref, grads()):
                 assert torch.equal(a, b), f"replay {rep}: {name}"
+        lib.mhc_tuning_get.restype = ctypes.c_int
+        lib.mhc_tuning_get.argtypes = [ctypes.c_int]
+        assert lib.mhc_tuning_get(7) >= 12, "the forced fork was not taken"  # 10 eager calls + warm-up + capture
     finally:
         lib.mhc_tuning_set(4, 0)
 
