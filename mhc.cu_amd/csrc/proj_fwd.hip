@@ -251,8 +251,10 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
 // fraction of the L1 rate, so here both operands are fetched with row-contiguous loads (8 lanes
 // per 128-byte line), parked in LDS and read back in MFMA layout.
 //   workgroup tile: 128 samples x (NT * 64) projection rows, K chunks of 64 elements
-//   NWM x 2 waves: a wave owns 128 / NWM samples x NT*32 rows.  Eight waves (NWM = 4, one 32 x 32
-//   accumulator tile each at NT = 1) are 12 % faster than four with two tiles each: the kernel is
+//   NWM x NWN waves: a wave owns 128 / NWM samples x NT*32 rows.  Eight waves (4 x 2, one 32 x 32
+//   accumulator tile each at NT = 1) are 12 % faster than four with two tiles each (sixteen waves on
+//   a 128 x 128 tile gain another 3 % at D = 1088 with exactly 24 K slabs and lose with any other
+//   count; not taken): the kernel is
 //   bound by its own pipeline (global loads, LDS parking, LDS reads and MFMAs take turns behind one
 //   barrier per chunk), and two waves per SIMD let one wave's MFMAs run under the other's LDS reads.
 //   P chunks of global loads are in flight per thread (register FIFO) ahead of the chunk being
@@ -264,8 +266,8 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
 // --------------------------------------------------------------------------------------------
 constexpr int kWideLd = 72;  // LDS row stride in bf16 elements: 128 data bytes + 16 pad
 
-template <int NT, int P, int NWM = 2>
-__global__ __launch_bounds__(128 * NWM) void proj_fwd_wide_kernel(const bf16_t *__restrict__ x,
+template <int NT, int P, int NWM = 2, int NWN = 2>
+__global__ __launch_bounds__(64 * NWM * NWN) void proj_fwd_wide_kernel(const bf16_t *__restrict__ x,
                                                             const bf16_t *__restrict__ phi,
                                                             float *__restrict__ Ppart,
                                                             float *__restrict__ ssqpart, int B,
@@ -273,8 +275,8 @@ __global__ __launch_bounds__(128 * NWM) void proj_fwd_wide_kernel(const bf16_t *
                                                             int sgroups, int KS,
                                                             int cpk /* chunks per K slab */) {
     static_assert(P % 2 == 0, "buffer parity is tied to the FIFO slot");
-    constexpr int R = NT * 64;   // projection rows per workgroup
-    constexpr int NTHR = 128 * NWM;          // NWM x 2 waves: a wave owns 128 / NWM samples x NT*32 rows
+    constexpr int R = NT * 32 * NWN;   // projection rows per workgroup
+    constexpr int NTHR = 64 * NWM * NWN;     // NWM x NWN waves: a wave owns 128 / NWM samples x NT*32 rows
     constexpr int MT = 4 / NWM;              // 32-sample tiles per wave
     constexpr int XJ = 128 * 8 / NTHR;       // 16-byte segments of the x tile per thread
     constexpr int PJ = R * 8 / NTHR;         // same for the phi tile
@@ -282,7 +284,7 @@ __global__ __launch_bounds__(128 * NWM) void proj_fwd_wide_kernel(const bf16_t *
     extern __shared__ __align__(16) bf16_t lds_w[];  // [2][128 + R][kWideLd]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = lane & 31, kh = lane >> 5;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / NWN, wn = wave % NWN;
     // work item = (K slab, sample group, row group), rows fastest.  Workgroup ids go round the 8 XCDs,
     // so XCD j takes the contiguous items [j * per_xcd, (j + 1) * per_xcd): the same number on every
     // XCD, and the items that share a slab of x sit on one XCD (two where a slab straddles the border).
@@ -416,21 +418,22 @@ __global__ __launch_bounds__(128 * NWM) void proj_fwd_wide_kernel(const bf16_t *
     }
 }
 
-template <int NT, int P, int NWM = 2>
+template <int NT, int P, int NWM = 2, int NWN = 2>
 static hipError_t launch_wide(const void *x, const void *phi, float *Ppart, float *ssqpart, int KS,
                               int B, int D, int DP, int nC, hipStream_t stream) {
     const int sgroups = (B + 127) / 128;
-    const int groups = (DP + NT * 64 - 1) / (NT * 64);
+    constexpr int R = NT * 32 * NWN;
+    const int groups = (DP + R - 1) / R;
     const int nch_all = (nC + 63) / 64;
     const int cpk = (nch_all + KS - 1) / KS;
     const int grid = 8 * ((groups * sgroups * KS + 7) / 8);
-    const size_t smem = sizeof(bf16_t) * 2 * (128 + NT * 64) * kWideLd;
+    const size_t smem = sizeof(bf16_t) * 2 * (128 + R) * kWideLd;
     if (smem > 64 * 1024) {  // above the default dynamic-LDS limit (the CU has 160 KB)
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&proj_fwd_wide_kernel<NT, P, NWM>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&proj_fwd_wide_kernel<NT, P, NWM, NWN>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return e;
     }
-    proj_fwd_wide_kernel<NT, P, NWM><<<grid, 128 * NWM, smem, stream>>>(
+    proj_fwd_wide_kernel<NT, P, NWM, NWN><<<grid, 64 * NWM * NWN, smem, stream>>>(
         static_cast<const bf16_t *>(x), static_cast<const bf16_t *>(phi), Ppart, ssqpart, B, D, DP,
         nC, groups, sgroups, KS, cpk);
     return hipGetLastError();
