@@ -36,8 +36,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # `--copy-calibration` (a 64 MiB copy).  Filled from the committed counter summary
 # (profiles/hbm_traffic_counters.txt); `commit` is the revision of the kernels the counters ran on.
 MEASURED_TRAFFIC = {
-    "commit": "ab7fbd7",
-    "bytes": {"c1": 13291318, "c2": 38566990, "c3": 248178695, "c4": 76819377, "c5": 552416086},
+    "commit": "141f0b8",
+    "bytes": {"c1": 13291313, "c2": 38566965, "c3": 248178194, "c4": 76819179, "c5": 552885517},
 }
 
 # The kernel with the largest share of a step's device time, from the committed kernel-trace summaries
@@ -45,11 +45,11 @@ MEASURED_TRAFFIC = {
 # needs that kernel to move (its own inputs and outputs once; for the split projections the partial
 # sums are not counted).
 PROFILED_DOMINANT = {
-    "c1": dict(kernel="layer_fwd_small_kernel<float,float,4,4,2>", us=6.58, bytes=2 * 4 * 320 * 4 * 1280),
-    "c2": dict(kernel="layer_fwd_onepass_kernel<bf16,1>", us=12.05, bytes=2 * 2 * 320 * 4 * 1280 + 2 * 24 * 5120),
-    "c3": dict(kernel="bwd_slab_kernel<bf16>", us=24.33, bytes=3 * 2 * 1280 * 4 * 2560 + 2 * 24 * 10240 + 4 * 24 * 10240),
+    "c1": dict(kernel="layer_fwd_small_kernel<float,float,4,4,2>", us=6.59, bytes=2 * 4 * 320 * 4 * 1280),
+    "c2": dict(kernel="layer_fwd_onepass_kernel<bf16,1>", us=11.92, bytes=2 * 2 * 320 * 4 * 1280 + 2 * 24 * 5120),
+    "c3": dict(kernel="bwd_slab_kernel<bf16>", us=24.26, bytes=3 * 2 * 1280 * 4 * 2560 + 2 * 24 * 10240 + 4 * 24 * 10240),
     "c4": dict(kernel="proj_bwd_mfma_kernel<1,1,true>", us=11.44, bytes=2 * 2 * 256 * 8 * 1280 + 2 * 80 * 10240 + 4 * 80 * 10240),
-    "c5": dict(kernel="dphi_large_kernel<9,true>", us=35.81, bytes=2 * 128 * 40960 + 4 * 1088 * 40960),
+    "c5": dict(kernel="dphi_large_kernel<9,true>", us=35.57, bytes=2 * 128 * 40960 + 4 * 1088 * 40960),
 }
 
 CONFIGS = {
@@ -409,10 +409,6 @@ def main():
     ap.add_argument("--graph-steps", type=int, default=10,
                     help="steps captured into one HIP graph (a replay costs ~5 us by itself); 1 = one step per replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--single-stream", action="store_true",
-                    help="profiling aid: keep every launch of the backward on the caller's stream (large shapes "
-                         "run one product beside the dx kernels otherwise), so that per-kernel durations in a "
-                         "trace do not overlap")
     ap.add_argument("--stream-probe", action="store_true",
                     help="run the library's plain streaming kernels (read-only, copy, write-only; 16-byte accesses, "
                          "all CUs) over 128 MiB .. 2 GiB and print what this GPU delivers to each, HIP events on the "
@@ -447,10 +443,6 @@ def main():
         return
     cfg = CONFIGS[a.config]
     step = Step(cfg, a.view, torch)
-    if a.single_stream:
-        step.lib.mhc_tuning_set.restype = ctypes.c_int
-        step.lib.mhc_tuning_set.argtypes = [ctypes.c_int, ctypes.c_int]
-        step.lib.mhc_tuning_set(4, 1)  # csrc/tuning.h: kTuneNoFork
 
     # ---- warm-up, optional graph capture ---------------------------------------------------
     # A HIP graph replay costs ~5 us on top of its kernels (measured: c2 37.1 us per step with one

@@ -110,14 +110,6 @@ MHC_API int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int
  * dw [C] fp32 is written only when f_inject == NULL.  dphi [D, nC], dbias [D], dalpha [3] fp32.
  * Every output is fully overwritten (no pre-zeroing needed); sums are order-deterministic.
  * sk_state: the tensor written by the forward call, or NULL (the iterations are then recomputed).
- * While `stream` is being captured, on large shapes of the bf16 tier with n > 4 (the launches in
- * question move 64 MB or more), one launch of the call, dphi = dP^T x, runs on a second stream of
- * the library's own, forked from `stream` and joined again before the call's last launch: it
- * shares no output with the launches beside it, and in a graph the fork and join are edges that
- * cost nothing (in an eager chain the event calls cost more than the overlap gains).  Those streams (a pool per GPU, default priority, one bound
- * to each caller stream on first use) are created by the first call outside a stream capture or by
- * mhc_device_init and live until the process ends; the fork and join are event record / wait
- * pairs, so the call can be captured in a HIP graph like any other.
  */
 MHC_API int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtype, const void *w,
                           int w_dtype, const void *phi, int phi_dtype, const float *bias,
@@ -155,11 +147,6 @@ MHC_API int mhc_pack_dynamic_params(const void *phi_pre, const void *phi_post, c
 MHC_API size_t mhc_static_scratch_capacity(void);
 MHC_API size_t mhc_layer_fwd_dynamic_scratch_bytes(int B, int n, int C);
 MHC_API int mhc_static_scratch_init(void);
-/* Optional: prepares everything the library keeps per GPU (the static scratch address above, the
- * second-stream pool of mhc_layer_bwd_dynamic) for the current device, so that a process whose
- * first layer call already sits inside a stream capture loses nothing.  No counterpart in the
- * reference. */
-MHC_API int mhc_device_init(void);
 MHC_API int mhc_layer_fwd_dynamic_static_scratch(const void *x, int x_dtype, const void *w, int w_dtype,
                                          const void *phi, int phi_dtype, const float *bias,
                                          const float *alpha, const void *f_inject, void *y, int y_dtype,

@@ -11,7 +11,7 @@ enum TuneKey {
     kTuneOnepassG = 1,      // samples per workgroup of the one-launch forward
     kTuneOnepassWaves = 2,  // waves per workgroup of the one-launch forward (4..8)
     kTuneSlabSplits = 3,    // batch splits of the slab backward
-    kTuneNoFork = 4,        // dphi beside the dx kernels on a second stream: 0 = by size, 1 = never, 2 = always
+    kTuneNoFork = 4,        // dphi beside the dx kernels on a second stream: 2 = always, anything else = never
     kTuneSpare1 = 5,
     kTuneSpare2 = 6,
     kTuneForkCount = 7,     // read-only use: backward calls that took the second stream so far (mhc_tuning_get)

@@ -43,7 +43,6 @@ _SIGNATURES = {
     "mhc_static_scratch_capacity": (_Z, []),
     "mhc_layer_fwd_dynamic_scratch_bytes": (_Z, [_I, _I, _I]),
     "mhc_static_scratch_init": (c_int, []),
-    "mhc_device_init": (c_int, []),
     "mhc_layer_fwd_dynamic_static_scratch": (c_int, [_P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P,
                                                      _P, _P, _P, _P, _I, _I, _I, _I, _F, _P]),
     "mhc_layer_static_workspace_bytes": (_Z, [_I, _I, _I]),

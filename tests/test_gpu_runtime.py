@@ -51,8 +51,7 @@ def test_graph_replay_matches_eager_and_is_deterministic(B, n, C):
 @pytest.mark.parametrize("shapes", [((64, 4, 512), (48, 4, 1024)), ((24, 32, 128), (16, 32, 256))])
 def test_two_streams_with_separate_workspaces(shapes):
     """Two layer calls in flight on two streams, each with its own workspace, give the results of
-    running them one after the other.  (n = 32: the backward forks its dphi product onto a second
-    stream of the library's own, one per caller stream.)"""
+    running them one after the other."""
     a, b = _bf16_step(*shapes[0]), _bf16_step(*shapes[1])
     for s in (a, b):
         s.step()
@@ -72,9 +71,9 @@ def test_two_streams_with_separate_workspaces(shapes):
 
 @pytest.mark.parametrize("B,n,C", [(40, 32, 256), (70, 8, 512), (33, 12, 256)])
 def test_forked_backward_matches_the_single_stream_backward(B, n, C):
-    """The backward with its dphi product on the library's second stream (forced for every shape
-    through the experiment hook; the default takes it for large shapes) against the same call kept
-    on one stream, bit for bit, repeated so that a missing fork or join edge would show as a race."""
+    """The backward with its dphi product on a second stream of the library's own (forced through the
+    experiment hook; the default keeps one stream) against the same call kept on one stream, bit for
+    bit, repeated so that a missing fork or join edge would show as a race."""
     import ctypes
 
     from mhc._lib import lib
