@@ -324,6 +324,51 @@ def cpu_baseline(step, torch, budget_s=20.0):
                       f"fp32 naive PyTorch layer, median"}
 
 
+def handoff_probe(torch):
+    """One kernel whose workgroups hand data to each other (write-through stores, arrival counter, bypassing
+    loads: csrc/stream_probe.hip) against the same work as two kernels, in graphs of ten, at the grid sizes and
+    partial-sum volumes of the n <= 4 backward (200 workgroups x 24 KB at B=320, C=1280; 480 at B=1280, C=2560)."""
+    from mhc import _lib
+
+    fn = _lib.lib.mhc_stream_probe
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
+                   ctypes.c_void_p]
+    rows = []
+    for blocks, per in ((200, 200 * 32), (200, 200 * 2), (480, 480 * 13), (480, 480 * 1), (1024, 1024 * 1)):
+        part = torch.zeros(blocks * per, dtype=torch.float32, device="cuda")
+        outs = [torch.zeros(blocks, dtype=torch.float32, device="cuda") for _ in range(2)]
+        sync = torch.zeros(3, dtype=torch.int32, device="cuda")
+
+        def chain(one, out, k=10):
+            cur = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            for _ in range(k):
+                for mode in ((7,) if one else (8, 9)):
+                    assert fn(mode, out.data_ptr(), part.data_ptr(), per * 4, blocks, sync.data_ptr(), cur) == 0
+        row = {"workgroups": blocks, "KB_per_workgroup": per * 4 / 1024}
+        for one in (False, True):
+            chain(one, outs[one], 1)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                chain(one, outs[one])
+            g.replay()
+            best_t = float("inf")
+            for _ in range(10):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(10):
+                    g.replay()
+                e1.record()
+                e1.synchronize()
+                best_t = min(best_t, e0.elapsed_time(e1) * 1e3 / 100)
+            row["one_kernel_us" if one else "two_kernels_us"] = round(best_t, 2)
+        row["results_equal"] = bool(torch.equal(outs[0], outs[1]))
+        row["gave_up"] = int(sync[2].item())
+        rows.append(row)
+    print(json.dumps({"handoff_probe": True, "protocol": "graphs of ten, best of 10 x 10 replays, HIP events", "rows": rows}))
+
+
 def stream_probe(torch):
     """Read-only / copy / write-only streaming rates of hand-written kernels (csrc/stream_probe.hip)."""
     from mhc import _lib
@@ -409,6 +454,10 @@ def main():
     ap.add_argument("--graph-steps", type=int, default=10,
                     help="steps captured into one HIP graph (a replay costs ~5 us by itself); 1 = one step per replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--handoff-probe", action="store_true",
+                    help="time one kernel whose workgroups exchange partial sums through memory (arrival counter, "
+                         "write-through stores) against the same work as two kernels: what a launch boundary costs "
+                         "next to an in-kernel grid-wide hand-off on this GPU")
     ap.add_argument("--stream-probe", action="store_true",
                     help="run the library's plain streaming kernels (read-only, copy, write-only; 16-byte accesses, "
                          "all CUs) over 128 MiB .. 2 GiB and print what this GPU delivers to each, HIP events on the "
@@ -428,6 +477,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if a.handoff_probe:
+        handoff_probe(torch)
+        return
     if a.stream_probe:
         stream_probe(torch)
         return

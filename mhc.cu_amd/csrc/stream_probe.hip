@@ -1,7 +1,7 @@
 // Streaming kernels that do nothing but move bytes: what this GPU delivers to a read-only, a copy
 // and a write-only pass over a large buffer.  They give the memory-bound kernels of the library a
 // measured ceiling next to the published 8 TB/s.  Not part of the layer path; exported for
-// bench.py --stream-probe only (no declaration in the public header).
+// bench.py --stream-probe and --handoff-probe only (no declaration in the public header).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -63,6 +63,57 @@ __global__ void probe_empty_kernel(uint32_t *sink) {
     if (sink == nullptr) __builtin_trap();  // never: the kernel has nothing to do
 }
 
+// Hand-off probe: what it costs to pass data between the workgroups of ONE kernel instead of between
+// two kernels.  Every workgroup writes `per` floats, all workgroups meet, every workgroup then sums its
+// slice of every workgroup's floats.  ONE: in one kernel - the floats leave with agent-scope relaxed atomic
+// stores (write-through, no cache write-back needed), one thread per workgroup counts its arrival with an
+// agent-scope atomic and polls the counter, the readers use agent-scope relaxed atomic loads; no fence
+// instruction anywhere.  The last workgroup to leave resets the counters, so launches need no host state.
+// The wait is bounded: a workgroup that gives up raises sync[2] and the results are garbage, but the kernel
+// ends.  PHASE 0 / 1: the same two halves as separate kernels with plain stores and loads.
+template <bool ONE, int PHASE>
+__global__ __launch_bounds__(256) void probe_handoff_kernel(float *part, float *out, unsigned *sync, int per) {
+    const int wg = blockIdx.x, N = gridDim.x, tid = threadIdx.x;
+    if (ONE || PHASE == 0) {
+        float *mine = part + (size_t)wg * per;
+        const float v = (float)(wg + 1);
+        for (int i = tid; i < per; i += 256) {
+            if (ONE) __hip_atomic_store(mine + i, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else mine[i] = v;
+        }
+    }
+    if (ONE) {
+        __builtin_amdgcn_s_waitcnt(0);  // every store of this wave has been acknowledged
+        __syncthreads();
+        if (tid == 0) {
+            __hip_atomic_fetch_add(sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned spins = 0;
+            while (__hip_atomic_load(sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)N) {
+                __builtin_amdgcn_s_sleep(1);
+                if (++spins > 2000000u) { sync[2] = 1; break; }
+            }
+            if (__hip_atomic_fetch_add(sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)N - 1) {
+                __hip_atomic_store(sync + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        __syncthreads();
+    }
+    if (ONE || PHASE == 1) {
+        const int w = per / N;  // this workgroup's slice of every producer: floats [wg*w, wg*w + w)
+        float s = 0.f;
+        for (int i = tid; i < N * w; i += 256) {
+            const float *p = part + (size_t)(i / w) * per + wg * w + i % w;
+            s += ONE ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *p;
+        }
+        for (int o = 32; o; o >>= 1) s += __shfl_xor(s, o);
+        __shared__ float sh[4];
+        if ((tid & 63) == 0) sh[tid >> 6] = s;
+        __syncthreads();
+        if (tid == 0) out[wg] = (sh[0] + sh[1]) + (sh[2] + sh[3]);
+    }
+}
+
 }  // namespace
 
 // mode 0 = read-only, 1 = copy, 2 = write-only, with the streaming (nt) hint on every access; 3, 4, 5 =
@@ -82,6 +133,18 @@ extern "C" __attribute__((visibility("default"))) int mhc_stream_probe(int mode,
     else if (mode == 4) probe_copy_kernel<4, false><<<grid, 256, 0, st>>>(s, d, words);
     else if (mode == 5) probe_write_kernel<false><<<grid, 256, 0, st>>>(d, words, 0x3f800000u);
     else if (mode == 6) probe_empty_kernel<<<grid, 256, 0, st>>>(static_cast<uint32_t *>(sink));  // launch floor
+    else if (mode >= 7 && mode <= 9) {
+        // hand-off probe: dst = blocks * (bytes / 4) floats of partial data, src = blocks floats of results (written),
+        // sink = 3 zeroed words (arrivals, departures, gave-up flag); bytes = per workgroup, a multiple of 4 * blocks;
+        // 7 = one kernel (blocks must all be resident: at most 8 per CU), 8 and 9 = its two halves as kernels
+        if (blocks <= 0 || blocks > 2048 || bytes % (4 * (size_t)blocks)) return (int)hipErrorInvalidValue;
+        float *part = static_cast<float *>(dst), *out = static_cast<float *>(const_cast<void *>(src));
+        unsigned *sync = static_cast<unsigned *>(sink);
+        const int per = (int)(bytes / 4);
+        if (mode == 7) probe_handoff_kernel<true, 0><<<blocks, 256, 0, st>>>(part, out, sync, per);
+        else if (mode == 8) probe_handoff_kernel<false, 0><<<blocks, 256, 0, st>>>(part, out, sync, per);
+        else probe_handoff_kernel<false, 1><<<blocks, 256, 0, st>>>(part, out, sync, per);
+    }
     else return (int)hipErrorInvalidValue;
     return (int)hipGetLastError();
 }
