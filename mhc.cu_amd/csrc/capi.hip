@@ -9,9 +9,8 @@
 #include "phase_profiler.h"
 #include "tuning.h"
 
-#include <stdint.h>
-
 #include <mutex>
+#include <stdint.h>
 
 using namespace mhc;
 
@@ -57,61 +56,6 @@ int ws_check(void *ws, size_t have, size_t need) {
     do {                                              \
         if ((expr) != hipSuccess) return MHC_ERR_LAUNCH; \
     } while (0)
-
-// ---- second stream for launches that share no output with their neighbours --------------------
-// Used only when the experiment hook asks for it (see mhc_layer_bwd_dynamic).
-// Per device a pool of non-blocking streams (default priority) with two events each, created by
-// the first forked call that is not inside a stream capture and kept until the process ends.  A caller stream is bound to one pool entry on first use and keeps it, so callers
-// on different streams never share a side stream; binding creates nothing and is therefore allowed
-// inside a capture.  fork() makes the side stream wait for everything enqueued on the caller's
-// stream so far; join() makes the caller's stream wait for the side stream.  Both are plain event
-// record / wait pairs, which a stream capture records as graph edges.  Without a pool (first call
-// of the process already inside a capture) or with every entry bound, the call runs unforked.
-struct SideStream { hipStream_t main, s; hipEvent_t fork, join; bool bound; };
-constexpr int kSideDevices = 16, kSidePool = 8;
-std::mutex g_side_mutex;
-SideStream g_side[kSideDevices][kSidePool];
-bool g_side_ready[kSideDevices];
-
-bool side_pool_create(int dev, hipStream_t probe, bool have_probe) {  // caller holds g_side_mutex
-    if (g_side_ready[dev]) return true;
-    if (have_probe) {
-        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(probe, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) return false;
-    }
-    for (int i = 0; i < kSidePool; i++) {
-        SideStream &e = g_side[dev][i];
-        if (hipStreamCreateWithFlags(&e.s, hipStreamNonBlocking) != hipSuccess ||
-            hipEventCreateWithFlags(&e.fork, hipEventDisableTiming) != hipSuccess ||
-            hipEventCreateWithFlags(&e.join, hipEventDisableTiming) != hipSuccess)
-            return false;  // what was created stays unused; the calls run unforked
-        e.bound = false;
-    }
-    g_side_ready[dev] = true;
-    return true;
-}
-
-SideStream *side_stream(hipStream_t main) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSideDevices) return nullptr;
-    std::lock_guard<std::mutex> lock(g_side_mutex);
-    if (!side_pool_create(dev, main, true)) return nullptr;
-    for (int i = 0; i < kSidePool; i++)
-        if (g_side[dev][i].bound && g_side[dev][i].main == main) return &g_side[dev][i];
-    for (int i = 0; i < kSidePool; i++)
-        if (!g_side[dev][i].bound) {
-            g_side[dev][i].bound = true;
-            g_side[dev][i].main = main;
-            return &g_side[dev][i];
-        }
-    return nullptr;
-}
-bool side_fork(SideStream *ss) {
-    return hipEventRecord(ss->fork, ss->main) == hipSuccess && hipStreamWaitEvent(ss->s, ss->fork, 0) == hipSuccess;
-}
-bool side_join(SideStream *ss) {
-    return hipEventRecord(ss->join, ss->s) == hipSuccess && hipStreamWaitEvent(ss->main, ss->join, 0) == hipSuccess;
-}
 
 // ---- dynamic workspace layout ----------------------------------------------------------------
 struct DynFwdWs { float *Ppart, *ssqpart, *agg; size_t bytes; };
@@ -333,25 +277,25 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     if (mfma) {
         // matrix cores: dphi and the projection term of dx (written into dx, then completed in place)
         S = proj_bwd_batch_splits(B, n, C);
-        // dphi = dP^T x shares no operand but dP and no output with dP phi and the dx kernel that
-        // follows it, so it can run on a second stream beside them (fork / join by events).  Measured on
-        // whole steps inside a captured graph of ten steps, where the edges cost nothing:
-        //   B=256 n=16 C=1280  111.6 -> 103.5 us     B=1024 n=8 C=1280  109.6 -> 106.5 us
-        //   B=512 n=12 C=1280  126.8 -> 129.2 us     B=128 n=32 C=1280  148.4 -> 154.6 us
-        // and in an eager chain the four event calls cost the host ~30 us (B=256 n=8: 49 -> 77 us per
-        // step).  No rule separates the wins from the losses, so the call stays on one stream; the
-        // experiment hook (kTuneNoFork = 2) forces the fork, which is how the numbers above were taken
-        // and how tests/test_gpu_runtime.py keeps the path alive.
-        const bool fork = tuning_get(kTuneNoFork) == 2;
-        SideStream *ss = fork ? side_stream(st) : nullptr;
-        if (ss && !side_fork(ss)) return MHC_ERR_LAUNCH;
-        if (ss) g_tuning[kTuneForkCount]++;
-        MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st,
-                                        ss ? ss->s : st));
-        MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
-                                     n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, ws.dt,
-                                     ws.dtpart, spg, B, n, C, st));
-        if (ss && !side_join(ss)) return MHC_ERR_LAUNCH;
+        if (proj_bwd_is_wide(n) && S == 1 && tuning_get(kTuneSeparateFinalize) != 1) {
+            // wide projection: the two products are separate kernels.  dphi goes last and its launch
+            // carries the batch sums (dw, dbias, dalpha) in a few extra workgroups, which run in the
+            // shadow of the dphi stores instead of as a launch of their own.
+            MHC_LAUNCH(launch_dxflat_wide(phi, ws.dPb, ws.BP, dx, B, n, C, st));
+            MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
+                                         n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, ws.dt,
+                                         ws.dtpart, spg, B, n, C, st));
+            const BatchSumArgs tail = make_batch_sums(ws.u, groups, C, f_inject ? nullptr : dw, ws.dtpart, groups,
+                                                      D, dbias, dalpha);
+            bool tail_taken = false;
+            MHC_LAUNCH(launch_dphi_large(x, ws.dPT, ws.BP, dphi, 1, B, n, C, &tail, &tail_taken, st));
+            if (tail_taken) return MHC_OK;
+        } else {
+            MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st));
+            MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
+                                         n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, ws.dt,
+                                         ws.dtpart, spg, B, n, C, st));
+        }
     } else if (gemm_f32_supported(x_dtype, phi_dtype, n, C)) {
         // exact float32 tier, wide projection: both products on the fp32 matrix cores; the projection
         // term of dx is written into dx and completed in place

@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 
+#include "batch_sums.h"
+
 namespace mhc {
 
 enum DType { kF32 = 0, kBF16 = 1 };
@@ -152,17 +154,20 @@ hipError_t launch_finalize(const float *u, int rows_u, int C, float *dw, const f
 // dxflat = dP phi (bf16 [B, nC]) in one pass over x and phi.  With S = proj_bwd_batch_splits() > 1
 // the S partial copies land in dphi_part and the caller's finalize launch sums them.
 bool proj_bwd_mfma_supported(int x_dtype, int phi_dtype, int C);
-// dphi_stream: the stream of the dphi product.  The two products share no operand but dP and no
-// output, so a caller may put dphi on a second stream that it has forked from `stream` and joins
-// later; with dphi_stream == stream the narrow shapes compute both in one launch.
-hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb, const void *dPT,
-                                 int BP, float *dphi_out, void *dxflat, int S, int B, int n, int C,
-                                 hipStream_t stream, hipStream_t dphi_stream);
-
 int proj_bwd_batch_splits(int B, int n, int C);
 hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,
                                 int BP, float *dphi, float *dphi_part, void *dxflat, int B, int n,
-                                int C, hipStream_t stream, hipStream_t dphi_stream);
+                                int C, hipStream_t stream);
+// Wide projections (proj_bwd_is_wide: more than 12 row tiles of 32, n > 18) run the two products as
+// two GEMM kernels that share no operand but dP and no output, so a caller may also launch them
+// apart.  `tail` (optional): batch sums that a few extra workgroups of the dphi launch compute
+// beside the product; they must depend on nothing that is still running.  *tail_taken tells whether
+// the launch had room for them (if not, the caller's finalize launch does them).
+bool proj_bwd_is_wide(int n);
+hipError_t launch_dxflat_wide(const void *phi, const void *dPb, int BP, void *dxflat, int B, int n, int C,
+                              hipStream_t stream);
+hipError_t launch_dphi_large(const void *x, const void *dPT, int BP, float *dphi_out, int S, int B, int n,
+                             int C, const BatchSumArgs *tail, bool *tail_taken, hipStream_t stream);
 
 // dphi[d, k] = sum_b dP[b, d] * x_flat[b, k].  `partial` holds dphi_batch_splits() copies of
 // dphi when that is > 1.

@@ -141,53 +141,19 @@ hipError_t launch_dphi(const void *x, int x_dtype, const float *dP, int DP, floa
 //   blocks [nblk_a, ...): 1024 columns each of the dphi batch-split partials [S, D*nC] -> dphi
 // --------------------------------------------------------------------------------------------
 struct FinalizeArgs {
-    const float *u; int rows_u, C; float *dw;
-    const float *dt; int rows_dt, D; float *dbias, *dalpha;
+    BatchSumArgs sums;
     const float *dphi_part; int S; size_t dphi_elems; float *dphi;
-    int nblk_a;
 };
 
 __global__ __launch_bounds__(1024) void finalize_kernel(FinalizeArgs a) {
-    // Batch sums in float64: dalpha (and the static coefficient gradients) are sums of B * n^2 terms of
-    // mixed sign whose total can be a hundred times smaller than the terms; a float32 running sum then
-    // loses what the 1e-5 parity tier needs.  The terms themselves stay float32.
-    __shared__ double red[16][65];
+    __shared__ double red[16 * 65];
     const int tid = threadIdx.x;
-    if ((int)blockIdx.x < a.nblk_a) {
-        const int cl = tid & 63, rg = tid >> 6;
-        const int col = blockIdx.x * 64 + cl;
-        const int ncol_u = a.dw ? a.C : 0;
-        const int ncols = ncol_u + a.D + 3;
-        double acc = 0.0;
-        if (col < ncols) {
-            const bool is_u = col < ncol_u;
-            const float *src = is_u ? a.u + col : a.dt + (col - ncol_u);
-            const int ld = is_u ? a.C : a.D + 3;
-            const int rows = is_u ? a.rows_u : a.rows_dt;
-            double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
-            int r = rg;
-            for (; r + 48 < rows; r += 64) {
-                const float t0 = src[(size_t)r * ld], t1 = src[(size_t)(r + 16) * ld];
-                const float t2 = src[(size_t)(r + 32) * ld], t3 = src[(size_t)(r + 48) * ld];
-                a0 += (double)t0; a1 += (double)t1; a2 += (double)t2; a3 += (double)t3;
-            }
-            for (; r < rows; r += 16) a0 += (double)src[(size_t)r * ld];
-            acc = (a0 + a1) + (a2 + a3);
-        }
-        red[rg][cl] = acc;
-        __syncthreads();
-        if (rg == 0 && col < ncols) {
-            double v = 0.0;
-#pragma unroll
-            for (int i = 0; i < 16; i++) v += red[i][cl];
-            if (col < ncol_u) a.dw[col] = (float)v;
-            else if (col - ncol_u < a.D) a.dbias[col - ncol_u] = (float)v;
-            else a.dalpha[col - ncol_u - a.D] = (float)v;
-        }
+    if ((int)blockIdx.x < a.sums.nblk) {
+        batch_sum_block<16>(a.sums, blockIdx.x, tid, red);
         return;
     }
     // dphi partial sums: one float per thread per 1024-column block (coalesced)
-    const size_t e = (size_t)(blockIdx.x - a.nblk_a) * 1024 + tid;
+    const size_t e = (size_t)(blockIdx.x - a.sums.nblk) * 1024 + tid;
     if (e < a.dphi_elems) {
         // all copies requested together (eight per round), added in split order
         float v = 0.f;
@@ -208,10 +174,10 @@ __global__ __launch_bounds__(1024) void finalize_kernel(FinalizeArgs a) {
 hipError_t launch_finalize(const float *u, int rows_u, int C, float *dw, const float *dt, int rows_dt,
                            int D, float *dbias, float *dalpha, const float *dphi_part, int S,
                            size_t dphi_elems, float *dphi, hipStream_t stream) {
-    const int ncols = (dw ? C : 0) + D + 3;
-    const int nblk_a = (ncols + 63) / 64;
+    const BatchSumArgs sums = make_batch_sums(u, rows_u, C, dw, dt, rows_dt, D, dbias, dalpha);
+    const int nblk_a = sums.nblk;
     const int nblk_b = S > 1 ? (int)((dphi_elems + 1023) / 1024) : 0;
-    FinalizeArgs a{u, rows_u, C, dw, dt, rows_dt, D, dbias, dalpha, dphi_part, S, dphi_elems, dphi, nblk_a};
+    FinalizeArgs a{sums, dphi_part, S, dphi_elems, dphi};
     finalize_kernel<<<nblk_a + nblk_b, 1024, 0, stream>>>(a);
     return hipGetLastError();
 }

@@ -305,20 +305,10 @@ static hipError_t launch_what(const ProjBwdArgs &a, int S, hipStream_t stream) {
     return hipGetLastError();
 }
 
-// One launch for both products, or (two streams given) one launch each.  The dxflat-only launch
-// ignores the batch split of dphi: it walks all samples.
-template <int NTK, int TPW, bool PHI_REGS>
-static hipError_t launch_shape(const ProjBwdArgs &a, int S, hipStream_t stream, hipStream_t dphi_stream) {
-    if (dphi_stream == stream) return launch_what<NTK, TPW, PHI_REGS, kProjBoth>(a, S, stream);
-    ProjBwdArgs ax = a;
-    ax.b_per_split = a.B;
-    if (hipError_t e = launch_what<NTK, TPW, PHI_REGS, kProjDx>(ax, 1, stream); e != hipSuccess) return e;
-    return launch_what<NTK, TPW, PHI_REGS, kProjDphi>(a, S, dphi_stream);
-}
 
 hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,
                                 int BP, float *dphi, float *dphi_part, void *dxflat, int B, int n,
-                                int C, hipStream_t stream, hipStream_t dphi_stream) {
+                                int C, hipStream_t stream) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
     const int S = proj_bwd_batch_splits(B, n, C);
     const int NTK = proj_bwd_ntk(B, n, C);
@@ -332,10 +322,12 @@ hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb,
     hipError_t e;
     // NTK == 1: dphi tiles per wave = ceil(NTD / 4); phi fragments in registers when 2*NTD <= 8.
     // Wide projections (more than 12 row tiles) run as two GEMM kernels that share no operand.
-    if (NTD <= 4) e = launch_shape<1, 1, true>(a, S, stream, dphi_stream);
-    else if (NTD <= 12) e = launch_shape<1, 3, false>(a, S, stream, dphi_stream);
-    else e = launch_proj_bwd_large(x, phi, dPb, dPT, BP, S > 1 ? dphi_part : dphi, dxflat, S, B, n, C, stream,
-                                   dphi_stream);
+    if (NTD <= 4) e = launch_what<1, 1, true, kProjBoth>(a, S, stream);
+    else if (NTD <= 12) e = launch_what<1, 3, false, kProjBoth>(a, S, stream);
+    else {
+        e = launch_dxflat_wide(phi, dPb, BP, dxflat, B, n, C, stream);
+        if (e == hipSuccess) e = launch_dphi_large(x, dPT, BP, S > 1 ? dphi_part : dphi, S, B, n, C, nullptr, nullptr, stream);
+    }
     return e;  // with S > 1 the caller's finalize launch sums the S partial copies
 }
 

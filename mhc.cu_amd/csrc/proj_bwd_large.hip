@@ -29,6 +29,8 @@ struct ProjBwdLargeArgs {
     bf16_t *dxflat;      // [B][nC]
     int B, BP, D, DP, nC, b_per_split;
     int tpw;             // row tiles per workgroup of the single-block dphi kernel
+    int tail_row;        // blockIdx.y of the extra row of workgroups that compute `tail` (-1: none)
+    BatchSumArgs tail;   // batch sums carried by the dphi launch (see launch_dphi_large)
 };
 
 // lane (n = lane & 31, kg = lane >> 5) gets tile[k0 + kg*8 + i][col0 + n], i = 0..7
@@ -50,9 +52,15 @@ __device__ __forceinline__ bf16x8_t pl_frag_t(const bf16_t *tile, int k0, int co
 // MFMAs and one accumulator is live at a time; otherwise TPW accumulators persist over the blocks.
 template <int TPW, bool SINGLE>
 __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
-    extern __shared__ bf16_t pl_lds[];
+    extern __shared__ __align__(16) bf16_t pl_lds[];
     bf16_t *x_s = pl_lds;  // [kPL_SB][kPL_LD]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if ((int)blockIdx.y == a.tail_row) {
+        // the extra row of the grid: its first workgroups do the batch sums, the others have nothing to do
+        if (blockIdx.z == 0 && (int)blockIdx.x < a.tail.nblk)
+            batch_sum_block<4>(a.tail, blockIdx.x, tid, reinterpret_cast<double *>(pl_lds));
+        return;
+    }
     const int row = lane & 31, kg = lane >> 5;
     const int k0 = blockIdx.x * kPL_KW;
     const int NTD = a.DP / 32;
@@ -299,22 +307,34 @@ __global__ __launch_bounds__(512 / MT) void dxflat_wide_kernel(ProjBwdLargeArgs 
     }
 }
 
-hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb, const void *dPT,
-                                 int BP, float *dphi_out, void *dxflat, int S, int B, int n, int C,
-                                 hipStream_t stream, hipStream_t dphi_stream) {
+bool proj_bwd_is_wide(int n) { return padded_D(n) / 32 > 12; }
+
+hipError_t launch_dxflat_wide(const void *phi, const void *dPb, int BP, void *dxflat, int B, int n, int C,
+                              hipStream_t stream) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
-    const int nblocks = (B + kPL_SB - 1) / kPL_SB;
-    const int bps = (nblocks + S - 1) / S * kPL_SB;
-    ProjBwdLargeArgs a{static_cast<const bf16_t *>(x), static_cast<const bf16_t *>(phi),
-                       static_cast<const bf16_t *>(dPb), static_cast<const bf16_t *>(dPT), dphi_out,
-                       static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, bps, 9};
-    const int slabs = (nC + kPL_KW - 1) / kPL_KW;
-    const int NTD = DP / 32;
+    ProjBwdLargeArgs a{nullptr, static_cast<const bf16_t *>(phi), static_cast<const bf16_t *>(dPb), nullptr,
+                       nullptr, static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, B, 0, -1, {}};
     // eight waves: 3 us faster than four at B=128 n=32 C=1280
     dxflat_wide_kernel<1><<<dim3((nC + kDxfCW - 1) / kDxfCW, (B + 127) / 128), 512,
                             sizeof(bf16_t) * 128 * kDxfLD, stream>>>(a);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    return hipGetLastError();
+}
+
+hipError_t launch_dphi_large(const void *x, const void *dPT, int BP, float *dphi_out, int S, int B, int n,
+                             int C, const BatchSumArgs *tail, bool *tail_taken, hipStream_t stream) {
+    const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
+    const int nblocks = (B + kPL_SB - 1) / kPL_SB;
+    const int bps = (nblocks + S - 1) / S * kPL_SB;
+    ProjBwdLargeArgs a{static_cast<const bf16_t *>(x), nullptr, nullptr, static_cast<const bf16_t *>(dPT),
+                       dphi_out, nullptr, B, BP, D, DP, nC, bps, 9, -1, {}};
+    const int slabs = (nC + kPL_KW - 1) / kPL_KW;
+    const int NTD = DP / 32;
+    // the batch sums ride along as one extra row of the grid when that row is long enough for them
+    const bool with_tail = tail && tail->nblk <= slabs;
+    if (tail_taken) *tail_taken = with_tail;
+    if (with_tail) a.tail = *tail;
+    const int extra = with_tail ? tail->nblk : 0;
+    hipError_t e;
     // the x block, later two operand tiles of 16 KB in the same memory
     const size_t smem = sizeof(bf16_t) * (kPL_SB * kPL_LD > 2 * 2 * 4096 ? kPL_SB * kPL_LD : 2 * 2 * 4096);
     if (bps <= kPL_SB) {
@@ -324,16 +344,20 @@ hipError_t launch_proj_bwd_large(const void *x, const void *phi, const void *dPb
         const int slots = 256 * 4;
         int tpw = NTD;
         for (int cand : {9, 12, 17})
-            if (cand < NTD && (long long)slabs * ((NTD + cand - 1) / cand) * S <= slots) { tpw = cand; break; }
+            if (cand < NTD && (long long)slabs * ((NTD + cand - 1) / cand) * S + extra <= slots) { tpw = cand; break; }
         if ((long long)slabs * S > slots) tpw = NTD < 9 ? NTD : 9;  // more than one round anyway
         a.tpw = tpw;
+        const int ytiles = (NTD + tpw - 1) / tpw;
+        if (with_tail) a.tail_row = ytiles;
         e = allow_dynamic_lds(&dphi_large_kernel<9, true>, smem);
         if (e != hipSuccess) return e;
-        dphi_large_kernel<9, true><<<dim3(slabs, (NTD + tpw - 1) / tpw, S), 256, smem, dphi_stream>>>(a);
+        dphi_large_kernel<9, true><<<dim3(slabs, ytiles + (with_tail ? 1 : 0), S), 256, smem, stream>>>(a);
     } else {
+        const int ytiles = (NTD + 2) / 3;
+        if (with_tail) a.tail_row = ytiles;
         e = allow_dynamic_lds(&dphi_large_kernel<3, false>, smem);
         if (e != hipSuccess) return e;
-        dphi_large_kernel<3, false><<<dim3(slabs, (NTD + 2) / 3, S), 256, smem, dphi_stream>>>(a);
+        dphi_large_kernel<3, false><<<dim3(slabs, ytiles + (with_tail ? 1 : 0), S), 256, smem, stream>>>(a);
     }
     return hipGetLastError();
 }

@@ -11,10 +11,10 @@ enum TuneKey {
     kTuneOnepassG = 1,      // samples per workgroup of the one-launch forward
     kTuneOnepassWaves = 2,  // waves per workgroup of the one-launch forward (4..8)
     kTuneSlabSplits = 3,    // batch splits of the slab backward
-    kTuneNoFork = 4,        // dphi beside the dx kernels on a second stream: 2 = always, anything else = never
+    kTuneSeparateFinalize = 4,  // wide projections: 1 = batch sums as a launch of their own, not inside the dphi launch
     kTuneSpare1 = 5,
     kTuneSpare2 = 6,
-    kTuneForkCount = 7,     // read-only use: backward calls that took the second stream so far (mhc_tuning_get)
+    kTuneSpare3 = 7,
     kTuneCount = 8
 };
 

@@ -69,11 +69,11 @@ def test_two_streams_with_separate_workspaces(shapes):
             assert torch.equal(got, want)
 
 
-@pytest.mark.parametrize("B,n,C", [(40, 32, 256), (70, 8, 512), (33, 12, 256)])
-def test_forked_backward_matches_the_single_stream_backward(B, n, C):
-    """The backward with its dphi product on a second stream of the library's own (forced through the
-    experiment hook; the default keeps one stream) against the same call kept on one stream, bit for
-    bit, repeated so that a missing fork or join edge would show as a race."""
+@pytest.mark.parametrize("B,n,C", [(40, 32, 256), (33, 20, 256), (128, 24, 64)])
+def test_batch_sums_inside_the_dphi_launch_match_the_separate_launch(B, n, C):
+    """Wide projections: dw, dbias and dalpha summed by extra workgroups of the dphi launch (the default)
+    against the same sums as a launch of their own (forced through the experiment hook), eagerly with
+    poisoned outputs and under graph replay."""
     import ctypes
 
     from mhc._lib import lib
@@ -81,22 +81,28 @@ def test_forked_backward_matches_the_single_stream_backward(B, n, C):
     lib.mhc_tuning_set.restype = ctypes.c_int
     lib.mhc_tuning_set.argtypes = [ctypes.c_int, ctypes.c_int]
     st = _bf16_step(B, n, C)
-    grads = lambda: [t.clone() for t in (st.dx, st.dw, st.dphi, st.dbias, st.dalpha)]
+    outs = (st.dx, st.dw, st.dphi, st.dbias, st.dalpha)
+    grads = lambda: [t.clone() for t in outs]
+
+    def check(what):
+        for name, a, b in zip(("dx", "dw", "dphi", "dbias", "dalpha"), ref, grads()):
+            if name in ("dx", "dphi"):
+                assert torch.equal(a, b), f"{what}: {name}"
+            else:  # float64 sums of the same float32 terms, grouped differently: equal up to the final rounding
+                torch.testing.assert_close(b, a, rtol=1e-6, atol=0, msg=f"{what}: {name}")
+
     try:
         assert lib.mhc_tuning_set(4, 1) == 0
         st.step()
         torch.cuda.synchronize()
         ref = grads()
-        assert lib.mhc_tuning_set(4, 2) == 0
-        for rep in range(10):
-            for t in (st.dx, st.dw, st.dphi, st.dbias, st.dalpha):
+        assert lib.mhc_tuning_set(4, 0) == 0
+        for rep in range(3):
+            for t in outs:
                 t.fill_(float("nan"))
             st.step()
-            st.dphi.sum()  # a consumer on the caller's stream right behind the call
             torch.cuda.synchronize()
-            for name, a, b in zip(("dx", "dw", "dphi", "dbias", "dalpha"), ref, grads()):
-                assert torch.equal(a, b), f"run {rep}: {name}"
-        # the same under capture: the fork and the join become edges of the graph
+            check(f"run {rep}")
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -108,16 +114,12 @@ def test_forked_backward_matches_the_single_stream_backward(B, n, C):
             st.step()
         scratch = torch.zeros(1 << 20, device="cuda")
         for rep in range(3):
-            for t in (st.dx, st.dw, st.dphi, st.dbias, st.dalpha):
+            for t in outs:
                 t.fill_(float("nan"))
             scratch.add_(1.0).sum().item()  # eager work + a host sync between replays
             graph.replay()
             torch.cuda.synchronize()
-            for name, a, b in zip(("dx", "dw", "dphi", "dbias", "dalpha"), ref, grads()):
-                assert torch.equal(a, b), f"replay {rep}: {name}"
-        lib.mhc_tuning_get.restype = ctypes.c_int
-        lib.mhc_tuning_get.argtypes = [ctypes.c_int]
-        assert lib.mhc_tuning_get(7) >= 12, "the forced fork was not taken"  # 10 eager calls + warm-up + capture
+            check(f"replay {rep}")
     finally:
         lib.mhc_tuning_set(4, 0)
 
