@@ -277,24 +277,35 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     if (mfma) {
         // matrix cores: dphi and the projection term of dx (written into dx, then completed in place)
         S = proj_bwd_batch_splits(B, n, C);
-        if (proj_bwd_is_wide(n) && S == 1 && tuning_get(kTuneSeparateFinalize) != 1) {
-            // wide projection: the two products are separate kernels.  dphi goes last and its launch
-            // carries the batch sums (dw, dbias, dalpha) in a few extra workgroups, which run in the
-            // shadow of the dphi stores instead of as a launch of their own.
-            MHC_LAUNCH(launch_dxflat_wide(phi, ws.dPb, ws.BP, dx, B, n, C, st));
-            MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
-                                         n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, ws.dt,
-                                         ws.dtpart, spg, B, n, C, st));
-            const BatchSumArgs tail = make_batch_sums(ws.u, groups, C, f_inject ? nullptr : dw, ws.dtpart, groups,
-                                                      D, dbias, dalpha);
-            bool tail_taken = false;
-            MHC_LAUNCH(launch_dphi_large(x, ws.dPT, ws.BP, dphi, 1, B, n, C, &tail, &tail_taken, st));
-            if (tail_taken) return MHC_OK;
+        // From D > 128 on the two products run as launches of their own (they share no operand but dP
+        // and no output): dP phi first, then the dx kernel that consumes it, dphi = dP^T x last.  The
+        // last launch carries the batch sums (dw, dbias, dalpha) in an extra row of workgroups, which
+        // run in the shadow of the dphi stores instead of as a launch of their own.  Measured on whole
+        // steps, graphs of ten (one launch for both products + finalize launch -> apart + carried sums):
+        //   B=256 n=8   47.7 -> 48.8 us (not taken)    B=256 n=10   79.8 -> 80.0 (not taken)
+        //   B=512 n=12 126.6 -> 125.9    B=256 n=13 101.6 -> 96.6    B=256 n=16 111.9 -> 104.4
+        //   B=256 n=18 127.5 -> 119.0    B=128 n=32 148.6 -> 145.8 (always two product kernels; sums carried)
+        const bool wide = proj_bwd_is_wide(n);
+        const int hook = tuning_get(kTuneProjApart);
+        const bool apart = wide || (hook ? hook == 2 : proj_bwd_products_apart(n));
+        if (apart) {
+            if (wide) MHC_LAUNCH(launch_dxflat_wide(phi, ws.dPb, ws.BP, dx, B, n, C, st));
+            else MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st, kProjPartDx));
         } else {
             MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st));
-            MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
-                                         n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, ws.dt,
-                                         ws.dtpart, spg, B, n, C, st));
+        }
+        MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
+                                     n, q, ws.s1, ws.cx, ws.dP, DP, nullptr, 0, dx, dx, df, ws.u, ws.dt,
+                                     ws.dtpart, spg, B, n, C, st));
+        if (apart) {
+            const BatchSumArgs sums = make_batch_sums(ws.u, groups, C, f_inject ? nullptr : dw, ws.dtpart, groups,
+                                                      D, dbias, dalpha);
+            const BatchSumArgs *tail = S == 1 && tuning_get(kTuneSeparateFinalize) != 1 ? &sums : nullptr;
+            bool tail_taken = false;
+            if (wide) MHC_LAUNCH(launch_dphi_large(x, ws.dPT, ws.BP, S > 1 ? ws.dphi_part : dphi, S, B, n, C, tail, &tail_taken, st));
+            else MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st,
+                                                 kProjPartDphi, tail, &tail_taken));
+            if (tail_taken) return MHC_OK;
         }
     } else if (gemm_f32_supported(x_dtype, phi_dtype, n, C)) {
         // exact float32 tier, wide projection: both products on the fp32 matrix cores; the projection

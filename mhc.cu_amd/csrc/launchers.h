@@ -155,14 +155,20 @@ hipError_t launch_finalize(const float *u, int rows_u, int C, float *dw, const f
 // the S partial copies land in dphi_part and the caller's finalize launch sums them.
 bool proj_bwd_mfma_supported(int x_dtype, int phi_dtype, int C);
 int proj_bwd_batch_splits(int B, int n, int C);
+// part: both products in one launch, or one of them (they share no operand but dP and no output, so a
+// caller may launch them apart, e.g. around the dx kernel that consumes dxflat).  `tail` (optional,
+// with kProjPartDphi): batch sums that a few extra workgroups of the dphi launch compute beside the
+// product; they must depend on nothing that is still running.  *tail_taken tells whether the launch
+// had room for them (if not, the caller's finalize launch does them).
+enum ProjBwdPart { kProjPartBoth = 0, kProjPartDphi = 1, kProjPartDx = 2 };
 hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,
                                 int BP, float *dphi, float *dphi_part, void *dxflat, int B, int n,
-                                int C, hipStream_t stream);
-// Wide projections (proj_bwd_is_wide: more than 12 row tiles of 32, n > 18) run the two products as
-// two GEMM kernels that share no operand but dP and no output, so a caller may also launch them
-// apart.  `tail` (optional): batch sums that a few extra workgroups of the dphi launch compute
-// beside the product; they must depend on nothing that is still running.  *tail_taken tells whether
-// the launch had room for them (if not, the caller's finalize launch does them).
+                                int C, hipStream_t stream, int part = kProjPartBoth,
+                                const BatchSumArgs *tail = nullptr, bool *tail_taken = nullptr);
+// n <= 18: whether the two products are faster apart (measured: from D > 128 on)
+bool proj_bwd_products_apart(int n);
+// Wide projections (more than 12 row tiles of 32, n > 18) always run the two products as two GEMM
+// kernels, launched through the two functions below; tail as above.
 bool proj_bwd_is_wide(int n);
 hipError_t launch_dxflat_wide(const void *phi, const void *dPb, int BP, void *dxflat, int B, int n, int C,
                               hipStream_t stream);

@@ -30,6 +30,8 @@ struct ProjBwdArgs {
     float *dphi;         // [S][D][nC]  (S = gridDim.y batch splits)
     bf16_t *dxflat;      // [B][nC]
     int B, BP, D, DP, nC, b_per_split;
+    int tail_row;        // kProjDphi only: blockIdx.y of the extra row of workgroups that compute `tail` (-1: none)
+    BatchSumArgs tail;   // batch sums carried by the dphi launch
 };
 
 // Transposed fragment: lane (n = lane & 31, kg = lane >> 5) gets tile[k0 + kg*8 + i][col0 + n], i = 0..7
@@ -38,9 +40,9 @@ __device__ __forceinline__ bf16x8_t lds_frag_t(const bf16_t *tile, int ld, int k
 }
 
 // WHAT: kProjBoth = both products in one pass; kProjDphi / kProjDx = one of them (they share no
-// operand but dP: dphi needs x and dP^T, dxflat needs phi and dP), for callers that run the two
-// side by side on two streams.
-enum { kProjBoth = 0, kProjDphi = 1, kProjDx = 2 };
+// operand but dP: dphi needs x and dP^T, dxflat needs phi and dP), for callers that launch the two
+// apart.
+enum { kProjBoth = kProjPartBoth, kProjDphi = kProjPartDphi, kProjDx = kProjPartDx };
 
 template <int NTK, int TPW, bool PHI_REGS, int WHAT = kProjBoth>
 __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
@@ -50,10 +52,17 @@ __global__ __launch_bounds__(256) void proj_bwd_mfma_kernel(ProjBwdArgs a) {
     constexpr int LD = KW + 8;           // LDS row pitch (elements), keeps 16-byte alignment
     constexpr int SBR = 32 * NSB;        // samples per block
     constexpr int CPR = KW / 8;          // 16-byte chunks per tile row
-    extern __shared__ bf16_t lds_bf[];
+    extern __shared__ __align__(16) bf16_t lds_bf[];
     bf16_t *phi_s = lds_bf;                       // [DP][LD]
     bf16_t *x_s = phi_s + (size_t)a.DP * LD;      // [SBR][LD]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if constexpr (WHAT == kProjDphi) {
+        if ((int)blockIdx.y == a.tail_row) {
+            // the extra row of the grid: its first workgroups do the batch sums, the others have nothing to do
+            if ((int)blockIdx.x < a.tail.nblk) batch_sum_block<4>(a.tail, blockIdx.x, tid, reinterpret_cast<double *>(lds_bf));
+            return;
+        }
+    }
     const int pwg = blockIdx.y * gridDim.x + blockIdx.x;
     (void)pwg;
     MHC_PHASE_ZERO(kPhaseProjBwd, pwg);
@@ -300,15 +309,17 @@ static hipError_t launch_what(const ProjBwdArgs &a, int S, hipStream_t stream) {
         if (e != hipSuccess) return e;
     }
     const int slabs = (a.nC + 32 * NTK - 1) / (32 * NTK);
-    dim3 grid(NTK == 1 ? round_up(slabs, 16) : slabs, S);
+    dim3 grid(NTK == 1 ? round_up(slabs, 16) : slabs, S + (WHAT == kProjDphi && a.tail_row >= 0 ? 1 : 0));
     kern<<<grid, 256, smem, stream>>>(a);
     return hipGetLastError();
 }
 
 
+bool proj_bwd_products_apart(int n) { return padded_D(n) / 32 > 4; }
+
 hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb, const void *dPT,
                                 int BP, float *dphi, float *dphi_part, void *dxflat, int B, int n,
-                                int C, hipStream_t stream) {
+                                int C, hipStream_t stream, int part, const BatchSumArgs *tail, bool *tail_taken) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
     const int S = proj_bwd_batch_splits(B, n, C);
     const int NTK = proj_bwd_ntk(B, n, C);
@@ -317,16 +328,28 @@ hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb,
     const int bps = (nblocks + S - 1) / S * sbr;
     ProjBwdArgs a{static_cast<const bf16_t *>(x), static_cast<const bf16_t *>(phi),
                   static_cast<const bf16_t *>(dPb), static_cast<const bf16_t *>(dPT),
-                  S > 1 ? dphi_part : dphi, static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, bps};
+                  S > 1 ? dphi_part : dphi, static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, bps, -1, {}};
     const int NTD = DP / 32;
     hipError_t e;
+    if (tail_taken) *tail_taken = false;
+    if (NTD <= 12 && part == kProjDphi && tail && tail->nblk <= (nC + 32 * NTK - 1) / (32 * NTK) && NTK == 1) {
+        a.tail = *tail;
+        a.tail_row = S;
+        if (tail_taken) *tail_taken = true;
+    }
     // NTK == 1: dphi tiles per wave = ceil(NTD / 4); phi fragments in registers when 2*NTD <= 8.
     // Wide projections (more than 12 row tiles) run as two GEMM kernels that share no operand.
-    if (NTD <= 4) e = launch_what<1, 1, true, kProjBoth>(a, S, stream);
-    else if (NTD <= 12) e = launch_what<1, 3, false, kProjBoth>(a, S, stream);
+    if (part == kProjDx) { a.b_per_split = B; }
+    if (NTD <= 4) e = part == kProjBoth ? launch_what<1, 1, true, kProjBoth>(a, S, stream)
+                    : part == kProjDx ? launch_what<1, 1, true, kProjDx>(a, 1, stream)
+                                      : launch_what<1, 1, true, kProjDphi>(a, S, stream);
+    else if (NTD <= 12) e = part == kProjBoth ? launch_what<1, 3, false, kProjBoth>(a, S, stream)
+                            : part == kProjDx ? launch_what<1, 3, false, kProjDx>(a, 1, stream)
+                                              : launch_what<1, 3, false, kProjDphi>(a, S, stream);
     else {
         e = launch_dxflat_wide(phi, dPb, BP, dxflat, B, n, C, stream);
         if (e == hipSuccess) e = launch_dphi_large(x, dPT, BP, S > 1 ? dphi_part : dphi, S, B, n, C, nullptr, nullptr, stream);
+        (void)part;  // wide shapes: callers that want the products apart use the two launchers themselves
     }
     return e;  // with S > 1 the caller's finalize launch sums the S partial copies
 }

@@ -11,8 +11,8 @@ enum TuneKey {
     kTuneOnepassG = 1,      // samples per workgroup of the one-launch forward
     kTuneOnepassWaves = 2,  // waves per workgroup of the one-launch forward (4..8)
     kTuneSlabSplits = 3,    // batch splits of the slab backward
-    kTuneSeparateFinalize = 4,  // wide projections: 1 = batch sums as a launch of their own, not inside the dphi launch
-    kTuneSpare1 = 5,
+    kTuneSeparateFinalize = 4,  // 1 = batch sums always as a launch of their own, never inside the dphi launch
+    kTuneProjApart = 5,     // n <= 18 projection backward: 1 = both products in one launch, 2 = two launches
     kTuneSpare2 = 6,
     kTuneSpare3 = 7,
     kTuneCount = 8

@@ -69,9 +69,39 @@ def test_two_streams_with_separate_workspaces(shapes):
             assert torch.equal(got, want)
 
 
-@pytest.mark.parametrize("B,n,C", [(40, 32, 256), (33, 20, 256), (128, 24, 64)])
+@pytest.mark.parametrize("B,n,C", [(70, 8, 512), (33, 10, 256), (64, 12, 256), (300, 16, 128)])
+def test_projection_backward_products_apart_match_one_launch(B, n, C):
+    """dphi = dP^T x and dP phi as two launches around the dx kernel (the default from n = 11 on) against
+    both in one launch, each forced through the experiment hook: same gradients bit for bit."""
+    import ctypes
+
+    from mhc._lib import lib
+
+    lib.mhc_tuning_set.restype = ctypes.c_int
+    lib.mhc_tuning_set.argtypes = [ctypes.c_int, ctypes.c_int]
+    st = _bf16_step(B, n, C)
+    outs = (st.dx, st.dw, st.dphi, st.dbias, st.dalpha)
+    try:
+        assert lib.mhc_tuning_set(4, 1) == 0  # batch sums in their own launch both times
+        res = []
+        for mode in (1, 2):
+            assert lib.mhc_tuning_set(5, mode) == 0
+            for t in outs:
+                t.fill_(float("nan"))
+            st.step()
+            torch.cuda.synchronize()
+            res.append([t.clone() for t in outs])
+        for name, a, b in zip(("dx", "dw", "dphi", "dbias", "dalpha"), *res):
+            assert torch.isfinite(a).all(), name
+            assert torch.equal(a, b), name
+    finally:
+        lib.mhc_tuning_set(4, 0)
+        lib.mhc_tuning_set(5, 0)
+
+
+@pytest.mark.parametrize("B,n,C", [(40, 32, 256), (33, 20, 256), (128, 24, 64), (33, 12, 256), (70, 16, 128)])
 def test_batch_sums_inside_the_dphi_launch_match_the_separate_launch(B, n, C):
-    """Wide projections: dw, dbias and dalpha summed by extra workgroups of the dphi launch (the default)
+    """From n = 11 on: dw, dbias and dalpha summed by extra workgroups of the dphi launch (the default)
     against the same sums as a launch of their own (forced through the experiment hook), eagerly with
     poisoned outputs and under graph replay."""
     import ctypes
