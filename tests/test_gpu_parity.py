@@ -336,6 +336,9 @@ _KEPT_CASES = [(260, 2, 100, 20, False, False, False), (1, 32, 1, 1, True, False
 _KEPT_CASES += [(3, 4, 32768, 20, True, True, False), (2, 32, 32768, 20, True, True, False),
                 (3, 8, 20000, 20, True, True, False), (33, 1, 32768, 20, False, False, False),
                 (3, 9, 16384, 20, True, False, False), (3, 4, 12296, 20, False, True, False)]
+# 11 <= n <= 18 with a large batch: the two projection-backward products as launches of their own, with batch
+# splits (the finalize launch sums the dphi copies) and, in the second case, without dw
+_KEPT_CASES += [(2000, 12, 32, 20, True, True, False), (3000, 16, 32, 20, True, True, True)]
 
 
 @pytest.mark.parametrize("B,n,C,T,dyn,bf16,inject", _random_cases(40, seed=2024) + _KEPT_CASES)
