@@ -155,17 +155,18 @@ __global__ __launch_bounds__(1024) void finalize_kernel(FinalizeArgs a) {
     // dphi partial sums: one float per thread per 1024-column block (coalesced)
     const size_t e = (size_t)(blockIdx.x - a.sums.nblk) * 1024 + tid;
     if (e < a.dphi_elems) {
-        // all copies requested together (eight per round), added in split order
+        // all copies requested together (sixteen per round: one round trip for the usual 8 to 13
+        // splits), added in split order
         float v = 0.f;
-        for (int s0 = 0; s0 < a.S; s0 += 8) {
-            float t[8];
+        for (int s0 = 0; s0 < a.S; s0 += 16) {
+            float t[16];
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
+            for (int u = 0; u < 16; u++) {
                 const int s = s0 + u < a.S ? s0 + u : a.S - 1;
                 t[u] = __builtin_nontemporal_load(a.dphi_part + (size_t)s * a.dphi_elems + e);
             }
 #pragma unroll
-            for (int u = 0; u < 8; u++) v += s0 + u < a.S ? t[u] : 0.f;
+            for (int u = 0; u < 16; u++) v += s0 + u < a.S ? t[u] : 0.f;
         }
         a.dphi[e] = v;
     }
