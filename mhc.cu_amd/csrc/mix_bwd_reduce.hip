@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
         const int c = c0 + e;
         if (r0 < n && c < n) {
             const int di = 2 * n + r0 * n + c;
-            const float dtr = d[e] * E[e];
+            const float dtr = d[e];  // the Sinkhorn backward hands back the gradient of the logits
             dt[di] = dtr;
             dpw.put(di, dtr * al2 * rinv);
             S2 += dtr * Pb[di];
@@ -386,7 +386,7 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
         if constexpr (GRAM) MHC_PHASE_ADD(kPhaseGramSmall, pwg_r, 5, rclk);
         if (mv) {
             const int di = 2 * n + r0 * n + c0;
-            const float dtr = d[0] * E;
+            const float dtr = d[0];  // the Sinkhorn backward hands back the gradient of the logits
             dt[di] = dtr;
             dpw.put(di, dtr * al2 * rinv);
             S2 = dtr * pres;
@@ -1053,7 +1053,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
         const int c = c0 + e;
         if (r0 < n && c < n) {
             const int di = 2 * n + r0 * n + c;
-            const float dtr = d[e] * E[e];
+            const float dtr = d[e];  // the Sinkhorn backward hands back the gradient of the logits
             dt[di] = dtr;
             dpw.put(di, dtr * al2 * rinv);
             S2 += dtr * pres[e];

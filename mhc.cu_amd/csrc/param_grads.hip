@@ -218,7 +218,7 @@ __global__ __launch_bounds__(256) void coef_bwd_static_kernel(const float *__res
     SK::template backward<true>(E, d, u, v, T, lds, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
-        if (r0 < n && c0 + e < n) dH_res[r0 * n + c0 + e] = d[e] * E[e];
+        if (r0 < n && c0 + e < n) dH_res[r0 * n + c0 + e] = d[e];  // gradient of the logits
 }
 
 hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const float *Hpost,

@@ -144,9 +144,16 @@ template <int NP> struct SkSmall {
     // one footprint for every layout: [T + 1][2][NP] (slot T is used by SkWg only)
     __host__ __device__ static constexpr int state_floats(int T) { return 2 * (T + 1) * NP; }
 
-    // d: in = dL/dM, out = dL/dE.  m: the final iterate from forward (destroyed).  The reverse
-    // sweep rebuilds the iterates it needs by undoing the scalings with the saved denominators
-    // (Out_t = m, R_t = Out_t s_t, Out_{t-1} = R_t rho_t) instead of reading stored copies.
+    // d: in = dL/dM, out = dL/dlogits (= dL/dE o E).  m: the final iterate from forward (destroyed).
+    // The reverse sweep runs on the PRODUCT p = (gradient o iterate) instead of on the gradient: through
+    // a normalisation Y = X / (sum X + eps) the gradient is dX = (dY - sum(dY o Y)) / den, and the product
+    // with the iterate before it is dX o X = (dY - sum(dY o Y)) o Y = p - sum(p) Y.  So one half-step is
+    //     p <- p - allreduce(p) * iterate
+    // with no division and no reciprocal; the iterates are rebuilt by undoing the scalings with the saved
+    // denominators (Out_t = m, R_t = Out_t s_t, Out_{t-1} = R_t rho_t), a chain of its own beside the
+    // one that carries p.  The dependent chain of an iteration is two all-reduces and two fused
+    // multiply-adds.  After the last step the iterate is E itself and p = dL/dE o E, which is what every
+    // caller wants.  PRECISE is kept for the callers' template argument; both tiers compute the same.
     template <bool PRECISE = false>
     __device__ static __forceinline__ void backward(float (&d)[EPL], float (&m)[EPL], int T,
                                                     const float *sc, int lane) {
@@ -158,13 +165,12 @@ template <int NP> struct SkSmall {
             rs = sc[(t * kRec) * kWave + lane];
             cs = sc[(t * kRec + 1) * kWave + lane];
         };
+        float p = d[0] * m[0];
         auto step = [&](float rs, float cs) {
-            const float cdot = col_allreduce(d[0] * m[0]);
-            const float dR = PRECISE ? (d[0] - cdot) / cs : (d[0] - cdot) * fast_rcp(cs);
-            m[0] *= cs;  // R_t
-            const float rdot = row_allreduce(dR * m[0]);
-            d[0] = PRECISE ? (dR - rdot) / rs : (dR - rdot) * fast_rcp(rs);
-            m[0] *= rs;  // Out_{t-1}
+            p = __builtin_fmaf(-col_allreduce(p), m[0], p);  // through the column normalisation: Out_t
+            m[0] *= cs;                                      // R_t
+            p = __builtin_fmaf(-row_allreduce(p), m[0], p);  // through the row normalisation
+            m[0] *= rs;                                      // Out_{t-1}
         };
         float rs0, cs0, rs1, cs1;
         int t = T - 1;
@@ -174,19 +180,14 @@ template <int NP> struct SkSmall {
             step(rs0, cs0);
             fetch(--t, rs0, cs0);
         }
-        // (the scheduling barriers keep the reciprocals of the values in flight, which do not depend
-        // on the chain, from being moved up into the step before and dragging the wait with them)
         for (; t >= 1; t -= 2) {
             fetch(t - 1, rs1, cs1);
-            __builtin_amdgcn_sched_barrier(0);
             step(rs0, cs0);
-            __builtin_amdgcn_sched_barrier(0);
             fetch(t - 2, rs0, cs0);
-            __builtin_amdgcn_sched_barrier(0);
             step(rs1, cs1);
-            __builtin_amdgcn_sched_barrier(0);
         }
         sk_chain_end();
+        d[0] = p;
     }
     __host__ __device__ static constexpr int scaling_floats(int T) { return T * kRec * kWave; }
 };
@@ -359,37 +360,45 @@ template <int NP> struct SkWg {
     }
     __host__ __device__ static constexpr int state_floats(int T) { return 2 * (T + 1) * NP; }
 
-    // d: in = dL/dM, out = dL/dE.  E, u, v, LDS contents: as left by forward() (u and v are
-    // destroyed).
+    // d: in = dL/dM, out = dL/dlogits (= dL/dE o E).  E, u, v, LDS contents: as left by forward() (u and
+    // v are destroyed).  Product form as in SkSmall::backward: p = gradient o iterate, one half-step is
+    // p <- p - allreduce(p) * iterate, no divisions; the iterate u E v is unwound with the saved
+    // denominators (v *= s, u *= rho).  Both tiers compute the same.
     template <bool PRECISE = true>
     __device__ static __forceinline__ void backward(const float (&E)[EPL], float (&d)[EPL], float u,
                                                     float (&v)[EPL], int T, float *lds, int tid) {
         float *cw = lds;  // the transpose tile is dead after forward()
         const float *rho = lds + kTile + 2 * NP, *s = rho + T * NP;
         const int r = row(tid), c0 = col0(tid);
+        float p[EPL], W[EPL];  // W = E v: the iterate without its row scaling
+#pragma unroll
+        for (int e = 0; e < EPL; e++) {
+            W[e] = E[e] * v[e];
+            p[e] = d[e] * (u * W[e]);
+        }
         for (int t = T - 1; t >= 0; t--) {
-            // column dots with the iterate after column step t: Out = u E v
-            float cd[EPL];
-#pragma unroll
-            for (int e = 0; e < EPL; e++) cd[e] = d[e] * u * E[e];
-            col_allreduce(cd, cw + (t & 1) * 4 * NP, tid);
-            float z = 0.f, sc[EPL];
+            float sc[EPL];
             ld_vec(s + t * NP + c0, sc);
-#pragma unroll
-            for (int e = 0; e < EPL; e++) {
-                d[e] -= cd[e] * v[e];
-                z += d[e] * E[e] * v[e];
-            }
-            const float rdot = u * seg_allreduce(z);
             const float rr = rho[t * NP + r];
-            const float rri = PRECISE ? 0.f : fast_rcp(rr);
+            // through column step t: iterate Out = u E v
+            float cd[EPL], out[EPL];
+#pragma unroll
+            for (int e = 0; e < EPL; e++) { cd[e] = p[e]; out[e] = u * W[e]; W[e] *= sc[e]; }
+            col_allreduce(cd, cw + (t & 1) * 4 * NP, tid);
+            float z = 0.f, rt[EPL];
 #pragma unroll
             for (int e = 0; e < EPL; e++) {
-                d[e] = PRECISE ? (d[e] / sc[e] - rdot) / rr : (d[e] * fast_rcp(sc[e]) - rdot) * rri;
-                v[e] *= sc[e];
+                p[e] = __builtin_fmaf(-cd[e], out[e], p[e]);
+                rt[e] = u * W[e];  // through row step t: iterate R = u E (v s)
+                z += p[e];
             }
+            const float rdot = seg_allreduce(z);
+#pragma unroll
+            for (int e = 0; e < EPL; e++) p[e] = __builtin_fmaf(-rdot, rt[e], p[e]);
             u *= rr;
         }
+#pragma unroll
+        for (int e = 0; e < EPL; e++) d[e] = p[e];
     }
 };
 
