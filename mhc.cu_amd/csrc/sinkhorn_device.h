@@ -2,7 +2,8 @@
 //
 // Semantics (reference: src/python/benchmarks/bench_layer.py:48-53 / :112-117): start from
 // E = exp(logits); T times: divide every row by (row sum + eps), then every column by
-// (column sum + eps).  The backward is the exact reverse sweep through all T iterations; only the
+// (column sum + eps).  The backward is the exact reverse sweep through all T iterations (carried on the
+// product gradient x iterate, which needs no division); only the
 // per-iteration denominators rho_t[r], s_t[c] are kept in LDS during the forward recompute, and
 // the iterates are rebuilt from them by undoing the scalings.
 //
@@ -201,7 +202,7 @@ template <int NP> struct SkSmall {
 // through LDS), so both the row sums and the column sums are an in-register dot product plus a
 // reduction over the LPR lanes of a DPP row; only the vectors u and v travel through LDS (one
 // barrier per half-step).  The denominators rho/s of every iteration stay in LDS.
-// backward(): one copy of the gradient; row dots inside a DPP row, column dots inside the wave
+// backward(): one copy of the product gradient x iterate; row sums inside a DPP row, column sums inside the wave
 // (DPP, v_permlane*_swap) and then across the 4 waves through a double-buffered LDS slot (one
 // barrier per iteration; keeping a transposed copy of the gradient as well needs two barriers and
 // measured 50 % slower); the scalings are unwound with the saved denominators (u *= rho, v *= s)
