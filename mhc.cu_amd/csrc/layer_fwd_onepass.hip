@@ -66,6 +66,7 @@ struct OnePassLds {
     }
 };
 
+constexpr int kOnePassWaves = 8;  // waves per workgroup (4..7 measured slower at every shape of the sweep)
 constexpr int kDppQuadBcast0 = 0x00, kDppQuadBcast1 = 0x55, kDppQuadBcast2 = 0xAA, kDppQuadBcast3 = 0xFF;
 
 template <typename TY, int GH>
@@ -74,7 +75,8 @@ __global__ __launch_bounds__(512) void layer_fwd_onepass_kernel(OnePassArgs a) {
     using SK = SkSmall<NP>;
     extern __shared__ __align__(16) unsigned char op_smem[];
     const int n = a.n, C = a.C, nC = n * C, G = a.G, D = n * n + 2 * n;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, NT = blockDim.x, NW = NT >> 6;
+    constexpr int NW = kOnePassWaves, NT = NW * 64;  // compile-time: the cross-wave sums below unroll without masks
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int b0 = blockIdx.x * G;
     const int Gv = min(G, a.B - b0);
     const int nch = C / 8, nchp = round_up(nch, 4);
@@ -458,7 +460,7 @@ bool layer_fwd_onepass_supported(int x_dtype, int phi_dtype, int B, int n, int C
     const int mode = tuning_get(kTuneOnepassOff);  // 0 = by cost, 1 = never, 2 = whenever the shape allows
     if (mode == 1) return false;
     if (x_dtype != kBF16 || phi_dtype != kBF16 || n > 4 || C % 8 != 0 || (n * C) % 64 != 0) return false;
-    if (OnePassLds(1, n * C, round_up(C / 8, 4), 8).total > 158 * 1024) return false;
+    if (OnePassLds(1, n * C, round_up(C / 8, 4), kOnePassWaves).total > 158 * 1024) return false;
     if (mode == 2) return true;
     (void)B;
     return 2ll * (n * n + 2 * n) * n * C <= 256 * 1024;
@@ -469,8 +471,7 @@ hipError_t launch_layer_fwd_onepass(const void *x, const void *w, int w_dtype, c
                                     float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
                                     float *sk_state, int B, int n, int C, int T, float eps, hipStream_t stream) {
     const int G = onepass_group(B, n, C);
-    int NW = tuning_get(kTuneOnepassWaves);
-    if (NW < 4 || NW > 8) NW = 8;
+    constexpr int NW = kOnePassWaves;
     OnePassArgs a{static_cast<const bf16_t *>(x), w, static_cast<const bf16_t *>(f_inject), y,
                   static_cast<const bf16_t *>(phi), alpha, bias, Hpre, Hpost, M, P, r, q,
                   w_dtype == kBF16, B, n, C, T, G, eps, sk_state};
