@@ -433,6 +433,23 @@ def stream_probe(torch):
                 e1.synchronize()
                 best_t = min(best_t, e0.elapsed_time(e1) * 1e3 / 100)
             floor[f"{name}_{blocks}_workgroups"] = round(best_t, 2)
+    # what ONE workgroup pulls out of the L2 when all workgroups stream the same small matrix (phi of the
+    # one-launch forward): 20 passes inside one launch, so the kernel start is amortised
+    pieces = {}
+    for nC, blocks in ((5120, 160), (10240, 256)):
+        phi = torch.ones(24 * nC, dtype=torch.bfloat16, device="cuda")
+        run = lambda: fn(10, phi.data_ptr(), None, 24 * nC * 2, blocks, sink.data_ptr(), stream)
+        assert run() == 0
+        best_t = float("inf")
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            assert run() == 0
+            e1.record()
+            e1.synchronize()
+            best_t = min(best_t, e0.elapsed_time(e1) * 1e-3 / 20)
+        pieces[f"phi_24x{nC}_{blocks}_workgroups"] = {"us_per_pass": round(best_t * 1e6, 2),
+                                                      "GB/s_per_workgroup": round(24 * nC * 2 / best_t / 1e9, 1)}
     best = {}
     for r in rows:
         key = (r["kernel"], r["MiB"], r["cache"])
@@ -440,7 +457,7 @@ def stream_probe(torch):
             best[key] = r
     print(json.dumps({"stream_probe": True, "protocol": "cold: 512 MiB fill before every timed launch; warm: back to back; median of 10, "
                       "HIP events on the launch stream", "rows": rows,
-                      "empty_kernel_us_per_launch": floor, "ceiling_GBs": {f"{k[0]}_{k[1]}MiB_{k[2]}": round(v["GB/s"], 1) for k, v in sorted(best.items())}}))
+                      "empty_kernel_us_per_launch": floor, "row_piece_stream_per_workgroup": pieces, "ceiling_GBs": {f"{k[0]}_{k[1]}MiB_{k[2]}": round(v["GB/s"], 1) for k, v in sorted(best.items())}}))
 
 
 def main():

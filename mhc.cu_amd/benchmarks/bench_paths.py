@@ -1,8 +1,8 @@
 #!/usr/bin/env python3
 """Two comparisons behind launch-path decisions of the library, each printed as a table.
 
-  --forward-paths   dynamic-H bf16 layer, forward alone (batched HIP events) and whole
-                    forward+backward step (graph replays): the two-launch forward (split-K
+  --forward-paths   dynamic-H bf16 layer, forward alone and whole forward+backward step (both as
+                    graphs of ten, like bench.py): the two-launch forward (split-K
                     projection, then the fused coefficient + mix kernel) against the one-launch
                     forward (csrc/layer_fwd_onepass.hip), forced through the library's experiment
                     hook mhc_tuning_set(0, 1 | 2).  The library's default takes the one-launch
@@ -42,6 +42,9 @@ def _events(fn, reps):
     return e0.elapsed_time(e1) / reps * 1e3
 
 
+_GRAPH_STEPS = 10  # steps per graph replay, as in bench.py: a replay costs ~5 us by itself
+
+
 def _graph(step):
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -51,7 +54,8 @@ def _graph(step):
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g):
-        step()
+        for _ in range(_GRAPH_STEPS):
+            step()
     g.replay()
     torch.cuda.synchronize()
     return g
@@ -75,10 +79,10 @@ def forward_paths(reps):
                     r = []
                     for mode in (1, 2):
                         lib.mhc_tuning_set(0, mode)
-                        r.append(_events(step.forward, reps))
+                        r.append(_events(_graph(step.forward).replay, reps // 2) / _GRAPH_STEPS)
                     for mode in (1, 2):
                         lib.mhc_tuning_set(0, mode)
-                        r.append(_events(_graph(step.step).replay, reps))
+                        r.append(_events(_graph(step.step).replay, reps // 2) / _GRAPH_STEPS)
                     print("%5d %3d %5d %8.0f | %8.1f %8.1f | %9.1f %9.1f" %
                           (B, n, C, 2 * (n * n + 2 * n) * n * C / 1024, *r), flush=True)
                     del step

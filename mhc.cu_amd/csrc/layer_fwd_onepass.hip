@@ -449,21 +449,23 @@ static int onepass_group(int B, int n, int C) {
     return G;
 }
 
-// Every workgroup streams all of phi through its CU's L1, which fills at about 50 GB/s (measured:
-// the same whether 2 or 4 steps are in flight, with or without the arithmetic), so phase A takes at
-// least |phi| / 50 GB/s whatever the batch.  Measured on whole forward+backward steps (graph replays,
-// B = 64 .. 4096, C = 512 .. 4096, n = 2, 3, 4): the one-launch forward wins by 3 - 15 % while phi is
-// below ~160 KB, ties up to ~256 KB (B=320 C=1280 n=4: 245 KB, 36.6 against 36.7 us) and loses beyond
-// (B=1280 C=2560 n=4: 491 KB, 70.4 against 68.6 us), where the two-launch forward (split-K
-// projection, then the fused mix kernel) stays.
+// Every workgroup streams all of phi out of the L2 (about 90 GB/s per CU in this access pattern, measured
+// by a stand-alone loop; more steps in flight change nothing), so phase A costs the kernel start plus
+// |phi| / 90 GB/s whatever the batch.  Measured on whole forward+backward steps (graphs of ten steps,
+// B = 64 .. 4096, C = 512 .. 4096, n = 2, 3, 4): the one-launch forward wins by 2 - 15 % while phi is
+// below ~120 KB; between 120 and 256 KB it wins only around B = 1280 (five samples per workgroup share
+// the phi stream: B=1280 C=1280 n=4 47.6 against 48.8 us) and loses at small and very large batches
+// (B=320 C=1280 n=4, 240 KB: 31.4 against 30.3 us); beyond 256 KB it loses everywhere (B=1280 C=2560
+// n=4: 64.1 against 62.2 us).  Elsewhere the two-launch forward (split-K projection, then the fused mix
+// kernel) stays.
 bool layer_fwd_onepass_supported(int x_dtype, int phi_dtype, int B, int n, int C) {
     const int mode = tuning_get(kTuneOnepassOff);  // 0 = by cost, 1 = never, 2 = whenever the shape allows
     if (mode == 1) return false;
     if (x_dtype != kBF16 || phi_dtype != kBF16 || n > 4 || C % 8 != 0 || (n * C) % 64 != 0) return false;
     if (OnePassLds(1, n * C, round_up(C / 8, 4), kOnePassWaves).total > 158 * 1024) return false;
     if (mode == 2) return true;
-    (void)B;
-    return 2ll * (n * n + 2 * n) * n * C <= 256 * 1024;
+    const long long phi_bytes = 2ll * (n * n + 2 * n) * n * C;
+    return phi_bytes <= 120 * 1024 || (phi_bytes <= 256 * 1024 && B >= 1024 && B <= 2048);
 }
 
 hipError_t launch_layer_fwd_onepass(const void *x, const void *w, int w_dtype, const void *f_inject, void *y,

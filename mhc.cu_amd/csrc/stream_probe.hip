@@ -114,6 +114,59 @@ __global__ __launch_bounds__(256) void probe_handoff_kernel(float *part, float *
     }
 }
 
+// Row-piece probe: what one workgroup of 8 waves pulls out of the L2 when every workgroup streams the
+// SAME [24][nC] bf16 matrix the way the one-launch forward streams phi: 64 contraction elements per step,
+// a wave fetches the step's 24 x 128 bytes row-contiguously (8 lanes per row piece), parks them in its own
+// LDS tile and reads them back in operand layout, two steps in flight.  `reps` passes inside one launch, so
+// the kernel start is amortised: the figure is the steady streaming rate of a CU, not a kernel time.
+__global__ __launch_bounds__(512) void probe_row_pieces_kernel(const unsigned short *phi, int nC, uint32_t *sink, int reps) {
+    __shared__ __align__(16) unsigned short tiles[8 * 32 * 72];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int steps = nC >> 6, r8 = lane >> 3, seg = lane & 7;
+    const int rot = (int)(((blockIdx.x >> 3) * (unsigned)steps) >> 5) % steps;  // workgroups of an XCD start apart
+    unsigned short *ps = tiles + wave * 32 * 72;
+    uint32_t acc = 0;
+    for (int r = 0; r < reps; r++) {
+        uint32_t q[2][3][4];
+        auto fetch = [&](int slot, int st) {
+            int p = st + rot;
+            p = p >= steps ? p - steps : p;
+#pragma unroll
+            for (int j = 0; j < 3; j++) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(phi + (size_t)(j * 8 + r8) * nC + (p << 6) + seg * 8);
+                q[slot][j][0] = v.x; q[slot][j][1] = v.y; q[slot][j][2] = v.z; q[slot][j][3] = v.w;
+            }
+        };
+        auto process = [&](int slot) {
+#pragma unroll
+            for (int j = 0; j < 3; j++)
+                *reinterpret_cast<uint4 *>(ps + (j * 8 + r8) * 72 + seg * 8) =
+                    make_uint4(q[slot][j][0], q[slot][j][1], q[slot][j][2], q[slot][j][3]);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            const uint4 v = *reinterpret_cast<const uint4 *>(ps + (lane & 15) * 72 + (lane >> 4) * 16);
+            acc += v.x ^ v.w;
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        };
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+            if (wave + u * 8 < steps) fetch(u, wave + u * 8);
+        for (int st = wave; st < steps; st += 16) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int su = st + u * 8;
+                if (su < steps) {
+                    process(u);
+                    if (su + 16 < steps) fetch(u, su + 16);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (acc == 0x12345678u) *sink = acc;  // never: keeps the reads alive
+}
+
 }  // namespace
 
 // mode 0 = read-only, 1 = copy, 2 = write-only, with the streaming (nt) hint on every access; 3, 4, 5 =
@@ -144,6 +197,12 @@ extern "C" __attribute__((visibility("default"))) int mhc_stream_probe(int mode,
         if (mode == 7) probe_handoff_kernel<true, 0><<<blocks, 256, 0, st>>>(part, out, sync, per);
         else if (mode == 8) probe_handoff_kernel<false, 0><<<blocks, 256, 0, st>>>(part, out, sync, per);
         else probe_handoff_kernel<false, 1><<<blocks, 256, 0, st>>>(part, out, sync, per);
+    }
+    else if (mode == 10) {
+        // row-piece probe: src = [24][nC] bf16, bytes = 24 * nC * 2 (nC a multiple of 64), dst unused; 20 passes per launch
+        const int nC = (int)(bytes / 48);
+        if (blocks <= 0 || nC <= 0 || nC % 64) return (int)hipErrorInvalidValue;
+        probe_row_pieces_kernel<<<blocks, 512, 0, st>>>(static_cast<const unsigned short *>(src), nC, static_cast<uint32_t *>(sink), 20);
     }
     else return (int)hipErrorInvalidValue;
     return (int)hipGetLastError();

@@ -1,9 +1,9 @@
 """The one-launch dynamic forward (projection + coefficients + mix, samples resident in LDS)
 through the C ABI: against the oracle at the bf16 tolerance, and against the two-launch path of the
 same library on the same inputs (both accumulate bf16 products in fp32, so their saved fp32
-tensors agree far inside the bf16 bar).  The group size G (samples per workgroup) and the wave
-count are forced through the library's experiment hook so that ragged last groups, G > 8 (two
-row pieces per lane) and every wave count are covered at small sizes."""
+tensors agree far inside the bf16 bar).  The group size G (samples per workgroup) is forced through
+the library's experiment hook so that ragged last groups and G > 8 (two row pieces per lane) are
+covered at small sizes."""
 import ctypes
 
 import pytest
@@ -14,7 +14,7 @@ from oracle import naive_mhc as nm
 
 pytestmark = pytest.mark.gpu
 
-K_OFF, K_G, K_WAVES = 0, 1, 2
+K_OFF, K_G = 0, 1
 
 
 def _tune(key, value):
@@ -28,7 +28,7 @@ def _tune(key, value):
 @pytest.fixture(autouse=True)
 def _reset_tuning():
     yield
-    for k in (K_OFF, K_G, K_WAVES):
+    for k in (K_OFF, K_G):
         _tune(k, 0)
 
 
@@ -54,17 +54,17 @@ def _forward(B, n, C, x, w, phi, bias, alpha, f, out_dtype, T, eps):
     return {k: v.float().cpu() for k, v in out.items()}
 
 
-CASES = [  # B, n, C, G, waves
-    (37, 4, 64, 0, 0), (37, 4, 64, 3, 4), (37, 4, 64, 16, 8), (37, 4, 64, 11, 5), (1, 4, 16, 0, 0),
-    (9, 2, 32, 4, 8), (13, 3, 64, 5, 6), (21, 4, 1280, 2, 8), (12, 4, 2560, 5, 8), (33, 1, 64, 9, 7),
-    (7, 4, 40, 2, 8), (300, 4, 128, 0, 0),
+CASES = [  # B, n, C, G
+    (37, 4, 64, 0), (37, 4, 64, 3), (37, 4, 64, 16), (37, 4, 64, 11), (1, 4, 16, 0),
+    (9, 2, 32, 4), (13, 3, 64, 5), (21, 4, 1280, 2), (12, 4, 2560, 5), (33, 1, 64, 9),
+    (7, 4, 40, 2), (300, 4, 128, 0),
 ]
 
 
-@pytest.mark.parametrize("B,n,C,G,waves", CASES)
+@pytest.mark.parametrize("B,n,C,G", CASES)
 @pytest.mark.parametrize("inject", [False, True])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-def test_onepass_forward(B, n, C, G, waves, inject, out_dtype):
+def test_onepass_forward(B, n, C, G, inject, out_dtype):
     from mhc._lib import lib
 
     T, eps = 20, 1e-6
@@ -90,7 +90,6 @@ def test_onepass_forward(B, n, C, G, waves, inject, out_dtype):
     two = _forward(B, n, C, x, w, phi, bias, alpha, f, out_dtype, T, eps)
     _tune(K_OFF, 2)
     _tune(K_G, G)
-    _tune(K_WAVES, waves)
     one = _forward(B, n, C, x, w, phi, bias, alpha, f, out_dtype, T, eps)
 
     # rows and columns n..NP-1 of the saved Sinkhorn denominators are padding nobody reads
