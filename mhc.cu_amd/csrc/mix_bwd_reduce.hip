@@ -17,6 +17,7 @@
 #include "launchers.h"
 #include "phase_profiler.h"
 #include "sinkhorn_device.h"
+#include "tuning.h"
 
 namespace mhc {
 
@@ -1084,6 +1085,7 @@ static int gram_small_parts(int B, int C) { return C >= 1024 && B < 1024 ? 2 : 1
 // Sinkhorn state would take the LDS that keeps several workgroups per CU resident, or the batch is
 // too small to do without column parts.
 static bool gram_small_fused(const BwdReduceArgs &a) {
+    if (const int hook = tuning_get(kTuneGramFused); hook && a.T <= 32) return hook == 2;  // experiment hook
     return a.T <= 32 && (a.B >= 128 || a.C <= 2048);
 }
 

@@ -9,7 +9,7 @@ namespace mhc {
 enum TuneKey {
     kTuneOnepassOff = 0,    // one-launch forward: 0 = by cost model, 1 = never, 2 = whenever the shape allows
     kTuneOnepassG = 1,      // samples per workgroup of the one-launch forward
-    kTuneSpare0 = 2,
+    kTuneGramFused = 2,     // n <= 8 channel sums and coefficient backward: 1 = two launches, 2 = one launch
     kTuneSlabSplits = 3,    // batch splits of the slab backward
     kTuneSeparateFinalize = 4,  // 1 = batch sums always as a launch of their own, never inside the dphi launch
     kTuneProjApart = 5,     // n <= 18 projection backward: 1 = both products in one launch, 2 = two launches
