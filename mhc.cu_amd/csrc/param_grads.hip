@@ -221,10 +221,49 @@ __global__ __launch_bounds__(256) void coef_bwd_static_kernel(const float *__res
         if (r0 < n && c0 + e < n) dH_res[r0 * n + c0 + e] = d[e];  // gradient of the logits
 }
 
+// n <= 8: one wave, one element per lane (SkSmall): the chain of an iteration is a dozen dependent
+// instructions instead of the LDS exchanges of the workgroup layout (10.7 -> about 4 us per call).
+template <int NP>
+__global__ __launch_bounds__(64) void coef_bwd_static_small_kernel(const float *__restrict__ red_sum,
+                                                                   const float *__restrict__ Hpre,
+                                                                   const float *__restrict__ Hpost,
+                                                                   const float *__restrict__ H_res_logits,
+                                                                   float *__restrict__ dH_pre,
+                                                                   float *__restrict__ dH_post,
+                                                                   float *__restrict__ dH_res, int n, int T,
+                                                                   float eps) {
+    using SK = SkSmall<NP>;
+    extern __shared__ float sc[];  // SK::scaling_floats(T)
+    const int lane = threadIdx.x, g = lane % SK::kGroup;
+    const bool first = lane < SK::kGroup;  // a 4 x 4 matrix takes 16 lanes: the other groups compute copies
+    if (first && g < n) {
+        const float hp = Hpre[g], ho = Hpost[g];
+        dH_pre[g] = red_sum[n * n + g] * hp * (1.0f - hp);
+        dH_post[g] = red_sum[n * n + n + g] * ho * (1.0f - 0.5f * ho);
+    }
+    const int r0 = SK::row(g), c0 = SK::col0(g);
+    const bool ok = r0 < n && c0 < n;
+    float m[1] = {ok ? expf(H_res_logits[r0 * n + c0]) : 0.f};
+    float d[1] = {ok ? red_sum[r0 * n + c0] : 0.f};
+    SK::template forward<true>(m, g, n, T, eps, sc, lane);
+    SK::template backward<true>(d, m, T, sc, lane);
+    if (first && ok) dH_res[r0 * n + c0] = d[0];  // gradient of the logits
+}
+
 hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const float *Hpost,
                                   const float *H_res_logits, float *dH_pre, float *dH_post,
                                   float *dH_res, int n, int T, float eps, hipStream_t stream) {
-    if (n <= 16) {
+    if (n <= 8) {
+        if (n <= 4) {
+            const size_t smem = sizeof(float) * SkSmall<4>::scaling_floats(T);
+            if (hipError_t e = allow_dynamic_lds(&coef_bwd_static_small_kernel<4>, smem); e != hipSuccess) return e;
+            coef_bwd_static_small_kernel<4><<<1, 64, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
+        } else {
+            const size_t smem = sizeof(float) * SkSmall<8>::scaling_floats(T);
+            if (hipError_t e = allow_dynamic_lds(&coef_bwd_static_small_kernel<8>, smem); e != hipSuccess) return e;
+            coef_bwd_static_small_kernel<8><<<1, 64, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
+        }
+    } else if (n <= 16) {
         const size_t smem = sizeof(float) * SkWg<16>::lds_floats(T);
         if (hipError_t e = allow_dynamic_lds(&coef_bwd_static_kernel<16>, smem); e != hipSuccess) return e;
         coef_bwd_static_kernel<16><<<1, 256, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
