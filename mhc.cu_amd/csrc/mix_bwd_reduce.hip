@@ -266,7 +266,10 @@ __global__ __launch_bounds__(256) void mix_bwd_reduce_small_kernel(BwdReduceArgs
 // with other work to do first has those values waiting; run() then forms dHpre / dHpost, the sigmoid
 // derivatives, the exact Sinkhorn backward, dP = dt * alpha / r in all three layouts, and cx.
 // =============================================================================================
-template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
+// STATIC (with GRAM): shared coefficients - prefetch() takes H from the [n] vectors and nothing else, and
+// run() stops after the channel-sum vectors: it writes the sample's raw gradients (dM | dHpre | dHpost)
+// as a row of `red` for the batch-sum launch; the Sinkhorn backward then runs once on the batch total.
+template <int NP, bool PRECISE, bool GRAM, bool STATIC = false> struct CoefBwdSmall {
     using SK = SkSmall<NP>;
     static constexpr int K = GRAM ? 3 * NP * NP : NP * NP + 3 * NP + 1;
     // LDS floats next to the Sinkhorn denominators, per group: the column results of the Gram sums
@@ -287,6 +290,13 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
         // PRECISE keeps IEEE divisions; otherwise v_rcp_f32 / v_exp_f32 (1 ulp) keep the step short
         qinv = inject ? 0.f : (PRECISE ? 1.0f / a.q[b] : fast_rcp(a.q[b]));
         inv_c = 1.0f / (float)a.C; inv_nc = 1.0f / (float)(n * a.C);
+        if constexpr (STATIC) {
+            hp = a.Hpre[gc]; ho = a.Hpost[gc];
+            hpre_r = a.Hpre[r0 < n ? r0 : 0];
+            hpost_r = a.Hpost[r0 < n ? r0 : 0];
+            rinv = al0 = al1 = al2 = pres = bres = ppre = ppost = 0.f;
+            return;
+        }
         const float *Pb = a.P + (size_t)b * D;
         al0 = a.alpha[0]; al1 = a.alpha[1]; al2 = a.alpha[2];
         rinv = PRECISE ? 1.0f / a.r[b] : fast_rcp(a.r[b]);
@@ -369,6 +379,15 @@ template <int NP, bool PRECISE, bool GRAM> struct CoefBwdSmall {
             tpost = s_a; tA1 = s_b; tA2 = s_c; s1 = s_d;
         }
         if (g == 0) a.out.s1[b] = s1;
+        if constexpr (STATIC) {
+            float *red = a.out.red + (size_t)b * (D + 3);  // rows padded like dt, for the batch-sum launch
+            if (mv) red[r0 * n + c0] = dMe;
+            if (g < n) {
+                red[n * n + g] = inject ? 0.f : tA1 * qinv - s1 * tA2 * qinv * qinv * qinv * inv_c;
+                red[n * n + n + g] = tpost;
+            }
+            return;
+        }
         float *dt = a.out.dt + (size_t)b * (D + 3);
         const DPWriter dpw{a.out, b, a.B, a.DP};
         float S0 = 0.f, S1 = 0.f, S2 = 0.f;  // sum_d dt_d p_d per alpha group
@@ -440,11 +459,14 @@ enum { kGramInject = 0, kGramWBf16 = 1, kGramWF32 = 2 };
 // backward (CoefBwdSmall) as soon as the sums are complete, its other inputs requested at the start;
 // with several workgroups per CU the serial Sinkhorn chain of one runs under the loads of the others,
 // and the launch of the coefficient kernel is saved.
-template <int NP, int WMODE, bool FUSED>
+// STATIC (with FUSED): shared coefficients; the tail only converts the sums into the sample's row of raw
+// gradients (see CoefBwdSmall).
+template <int NP, int WMODE, bool FUSED, bool STATIC = false>
 __global__ __launch_bounds__(256, NP == 4 ? 4 : 1) void gram_small_kernel(BwdReduceArgs a) {
     static_assert(NP == 4 || NP == 8, "stream groups of four");
+    static_assert(FUSED || !STATIC, "the static tail runs inside the launch");
     using SK = SkSmall<NP>;
-    using CB = CoefBwdSmall<NP, false, true>;
+    using CB = CoefBwdSmall<NP, false, true, STATIC>;
     constexpr int NB = NP / 4;            // stream groups
     constexpr int U = 2;                  // steps of a wave in flight
     constexpr int K = 3 * NP * NP;
@@ -464,7 +486,7 @@ __global__ __launch_bounds__(256, NP == 4 ? 4 : 1) void gram_small_kernel(BwdRed
         // wave 0, while the other waves already stream (and not at the tail of the workgroup)
         if (tid < SK::kGroup) {
             cb.prefetch(a, b, tid);
-            cb.forward_recompute(a, b, tid, tid, sc);
+            if constexpr (!STATIC) cb.forward_recompute(a, b, tid, tid, sc);
         }
     }
     const int blk = lane >> 2, i = lane & 3;
@@ -595,7 +617,7 @@ __global__ __launch_bounds__(256, NP == 4 ? 4 : 1) void gram_small_kernel(BwdRed
         MHC_PHASE_ADD(kPhaseGramSmall, pwg, 2, pclk);
         if (tid < SK::kGroup) {
             cb.fetch_sums(tot_s, 1);
-            cb.run(a, b, tid, tid, sc, sc + SK::scaling_floats(a.T));
+            cb.run(a, b, tid, tid, sc, sc + (STATIC ? 0 : SK::scaling_floats(a.T)));
         }
         MHC_PHASE_ADD(kPhaseGramSmall, pwg, 3, pclk);
     }
@@ -1117,10 +1139,26 @@ static hipError_t launch_gram_small(BwdReduceArgs a, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// Static H with bf16 dy and x: the same Gram kernel, one launch, the tail writes the rows of `red`.
+template <int NP>
+static hipError_t launch_gram_small_static(BwdReduceArgs a, hipStream_t stream) {
+    using CB = CoefBwdSmall<NP, false, true, true>;
+    a.parts = 1;
+    const size_t smem = sizeof(float) * CB::kXch;
+    const dim3 grid(a.B, 1);
+    if (a.f_inject) gram_small_kernel<NP, kGramInject, true, true><<<grid, 256, smem, stream>>>(a);
+    else if (a.w_bf16) gram_small_kernel<NP, kGramWBf16, true, true><<<grid, 256, smem, stream>>>(a);
+    else gram_small_kernel<NP, kGramWF32, true, true><<<grid, 256, smem, stream>>>(a);
+    return hipGetLastError();
+}
+
 template <typename TG, typename TX, int NP, int V>
 static hipError_t launch_small(const BwdReduceArgs &a, hipStream_t stream) {
-    if constexpr (std::is_same<TG, bf16_t>::value && std::is_same<TX, bf16_t>::value)
+    if constexpr (std::is_same<TG, bf16_t>::value && std::is_same<TX, bf16_t>::value) {
         if (gram_small_supported(a)) return launch_gram_small<NP>(a, stream);
+        // static H: worth it once the batch fills the chip (one workgroup per sample)
+        if (a.hstride == 0 && a.C % 8 == 0 && a.B >= 128) return launch_gram_small_static<NP>(a, stream);
+    }
     const int nch = (a.C / V + a.parts - 1) / a.parts;  // chunks per column part
     // every thread gets the same number of chunks (whole 16-lane rows: the reduction works on them)
     const int rounds = (nch + 255) / 256;

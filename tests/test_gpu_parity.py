@@ -242,7 +242,9 @@ def test_bf16_small_n_coefficient_gradients_are_tight(B, n, C, inject, w_dtype):
 
 
 @pytest.mark.parametrize("B,n,C", [(16, 4, 256), (8, 8, 128), (4, 16, 64), (3, 32, 72), (5, 32, 1040),
-                                   (5, 4, 2568), (3, 7, 2176)])
+                                   (5, 4, 2568), (3, 7, 2176),
+                                   # 128 samples and more: the channel sums run on the matrix cores
+                                   (130, 4, 264), (128, 7, 136), (300, 3, 1288), (129, 8, 2048)])
 @pytest.mark.parametrize("inject", [False, True])
 def test_static_bf16_vs_oracle(B, n, C, inject):
     """Static H with bf16 activations: the shared-coefficient mode of the bf16 kernels."""
