@@ -13,7 +13,7 @@ enum TuneKey {
     kTuneSlabSplits = 3,    // batch splits of the slab backward
     kTuneSeparateFinalize = 4,  // 1 = batch sums always as a launch of their own, never inside the dphi launch
     kTuneProjApart = 5,     // n <= 18 projection backward: 1 = both products in one launch, 2 = two launches
-    kTuneSpare2 = 6,
+    kTuneStaticSpg = 6,     // static backward: samples per workgroup of the dx kernel (n <= 8)
     kTuneSpare3 = 7,
     kTuneCount = 8
 };

@@ -244,7 +244,9 @@ def test_bf16_small_n_coefficient_gradients_are_tight(B, n, C, inject, w_dtype):
 @pytest.mark.parametrize("B,n,C", [(16, 4, 256), (8, 8, 128), (4, 16, 64), (3, 32, 72), (5, 32, 1040),
                                    (5, 4, 2568), (3, 7, 2176),
                                    # 128 samples and more: the channel sums run on the matrix cores
-                                   (130, 4, 264), (128, 7, 136), (300, 3, 1288), (129, 8, 2048)])
+                                   (130, 4, 264), (128, 7, 136), (300, 3, 1288), (129, 8, 2048),
+                                   # 1024 samples and more with n <= 4: the dx kernel takes four samples per workgroup
+                                   (1100, 4, 72)])
 @pytest.mark.parametrize("inject", [False, True])
 def test_static_bf16_vs_oracle(B, n, C, inject):
     """Static H with bf16 activations: the shared-coefficient mode of the bf16 kernels."""
@@ -260,7 +262,7 @@ def test_static_bf16_vs_oracle(B, n, C, inject):
         _check(g[k], ref, "bf16", "d" + k)
 
 
-@pytest.mark.parametrize("B,n,C", [(32, 4, 1280), (3, 4, 20), (8, 8, 128), (4, 16, 64), (3, 32, 72)])
+@pytest.mark.parametrize("B,n,C", [(32, 4, 1280), (3, 4, 20), (8, 8, 128), (4, 16, 64), (3, 32, 72), (1030, 3, 40)])
 @pytest.mark.parametrize("inject", [False, True])
 def test_static_fp32_vs_oracle(B, n, C, inject):
     x, dy, f, p = nm.make_static_inputs(B, n, C, with_f=inject)
