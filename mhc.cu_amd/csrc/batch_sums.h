@@ -39,6 +39,16 @@ __device__ __forceinline__ void batch_sum_block(const BatchSumArgs &a, int blk, 
         const int rows = is_u ? a.rows_u : a.rows_dt;
         double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
         int r = rg;
+        // many rows (per-sample rows of a large batch): sixteen loads in flight, the round trips decide
+        for (; r + 15 * RG < rows; r += 16 * RG) {
+            float t[16];
+#pragma unroll
+            for (int k = 0; k < 16; k++) t[k] = src[(size_t)(r + k * RG) * ld];
+#pragma unroll
+            for (int k = 0; k < 16; k += 4) {
+                a0 += (double)t[k]; a1 += (double)t[k + 1]; a2 += (double)t[k + 2]; a3 += (double)t[k + 3];
+            }
+        }
         for (; r + 3 * RG < rows; r += 4 * RG) {
             const float t0 = src[(size_t)r * ld], t1 = src[(size_t)(r + RG) * ld];
             const float t2 = src[(size_t)(r + 2 * RG) * ld], t3 = src[(size_t)(r + 3 * RG) * ld];
