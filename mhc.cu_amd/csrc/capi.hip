@@ -471,8 +471,8 @@ int mhc_rmsnorm_fwd(const void *inp, int dtype, const void *w, int w_dtype, void
 size_t mhc_rmsnorm_bwd_workspace_bytes(int rows, int C) {
     if (rows < 1 || C < 1) return 0;
     Carver c(nullptr);
-    c.floats((size_t)rows * C);
-    c.floats(colsum_workspace_floats(rows, C));
+    c.floats((size_t)(rows + 3) * C);  // dw terms: a row per input row, or per row slot of the persistent kernel
+    c.floats(colsum_workspace_floats(rows + 3, C));
     return c.off;
 }
 
@@ -484,11 +484,12 @@ int mhc_rmsnorm_bwd(const void *grad_out, const void *inp, int dtype, const void
     if (!valid_dtype(dtype) || !valid_dtype(w_dtype)) return MHC_ERR_BAD_DTYPE;
     if (int s = ws_check(workspace, workspace_bytes, mhc_rmsnorm_bwd_workspace_bytes(rows, C))) return s;
     Carver c(workspace);
-    float *u = c.floats((size_t)rows * C);
-    float *part = c.floats(colsum_workspace_floats(rows, C));
+    float *u = c.floats((size_t)(rows + 3) * C);
+    float *part = c.floats(colsum_workspace_floats(rows + 3, C));
     hipStream_t st = static_cast<hipStream_t>(stream);
-    MHC_LAUNCH(launch_rmsnorm_bwd(grad_out, inp, dtype, w, w_dtype, rms, d_inp, u, rows, C, st));
-    MHC_LAUNCH(launch_colsum(u, rows, C, C, d_w, part, st));
+    int u_rows = rows;  // rows of u whose column sums are dw (fewer when the kernel sums its own rows)
+    MHC_LAUNCH(launch_rmsnorm_bwd(grad_out, inp, dtype, w, w_dtype, rms, d_inp, u, rows, C, &u_rows, st));
+    MHC_LAUNCH(launch_colsum(u, u_rows, C, C, d_w, part, st));
     return MHC_OK;
 }
 

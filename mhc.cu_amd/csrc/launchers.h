@@ -212,6 +212,6 @@ hipError_t launch_rmsnorm_fwd(const void *inp, int dtype, const void *w, int w_d
                               float *rms, int rows, int C, float eps, hipStream_t stream);
 hipError_t launch_rmsnorm_bwd(const void *grad, const void *inp, int dtype, const void *w,
                               int w_dtype, const float *rms, void *d_inp, float *u, int rows, int C,
-                              hipStream_t stream);
+                              int *u_rows, hipStream_t stream);  // u: (rows + 3) * C floats
 
 }  // namespace mhc

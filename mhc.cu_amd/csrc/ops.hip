@@ -191,8 +191,177 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T *__restrict__ 
     }
 }
 
+// --------------------------------------------------------------------------------------------
+// Rows in registers: TPR threads share a row (64: one wave, four rows per workgroup; 256: the whole
+// workgroup), a thread holds VPT 16-byte pieces of it (piece k of thread t = columns (k TPR + t) V ...),
+// all requested before the first is used.  One pass over the row: x is read once (forward) and dy and
+// x once (backward), 16-byte loads and stores.  Needs C % V == 0, 16-byte aligned rows and
+// C <= TPR * V * VPT; other shapes take the kernels above.
+// --------------------------------------------------------------------------------------------
+template <int V> __device__ __forceinline__ void load_w_vec(const void *w, int w_bf16, int c, float (&wv)[V]) {
+    if (w_bf16) load_vec<bf16_t, V>(static_cast<const bf16_t *>(w) + c, wv);
+    else load_vec<float, V>(static_cast<const float *>(w) + c, wv);
+}
+
+template <int TPR> __device__ __forceinline__ float row_allreduce(float v, float *red) {
+    if constexpr (TPR == 64) return wave_allreduce_sum(v);
+    else return block_allreduce_sum<256>(v, red);
+}
+
+template <typename T, int VPT, int TPR>
+__global__ __launch_bounds__(256) void rmsnorm_fwd_rows_kernel(const T *__restrict__ inp, const void *w, int w_bf16,
+                                                               T *__restrict__ out, float *__restrict__ rms,
+                                                               int rows, int C, float eps) {
+    constexpr int V = 16 / (int)sizeof(T), RPW = 256 / TPR;
+    __shared__ float red[4];
+    const int tid = threadIdx.x, t = tid % TPR;
+    const int row = blockIdx.x * RPW + tid / TPR;
+    const bool live = row < rows;  // TPR == 64: whole waves; nothing below synchronises across waves
+    const T *x = inp + (size_t)(live ? row : 0) * C;
+    RawVec<T, V> xr[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; k++) {
+        const int c = (k * TPR + t) * V;
+        xr[k].load(x + (c < C ? c : 0));
+    }
+    float ssq = 0.f;
+#pragma unroll
+    for (int k = 0; k < VPT; k++) {
+        float v[V];
+        xr[k].get(v);
+        if ((k * TPR + t) * V < C) {
+#pragma unroll
+            for (int j = 0; j < V; j++) ssq += v[j] * v[j];
+        }
+    }
+    ssq = row_allreduce<TPR>(ssq, red);
+    const float r = sqrtf(ssq / (float)C + eps);
+    if (t == 0 && rms && live) rms[row] = r;
+    const float rinv = 1.0f / r;
+    if (!live) return;
+#pragma unroll
+    for (int k = 0; k < VPT; k++) {
+        const int c = (k * TPR + t) * V;
+        if (c < C) {
+            float v[V], wv[V];
+            xr[k].get(v);
+            load_w_vec<V>(w, w_bf16, c, wv);
+#pragma unroll
+            for (int j = 0; j < V; j++) v[j] = v[j] * rinv * wv[j];
+            store_vec<T, V, true>(out + (size_t)row * C + c, v);
+        }
+    }
+}
+
+// Backward, persistent: workgroup g takes the row groups g, g + gridDim.x, ...; a thread keeps the dw
+// terms of its own columns in registers over all its rows and writes them once, as row
+// (blockIdx.x * RPW + row lane) of `part` [gridDim.x * RPW][C]; a column sum over those rows gives dw.
+template <typename T, int VPT, int TPR>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_rows_kernel(const T *__restrict__ grad, const T *__restrict__ inp,
+                                                               const void *w, int w_bf16, const float *__restrict__ rms,
+                                                               T *__restrict__ d_inp, float *__restrict__ part,
+                                                               int rows, int C) {
+    constexpr int V = 16 / (int)sizeof(T), RPW = 256 / TPR;
+    __shared__ float red[4];
+    const int tid = threadIdx.x, t = tid % TPR, rl = tid / TPR;
+    float acc[VPT][V];
+#pragma unroll
+    for (int k = 0; k < VPT; k++)
+#pragma unroll
+        for (int j = 0; j < V; j++) acc[k][j] = 0.f;
+    const int ngroups = (rows + RPW - 1) / RPW;
+    for (int grp = blockIdx.x; grp < ngroups; grp += gridDim.x) {
+        const int row = grp * RPW + rl;
+        const bool live = row < rows;
+        const size_t base = (size_t)(live ? row : 0) * C;
+        RawVec<T, V> xr[VPT], gr[VPT];
+#pragma unroll
+        for (int k = 0; k < VPT; k++) {
+            const int c = (k * TPR + t) * V, cc = c < C ? c : 0;
+            xr[k].load(inp + base + cc);
+            gr[k].load(grad + base + cc);
+        }
+        const float rinv = 1.0f / rms[live ? row : 0];
+        float dot = 0.f;
+#pragma unroll
+        for (int k = 0; k < VPT; k++) {
+            const int c = (k * TPR + t) * V;
+            if (c < C) {
+                float xv[V], gv[V], wv[V];
+                xr[k].get(xv); gr[k].get(gv);
+                load_w_vec<V>(w, w_bf16, c, wv);
+#pragma unroll
+                for (int j = 0; j < V; j++) dot += gv[j] * wv[j] * xv[j];
+            }
+        }
+        dot = row_allreduce<TPR>(dot, red);  // TPR == 256: every thread of the workgroup gets here (grp is uniform)
+        const float k2 = dot * rinv * rinv * rinv / (float)C;
+#pragma unroll
+        for (int k = 0; k < VPT; k++) {
+            const int c = (k * TPR + t) * V;
+            if (c < C && live) {
+                float xv[V], gv[V], wv[V], dv[V];
+                xr[k].get(xv); gr[k].get(gv);
+                load_w_vec<V>(w, w_bf16, c, wv);
+#pragma unroll
+                for (int j = 0; j < V; j++) {
+                    dv[j] = gv[j] * wv[j] * rinv - xv[j] * k2;
+                    acc[k][j] += gv[j] * xv[j] * rinv;
+                }
+                store_vec<T, V, true>(d_inp + base + c, dv);
+            }
+        }
+    }
+    float *prow = part + (size_t)(blockIdx.x * RPW + rl) * C;
+#pragma unroll
+    for (int k = 0; k < VPT; k++) {
+        const int c = (k * TPR + t) * V;
+        if (c < C) store_vec<float, V>(prow + c, acc[k]);
+    }
+}
+
+// VPT (pieces per thread) and TPR (threads per row) of the row kernels, 0 when the shape does not fit
+static int rows_kernel_vpt(int dtype, int C, int max_vpt, int *tpr) {
+    const int V = dtype == kBF16 ? 8 : 4;
+    if (C % V != 0) return 0;
+    const int pieces = C / V;
+    *tpr = pieces <= 64 * 4 ? 64 : 256;
+    const int need = (pieces + *tpr - 1) / *tpr;
+    for (int v : {1, 2, 4, 8, 16})
+        if (need <= v) return v <= max_vpt ? v : 0;
+    return 0;
+}
+static bool aligned16_(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// number of partial dw rows the backward row kernel writes (0: the generic kernel runs, rows of u)
+int rmsnorm_bwd_partial_rows(int dtype, int rows, int C) {
+    int tpr = 0;
+    if (rows_kernel_vpt(dtype, C, 8, &tpr) == 0) return 0;
+    const int rpw = 256 / tpr, groups = (rows + rpw - 1) / rpw;
+    return (groups < 1024 ? groups : 1024) * rpw;
+}
+
 hipError_t launch_rmsnorm_fwd(const void *inp, int dtype, const void *w, int w_dtype, void *out,
                               float *rms, int rows, int C, float eps, hipStream_t stream) {
+    int tpr = 0;
+    const int vpt = rows_kernel_vpt(dtype, C, 16, &tpr);
+    if (vpt && aligned16_(inp) && aligned16_(out) && aligned16_(w)) {
+        const int wb = w_dtype == kBF16, grid = (rows + 256 / tpr - 1) / (256 / tpr);
+#define MHC_RMS_FWD(T, VPT, TPR) \
+    rmsnorm_fwd_rows_kernel<T, VPT, TPR><<<grid, 256, 0, stream>>>(static_cast<const T *>(inp), w, wb, static_cast<T *>(out), rms, rows, C, eps)
+#define MHC_RMS_FWD_T(T)                                                                  \
+    do {                                                                                  \
+        if (tpr == 64) { if (vpt == 1) MHC_RMS_FWD(T, 1, 64); else if (vpt == 2) MHC_RMS_FWD(T, 2, 64); else MHC_RMS_FWD(T, 4, 64); } \
+        else if (vpt <= 2) MHC_RMS_FWD(T, 2, 256);                                        \
+        else if (vpt == 4) MHC_RMS_FWD(T, 4, 256);                                        \
+        else if (vpt == 8) MHC_RMS_FWD(T, 8, 256);                                        \
+        else MHC_RMS_FWD(T, 16, 256);                                                     \
+    } while (0)
+        if (dtype == kBF16) MHC_RMS_FWD_T(bf16_t); else MHC_RMS_FWD_T(float);
+#undef MHC_RMS_FWD_T
+#undef MHC_RMS_FWD
+        return hipGetLastError();
+    }
     if (dtype == kBF16)
         rmsnorm_fwd_kernel<bf16_t><<<rows, 256, 0, stream>>>(static_cast<const bf16_t *>(inp), w, w_dtype == kBF16,
                                                              static_cast<bf16_t *>(out), rms, C, eps);
@@ -202,9 +371,32 @@ hipError_t launch_rmsnorm_fwd(const void *inp, int dtype, const void *w, int w_d
     return hipGetLastError();
 }
 
+// u: rows x C floats of workspace.  *u_rows receives the number of rows of u whose column sums are dw:
+// `rows` from the generic kernel, rmsnorm_bwd_partial_rows() from the row kernel.
 hipError_t launch_rmsnorm_bwd(const void *grad, const void *inp, int dtype, const void *w,
                               int w_dtype, const float *rms, void *d_inp, float *u, int rows, int C,
-                              hipStream_t stream) {
+                              int *u_rows, hipStream_t stream) {
+    int tpr = 0;
+    const int vpt = rows_kernel_vpt(dtype, C, 8, &tpr);
+    if (vpt && aligned16_(grad) && aligned16_(inp) && aligned16_(d_inp) && aligned16_(w) && aligned16_(u)) {
+        const int wb = w_dtype == kBF16, rpw = 256 / tpr;
+        const int prow = rmsnorm_bwd_partial_rows(dtype, rows, C), grid = prow / rpw;
+        *u_rows = prow;
+#define MHC_RMS_BWD(T, VPT, TPR) \
+    rmsnorm_bwd_rows_kernel<T, VPT, TPR><<<grid, 256, 0, stream>>>(static_cast<const T *>(grad), static_cast<const T *>(inp), w, wb, rms, static_cast<T *>(d_inp), u, rows, C)
+#define MHC_RMS_BWD_T(T)                                                                  \
+    do {                                                                                  \
+        if (tpr == 64) { if (vpt == 1) MHC_RMS_BWD(T, 1, 64); else if (vpt == 2) MHC_RMS_BWD(T, 2, 64); else MHC_RMS_BWD(T, 4, 64); } \
+        else if (vpt <= 2) MHC_RMS_BWD(T, 2, 256);                                        \
+        else if (vpt == 4) MHC_RMS_BWD(T, 4, 256);                                        \
+        else MHC_RMS_BWD(T, 8, 256);                                                      \
+    } while (0)
+        if (dtype == kBF16) MHC_RMS_BWD_T(bf16_t); else MHC_RMS_BWD_T(float);
+#undef MHC_RMS_BWD_T
+#undef MHC_RMS_BWD
+        return hipGetLastError();
+    }
+    *u_rows = rows;
     if (dtype == kBF16)
         rmsnorm_bwd_kernel<bf16_t><<<rows, 256, 0, stream>>>(static_cast<const bf16_t *>(grad),
                                                              static_cast<const bf16_t *>(inp), w, w_dtype == kBF16,

@@ -47,7 +47,12 @@ def test_sinkhorn_knopp_stability_and_zero_rows():
     assert torch.equal(sinkhorn_knopp(z, num_iters=3), z)   # thresholded division: no 0/0
 
 
-@pytest.mark.parametrize("rows,C", [(8, 128), (128, 4096), (16, 64), (5, 100), (3, 100000), (70000, 64), (1, 1)])
+@pytest.mark.parametrize("rows,C", [(8, 128), (128, 4096), (16, 64), (5, 100), (3, 100000), (70000, 64), (1, 1),
+                                    # rows in registers: one wave per row (1, 2, 4 pieces per thread), a workgroup per row
+                                    # (2, 4, 8, 16 pieces), ragged last pieces, row counts off the rows-per-workgroup grid;
+                                    # 32768 channels: row kernel forward, generic kernel backward
+                                    (5, 1024), (1030, 2048), (7, 8192), (3, 16384), (2, 32768), (9, 4104), (6, 520),
+                                    (2500, 264)])
 def test_rmsnorm_forward_backward_vs_oracle(rows, C):
     """bf16 operator as in the reference (test_rmsnorm.cu tolerance 1e-2, backward 2e-2)."""
     from mhc import rmsnorm
@@ -66,12 +71,13 @@ def test_rmsnorm_forward_backward_vs_oracle(rows, C):
     assert rel_err(wd.grad.float(), wr.grad) < 2e-2
 
 
-def test_rmsnorm_fp32_through_c_abi():
+@pytest.mark.parametrize("rows,C", [(16, 64), (37, 1028), (9, 8192), (1100, 260), (3, 12288), (5, 1023)])
+def test_rmsnorm_fp32_through_c_abi(rows, C):
     from mhc.ops import RMSNormFunction
     g = torch.Generator().manual_seed(3)
-    inp = torch.randn(16, 64, generator=g)
-    w = 1 + 0.2 * torch.randn(64, generator=g)
-    go = torch.randn(16, 64, generator=g)
+    inp = torch.randn(rows, C, generator=g)
+    w = 1 + 0.2 * torch.randn(C, generator=g)
+    go = torch.randn(rows, C, generator=g)
     dx_ref, dw_ref = nm.rmsnorm_backward_ref(go.double(), inp.double(), w.double(), 1e-5)
     x, wd = inp.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
     out = RMSNormFunction.apply(x, wd, 1e-5)
