@@ -387,7 +387,7 @@ def stream_probe(torch):
         dst = torch.empty_like(src)
         for mode, name, moved in ((0, "read", nbytes), (1, "copy", 2 * nbytes), (2, "write", nbytes),
                                   (3, "read", nbytes), (4, "copy", 2 * nbytes), (5, "write", nbytes)):
-            for blocks in (2048, 4096):
+            for blocks in (2048, 4096, 16384, 65536, 131072):  # few persistent workgroups .. one pass of short ones
                 def run():
                     st = fn(mode, src.data_ptr(), dst.data_ptr(), nbytes, blocks, sink.data_ptr(), stream)
                     assert st == 0, st
