@@ -4,6 +4,7 @@
 // src/csrc/tests/test_rmsnorm.cu:17-30 and test_rmsnorm_backward.cu:17-39.
 #include "launchers.h"
 #include "mhc_common.h"
+#include "sinkhorn_device.h"
 
 namespace mhc {
 
@@ -129,8 +130,76 @@ __global__ __launch_bounds__(256) void sinkhorn_plain_bwd_kernel(const float *__
     }
 }
 
+// --------------------------------------------------------------------------------------------
+// Square matrices up to 8 x 8: one element per lane (four 4 x 4 matrices or one 8 x 8 matrix per wave,
+// the lane layout and the DPP reductions of SkSmall), the whole iteration in registers.  Same
+// operator: no exp, a row / column is divided only where its sum exceeds eps.  BWD: the forward keeps
+// the divisors in LDS (-1 where the division was skipped) and the reverse sweep follows in the same
+// launch; it rebuilds the iterates by multiplying the divisors back.
+// --------------------------------------------------------------------------------------------
+template <int NP, bool BWD>
+__global__ __launch_bounds__(64) void sinkhorn_small_kernel(const float *__restrict__ inp, float *__restrict__ out,
+                                                            const float *__restrict__ grad, float *__restrict__ d_inp,
+                                                            int batch, int n, int T, float eps) {
+    using SK = SkSmall<NP>;
+    extern __shared__ float sc[];  // BWD: [T][2][64] divisors per lane
+    const int lane = threadIdx.x, g = lane % SK::kGroup;
+    const int b = blockIdx.x * SK::kPerWave + lane / SK::kGroup;
+    const int r = SK::row(g), c = SK::col0(g);
+    const bool ok = b < batch && r < n && c < n;  // lanes of absent matrices run on zeros
+    const size_t e = ok ? (size_t)b * n * n + r * n + c : 0;
+    float m = ok ? inp[e] : 0.f;
+    float d = 0.f;
+    if constexpr (BWD) d = ok ? grad[e] : 0.f;
+    for (int t = 0; t < T; t++) {
+        const float rs = SK::row_allreduce(m);
+        const bool dr = rs > eps;
+        m = dr ? m / rs : m;
+        const float cs = SK::col_allreduce(m);
+        const bool dc = cs > eps;
+        m = dc ? m / cs : m;
+        if constexpr (BWD) {
+            sc[(t * 2) * 64 + lane] = dr ? rs : -1.0f;
+            sc[(t * 2 + 1) * 64 + lane] = dc ? cs : -1.0f;
+        }
+    }
+    if constexpr (!BWD) {
+        if (ok) out[e] = m;
+        return;
+    } else {
+        // through column step t: Out = R / s, dR = (dOut - sum_col(dOut Out)) / s; then the row step alike
+        for (int t = T - 1; t >= 0; t--) {
+            const float rs = sc[(t * 2) * 64 + lane], cs = sc[(t * 2 + 1) * 64 + lane];
+            // (selects, not branches: the reductions run on every lane)
+            const float cdot = SK::col_allreduce(d * m);
+            d = cs > 0.f ? (d - cdot) / cs : d;
+            m = cs > 0.f ? m * cs : m;
+            const float rdot = SK::row_allreduce(d * m);
+            d = rs > 0.f ? (d - rdot) / rs : d;
+            m = rs > 0.f ? m * rs : m;
+        }
+        if (ok) d_inp[e] = d;
+    }
+}
+
+static bool sinkhorn_small_supported(int rows, int cols, int T) { return rows == cols && rows <= 8 && T <= 96; }
+
+template <bool BWD>
+static hipError_t launch_sinkhorn_small(const float *inp, float *out, const float *grad, float *d_inp, int batch,
+                                        int n, int T, float eps, hipStream_t stream) {
+    const size_t smem = BWD ? sizeof(float) * (size_t)(T > 0 ? T : 1) * 2 * 64 : 0;
+    if (n <= 4) {
+        sinkhorn_small_kernel<4, BWD><<<(batch + 3) / 4, 64, smem, stream>>>(inp, out, grad, d_inp, batch, n, T, eps);
+    } else {
+        sinkhorn_small_kernel<8, BWD><<<batch, 64, smem, stream>>>(inp, out, grad, d_inp, batch, n, T, eps);
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_sinkhorn_plain_fwd(const float *inp, float *out, int batch, int rows, int cols,
                                      int T, float eps, hipStream_t stream) {
+    if (sinkhorn_small_supported(rows, cols, T))
+        return launch_sinkhorn_small<false>(inp, out, nullptr, nullptr, batch, rows, T, eps, stream);
     sinkhorn_plain_fwd_kernel<<<batch, 256, 0, stream>>>(inp, out, rows, cols, T, eps, nullptr);
     return hipGetLastError();
 }
@@ -138,6 +207,8 @@ hipError_t launch_sinkhorn_plain_fwd(const float *inp, float *out, int batch, in
 hipError_t launch_sinkhorn_plain_bwd(const float *grad, const float *inp, float *d_inp, int batch,
                                      int rows, int cols, int T, float eps, float *scal,
                                      hipStream_t stream) {
+    if (sinkhorn_small_supported(rows, cols, T))
+        return launch_sinkhorn_small<true>(inp, nullptr, grad, d_inp, batch, rows, T, eps, stream);
     sinkhorn_plain_fwd_kernel<<<batch, 256, 0, stream>>>(inp, nullptr, rows, cols, T, eps, scal);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

@@ -22,7 +22,10 @@ def test_sinkhorn_knopp_doubly_stochastic():
 @pytest.mark.parametrize("shape,iters", [((32, 32), 10), ((64, 64), 20), ((4, 4), 20), ((5, 9), 7),
                                          ((3, 16, 16), 10), ((128, 128), 5), ((2, 8, 8), 20),
                                          ((70000, 4, 4), 20), ((3000, 32, 32), 3), ((7, 128, 3), 1024),
-                                         ((4, 3, 100), 200), ((2, 64, 128), 60)])
+                                         ((4, 3, 100), 200), ((2, 64, 128), 60),
+                                         # square matrices up to 8 x 8 with at most 96 iterations: the in-register kernel
+                                         ((9, 3, 3), 20), ((5, 7, 7), 96), ((1030, 8, 8), 20), ((6, 5, 5), 0), ((3, 2, 2), 1),
+                                         ((3, 8, 8), 97), ((7, 1, 1), 5)])
 def test_sinkhorn_knopp_forward_backward_vs_oracle(shape, iters):
     from mhc import sinkhorn_knopp
     g = torch.Generator().manual_seed(1)
