@@ -171,7 +171,7 @@ template <bool AK, bool BK> static hipError_t launch_gemm(const GemmArgs &a, int
 }
 
 bool gemm_f32_supported(int x_dtype, int phi_dtype, int n, int C) {
-    return x_dtype == kF32 && phi_dtype == kF32 && n > 8 && (n * C) % 4 == 0;
+    return x_dtype == kF32 && phi_dtype == kF32 && (n * C) % 4 == 0 && n * C >= 256;
 }
 
 int gemm_f32_proj_ksplit(int B, int n, int C, int max_splits) {
@@ -181,6 +181,8 @@ int gemm_f32_proj_ksplit(int B, int n, int C, int max_splits) {
     const int cap = nC / (8 * kGK);  // at least 8 slices per split
     if (ks > cap) ks = cap;
     if (ks > max_splits) ks = max_splits;
+    // n <= 8: the fused forward kernel sums at most 24 splits (16 for rows longer than 2048) in its one round of loads
+    if (n <= 8 && ks > (C <= 2048 ? 24 : 16)) ks = C <= 2048 ? 24 : 16;
     if (ks < 1) ks = 1;
     // whole slices per split; drop the splits that would get none
     const int kps = ((nC + ks - 1) / ks + kGK - 1) / kGK * kGK;
