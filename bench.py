@@ -123,10 +123,10 @@ def synthetic_inputs(torch, cfg, with_f):
 class Step:
     """Pre-allocated tensors and the two C-ABI calls of one configuration."""
 
-    def __init__(self, cfg, view, torch):
+    def __init__(self, cfg, view, torch, lib=None):
         from mhc import _lib
 
-        self.torch, self.lib, self._lib = torch, _lib.lib, _lib
+        self.torch, self.lib, self._lib = torch, (lib if lib is not None else _lib.lib), _lib
         self.cfg, self.view = cfg, view
         B, n, C = cfg["B"], cfg["n"], cfg["C"]
         dev = torch.device("cuda:0")

@@ -1,6 +1,6 @@
 """Builds libmhc_hip.so (hand-written HIP kernels + C ABI) for gfx950 with hipcc.
 
-    python mhc.cu_amd/build.py [--jobs N] [--profile] [--no-ext]
+    python mhc.cu_amd/build.py [--jobs N] [--profile | --tuning] [--no-ext]
 
 hipcc cross-compiles for gfx950 without a GPU.  The library lands in mhc.cu_amd/mhc/ next to
 the Python package that loads it; object files go to mhc.cu_amd/build/.
@@ -18,8 +18,8 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "mhc", "libmhc_hip.so")
 
-SOURCES = ["capi.hip", "proj_fwd.hip", "gemm_f32.hip", "proj_bwd.hip", "proj_bwd_large.hip", "bwd_slab.hip", "coef_fwd.hip", "mix_fwd.hip", "layer_fwd_onepass.hip", "mix_bwd_reduce.hip",
-           "mix_bwd_dx.hip", "param_grads.hip", "pack_params.hip", "ops.hip", "stream_probe.hip"]
+SOURCES = ["capi.hip", "proj_fwd.hip", "gemm_f32.hip", "proj_bwd.hip", "proj_bwd_addx.hip", "proj_bwd_large.hip", "bwd_slab.hip", "coef_fwd.hip", "mix_fwd.hip", "layer_fwd_onepass.hip", "mix_bwd_reduce.hip",
+           "bwd_resident.hip", "mix_bwd_dx.hip", "param_grads.hip", "pack_params.hip", "ops.hip", "stream_probe.hip"]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are not trusted on this hardware pool.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -35,6 +35,7 @@ def _hipcc():
 
 
 PROFILE_LIB = os.path.join(HERE, "mhc", "libmhc_hip_profile.so")
+TUNING_LIB = os.path.join(HERE, "mhc", "libmhc_hip_tuning.so")
 
 
 def _compile(src, extra=(), suffix=""):
@@ -45,12 +46,16 @@ def _compile(src, extra=(), suffix=""):
     return src, obj, p.returncode, err
 
 
-def build(jobs: int = 8, verbose: bool = True, profile: bool = False):
+def build(jobs: int = 8, verbose: bool = True, profile: bool = False, tuning: bool = False):
     """profile=True builds libmhc_hip_profile.so instead: the same library with the in-kernel phase
-    profiler compiled in (csrc/phase_profiler.h) and the extra entry point mhc_phase_read."""
+    profiler compiled in (csrc/phase_profiler.h) and the extra entry point mhc_phase_read.
+    tuning=True builds libmhc_hip_tuning.so instead: the same library with the launch-heuristic
+    overrides of csrc/tuning.h and their setter mhc_tuning_set, for experiments and for the tests that
+    compare two launch paths on the same inputs; the product library has neither."""
     os.makedirs(OBJ, exist_ok=True)
     objs = []
-    extra, suffix, lib = ((("-DMHC_PHASE_PROFILE", "-fgpu-rdc"), "_prof", PROFILE_LIB) if profile else ((), "", LIB))
+    extra, suffix, lib = ((("-DMHC_PHASE_PROFILE", "-fgpu-rdc"), "_prof", PROFILE_LIB) if profile
+                          else ((("-DMHC_TUNING",), "_tune", TUNING_LIB) if tuning else ((), "", LIB)))
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
         for src, obj, rc, err in ex.map(lambda s_: _compile(s_, extra, suffix), SOURCES):
             if err.strip() and verbose:
@@ -107,8 +112,9 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
     ap.add_argument("--profile", action="store_true", help="build libmhc_hip_profile.so (in-kernel phase profiler)")
+    ap.add_argument("--tuning", action="store_true", help="build libmhc_hip_tuning.so (launch-heuristic overrides)")
     ap.add_argument("--no-ext", action="store_true", help="skip the PyTorch extension (about a minute of g++)")
     a = ap.parse_args()
-    build(a.jobs, profile=a.profile)
-    if not a.profile and not a.no_ext:
+    build(a.jobs, profile=a.profile, tuning=a.tuning)
+    if not a.profile and not a.tuning and not a.no_ext:
         build_torch_ext()

@@ -14,9 +14,11 @@
 
 using namespace mhc;
 
+#ifdef MHC_TUNING
 namespace mhc {
 int g_tuning[kTuneCount];
 }
+#endif
 
 namespace {
 
@@ -60,6 +62,14 @@ int ws_check(void *ws, size_t have, size_t need) {
 // ---- dynamic workspace layout ----------------------------------------------------------------
 struct DynFwdWs { float *Ppart, *ssqpart, *agg; size_t bytes; };
 struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *raw, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
+
+// Whether the sample-resident backward (bwd_resident.hip + the column-slab kernel without batch split)
+// is taken where it is supported.  Experiment hook: 1 = never, 2 = always.
+bool bwd_resident_preferred(int B, int n, int C) {
+    if (const int hook = tuning_get(kTuneResident)) return hook == 2;
+    (void)B; (void)n; (void)C;
+    return false;
+}
 
 int max_ksplit(int B, int n, int C) {
     const int a = proj_fwd_ksplit(kBF16, kBF16, B, n, C), b = proj_fwd_ksplit(kF32, kF32, B, n, C);
@@ -150,7 +160,8 @@ __attribute__((visibility("default"))) int mhc_phase_read(int kernel, unsigned l
 
 int mhc_abi_version(void) { return MHC_ABI_VERSION; }
 
-// Experiment hook (csrc/tuning.h), deliberately absent from the public header.
+#ifdef MHC_TUNING
+// Experiment hooks (csrc/tuning.h): only in the -DMHC_TUNING build, never in the product library.
 __attribute__((visibility("default"))) int mhc_tuning_set(int key, int value) {
     if (key < 0 || key >= kTuneCount) return -1;
     g_tuning[key] = value;
@@ -159,6 +170,7 @@ __attribute__((visibility("default"))) int mhc_tuning_set(int key, int value) {
 __attribute__((visibility("default"))) int mhc_tuning_get(int key) {
     return (key < 0 || key >= kTuneCount) ? -1 : g_tuning[key];
 }
+#endif
 
 int mhc_max_sinkhorn_iters(int n) { return (n < 1 || n > MHC_MAX_N) ? 0 : max_layer_sinkhorn_iters(n); }
 
@@ -258,6 +270,23 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     const int D = n * n + 2 * n, DP = padded_D(n);
     const bool mfma = proj_bwd_mfma_supported(x_dtype, phi_dtype, C);
     BwdCoefOut out{ws.dt, ws.dP, ws.cx, ws.s1, nullptr, mfma ? ws.dPb : nullptr, ws.dPT, ws.BP};
+    if (mfma && bwd_resident_supported(x_dtype, y_dtype, phi_dtype, n, C, iters) && proj_bwd_addx_supported(n) &&
+        bwd_resident_preferred(B, n, C)) {
+        // two launches: (1) one workgroup per sample keeps the sample's rows of dy and x in registers for
+        // the channel sums, the coefficient backward and the mixing part of dx; (2) a column-slab
+        // kernel over all samples adds dP phi - cx x, finishes dphi without batch-split partial sums
+        // and sums dw, dbias and dalpha in a few extra workgroups
+        MHC_LAUNCH(launch_bwd_resident(dy, x, w, w_dtype, f_inject, H_pre, H_post, M, q, P, r, alpha, bias + 2 * n,
+                                       sk_state, out, dx, df, ws.u, B, n, C, iters, eps, st));
+        const BatchSumArgs sums = make_batch_sums(ws.u, B, C, f_inject ? nullptr : dw, ws.dt, B, D, dbias, dalpha);
+        bool tail_taken = false;
+        MHC_LAUNCH(launch_proj_bwd_addx(x, phi, ws.dPb, ws.dPT, ws.BP, ws.cx, dphi, dx, B, n, C,
+                                        tuning_get(kTuneSeparateFinalize) == 1 ? nullptr : &sums, &tail_taken, st));
+        if (!tail_taken)
+            MHC_LAUNCH(launch_finalize(ws.u, B, C, f_inject ? nullptr : dw, ws.dt, B, D, dbias, dalpha, nullptr, 1,
+                                       0, nullptr, st));
+        return MHC_OK;
+    }
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      n, q, P, r, alpha, bias + 2 * n, sk_state, out, ws.raw, B, n, C, iters, eps,
                                      st));

@@ -165,6 +165,23 @@ hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb,
                                 int BP, float *dphi, float *dphi_part, void *dxflat, int B, int n,
                                 int C, hipStream_t stream, int part = kProjPartBoth,
                                 const BatchSumArgs *tail = nullptr, bool *tail_taken = nullptr);
+
+// Sample-resident first launch of the n <= 8 bf16 backward: channel sums, coefficient backward (all
+// outputs of launch_mix_bwd_reduce) and dxp = M^T dy + Hpre (x) da from ONE pass over dy and x, one
+// workgroup per sample; u [B, C] = the samples' summands of dw, df with an injected f.
+bool bwd_resident_supported(int x_dtype, int y_dtype, int phi_dtype, int n, int C, int T);
+hipError_t launch_bwd_resident(const void *dy, const void *x, const void *w, int w_dtype, const void *f_inject,
+                               const float *Hpre, const float *Hpost, const float *M, const float *q,
+                               const float *P, const float *r, const float *alpha, const float *b_res,
+                               const float *sk_state, BwdCoefOut out, void *dxp, void *df, float *u, int B, int n,
+                               int C, int T, float eps, hipStream_t stream);
+// Second and last launch of that backward (D <= 96): a column slab for all samples per workgroup;
+// dphi = dP^T x_flat without batch split, dx completed in place (dx = dxp + dP phi - cx x), and `tail`
+// (dw, dbias, dalpha) summed by extra workgroups when the grid has room (*tail_taken).
+bool proj_bwd_addx_supported(int n);
+hipError_t launch_proj_bwd_addx(const void *x, const void *phi, const void *dPb, const void *dPT, int BP,
+                                const float *cx, float *dphi, void *dx, int B, int n, int C, const BatchSumArgs *tail,
+                                bool *tail_taken, hipStream_t stream);
 // n <= 18: whether the two products are faster apart (measured: from D > 128 on)
 bool proj_bwd_products_apart(int n);
 // Wide projections (more than 12 row tiles of 32, n > 18) always run the two products as two GEMM

@@ -1,0 +1,270 @@
+// Backward, second (and last) launch behind the sample-resident kernel (bwd_resident.hip), bf16 tier,
+// D <= 96 (n <= 8): a workgroup owns a slab of 32 columns of x_flat / phi for ALL samples, so that
+//
+//   dphi[d, k] = sum_b dP[b, d] x_flat[b, k]                      (reference ops.py:332-334)
+//
+// is finished here without batch-split partial sums, and completes dx in place,
+//
+//   dx[b, k] = dxp[b, k] + sum_d dP[b, d] phi[d, k] - cx[b] x_flat[b, k]      (reference ops.py:336-351)
+//
+// where dxp = M^T dy + Hpre (x) da was left in the dx buffer by the first launch.  A few extra
+// workgroups (one more grid row) add up dw, dbias and dalpha (batch_sums.h), so the backward needs no
+// third launch.
+//
+// Samples are walked in blocks of 256.  Per block every thread requests its 16-byte chunks of x and
+// dxp up front (row-contiguous, next block in flight while this one is worked on); x is parked in
+// LDS as [sample][column] and read back transposed as the B operand of v_mfma_f32_32x32x16_bf16 (the
+// contraction of dphi runs over samples, the strided axis).  Wave w owns samples 64w .. 64w+63 of
+// the block: it accumulates their share of every dphi tile (dP^T from global memory in fragment
+// order, rounded value + remainder), forms dP phi for them (phi fragments from the slab in LDS),
+// hands the result through a wave-private LDS tile to a row-major epilogue - 16-byte loads of dxp,
+// 16-byte stores of dx - and at the very end the four waves' dphi shares are summed through LDS.
+#include "launchers.h"
+
+#include <type_traits>
+#include "mhc_common.h"
+
+namespace mhc {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+struct ProjAddxArgs {
+    const bf16_t *x;     // [B][nC]
+    const bf16_t *phi;   // [D][nC]
+    const bf16_t *dPb;   // dP, fragment-major (frag_dpb); columns >= D are zero
+    const bf16_t *dPT;   // dP^T hi and lo bf16 planes, fragment-major (frag_dpt); rows >= D, columns >= B zero
+    const float *cx;     // [B]
+    float *dphi;         // [D][nC]
+    bf16_t *dx;          // [B][nC]: in dxp, out dx
+    int B, BP, D, DP, nC;
+    int tail_row;        // blockIdx.y of the workgroups that compute `tail` (-1: none)
+    BatchSumArgs tail;
+};
+
+constexpr int kAxKW = 32;          // slab width (columns)
+constexpr int kAxLD = kAxKW + 8;   // LDS pitch of the bf16 tiles (elements): rows stay 16-byte aligned
+constexpr int kAxLDO = kAxKW + 4;  // LDS pitch of the fp32 tile of dP phi
+constexpr int kAxSBR = 256;        // samples per block
+constexpr int kAxLDR = 33;         // LDS pitch of the dphi tiles in the final cross-wave sum
+
+template <int NTD>
+__global__ __launch_bounds__(256) void proj_bwd_addx_kernel(ProjAddxArgs a) {
+    extern __shared__ __align__(16) unsigned char ax_smem[];
+    bf16_t *phi_s = reinterpret_cast<bf16_t *>(ax_smem);                 // [32 NTD][LD]
+    bf16_t *x_s = phi_s + (size_t)32 * NTD * kAxLD;                       // [SBR][LD]
+    float *o_s = reinterpret_cast<float *>(x_s + (size_t)kAxSBR * kAxLD);  // [SBR][LDO]
+    float *red_s = reinterpret_cast<float *>(x_s);                        // final sum: [4][NTD][32][LDR], over x_s and o_s
+    static_assert(sizeof(float) * 4 * NTD * 32 * kAxLDR <= sizeof(bf16_t) * kAxSBR * kAxLD + sizeof(float) * kAxSBR * kAxLDO,
+                  "the cross-wave sum of dphi reuses the x and output tiles");
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if ((int)blockIdx.y == a.tail_row) {
+        // the extra row of the grid: its first workgroups do the batch sums, the others have nothing to do
+        if ((int)blockIdx.x < a.tail.nblk) batch_sum_block<4>(a.tail, blockIdx.x, tid, reinterpret_cast<double *>(ax_smem));
+        return;
+    }
+    // Workgroup ids go round robin over the 8 XCDs (each with its own L2, 128-byte lines).  A slab
+    // row of 32 columns is half a line: neighbouring slabs are given to the same XCD (ids x and
+    // x + 8 of a group of 16), otherwise two L2s fetch every line of x, dxp and phi.
+    const int slab = (blockIdx.x >> 4) * 16 + (blockIdx.x & 7) * 2 + ((blockIdx.x >> 3) & 1);
+    const int k0 = slab * kAxKW;
+    if (k0 >= a.nC) return;  // ids of the padded grid; the whole workgroup, before any barrier
+    const int row = lane & 31, kg = lane >> 5;
+    const int D = a.D, nC = a.nC, B = a.B;
+
+    // ---- per-block loads: x for the LDS tile (thread -> chunks tid + 256 u) and, for the epilogue,
+    // the chunks of dxp this thread completes: sample 64 wave + lane / 4 + 16 t, chunk lane % 4 -------
+    const int ech = lane & 3, erow = 64 * wave + (lane >> 2);
+    const int kc = k0 + ech * 8;
+    const bool kok = kc < nC;  // nC % 8 == 0: a chunk is inside or outside
+    uint32_t xr[2][4][4], pr[2][4][4];
+    float cxr[2][4];
+    auto load_block = [&](int sb, auto slot) {
+        constexpr int S = decltype(slot)::value;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int ch = tid + u * 256;
+            const int b = sb + (ch >> 2), k = k0 + (ch & 3) * 8;
+            const bool ok = b < B && k < nC;
+            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(a.x + (ok ? (size_t)b * nC + k : 0)), ok);
+            xr[S][u][0] = v.x; xr[S][u][1] = v.y; xr[S][u][2] = v.z; xr[S][u][3] = v.w;
+        }
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int b = sb + erow + 16 * t;
+            const bool ok = b < B && kok;
+            const uint4 v = *reinterpret_cast<const uint4 *>(a.dx + (ok ? (size_t)b * nC + kc : 0));
+            pr[S][t][0] = v.x; pr[S][t][1] = v.y; pr[S][t][2] = v.z; pr[S][t][3] = v.w;
+            cxr[S][t] = a.cx[b < B ? b : 0];
+        }
+    };
+    using Slot0 = std::integral_constant<int, 0>;
+    using Slot1 = std::integral_constant<int, 1>;
+
+    // ---- phi slab -> LDS (rows >= D and columns >= nC read as zero), first blocks requested ---------
+    constexpr int PCH = 32 * NTD * 4;  // 16-byte chunks of the slab
+    uint4 phir[(PCH + 255) / 256];
+#pragma unroll
+    for (int u = 0; u < (PCH + 255) / 256; u++) {
+        const int ch = tid + u * 256;
+        const int d = ch >> 2, k = k0 + (ch & 3) * 8;
+        const bool ok = ch < PCH && d < D && k < nC;
+        phir[u] = load16_masked(reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * nC + k : 0)), ok);
+    }
+    load_block(0, Slot0{});
+    if (kAxSBR < B) load_block(kAxSBR, Slot1{});
+#pragma unroll
+    for (int u = 0; u < (PCH + 255) / 256; u++) {
+        const int ch = tid + u * 256;
+        if (ch < PCH) *reinterpret_cast<uint4 *>(phi_s + (size_t)(ch >> 2) * kAxLD + (ch & 3) * 8) = phir[u];
+    }
+    __syncthreads();
+    bf16x8_t phif[2 * NTD];
+#pragma unroll
+    for (int ks = 0; ks < 2 * NTD; ks++)
+        phif[ks] = __builtin_bit_cast(bf16x8_t, lds_frag_tr(phi_s, kAxLD, ks * 16, 0, lane));
+
+    f32x16_t acc[NTD];
+#pragma unroll
+    for (int m = 0; m < NTD; m++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[m][i] = 0.f;
+
+    auto process_block = [&](int sb, auto slot) {
+        constexpr int S = decltype(slot)::value;
+        // ---- operands that come straight from global memory, requested ahead of the barriers ----------
+        // dP^T of this wave's 64 samples (k-steps 4 wave .. + 3 of the block) for every dphi tile, and dP
+        // of its two 32-sample tiles.  Steps and tiles beyond the padded batch read zeros.
+        const int step0 = (sb >> 4) + 4 * wave, nsteps = a.BP >> 4;
+        uint4 ah[NTD][4], al[NTD][4], av[2][2 * NTD];
+#pragma unroll
+        for (int m = 0; m < NTD; m++)
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                const bool ok = step0 + ks < nsteps;
+                const bf16_t *ap = a.dPT + (ok ? frag_base(m, nsteps, step0 + ks) : 0) + lane * 8;
+                ah[m][ks] = load16_masked(reinterpret_cast<const uint4 *>(ap), ok);
+                al[m][ks] = load16_masked(reinterpret_cast<const uint4 *>(ap + (size_t)a.DP * a.BP), ok);
+            }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const int tile = (sb >> 5) + 2 * wave + t;
+            const bool ok = tile < (a.BP >> 5);
+#pragma unroll
+            for (int ks = 0; ks < 2 * NTD; ks++)
+                av[t][ks] = load16_masked(
+                    reinterpret_cast<const uint4 *>(a.dPb + (ok ? frag_base(tile, a.DP >> 4, ks) : 0) + lane * 8), ok);
+        }
+        // ---- x block -> LDS ---------------------------------------------------------------------------
+        if (sb != 0) __syncthreads();  // every wave is done with the previous block's tile
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int ch = tid + u * 256;
+            *reinterpret_cast<uint4 *>(x_s + (size_t)(ch >> 2) * kAxLD + (ch & 3) * 8) =
+                make_uint4(xr[S][u][0], xr[S][u][1], xr[S][u][2], xr[S][u][3]);
+        }
+        __syncthreads();
+        // ---- dphi: this wave's samples, every row tile ------------------------------------------------
+        bf16x8_t xf[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+            xf[ks] = __builtin_bit_cast(bf16x8_t, lds_frag_tr(x_s, kAxLD, (4 * wave + ks) * 16, 0, lane));
+#pragma unroll
+        for (int m = 0; m < NTD; m++)
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ah[m][ks]), xf[ks], acc[m], 0, 0, 0);
+                acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, al[m][ks]), xf[ks], acc[m], 0, 0, 0);
+            }
+        // ---- dP phi of this wave's two sample tiles -> its own rows of o_s ------------------------------
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            f32x16_t o;
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[i] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 2 * NTD; ks++)
+                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av[t][ks]), phif[ks], o, 0, 0, 0);
+            // accumulator layout: column = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                o_s[(size_t)(64 * wave + 32 * t + 8 * (i >> 2) + 4 * kg + (i & 3)) * kAxLDO + row] = o[i];
+        }
+        // ---- epilogue, row-major: the wave reads back only rows it wrote itself (its LDS accesses
+        // complete in order), x from the block's tile ------------------------------------------------------
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int r = erow + 16 * t, b = sb + r;
+            const float4 o0 = *reinterpret_cast<const float4 *>(o_s + (size_t)r * kAxLDO + ech * 8);
+            const float4 o1 = *reinterpret_cast<const float4 *>(o_s + (size_t)r * kAxLDO + ech * 8 + 4);
+            const uint4 xv = *reinterpret_cast<const uint4 *>(x_s + (size_t)r * kAxLD + ech * 8);
+            const float cxv = cxr[S][t];
+            const float ov[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
+            const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+            uint32_t outw[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const float lo = bf16lo_to_f32(pr[S][t][p]) + ov[2 * p] - cxv * bf16lo_to_f32(xw[p]);
+                const float hi = bf16hi_to_f32(pr[S][t][p]) + ov[2 * p + 1] - cxv * bf16hi_to_f32(xw[p]);
+                outw[p] = pack_bf16x2(lo, hi);
+            }
+            if (b < B && kok) st16<true>(a.dx + (size_t)b * nC + kc, outw[0], outw[1], outw[2], outw[3]);
+        }
+        if (sb + 2 * kAxSBR < B) load_block(sb + 2 * kAxSBR, slot);
+    };
+    for (int sb = 0; sb < B; sb += 2 * kAxSBR) {
+        process_block(sb, Slot0{});
+        if (sb + kAxSBR < B) process_block(sb + kAxSBR, Slot1{});
+    }
+
+    // ---- dphi: sum the four waves' shares through LDS, store row-major --------------------------------
+    __syncthreads();  // all tiles consumed; the region becomes red_s
+#pragma unroll
+    for (int m = 0; m < NTD; m++)
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            red_s[((size_t)(wave * NTD + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3)) * kAxLDR + row] = acc[m][i];
+    __syncthreads();
+    for (int e = tid; e < NTD * 32 * 32; e += 256) {
+        const int d = e >> 5, c = e & 31;
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) s += red_s[((size_t)w * NTD * 32 + d) * kAxLDR + c];
+        if (d < D && k0 + c < nC) a.dphi[(size_t)d * nC + k0 + c] = s;
+    }
+}
+
+bool proj_bwd_addx_supported(int n) { return padded_D(n) / 32 <= 3; }
+
+template <int NTD>
+static hipError_t launch_addx(const ProjAddxArgs &a, hipStream_t stream) {
+    const size_t smem = sizeof(bf16_t) * (size_t)kAxLD * (32 * NTD + kAxSBR) + sizeof(float) * kAxSBR * kAxLDO;
+    hipError_t e = allow_dynamic_lds(&proj_bwd_addx_kernel<NTD>, smem);
+    if (e != hipSuccess) return e;
+    const int slabs = (a.nC + kAxKW - 1) / kAxKW;
+    dim3 grid(round_up(slabs, 16), 1 + (a.tail_row >= 0 ? 1 : 0));
+    proj_bwd_addx_kernel<NTD><<<grid, 256, smem, stream>>>(a);
+    return hipGetLastError();
+}
+
+hipError_t launch_proj_bwd_addx(const void *x, const void *phi, const void *dPb, const void *dPT, int BP,
+                                const float *cx, float *dphi, void *dx, int B, int n, int C, const BatchSumArgs *tail,
+                                bool *tail_taken, hipStream_t stream) {
+    const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n), NTD = DP / 32;
+    ProjAddxArgs a{static_cast<const bf16_t *>(x), static_cast<const bf16_t *>(phi), static_cast<const bf16_t *>(dPb),
+                   static_cast<const bf16_t *>(dPT), cx, dphi, static_cast<bf16_t *>(dx), B, BP, D, DP, nC, -1, {}};
+    if (tail_taken) *tail_taken = false;
+    if (tail && tail->nblk <= round_up((nC + kAxKW - 1) / kAxKW, 16)) {
+        a.tail = *tail;
+        a.tail_row = 1;
+        if (tail_taken) *tail_taken = true;
+    }
+    switch (NTD) {
+        case 1: return launch_addx<1>(a, stream);
+        case 2: return launch_addx<2>(a, stream);
+        case 3: return launch_addx<3>(a, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace mhc

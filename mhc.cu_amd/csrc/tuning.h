@@ -1,7 +1,8 @@
-// Launch-heuristic overrides for experiments (host side only).  Every knob defaults to 0 = "use
-// the built-in heuristic"; mhc_tuning_set (exported, but not part of the public header) changes
-// one for the whole process.  Not thread-safe and not meant for production callers: the public
-// entry points behave identically with all knobs at 0.
+// Launch-heuristic overrides for experiments and for tests that must reach a path the heuristics
+// would not pick at the test's shape (host side only).  They exist only in a build with -DMHC_TUNING
+// (libmhc_hip_tuning.so, `build.py --tuning`): there, mhc_tuning_set changes a knob for the whole
+// process, unsynchronised.  In the product library tuning_get() is the constant 0 = "use the built-in
+// heuristic", no knob and no setter exist, and the dispatch code reads no global state.
 #pragma once
 
 namespace mhc {
@@ -14,11 +15,15 @@ enum TuneKey {
     kTuneSeparateFinalize = 4,  // 1 = batch sums always as a launch of their own, never inside the dphi launch
     kTuneProjApart = 5,     // n <= 18 projection backward: 1 = both products in one launch, 2 = two launches
     kTuneStaticSpg = 6,     // static backward: samples per workgroup of the dx kernel (n <= 8)
-    kTuneSpare3 = 7,
+    kTuneResident = 7,      // n <= 8 sample-resident backward: 0 = by heuristic, 1 = never, 2 = whenever the shape allows
     kTuneCount = 8
 };
 
+#ifdef MHC_TUNING
 extern int g_tuning[kTuneCount];
 inline int tuning_get(int key) { return g_tuning[key]; }
+#else
+constexpr int tuning_get(int) { return 0; }
+#endif
 
 }  // namespace mhc

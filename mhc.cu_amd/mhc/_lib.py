@@ -58,13 +58,38 @@ _SIGNATURES = {
     "mhc_rmsnorm_bwd_workspace_bytes": (_Z, [_I, _I]),
 }
 
-for _name, (_res, _args) in _SIGNATURES.items():
-    _fn = getattr(lib, _name)  # AttributeError here means the library does not match the header
-    _fn.restype = _res
-    _fn.argtypes = _args
+def _bind(handle):
+    for _name, (_res, _args) in _SIGNATURES.items():
+        _fn = getattr(handle, _name)  # AttributeError here means the library does not match the header
+        _fn.restype = _res
+        _fn.argtypes = _args
+    if handle.mhc_abi_version() != ABI_VERSION:
+        raise ImportError(f"{handle._name}: ABI {handle.mhc_abi_version()} != binding ABI {ABI_VERSION}")
+    return handle
 
-if lib.mhc_abi_version() != ABI_VERSION:
-    raise ImportError(f"libmhc_hip.so ABI {lib.mhc_abi_version()} != binding ABI {ABI_VERSION}")
+
+_bind(lib)
+
+_TUNING_LIB = None
+
+
+def tuning_lib():
+    """The test/experiment build of the same library (libmhc_hip_tuning.so, `build.py --tuning`): the same
+    entry points plus mhc_tuning_set / mhc_tuning_get, which override the launch heuristics
+    (csrc/tuning.h) for the whole process.  The product library above has no such hooks; tests load
+    this one to compare two launch paths on the same inputs."""
+    global _TUNING_LIB
+    if _TUNING_LIB is None:
+        path = os.path.join(_HERE, "libmhc_hip_tuning.so")
+        if not os.path.exists(path):
+            raise ImportError(f"{path} not found: python mhc.cu_amd/build.py --tuning")
+        handle = _bind(ctypes.CDLL(path))
+        handle.mhc_tuning_set.restype = c_int
+        handle.mhc_tuning_set.argtypes = [c_int, c_int]
+        handle.mhc_tuning_get.restype = c_int
+        handle.mhc_tuning_get.argtypes = [c_int]
+        _TUNING_LIB = handle
+    return _TUNING_LIB
 
 
 class MHCError(RuntimeError):
