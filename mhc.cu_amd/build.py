@@ -48,13 +48,14 @@ def _compile(src, extra=(), suffix=""):
 
 def build(jobs: int = 8, verbose: bool = True, profile: bool = False, tuning: bool = False):
     """profile=True builds libmhc_hip_profile.so instead: the same library with the in-kernel phase
-    profiler compiled in (csrc/phase_profiler.h) and the extra entry point mhc_phase_read.
+    profiler compiled in (csrc/phase_profiler.h), the extra entry point mhc_phase_read and the
+    launch-heuristic overrides of the tuning build.
     tuning=True builds libmhc_hip_tuning.so instead: the same library with the launch-heuristic
     overrides of csrc/tuning.h and their setter mhc_tuning_set, for experiments and for the tests that
     compare two launch paths on the same inputs; the product library has neither."""
     os.makedirs(OBJ, exist_ok=True)
     objs = []
-    extra, suffix, lib = ((("-DMHC_PHASE_PROFILE", "-fgpu-rdc"), "_prof", PROFILE_LIB) if profile
+    extra, suffix, lib = ((("-DMHC_PHASE_PROFILE", "-DMHC_TUNING", "-fgpu-rdc"), "_prof", PROFILE_LIB) if profile
                           else ((("-DMHC_TUNING",), "_tune", TUNING_LIB) if tuning else ((), "", LIB)))
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
         for src, obj, rc, err in ex.map(lambda s_: _compile(s_, extra, suffix), SOURCES):

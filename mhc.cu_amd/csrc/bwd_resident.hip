@@ -61,6 +61,12 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
     extern __shared__ float sc[];         // Sinkhorn denominators, SK::scaling_floats(T), then CB::kXch
     const int b = blockIdx.x, n = a.n, C = a.C;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int pwg = blockIdx.x;
+    (void)pwg;
+    MHC_PHASE_ZERO(kPhaseGramSmall, pwg);
+    MHC_PHASE_ZERO(kPhaseDxSmall, pwg);   // second timeline: the first tile wave (thread 64)
+    MHC_PHASE_BEGIN(pclk);
+    MHC_PHASE_BEGIN(tclk);
     CB cb;
     if (tid < SK::kGroup) {
         // everything the coefficient backward needs besides the sums, requested at once
@@ -75,6 +81,7 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
         const float ho = a.Hpost[(size_t)b * n + (r < n ? r : 0)], hp = a.Hpre[(size_t)b * n + (c < n ? c : 0)];
         hohp = (r < n && c < n) ? ho * hp : 0.f;
     }
+    MHC_PHASE_ADD(kPhaseGramSmall, pwg, 0, pclk);
     const int blk = lane >> 2, i = lane & 3;
     const int tw = wave - 1;              // tile wave index, -1 for the coefficient wave
     const bool tile = tw >= 0;
@@ -131,6 +138,7 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
             if (!sv[I]) { hpre[I] = 0.f; hpost[I] = 0.f; }
     }
 
+    MHC_PHASE_ADD_BY(64, kPhaseDxSmall, pwg, 0, tclk);
     // ---- 1. Gram sums -------------------------------------------------------------------------------
     if (tile) {
         f32x4_t acc[3][NB][NB];
@@ -208,7 +216,9 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
                             slot_s[(m * NP * NP + (4 * I + r) * NP + 4 * J + (tid & 3)) * (TW * 4) + slot] = v;
                     }
     }
+    MHC_PHASE_ADD_BY(64, kPhaseDxSmall, pwg, 1, tclk);
     __syncthreads();
+    MHC_PHASE_ADD(kPhaseGramSmall, pwg, 1, pclk);
     // K threads finish the sums; the NP^2 threads that hold W1 (one DPP row for 4x4, wave 1 for 8x8)
     // also form s1 = Hpost^T W1 Hpre, which the tile waves need for da
     if (tid < K) {
@@ -225,11 +235,14 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
     }
     __syncthreads();
 
+    MHC_PHASE_ADD(kPhaseGramSmall, pwg, 2, pclk);
+    MHC_PHASE_ADD_BY(64, kPhaseDxSmall, pwg, 2, tclk);
     // ---- 2. coefficient backward on the first lanes of wave 0 -----------------------------------------
     if (tid < SK::kGroup) {
         cb.fetch_sums(tot_s, 1);
         cb.run(a, b, tid, tid, sc, sc + SK::scaling_floats(a.T));
     }
+    MHC_PHASE_ADD(kPhaseGramSmall, pwg, 3, pclk);
     if (!tile) return;
 
     // ---- 3. tile waves: dxp, u, df ---------------------------------------------------------------------
@@ -298,6 +311,7 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
             if (sv[I]) store_vec<bf16_t, 8>(ra.dxp + ((size_t)b * n + 4 * I + i) * C + c, out);
         }
     }
+    MHC_PHASE_ADD_BY(64, kPhaseDxSmall, pwg, 3, tclk);
 }
 
 // The rows of a sample must fit the tile waves' registers; the Sinkhorn state shares the LDS.

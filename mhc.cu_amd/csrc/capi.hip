@@ -64,11 +64,17 @@ struct DynFwdWs { float *Ppart, *ssqpart, *agg; size_t bytes; };
 struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *raw, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
 
 // Whether the sample-resident backward (bwd_resident.hip + the column-slab kernel without batch split)
-// is taken where it is supported.  Experiment hook: 1 = never, 2 = always.
+// is taken where it is supported.  Its second launch walks all samples of a column slab in one
+// workgroup, which stops paying once the batch is large enough to fill the chip with batch splits.
+// Measured, backward in graphs of ten, slab / Gram path -> resident path (us):
+//   n=4 C=1280: B=64 17.1 -> 9.2, 128 17.2 -> 9.7, 320 19.1 -> 16.1, 512 23.6 -> 19.8, 768 25.3 -> 26.0,
+//               1024 29.8 -> 30.5, 2560 46.2 -> 62.5;  n=4 C=2560: B=256 23.9 -> 17.8, 512 32.1 -> 27.7, 1280 42.4 -> 53.9
+//   n=8 C=1280: B=128 25.1 -> 16.9, 256 30.5 -> 22.0, 512 46.1 -> 36.1, 1024 77.3 -> 62.7
+// Experiment hook: 1 = never, 2 = always.
 bool bwd_resident_preferred(int B, int n, int C) {
     if (const int hook = tuning_get(kTuneResident)) return hook == 2;
-    (void)B; (void)n; (void)C;
-    return false;
+    (void)C;
+    return n > 4 || B <= 640;
 }
 
 int max_ksplit(int B, int n, int C) {

@@ -36,6 +36,13 @@ __device__ __forceinline__ unsigned long long phase_add(int kernel, int wg, int 
     if (threadIdx.x == 0 && wg < kPhaseMaxWg) g_phase[kernel][wg][mark] += t - since;
     return t;
 }
+// the same from a chosen thread of the workgroup (a second timeline, e.g. of another wave)
+__device__ __forceinline__ unsigned long long phase_add_by(int thread, int kernel, int wg, int mark, unsigned long long since) {
+    const unsigned long long t = phase_clock();
+    if ((int)threadIdx.x == thread && wg < kPhaseMaxWg) g_phase[kernel][wg][mark] += t - since;
+    return t;
+}
+#define MHC_PHASE_ADD_BY(thread, kernel, wg, mark, var) var = ::mhc::phase_add_by(thread, kernel, wg, mark, var)
 #define MHC_PHASE(kernel, wg, mark) ::mhc::phase_mark(kernel, wg, mark)
 #define MHC_PHASE_BEGIN(var) unsigned long long var = ::mhc::phase_clock()
 #define MHC_PHASE_ZERO(kernel, wg)                                                        \
@@ -49,6 +56,7 @@ __device__ __forceinline__ unsigned long long phase_add(int kernel, int wg, int 
 #define MHC_PHASE_BEGIN(var) ((void)0)
 #define MHC_PHASE_ZERO(kernel, wg) ((void)0)
 #define MHC_PHASE_ADD(kernel, wg, mark, var) ((void)0)
+#define MHC_PHASE_ADD_BY(thread, kernel, wg, mark, var) ((void)0)
 #endif
 
 }  // namespace mhc

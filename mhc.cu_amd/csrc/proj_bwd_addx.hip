@@ -11,11 +11,11 @@
 // workgroups (one more grid row) add up dw, dbias and dalpha (batch_sums.h), so the backward needs no
 // third launch.
 //
-// Samples are walked in blocks of 256.  Per block every thread requests its 16-byte chunks of x and
-// dxp up front (row-contiguous, next block in flight while this one is worked on); x is parked in
-// LDS as [sample][column] and read back transposed as the B operand of v_mfma_f32_32x32x16_bf16 (the
-// contraction of dphi runs over samples, the strided axis).  Wave w owns samples 64w .. 64w+63 of
-// the block: it accumulates their share of every dphi tile (dP^T from global memory in fragment
+// Samples are walked in blocks of 256 (D <= 32) or 128.  Per block every thread requests its 16-byte
+// chunks of x and dxp up front (row-contiguous, next block in flight while this one is worked on); x is
+// parked in LDS as [sample][column] and read back transposed as the B operand of
+// v_mfma_f32_32x32x16_bf16 (the contraction of dphi runs over samples, the strided axis).  Wave w owns a
+// quarter of the block's samples: it accumulates their share of every dphi tile (dP^T from global memory in fragment
 // order, rounded value + remainder), forms dP phi for them (phi fragments from the slab in LDS),
 // hands the result through a wave-private LDS tile to a row-major epilogue - 16-byte loads of dxp,
 // 16-byte stores of dx - and at the very end the four waves' dphi shares are summed through LDS.
@@ -45,18 +45,22 @@ struct ProjAddxArgs {
 constexpr int kAxKW = 32;          // slab width (columns)
 constexpr int kAxLD = kAxKW + 8;   // LDS pitch of the bf16 tiles (elements): rows stay 16-byte aligned
 constexpr int kAxLDO = kAxKW + 4;  // LDS pitch of the fp32 tile of dP phi
-constexpr int kAxSBR = 256;        // samples per block
 constexpr int kAxLDR = 33;         // LDS pitch of the dphi tiles in the final cross-wave sum
 
-template <int NTD>
-__global__ __launch_bounds__(256) void proj_bwd_addx_kernel(ProjAddxArgs a) {
+// NTD: 32-row tiles of dphi (D <= 32 NTD).  SPW: samples a wave owns per block (32 or 64; a block is
+// 4 SPW samples).  PFOP: the dP operands of the next block are requested a block ahead like x and dxp.
+// Measured at B=320, C=1280, n=4 (backward, graphs of ten): SPW 32 without / with PFOP 16.1 / 16.1 us,
+// SPW 64 without PFOP 19.1 us, with PFOP 23.0 us (registers spill).
+template <int NTD, int SPW, bool PFOP>
+__global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
+    constexpr int SBR = 4 * SPW;   // samples per block
+    constexpr int KS = SPW / 16;   // k-steps (16 samples) of a wave per block = its 16-byte chunks of x and of dxp
+    constexpr int TT = SPW / 32;   // 32-sample tiles of a wave per block
     extern __shared__ __align__(16) unsigned char ax_smem[];
     bf16_t *phi_s = reinterpret_cast<bf16_t *>(ax_smem);                 // [32 NTD][LD]
     bf16_t *x_s = phi_s + (size_t)32 * NTD * kAxLD;                       // [SBR][LD]
-    float *o_s = reinterpret_cast<float *>(x_s + (size_t)kAxSBR * kAxLD);  // [SBR][LDO]
-    float *red_s = reinterpret_cast<float *>(x_s);                        // final sum: [4][NTD][32][LDR], over x_s and o_s
-    static_assert(sizeof(float) * 4 * NTD * 32 * kAxLDR <= sizeof(bf16_t) * kAxSBR * kAxLD + sizeof(float) * kAxSBR * kAxLDO,
-                  "the cross-wave sum of dphi reuses the x and output tiles");
+    float *o_s = reinterpret_cast<float *>(x_s + (size_t)SBR * kAxLD);    // [SBR][LDO]
+    float *red_s = reinterpret_cast<float *>(ax_smem);                    // final sum: [4][NTD][32][LDR], over everything
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if ((int)blockIdx.y == a.tail_row) {
         // the extra row of the grid: its first workgroups do the batch sums, the others have nothing to do
@@ -73,16 +77,16 @@ __global__ __launch_bounds__(256) void proj_bwd_addx_kernel(ProjAddxArgs a) {
     const int D = a.D, nC = a.nC, B = a.B;
 
     // ---- per-block loads: x for the LDS tile (thread -> chunks tid + 256 u) and, for the epilogue,
-    // the chunks of dxp this thread completes: sample 64 wave + lane / 4 + 16 t, chunk lane % 4 -------
-    const int ech = lane & 3, erow = 64 * wave + (lane >> 2);
+    // the chunks of dxp this thread completes: sample SPW wave + lane / 4 + 16 t, chunk lane % 4 ------
+    const int ech = lane & 3, erow = SPW * wave + (lane >> 2);
     const int kc = k0 + ech * 8;
     const bool kok = kc < nC;  // nC % 8 == 0: a chunk is inside or outside
-    uint32_t xr[2][4][4], pr[2][4][4];
-    float cxr[2][4];
+    uint32_t xr[2][KS][4], pr[2][KS][4];
+    float cxr[2][KS];
     auto load_block = [&](int sb, auto slot) {
         constexpr int S = decltype(slot)::value;
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < KS; u++) {
             const int ch = tid + u * 256;
             const int b = sb + (ch >> 2), k = k0 + (ch & 3) * 8;
             const bool ok = b < B && k < nC;
@@ -90,7 +94,7 @@ __global__ __launch_bounds__(256) void proj_bwd_addx_kernel(ProjAddxArgs a) {
             xr[S][u][0] = v.x; xr[S][u][1] = v.y; xr[S][u][2] = v.z; xr[S][u][3] = v.w;
         }
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
+        for (int t = 0; t < KS; t++) {
             const int b = sb + erow + 16 * t;
             const bool ok = b < B && kok;
             const uint4 v = *reinterpret_cast<const uint4 *>(a.dx + (ok ? (size_t)b * nC + kc : 0));
@@ -98,11 +102,39 @@ __global__ __launch_bounds__(256) void proj_bwd_addx_kernel(ProjAddxArgs a) {
             cxr[S][t] = a.cx[b < B ? b : 0];
         }
     };
+    // Operands that come straight from global memory in fragment order: dP^T (rounded value and
+    // remainder) of this wave's samples for every dphi tile, and dP of its sample tiles.  Steps and
+    // tiles beyond the padded batch read zeros.
+    struct Ops {
+        uint4 ah[NTD][KS], al[NTD][KS], av[TT][2 * NTD];
+    };
+    Ops ops[PFOP ? 2 : 1];
+    auto load_ops = [&](int sb, Ops &o) {
+        const int step0 = (sb >> 4) + KS * wave, nsteps = a.BP >> 4;
+#pragma unroll
+        for (int m = 0; m < NTD; m++)
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                const bool ok = step0 + ks < nsteps;
+                const bf16_t *ap = a.dPT + (ok ? frag_base(m, nsteps, step0 + ks) : 0) + lane * 8;
+                o.ah[m][ks] = load16_masked(reinterpret_cast<const uint4 *>(ap), ok);
+                o.al[m][ks] = load16_masked(reinterpret_cast<const uint4 *>(ap + (size_t)a.DP * a.BP), ok);
+            }
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const int tile = (sb >> 5) + TT * wave + t;
+            const bool ok = tile < (a.BP >> 5);
+#pragma unroll
+            for (int ks = 0; ks < 2 * NTD; ks++)
+                o.av[t][ks] = load16_masked(
+                    reinterpret_cast<const uint4 *>(a.dPb + (ok ? frag_base(tile, a.DP >> 4, ks) : 0) + lane * 8), ok);
+        }
+    };
     using Slot0 = std::integral_constant<int, 0>;
     using Slot1 = std::integral_constant<int, 1>;
 
-    // ---- phi slab -> LDS (rows >= D and columns >= nC read as zero), first blocks requested ---------
-    constexpr int PCH = 32 * NTD * 4;  // 16-byte chunks of the slab
+    // ---- every load of the first block (and the next one) is requested before anything is waited for ---
+    constexpr int PCH = 32 * NTD * 4;  // 16-byte chunks of the phi slab (rows >= D, columns >= nC read as zero)
     uint4 phir[(PCH + 255) / 256];
 #pragma unroll
     for (int u = 0; u < (PCH + 255) / 256; u++) {
@@ -112,17 +144,16 @@ __global__ __launch_bounds__(256) void proj_bwd_addx_kernel(ProjAddxArgs a) {
         phir[u] = load16_masked(reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * nC + k : 0)), ok);
     }
     load_block(0, Slot0{});
-    if (kAxSBR < B) load_block(kAxSBR, Slot1{});
+    load_ops(0, ops[0]);
+    if (SBR < B) {
+        load_block(SBR, Slot1{});
+        if constexpr (PFOP) load_ops(SBR, ops[1]);
+    }
 #pragma unroll
     for (int u = 0; u < (PCH + 255) / 256; u++) {
         const int ch = tid + u * 256;
         if (ch < PCH) *reinterpret_cast<uint4 *>(phi_s + (size_t)(ch >> 2) * kAxLD + (ch & 3) * 8) = phir[u];
     }
-    __syncthreads();
-    bf16x8_t phif[2 * NTD];
-#pragma unroll
-    for (int ks = 0; ks < 2 * NTD; ks++)
-        phif[ks] = __builtin_bit_cast(bf16x8_t, lds_frag_tr(phi_s, kAxLD, ks * 16, 0, lane));
 
     f32x16_t acc[NTD];
 #pragma unroll
@@ -132,68 +163,53 @@ __global__ __launch_bounds__(256) void proj_bwd_addx_kernel(ProjAddxArgs a) {
 
     auto process_block = [&](int sb, auto slot) {
         constexpr int S = decltype(slot)::value;
-        // ---- operands that come straight from global memory, requested ahead of the barriers ----------
-        // dP^T of this wave's 64 samples (k-steps 4 wave .. + 3 of the block) for every dphi tile, and dP
-        // of its two 32-sample tiles.  Steps and tiles beyond the padded batch read zeros.
-        const int step0 = (sb >> 4) + 4 * wave, nsteps = a.BP >> 4;
-        uint4 ah[NTD][4], al[NTD][4], av[2][2 * NTD];
-#pragma unroll
-        for (int m = 0; m < NTD; m++)
-#pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                const bool ok = step0 + ks < nsteps;
-                const bf16_t *ap = a.dPT + (ok ? frag_base(m, nsteps, step0 + ks) : 0) + lane * 8;
-                ah[m][ks] = load16_masked(reinterpret_cast<const uint4 *>(ap), ok);
-                al[m][ks] = load16_masked(reinterpret_cast<const uint4 *>(ap + (size_t)a.DP * a.BP), ok);
-            }
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-            const int tile = (sb >> 5) + 2 * wave + t;
-            const bool ok = tile < (a.BP >> 5);
-#pragma unroll
-            for (int ks = 0; ks < 2 * NTD; ks++)
-                av[t][ks] = load16_masked(
-                    reinterpret_cast<const uint4 *>(a.dPb + (ok ? frag_base(tile, a.DP >> 4, ks) : 0) + lane * 8), ok);
+        Ops &op = ops[PFOP ? S : 0];
+        if (sb != 0) {
+            if constexpr (!PFOP) load_ops(sb, op);
+            __syncthreads();  // every wave is done with the previous block's tile
         }
-        // ---- x block -> LDS ---------------------------------------------------------------------------
-        if (sb != 0) __syncthreads();  // every wave is done with the previous block's tile
+        // ---- x block -> LDS (the first barrier also covers the phi slab) -------------------------------
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < KS; u++) {
             const int ch = tid + u * 256;
             *reinterpret_cast<uint4 *>(x_s + (size_t)(ch >> 2) * kAxLD + (ch & 3) * 8) =
                 make_uint4(xr[S][u][0], xr[S][u][1], xr[S][u][2], xr[S][u][3]);
         }
         __syncthreads();
         // ---- dphi: this wave's samples, every row tile ------------------------------------------------
-        bf16x8_t xf[4];
+        {
+            bf16x8_t xf[KS];
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++)
-            xf[ks] = __builtin_bit_cast(bf16x8_t, lds_frag_tr(x_s, kAxLD, (4 * wave + ks) * 16, 0, lane));
+            for (int ks = 0; ks < KS; ks++)
+                xf[ks] = __builtin_bit_cast(bf16x8_t, lds_frag_tr(x_s, kAxLD, (KS * wave + ks) * 16, 0, lane));
 #pragma unroll
-        for (int m = 0; m < NTD; m++)
+            for (int m = 0; m < NTD; m++)
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ah[m][ks]), xf[ks], acc[m], 0, 0, 0);
-                acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, al[m][ks]), xf[ks], acc[m], 0, 0, 0);
-            }
-        // ---- dP phi of this wave's two sample tiles -> its own rows of o_s ------------------------------
+                for (int ks = 0; ks < KS; ks++) {
+                    acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, op.ah[m][ks]), xf[ks], acc[m], 0, 0, 0);
+                    acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, op.al[m][ks]), xf[ks], acc[m], 0, 0, 0);
+                }
+        }
+        // ---- dP phi of this wave's sample tiles -> its own rows of o_s (phi fragments from the slab) -----
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
+        for (int t = 0; t < TT; t++) {
             f32x16_t o;
 #pragma unroll
             for (int i = 0; i < 16; i++) o[i] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < 2 * NTD; ks++)
-                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av[t][ks]), phif[ks], o, 0, 0, 0);
+            for (int ks = 0; ks < 2 * NTD; ks++) {
+                const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, lds_frag_tr(phi_s, kAxLD, ks * 16, 0, lane));
+                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, op.av[t][ks]), pf, o, 0, 0, 0);
+            }
             // accumulator layout: column = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4
 #pragma unroll
             for (int i = 0; i < 16; i++)
-                o_s[(size_t)(64 * wave + 32 * t + 8 * (i >> 2) + 4 * kg + (i & 3)) * kAxLDO + row] = o[i];
+                o_s[(size_t)(SPW * wave + 32 * t + 8 * (i >> 2) + 4 * kg + (i & 3)) * kAxLDO + row] = o[i];
         }
         // ---- epilogue, row-major: the wave reads back only rows it wrote itself (its LDS accesses
         // complete in order), x from the block's tile ------------------------------------------------------
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
+        for (int t = 0; t < KS; t++) {
             const int r = erow + 16 * t, b = sb + r;
             const float4 o0 = *reinterpret_cast<const float4 *>(o_s + (size_t)r * kAxLDO + ech * 8);
             const float4 o1 = *reinterpret_cast<const float4 *>(o_s + (size_t)r * kAxLDO + ech * 8 + 4);
@@ -210,15 +226,18 @@ __global__ __launch_bounds__(256) void proj_bwd_addx_kernel(ProjAddxArgs a) {
             }
             if (b < B && kok) st16<true>(a.dx + (size_t)b * nC + kc, outw[0], outw[1], outw[2], outw[3]);
         }
-        if (sb + 2 * kAxSBR < B) load_block(sb + 2 * kAxSBR, slot);
+        if (sb + 2 * SBR < B) {
+            load_block(sb + 2 * SBR, slot);
+            if constexpr (PFOP) load_ops(sb + 2 * SBR, op);
+        }
     };
-    for (int sb = 0; sb < B; sb += 2 * kAxSBR) {
+    for (int sb = 0; sb < B; sb += 2 * SBR) {
         process_block(sb, Slot0{});
-        if (sb + kAxSBR < B) process_block(sb + kAxSBR, Slot1{});
+        if (sb + SBR < B) process_block(sb + SBR, Slot1{});
     }
 
     // ---- dphi: sum the four waves' shares through LDS, store row-major --------------------------------
-    __syncthreads();  // all tiles consumed; the region becomes red_s
+    __syncthreads();  // all tiles consumed; the memory becomes red_s
 #pragma unroll
     for (int m = 0; m < NTD; m++)
 #pragma unroll
@@ -236,14 +255,17 @@ __global__ __launch_bounds__(256) void proj_bwd_addx_kernel(ProjAddxArgs a) {
 
 bool proj_bwd_addx_supported(int n) { return padded_D(n) / 32 <= 3; }
 
-template <int NTD>
+template <int NTD, int SPW, bool PFOP>
 static hipError_t launch_addx(const ProjAddxArgs &a, hipStream_t stream) {
-    const size_t smem = sizeof(bf16_t) * (size_t)kAxLD * (32 * NTD + kAxSBR) + sizeof(float) * kAxSBR * kAxLDO;
-    hipError_t e = allow_dynamic_lds(&proj_bwd_addx_kernel<NTD>, smem);
+    constexpr int SBR = 4 * SPW;
+    const size_t tiles = sizeof(bf16_t) * (size_t)kAxLD * (32 * NTD + SBR) + sizeof(float) * SBR * kAxLDO;
+    const size_t red = sizeof(float) * 4 * NTD * 32 * kAxLDR;  // the final cross-wave sum reuses the tiles' memory
+    const size_t smem = tiles > red ? tiles : red;
+    hipError_t e = allow_dynamic_lds(&proj_bwd_addx_kernel<NTD, SPW, PFOP>, smem);
     if (e != hipSuccess) return e;
     const int slabs = (a.nC + kAxKW - 1) / kAxKW;
     dim3 grid(round_up(slabs, 16), 1 + (a.tail_row >= 0 ? 1 : 0));
-    proj_bwd_addx_kernel<NTD><<<grid, 256, smem, stream>>>(a);
+    proj_bwd_addx_kernel<NTD, SPW, PFOP><<<grid, 256, smem, stream>>>(a);
     return hipGetLastError();
 }
 
@@ -260,9 +282,9 @@ hipError_t launch_proj_bwd_addx(const void *x, const void *phi, const void *dPb,
         if (tail_taken) *tail_taken = true;
     }
     switch (NTD) {
-        case 1: return launch_addx<1>(a, stream);
-        case 2: return launch_addx<2>(a, stream);
-        case 3: return launch_addx<3>(a, stream);
+        case 1: return launch_addx<1, 32, false>(a, stream);
+        case 2: return launch_addx<2, 32, false>(a, stream);
+        case 3: return launch_addx<3, 32, false>(a, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -1,7 +1,7 @@
 // Native benchmark of the mHC layer over the C ABI (libmhc_hip.so): no Python, no PyTorch.
 //
 //   bench_mhc_layer [--batch B] [--hidden C] [--expansion n] [--iters T] [--runs R] [--warmup W]
-//                   [--static] [--fp32] [--all-configs] [--tune KEY VALUE   (experiment hook, csrc/tuning.h)]
+//                   [--static] [--fp32] [--all-configs]
 //
 // Counterpart of the reference's native layer benchmark (src/csrc/benchmarks/bench_mhc_layer.cu:
 // warm-up, an L2 / cache flush before every timed run, event timing, bytes-moved bandwidth) for
@@ -21,7 +21,6 @@
 
 #include "../../include/mhc_hip.h"
 
-extern "C" int mhc_tuning_set(int key, int value);  // experiment hook of the library (csrc/tuning.h)
 
 #define HIP_OK(e)                                                                      \
     do {                                                                               \
@@ -169,7 +168,6 @@ int main(int argc, char **argv) {
         else if (is("--static")) dynamic = false;
         else if (is("--fp32")) bf16 = false;
         else if (is("--all-configs")) all = true;
-        else if (is("--tune") && i + 2 < argc) { mhc_tuning_set(atoi(argv[i + 1]), atoi(argv[i + 2])); i += 2; }
         else { fprintf(stderr, "unknown argument %s\n", argv[i]); return 2; }
     }
     printf("mHC layer native benchmark over the C ABI (ABI version %d); cold caches (512 MiB flush per call)\n",

@@ -21,7 +21,7 @@
 #include "../../include/mhc_hip.h"
 
 extern "C" int mhc_phase_read(int kernel, unsigned long long *host, int workgroups);
-extern "C" int mhc_tuning_set(int key, int value);  // experiment hook of the library (csrc/tuning.h)
+extern "C" int mhc_tuning_set(int key, int value);  // launch-heuristic override; the profile build has it (csrc/tuning.h)
 
 #define HIP_OK(e) do { hipError_t _e = (e); if (_e != hipSuccess) { fprintf(stderr, "HIP error %s at line %d\n", hipGetErrorString(_e), __LINE__); exit(1); } } while (0)
 #define MHC_OK_(e) do { int _s = (e); if (_s != MHC_OK) { fprintf(stderr, "mhc error %d (%s) at line %d\n", _s, mhc_status_string(_s), __LINE__); exit(1); } } while (0)
@@ -129,6 +129,9 @@ int main(int argc, char **argv) {
             {"start: coefficient inputs, Sinkhorn state (wave 0)", "streaming loop (wave 0's steps)",
              "workgroup sums", "coefficient backward (all of it: the three lines below)",
              "  channel-sum vectors, dHpre / dHpost", "  Sinkhorn reverse sweep", "  dt / dP stores, alpha sums"}, false);
+    summary("sample-resident backward (--tune 7 2 only), first tile wave of each workgroup", 5, std::min(B, 4096),
+            {"loads requested", "tile arrives, Gram sums, slots written", "two barriers (workgroup sums between them)",
+             "dxp / u computed, stores issued"}, false);
     if (n > 4) {
         summary("dx kernel (generic, one wave per workgroup)", 5, std::min(B * ((C / 4 + 63) / 64), 4096),
                 {"start: coefficients and all loads requested", "data arrives, df / a / da", "mixing, dx stores issued", "dw / dt partial sums"}, false);

@@ -4,8 +4,6 @@ same library on the same inputs (both accumulate bf16 products in fp32, so their
 tensors agree far inside the bf16 bar).  The group size G (samples per workgroup) is forced through
 the library's experiment hook so that ragged last groups and G > 8 (two row pieces per lane) are
 covered at small sizes."""
-import ctypes
-
 import pytest
 import torch
 
@@ -18,11 +16,9 @@ K_OFF, K_G = 0, 1
 
 
 def _tune(key, value):
-    from mhc._lib import lib
+    from mhc._lib import tuning_lib
 
-    lib.mhc_tuning_set.restype = ctypes.c_int
-    lib.mhc_tuning_set.argtypes = [ctypes.c_int, ctypes.c_int]
-    assert lib.mhc_tuning_set(key, value) == 0
+    assert tuning_lib().mhc_tuning_set(key, value) == 0
 
 
 @pytest.fixture(autouse=True)
@@ -34,7 +30,9 @@ def _reset_tuning():
 
 def _forward(B, n, C, x, w, phi, bias, alpha, f, out_dtype, T, eps):
     from mhc import _lib
-    from mhc._lib import check, dtype_code, lib, ptr
+    from mhc._lib import check, dtype_code, ptr
+
+    lib = _lib.tuning_lib()  # the build of the library whose launch heuristics can be overridden
 
     D = n * n + 2 * n
     f32 = dict(dtype=torch.float32, device="cuda")
@@ -65,8 +63,6 @@ CASES = [  # B, n, C, G
 @pytest.mark.parametrize("inject", [False, True])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_onepass_forward(B, n, C, G, inject, out_dtype):
-    from mhc._lib import lib
-
     T, eps = 20, 1e-6
     xh, _, fh, p = nm.make_dynamic_inputs(B, n, C, bf16_round=True, with_f=True)
     for k in ("alpha_pre", "alpha_post", "alpha_res"):

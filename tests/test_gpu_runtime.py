@@ -8,11 +8,11 @@ from oracle import naive_mhc as nm
 pytestmark = pytest.mark.gpu
 
 
-def _bf16_step(B, n, C):
+def _bf16_step(B, n, C, lib=None):
     import bench
 
     cfg = dict(kind="dynamic", B=B, n=n, C=C, dtype="bf16", bwd=True)
-    return bench.Step(cfg, "L", torch)
+    return bench.Step(cfg, "L", torch, lib=lib)
 
 
 @pytest.mark.parametrize("B,n,C", [(96, 4, 512), (40, 8, 256), (24, 32, 256)])
@@ -73,13 +73,10 @@ def test_two_streams_with_separate_workspaces(shapes):
 def test_projection_backward_products_apart_match_one_launch(B, n, C):
     """dphi = dP^T x and dP phi as two launches around the dx kernel (the default from n = 11 on) against
     both in one launch, each forced through the experiment hook: same gradients bit for bit."""
-    import ctypes
+    from mhc._lib import tuning_lib
 
-    from mhc._lib import lib
-
-    lib.mhc_tuning_set.restype = ctypes.c_int
-    lib.mhc_tuning_set.argtypes = [ctypes.c_int, ctypes.c_int]
-    st = _bf16_step(B, n, C)
+    lib = tuning_lib()  # the build of the library whose launch heuristics can be overridden
+    st = _bf16_step(B, n, C, lib)
     outs = (st.dx, st.dw, st.dphi, st.dbias, st.dalpha)
     try:
         assert lib.mhc_tuning_set(4, 1) == 0  # batch sums in their own launch both times
@@ -104,13 +101,10 @@ def test_batch_sums_inside_the_dphi_launch_match_the_separate_launch(B, n, C):
     """From n = 11 on: dw, dbias and dalpha summed by extra workgroups of the dphi launch (the default)
     against the same sums as a launch of their own (forced through the experiment hook), eagerly with
     poisoned outputs and under graph replay."""
-    import ctypes
+    from mhc._lib import tuning_lib
 
-    from mhc._lib import lib
-
-    lib.mhc_tuning_set.restype = ctypes.c_int
-    lib.mhc_tuning_set.argtypes = [ctypes.c_int, ctypes.c_int]
-    st = _bf16_step(B, n, C)
+    lib = tuning_lib()  # the build of the library whose launch heuristics can be overridden
+    st = _bf16_step(B, n, C, lib)
     outs = (st.dx, st.dw, st.dphi, st.dbias, st.dalpha)
     grads = lambda: [t.clone() for t in outs]
 
