@@ -44,6 +44,7 @@ MEASURED_TRAFFIC = {
 # (profiles/layer_step_<config>.txt): average duration per dispatch and the HBM bytes the algorithm
 # needs that kernel to move (its own inputs and outputs once; for the split projections the partial
 # sums are not counted).
+PROFILED_AT = "7fb7ec3"
 PROFILED_DOMINANT = {
     "c1": dict(kernel="layer_fwd_small_kernel<float,float,4,4,2>", us=6.53, bytes=2 * 4 * 320 * 4 * 1280),
     "c2": dict(kernel="bwd_slab_kernel<bf16>", us=9.53, bytes=3 * 2 * 320 * 4 * 1280 + 2 * 24 * 5120 + 4 * 24 * 5120),
@@ -82,10 +83,11 @@ def algorithmic_bytes(cfg, view):
 
 def dominant_kernel(config):
     """roofline.dominant: the step's largest kernel as profiled (not re-timed here: HIP events see whole
-    entry points, not the launches inside them)."""
+    entry points, not the launches inside them); `profiled_at` is the revision the profile ran on."""
     d = dict(PROFILED_DOMINANT[config])
     d["frac"] = d["bytes"] / (d["us"] * 1e-6) / 1e9 / HBM_PEAK_GBS
     d["source"] = f"profiles/layer_step_{config}.txt"
+    d["profiled_at"] = PROFILED_AT
     return d
 
 
@@ -324,56 +326,13 @@ def cpu_baseline(step, torch, budget_s=20.0):
                       f"fp32 naive PyTorch layer, median"}
 
 
-def handoff_probe(torch):
-    """One kernel whose workgroups hand data to each other (write-through stores, arrival counter, bypassing
-    loads: csrc/stream_probe.hip) against the same work as two kernels, in graphs of ten, at the grid sizes and
-    partial-sum volumes of the n <= 4 backward (200 workgroups x 24 KB at B=320, C=1280; 480 at B=1280, C=2560)."""
-    from mhc import _lib
-
-    fn = _lib.lib.mhc_stream_probe
-    fn.restype = ctypes.c_int
-    fn.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
-                   ctypes.c_void_p]
-    rows = []
-    for blocks, per in ((200, 200 * 32), (200, 200 * 2), (480, 480 * 13), (480, 480 * 1), (1024, 1024 * 1)):
-        part = torch.zeros(blocks * per, dtype=torch.float32, device="cuda")
-        outs = [torch.zeros(blocks, dtype=torch.float32, device="cuda") for _ in range(2)]
-        sync = torch.zeros(3, dtype=torch.int32, device="cuda")
-
-        def chain(one, out, k=10):
-            cur = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            for _ in range(k):
-                for mode in ((7,) if one else (8, 9)):
-                    assert fn(mode, out.data_ptr(), part.data_ptr(), per * 4, blocks, sync.data_ptr(), cur) == 0
-        row = {"workgroups": blocks, "KB_per_workgroup": per * 4 / 1024}
-        for one in (False, True):
-            chain(one, outs[one], 1)
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                chain(one, outs[one])
-            g.replay()
-            best_t = float("inf")
-            for _ in range(10):
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                for _ in range(10):
-                    g.replay()
-                e1.record()
-                e1.synchronize()
-                best_t = min(best_t, e0.elapsed_time(e1) * 1e3 / 100)
-            row["one_kernel_us" if one else "two_kernels_us"] = round(best_t, 2)
-        row["results_equal"] = bool(torch.equal(outs[0], outs[1]))
-        row["gave_up"] = int(sync[2].item())
-        rows.append(row)
-    print(json.dumps({"handoff_probe": True, "protocol": "graphs of ten, best of 10 x 10 replays, HIP events", "rows": rows}))
-
-
 def stream_probe(torch):
-    """Read-only / copy / write-only streaming rates of hand-written kernels (csrc/stream_probe.hip)."""
-    from mhc import _lib
-
-    fn = _lib.lib.mhc_stream_probe
+    """Read-only / copy / write-only streaming rates of hand-written kernels and the cost of an empty launch
+    (csrc/stream_probe.hip, built into its own libmhc_probe.so)."""
+    path = os.path.join(ROOT, "mhc.cu_amd", "mhc", "libmhc_probe.so")
+    if not os.path.exists(path):
+        raise SystemExit(f"{path} not found: python mhc.cu_amd/build.py")
+    fn = ctypes.CDLL(path).mhc_stream_probe
     fn.restype = ctypes.c_int
     fn.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
                    ctypes.c_void_p]
@@ -433,23 +392,6 @@ def stream_probe(torch):
                 e1.synchronize()
                 best_t = min(best_t, e0.elapsed_time(e1) * 1e3 / 100)
             floor[f"{name}_{blocks}_workgroups"] = round(best_t, 2)
-    # what ONE workgroup pulls out of the L2 when all workgroups stream the same small matrix (phi of the
-    # one-launch forward): 20 passes inside one launch, so the kernel start is amortised
-    pieces = {}
-    for nC, blocks in ((5120, 160), (10240, 256)):
-        phi = torch.ones(24 * nC, dtype=torch.bfloat16, device="cuda")
-        run = lambda: fn(10, phi.data_ptr(), None, 24 * nC * 2, blocks, sink.data_ptr(), stream)
-        assert run() == 0
-        best_t = float("inf")
-        for _ in range(5):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            assert run() == 0
-            e1.record()
-            e1.synchronize()
-            best_t = min(best_t, e0.elapsed_time(e1) * 1e-3 / 20)
-        pieces[f"phi_24x{nC}_{blocks}_workgroups"] = {"us_per_pass": round(best_t * 1e6, 2),
-                                                      "GB/s_per_workgroup": round(24 * nC * 2 / best_t / 1e9, 1)}
     best = {}
     for r in rows:
         key = (r["kernel"], r["MiB"], r["cache"])
@@ -457,7 +399,7 @@ def stream_probe(torch):
             best[key] = r
     print(json.dumps({"stream_probe": True, "protocol": "cold: 512 MiB fill before every timed launch; warm: back to back; median of 10, "
                       "HIP events on the launch stream", "rows": rows,
-                      "empty_kernel_us_per_launch": floor, "row_piece_stream_per_workgroup": pieces, "ceiling_GBs": {f"{k[0]}_{k[1]}MiB_{k[2]}": round(v["GB/s"], 1) for k, v in sorted(best.items())}}))
+                      "empty_kernel_us_per_launch": floor, "ceiling_GBs": {f"{k[0]}_{k[1]}MiB_{k[2]}": round(v["GB/s"], 1) for k, v in sorted(best.items())}}))
 
 
 def main():
@@ -471,10 +413,6 @@ def main():
     ap.add_argument("--graph-steps", type=int, default=10,
                     help="steps captured into one HIP graph (a replay costs ~5 us by itself); 1 = one step per replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--handoff-probe", action="store_true",
-                    help="time one kernel whose workgroups exchange partial sums through memory (arrival counter, "
-                         "write-through stores) against the same work as two kernels: what a launch boundary costs "
-                         "next to an in-kernel grid-wide hand-off on this GPU")
     ap.add_argument("--stream-probe", action="store_true",
                     help="run the library's plain streaming kernels (read-only, copy, write-only; 16-byte accesses, "
                          "all CUs) over 128 MiB .. 2 GiB and print what this GPU delivers to each, HIP events on the "
@@ -494,9 +432,6 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
-    if a.handoff_probe:
-        handoff_probe(torch)
-        return
     if a.stream_probe:
         stream_probe(torch)
         return
@@ -606,7 +541,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC["bytes"].get(a.config) if a.view == "L" else None,
-                     "traffic_commit": MEASURED_TRAFFIC["commit"],
+                     "traffic_profiled_at": MEASURED_TRAFFIC["commit"],
+                     # the same step with a 512 MiB fill before every one (nothing served from the caches)
+                     "cold_us": cold_step, "cold_frac": alg / (cold_step * 1e-6) / 1e9 / HBM_PEAK_GBS,
                      "dominant": dominant_kernel(a.config),
                      "kernel": "whole step (all launches of one forward+backward)",
                      "algorithmic_bytes": alg, "device_us": dev_step, "single_step_graph_us": dev_single,
@@ -617,6 +554,10 @@ def main():
                      "cold_cache": {"device_us": cold_step, "achieved": alg / (cold_step * 1e-6) / 1e9,
                                     "flush": "512 MiB fill before every step"}},
     }
+    # the three protocols side by side at top level: `value` above (warm, G steps per graph replay), one
+    # step per replay (warm), and cold (one step per replay behind a 512 MiB fill)
+    out["single_step_graph_us"] = dev_single
+    out["cold_us"] = cold_step
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(step, torch)
     print(json.dumps(out))

@@ -6,7 +6,8 @@
  * default stream) and returns a status immediately.  The library keeps no global mutable
  * state, never allocates, never synchronises, never prints and never exits: the caller owns
  * all memory, including the scratch `workspace` (size from the *_workspace_bytes queries,
- * 256-byte aligned).  Calls are re-entrant across streams as long as each in-flight call has
+ * 256-byte aligned).  (One documented exception at the end of this header: the entry point
+ * that takes no workspace uses a device array owned by the library and remembers its address.)  Calls are re-entrant across streams as long as each in-flight call has
  * its own workspace.
  *
  * Each entry point names the interface of the reference (AndreSlavescu/mHC.cu) that it
@@ -69,9 +70,9 @@ MHC_API const char *mhc_status_string(int status);
 
 /*
  * Largest `iters` the layer entry points below accept for expansion rate n (0 for an invalid n):
- * 256 for every n in 1..32.  The exact Sinkhorn backward
- * keeps the scalings of every iteration in LDS, and for n > 8 its float32 round-off grows with the
- * iteration count (2-3e-8 per iteration relative to float64: 5e-7 at 20, up to 8e-6 at 256).  The reference's interface states no bound
+ * 256 for every n in 1..32.  The exact Sinkhorn backward keeps the scalings of every iteration in
+ * LDS, which bounds the count; its float32 round-off does not grow with it (about 2e-7 relative to
+ * float64 on the bias gradients from 20 to 256 iterations).  The reference's interface states no bound
  * (sinkhorn_iters of mhc.MHCLayer, src/python/mhc/layer.py:21-29, default 20).
  * The stand-alone mhc_sinkhorn_knopp_* take up to 1024 iterations for any shape.
  */

@@ -19,7 +19,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "mhc", "libmhc_hip.so")
 
 SOURCES = ["capi.hip", "proj_fwd.hip", "gemm_f32.hip", "proj_bwd.hip", "proj_bwd_addx.hip", "proj_bwd_large.hip", "bwd_slab.hip", "coef_fwd.hip", "mix_fwd.hip", "layer_fwd_onepass.hip", "mix_bwd_reduce.hip",
-           "bwd_resident.hip", "mix_bwd_dx.hip", "param_grads.hip", "pack_params.hip", "ops.hip", "stream_probe.hip"]
+           "bwd_resident.hip", "mix_bwd_dx.hip", "param_grads.hip", "pack_params.hip", "ops.hip"]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are not trusted on this hardware pool.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -71,6 +71,21 @@ def build(jobs: int = 8, verbose: bool = True, profile: bool = False, tuning: bo
     return lib
 
 
+PROBE_LIB = os.path.join(HERE, "mhc", "libmhc_probe.so")
+
+
+def build_probe(verbose: bool = True):
+    """libmhc_probe.so: the plain streaming kernels of csrc/stream_probe.hip (measured bandwidth ceilings
+    and launch floor for bench.py --stream-probe).  Deliberately not part of libmhc_hip.so."""
+    cmd = [_hipcc(), *FLAGS, "-shared", os.path.join(CSRC, "stream_probe.hip"), "-o", PROBE_LIB]
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("hipcc failed on stream_probe.hip:\n" + p.stderr)
+    if verbose:
+        print("built", PROBE_LIB)
+    return PROBE_LIB
+
+
 EXT_SRC = os.path.join(HERE, "torch_ext", "mhc_torch_ext.cpp")
 EXT_NAME = "mhc_torch_ext"
 
@@ -117,5 +132,7 @@ if __name__ == "__main__":
     ap.add_argument("--no-ext", action="store_true", help="skip the PyTorch extension (about a minute of g++)")
     a = ap.parse_args()
     build(a.jobs, profile=a.profile, tuning=a.tuning)
+    if not a.profile and not a.tuning:
+        build_probe()
     if not a.profile and not a.tuning and not a.no_ext:
         build_torch_ext()

@@ -84,6 +84,7 @@ template <int NP> __global__ __launch_bounds__(64) void coef_fwd_small_kernel(Co
     float *st = a.sk_state ? a.sk_state + (size_t)b * SK::state_floats(a.T) : nullptr;
     if (st && a.precise) SK::template forward_save<true>(m, g, n, a.T, a.eps, st);
     else if (st) SK::template forward_save<false>(m, g, n, a.T, a.eps, st);
+    else if (a.precise) SK::template forward<true, false>(m, g, n, a.T, a.eps, nullptr, lane);
     else SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, lane);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++) {

@@ -306,8 +306,10 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             }
             // kept denominators: the fp32 tier divides, so that the backward call can undo the
             // scalings (m * s * rho) without a bias that grows with the iteration count
+            // (the same arithmetic with and without the state: the forward result does not depend on
+            // whether the caller keeps it)
             if (dyn && a.sk_state) SK::template forward_save<!kFast>(m, g, n, a.T, a.eps, a.sk_state + (size_t)b * SK::state_floats(a.T));
-            else SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, tid);
+            else SK::template forward<!kFast, false>(m, g, n, a.T, a.eps, nullptr, tid);
             coef_s[r0 * NP + c0] = m[0];
             if (wr && a.M && mv) a.M[ms + r0 * n + c0] = m[0];
         }

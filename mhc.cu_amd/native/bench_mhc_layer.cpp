@@ -2,12 +2,17 @@
 //
 //   bench_mhc_layer [--batch B] [--hidden C] [--expansion n] [--iters T] [--runs R] [--warmup W]
 //                   [--static] [--fp32] [--all-configs]
+//   bench_mhc_layer --ops [--runs R] [--warmup W]
 //
 // Counterpart of the reference's native layer benchmark (src/csrc/benchmarks/bench_mhc_layer.cu:
 // warm-up, an L2 / cache flush before every timed run, event timing, bytes-moved bandwidth) for
 // this library's entry points.  Times the forward and the backward call separately with HIP
 // events, flushing 512 MiB before each timed call, and prints microseconds and the achieved
 // fraction of the configuration's algorithmic HBM bytes at 8 TB/s.
+// --ops: the two stand-alone operators at the shapes of the reference's per-operator benchmarks
+// (src/csrc/benchmarks/bench_rmsnorm.cu:104-107, bench_rmsnorm_backward.cu:17-20,
+// bench_sinkhorn_knopp.cu:117-120, bench_sinkhorn_knopp_backward.cu:23-25; CMake targets
+// src/csrc/CMakeLists.txt:38-48), same protocol, bytes as those benchmarks count them.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -154,9 +159,77 @@ static void run_config(int B, int C, int n, int T, bool dynamic, bool bf16, int 
     HIP_OK(hipEventDestroy(e1));
 }
 
+template <typename F> static float time_cold(F &&fn, DeviceBuf &flush, int warmup, int runs) {
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    std::vector<float> t;
+    for (int i = 0; i < warmup + runs; i++) {
+        HIP_OK(hipMemsetAsync(flush.p, i & 0xff, flush.bytes, nullptr));
+        HIP_OK(hipEventRecord(e0, nullptr));
+        fn();
+        HIP_OK(hipEventRecord(e1, nullptr));
+        HIP_OK(hipEventSynchronize(e1));
+        float ms;
+        HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+        if (i >= warmup) t.push_back(ms * 1e3f);
+    }
+    HIP_OK(hipEventDestroy(e0));
+    HIP_OK(hipEventDestroy(e1));
+    return trimmed_mean(t);
+}
+
+static void run_ops(int warmup, int runs) {
+    DeviceBuf flush(512u << 20);
+    std::mt19937 gen(0);
+    printf("\nRMSNorm (bf16 rows, bf16 weight; bytes = rows read + written [+ gradient read])\n");
+    printf("%6s %6s %10s %9s %10s %9s\n", "N", "C", "fwd us", "fwd GB/s", "bwd us", "bwd GB/s");
+    const int rc[7][2] = {{128, 4096}, {256, 4096}, {512, 4096}, {1024, 4096}, {2048, 4096}, {1024, 8192}, {2048, 8192}};
+    for (auto &c : rc) {
+        const int N = c[0], C = c[1];
+        const size_t NC = (size_t)N * C;
+        DeviceBuf inp(NC * 2), out(NC * 2), grad(NC * 2), dinp(NC * 2), w(C * 2), rms(N * 4), dw(C * 4);
+        upload(inp, randn(NC, 1.f, gen), true);
+        upload(grad, randn(NC, 1.f, gen), true);
+        upload(w, std::vector<float>(C, 1.f), true);
+        const size_t wsb = mhc_rmsnorm_bwd_workspace_bytes(N, C);
+        DeviceBuf ws(wsb);
+        auto fwd = [&]() { MHC_OK_(mhc_rmsnorm_fwd(inp.p, MHC_BF16, w.p, MHC_BF16, out.p, (float *)rms.p, N, C, 1e-5f, nullptr)); };
+        auto bwd = [&]() {
+            MHC_OK_(mhc_rmsnorm_bwd(grad.p, inp.p, MHC_BF16, w.p, MHC_BF16, (const float *)rms.p, dinp.p, (float *)dw.p, N, C,
+                                    ws.p, wsb, nullptr));
+        };
+        fwd();
+        const float tf = time_cold(fwd, flush, warmup, runs), tb = time_cold(bwd, flush, warmup, runs);
+        printf("%6d %6d %10.1f %9.0f %10.1f %9.0f\n", N, C, tf, 2.0 * NC * 2 / tf * 1e-3, tb, 3.0 * NC * 2 / tb * 1e-3);
+    }
+    printf("\nSinkhorn-Knopp, one fp32 matrix (threshold form, eps = 1e-8)\n");
+    printf("%6s %6s %6s %10s %12s %10s %12s\n", "M", "N", "iters", "fwd us", "fwd us/iter", "bwd us", "bwd us/iter");
+    const int sc[9][3] = {{32, 32, 5}, {32, 32, 10}, {32, 32, 20}, {64, 64, 5}, {64, 64, 10}, {64, 64, 20},
+                          {128, 128, 5}, {128, 128, 10}, {128, 128, 20}};
+    for (auto &c : sc) {
+        const int M = c[0], N = c[1], it = c[2];
+        const size_t MN = (size_t)M * N;
+        DeviceBuf inp(MN * 4), out(MN * 4), grad(MN * 4), dinp(MN * 4);
+        std::vector<float> h = randn(MN, 1.f, gen);
+        for (auto &v : h) v = std::fabs(v) + 0.1f;  // positive entries, like the reference's benchmark input
+        upload(inp, h, false);
+        upload(grad, randn(MN, 1.f, gen), false);
+        const size_t wsb = mhc_sinkhorn_knopp_bwd_workspace_bytes(1, M, N, it);
+        DeviceBuf ws(wsb);
+        auto fwd = [&]() { MHC_OK_(mhc_sinkhorn_knopp_fwd((const float *)inp.p, (float *)out.p, 1, M, N, it, 1e-8f, nullptr)); };
+        auto bwd = [&]() {
+            MHC_OK_(mhc_sinkhorn_knopp_bwd((const float *)grad.p, (const float *)inp.p, (float *)dinp.p, 1, M, N, it, 1e-8f, ws.p,
+                                           wsb, nullptr));
+        };
+        const float tf = time_cold(fwd, flush, warmup, runs), tb = time_cold(bwd, flush, warmup, runs);
+        printf("%6d %6d %6d %10.1f %12.2f %10.1f %12.2f\n", M, N, it, tf, tf / it, tb, tb / it);
+    }
+}
+
 int main(int argc, char **argv) {
     int B = 320, C = 1280, n = 4, T = 20, runs = 50, warmup = 5;
-    bool dynamic = true, bf16 = true, all = false;
+    bool dynamic = true, bf16 = true, all = false, ops = false;
     for (int i = 1; i < argc; i++) {
         auto is = [&](const char *s) { return strcmp(argv[i], s) == 0; };
         if (is("--batch") && i + 1 < argc) B = atoi(argv[++i]);
@@ -168,10 +241,15 @@ int main(int argc, char **argv) {
         else if (is("--static")) dynamic = false;
         else if (is("--fp32")) bf16 = false;
         else if (is("--all-configs")) all = true;
+        else if (is("--ops")) ops = true;
         else { fprintf(stderr, "unknown argument %s\n", argv[i]); return 2; }
     }
     printf("mHC layer native benchmark over the C ABI (ABI version %d); cold caches (512 MiB flush per call)\n",
            mhc_abi_version());
+    if (ops) {
+        run_ops(warmup, runs);
+        return 0;
+    }
     printf("%-7s %-4s %6s %6s %4s %10s %10s %9s %9s %8s %8s\n", "H", "act", "batch", "hidden", "n", "fwd us", "bwd us",
            "fwd GB/s", "bwd GB/s", "fwd roof", "bwd roof");
     if (all) {

@@ -27,6 +27,18 @@ def test_library_exports_every_declared_symbol():
     assert _lib.lib.mhc_abi_version() == 2
 
 
+def test_library_exports_nothing_the_header_does_not_declare():
+    """The product library carries no experiment hooks, probes or other undeclared entry points (those
+    live in libmhc_hip_tuning.so / libmhc_probe.so)."""
+    import subprocess
+
+    from mhc import _lib
+
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = sorted(l.split()[-1] for l in out.splitlines() if " T " in l)
+    assert exported == _declared_symbols()
+
+
 def test_status_strings():
     from mhc import _lib
 

@@ -62,6 +62,60 @@ def test_static_scratch_forward_matches_workspace_forward(n, C, dtype):
             assert torch.equal(got[k], ref[k]), (call, k, float((got[k] - ref[k]).abs().max()))
 
 
+def test_static_scratch_forward_allocates_nothing_and_replays_in_a_graph():
+    """What the entry point is for: no device memory is taken by a call (free memory is unchanged over
+    eager calls once the array's address has been looked up), and after mhc_static_scratch_init() it
+    can be captured into a HIP graph; every replay, with unrelated eager work and synchronisations
+    between the replays, reproduces the eager result bit for bit."""
+    from mhc import _lib
+    from mhc._lib import check, dtype_code, lib, ptr
+
+    B, n, C, T, eps, dtype = 64, 8, 256, 20, 1e-6, torch.bfloat16
+    x, w, phi, bias, alpha = _inputs(B, n, C, dtype, 5)
+    D = n * n + 2 * n
+    f32 = dict(dtype=torch.float32, device="cuda")
+    out = dict(y=torch.empty_like(x), Hp=torch.empty(B, n, **f32), Ho=torch.empty(B, n, **f32),
+               M=torch.empty(B, n, n, **f32), P=torch.empty(B, D, **f32), r=torch.empty(B, **f32),
+               q=torch.empty(B, **f32))
+    scratch = torch.zeros(1 << 20, device="cuda")  # allocated before the free-memory readings
+    assert lib.mhc_static_scratch_init() == 0
+
+    def call():
+        st = _lib.stream_ptr(x.device)
+        check("mhc_layer_fwd_dynamic_static_scratch",
+              lib.mhc_layer_fwd_dynamic_static_scratch(ptr(x), dtype_code(x), ptr(w), dtype_code(w), ptr(phi),
+                                                       dtype_code(phi), ptr(bias), ptr(alpha), None, ptr(out["y"]),
+                                                       dtype_code(out["y"]), ptr(out["Hp"]), ptr(out["Ho"]), ptr(out["M"]),
+                                                       ptr(out["P"]), ptr(out["r"]), ptr(out["q"]), None, B, n, C, T, eps, st))
+
+    call()
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "a call through the no-allocation entry point took device memory"
+    eager = {k: v.clone() for k, v in out.items()}
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for rep in range(3):
+        for t in out.values():
+            t.fill_(float("nan"))
+        scratch.add_(1.0).sum().item()  # eager work + a host sync between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        for k, v in out.items():
+            assert torch.equal(v, eager[k]), (rep, k)
+
+
 def test_static_scratch_refuses_shapes_beyond_its_array():
     from mhc._lib import lib
 
