@@ -48,7 +48,17 @@ extern "C" {
 #define MHC_MAX_N 32
 #define MHC_MAX_C 32768 /* largest hidden size C of the layer entry points (a [C] float row is kept in LDS) */
 
-enum mhc_dtype { MHC_F32 = 0, MHC_BF16 = 1 };
+/*
+ * MHC_F32_AS_BF16: fp32 storage that the kernels consume as bf16 - every kernel rounds the values to
+ * bf16 (nearest even) in registers as it loads them and then computes exactly as for MHC_BF16, so no
+ * cast pass over the tensor is needed.  This is the reference's default contract (float32
+ * activations in and out around a bf16 kernel path: src/python/mhc/ops.py:129,404,
+ * src/python/bindings.cu:280,421-423,462).  Accepted as x_dtype by mhc_layer_fwd_dynamic and
+ * mhc_layer_bwd_dynamic only, with y_dtype = MHC_F32 (y, dy and dx are then fp32; an injected f and df
+ * are fp32 like x), phi in bf16, and only for the shapes mhc_layer_dynamic_accepts_f32_as_bf16()
+ * reports; MHC_ERR_BAD_DTYPE otherwise.
+ */
+enum mhc_dtype { MHC_F32 = 0, MHC_BF16 = 1, MHC_F32_AS_BF16 = 2 };
 
 enum mhc_status {
     MHC_OK = 0,
@@ -77,6 +87,14 @@ MHC_API const char *mhc_status_string(int status);
  * The stand-alone mhc_sinkhorn_knopp_* take up to 1024 iterations for any shape.
  */
 MHC_API int mhc_max_sinkhorn_iters(int n);
+
+/*
+ * 1 when the two dynamic-H entry points below take x_dtype = MHC_F32_AS_BF16 for this shape (the
+ * kernels that load fp32 storage directly serve n <= 8 and the batch sizes for which the two-launch
+ * backward is taken), else 0: the caller then rounds x to bf16 itself, as the reference does
+ * (src/python/bindings.cu:421-423).
+ */
+MHC_API int mhc_layer_dynamic_accepts_f32_as_bf16(int B, int n, int C, int iters);
 
 /* ------------------------------------------------------------------------------------------
  * Dynamic-H layer.  Replaces mhc_cuda.mhc_layer_fwd_dynamic / mhc_layer_bwd_dynamic

@@ -22,14 +22,16 @@
 // The mixing uses the VALU with DPP quad broadcasts: the contraction runs over streams, which lie
 // across the four lanes of a quad.
 #include "coef_bwd_small.h"
+
+#include <type_traits>
 #include "tuning.h"
 
 namespace mhc {
 
 struct BwdResidentArgs {
     BwdReduceArgs r;   // inputs and the outputs of the coefficient backward
-    bf16_t *dxp;       // [B, n, C]
-    bf16_t *df;        // [B, C] or nullptr (only with r.f_inject)
+    void *dxp;         // [B, n, C], stored like x (bf16, or fp32 with F32)
+    void *df;          // [B, C] or nullptr (only with r.f_inject), stored like x
     float *u;          // [B, C] (unused with r.f_inject)
 };
 
@@ -46,8 +48,35 @@ __device__ __forceinline__ float quad_allreduce(float v) {
     return v;
 }
 
-template <int NP, int WMODE, int ITEMS>
+// Eight consecutive activation values as four words of bf16 pairs.  bf16 storage: the 16 bytes as
+// loaded.  fp32 storage (F32): two 16-byte loads, rounded to bf16 (nearest even) by get() - called
+// once all loads of the workgroup have been requested.
+template <bool F32> struct Act8;
+template <> struct Act8<false> {
+    uint4 r;
+    __device__ __forceinline__ void load(const void *base, size_t elem, bool ok) {
+        r = load16_masked(reinterpret_cast<const uint4 *>(static_cast<const bf16_t *>(base) + (ok ? elem : 0)), ok);
+    }
+    __device__ __forceinline__ uint4 get() const { return r; }
+};
+template <> struct Act8<true> {
+    uint4 r0, r1;
+    __device__ __forceinline__ void load(const void *base, size_t elem, bool ok) {
+        const uint4 *p = reinterpret_cast<const uint4 *>(static_cast<const float *>(base) + (ok ? elem : 0));
+        r0 = load16_masked(p, ok);
+        r1 = load16_masked(p + 1, ok);
+    }
+    __device__ __forceinline__ uint4 get() const {
+        return make_uint4(pack_bf16x2(__uint_as_float(r0.x), __uint_as_float(r0.y)), pack_bf16x2(__uint_as_float(r0.z), __uint_as_float(r0.w)),
+                          pack_bf16x2(__uint_as_float(r1.x), __uint_as_float(r1.y)), pack_bf16x2(__uint_as_float(r1.z), __uint_as_float(r1.w)));
+    }
+};
+
+// F32: dy, x (and an injected f) are stored as fp32 and rounded to bf16 as they are loaded; dxp and df
+// are written as fp32.  The arithmetic is the same either way.
+template <int NP, int WMODE, int ITEMS, bool F32>
 __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentArgs ra) {
+    using TS = typename std::conditional<F32, float, bf16_t>::type;  // storage type of the activations
     static_assert(NP == 4 || NP == 8, "stream groups of four");
     using SK = SkSmall<NP>;
     using CB = CoefBwdSmall<NP, false, true>;
@@ -88,20 +117,18 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
 
     // ---- tile waves: every load of the sample up front -----------------------------------------
     uint4 gr[ITEMS][NB], xr[ITEMS][NB], fr[ITEMS];
+    Act8<F32> graw[ITEMS][NB], xraw[ITEMS][NB], fraw[ITEMS];
     RawVec<bf16_t, 8> wb[ITEMS];
     RawVec<float, 8> wf[ITEMS];
     bool in[ITEMS], sv[NB];
     float hpre[NB], hpost[NB], Mc[NB][NB][4], qraw = 1.f;
     if (tile) {
-        const bf16_t *gb[NB], *xb[NB];
+        size_t rowoff[NB];
 #pragma unroll
         for (int I = 0; I < NB; I++) {
             sv[I] = 4 * I + i < n;  // streams >= n: masked, they alias stream 0
-            const size_t row = (size_t)b * n * C + (size_t)(sv[I] ? 4 * I + i : 0) * C;
-            gb[I] = static_cast<const bf16_t *>(a.dy) + row;
-            xb[I] = static_cast<const bf16_t *>(a.x) + row;
+            rowoff[I] = (size_t)b * n * C + (size_t)(sv[I] ? 4 * I + i : 0) * C;
         }
-        const bf16_t *fb = inject ? static_cast<const bf16_t *>(a.f_inject) + (size_t)b * C : nullptr;
 #pragma unroll
         for (int it = 0; it < ITEMS; it++) {
             const int c = (tw + TW * it) * 128 + blk * 8;
@@ -109,10 +136,10 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
             const int cc = in[it] ? c : 0;
 #pragma unroll
             for (int I = 0; I < NB; I++) {
-                gr[it][I] = load16_masked(reinterpret_cast<const uint4 *>(gb[I] + cc), in[it] && sv[I]);
-                xr[it][I] = load16_masked(reinterpret_cast<const uint4 *>(xb[I] + cc), in[it] && sv[I]);
+                graw[it][I].load(a.dy, rowoff[I] + cc, in[it] && sv[I]);
+                xraw[it][I].load(a.x, rowoff[I] + cc, in[it] && sv[I]);
             }
-            if constexpr (inject) fr[it] = load16_masked(reinterpret_cast<const uint4 *>(fb + cc), in[it] && i == 0);
+            if constexpr (inject) fraw[it].load(a.f_inject, (size_t)b * C + cc, in[it] && i == 0);
             else if constexpr (WMODE == kGramWBf16) wb[it].load(static_cast<const bf16_t *>(a.w) + cc);
             else wf[it].load(static_cast<const float *>(a.w) + cc);
         }
@@ -136,6 +163,13 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
 #pragma unroll
         for (int I = 0; I < NB; I++)
             if (!sv[I]) { hpre[I] = 0.f; hpost[I] = 0.f; }
+        // every load is requested: from here on the tile is four words of bf16 pairs per chunk
+#pragma unroll
+        for (int it = 0; it < ITEMS; it++) {
+#pragma unroll
+            for (int I = 0; I < NB; I++) { gr[it][I] = graw[it][I].get(); xr[it][I] = xraw[it][I].get(); }
+            if constexpr (inject) fr[it] = fraw[it].get();
+        }
     }
 
     MHC_PHASE_ADD_BY(64, kPhaseDxSmall, pwg, 0, tclk);
@@ -277,7 +311,7 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
         if constexpr (inject) {
 #pragma unroll
             for (int v = 0; v < 8; v++) da[v] = 0.f;
-            if (ra.df && i == 0) store_vec<bf16_t, 8>(ra.df + (size_t)b * C + c, dfv);
+            if (ra.df && i == 0) store_vec<TS, 8>(static_cast<TS *>(ra.df) + (size_t)b * C + c, dfv);
         } else {
             float wv[8], uv[8];
             if constexpr (WMODE == kGramWBf16) wb[it].get(wv);
@@ -308,19 +342,20 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
                     out[v] += Mc[I][J][3] * quad_bcast<3>(gv[J][v]);
                 }
             // plain stores: the projection-backward launch reads dxp back right away
-            if (sv[I]) store_vec<bf16_t, 8>(ra.dxp + ((size_t)b * n + 4 * I + i) * C + c, out);
+            if (sv[I]) store_vec<TS, 8>(static_cast<TS *>(ra.dxp) + ((size_t)b * n + 4 * I + i) * C + c, out);
         }
     }
     MHC_PHASE_ADD_BY(64, kPhaseDxSmall, pwg, 3, tclk);
 }
 
 // The rows of a sample must fit the tile waves' registers; the Sinkhorn state shares the LDS.
+// Activations: dy and x both bf16, or both fp32 with x marked as "consumed as bf16".
 bool bwd_resident_supported(int x_dtype, int y_dtype, int phi_dtype, int n, int C, int T) {
-    return x_dtype == kBF16 && y_dtype == kBF16 && phi_dtype == kBF16 && n <= 8 && C % 8 == 0 &&
-           C <= 128 * kResTileWaves * kResMaxItems && T <= 32;
+    const bool io = (x_dtype == kBF16 && y_dtype == kBF16) || (x_dtype == kF32AsBF16 && y_dtype == kF32);
+    return io && phi_dtype == kBF16 && n <= 8 && C % 8 == 0 && C <= 128 * kResTileWaves * kResMaxItems && T <= 32;
 }
 
-template <int NP, int WMODE>
+template <int NP, int WMODE, bool F32>
 static hipError_t launch_items(const BwdResidentArgs &ra, hipStream_t stream) {
     using SK = SkSmall<NP>;
     using CB = CoefBwdSmall<NP, false, true>;
@@ -328,30 +363,34 @@ static hipError_t launch_items(const BwdResidentArgs &ra, hipStream_t stream) {
     const int items = (ra.r.C + 128 * kResTileWaves - 1) / (128 * kResTileWaves);
     const dim3 grid(ra.r.B);
     switch (items) {
-        case 1: bwd_resident_kernel<NP, WMODE, 1><<<grid, kResThreads, smem, stream>>>(ra); break;
-        case 2: bwd_resident_kernel<NP, WMODE, 2><<<grid, kResThreads, smem, stream>>>(ra); break;
-        case 3: bwd_resident_kernel<NP, WMODE, 3><<<grid, kResThreads, smem, stream>>>(ra); break;
-        case 4: bwd_resident_kernel<NP, WMODE, 4><<<grid, kResThreads, smem, stream>>>(ra); break;
-        case 5: bwd_resident_kernel<NP, WMODE, 5><<<grid, kResThreads, smem, stream>>>(ra); break;
+        case 1: bwd_resident_kernel<NP, WMODE, 1, F32><<<grid, kResThreads, smem, stream>>>(ra); break;
+        case 2: bwd_resident_kernel<NP, WMODE, 2, F32><<<grid, kResThreads, smem, stream>>>(ra); break;
+        case 3: bwd_resident_kernel<NP, WMODE, 3, F32><<<grid, kResThreads, smem, stream>>>(ra); break;
+        case 4: bwd_resident_kernel<NP, WMODE, 4, F32><<<grid, kResThreads, smem, stream>>>(ra); break;
+        case 5: bwd_resident_kernel<NP, WMODE, 5, F32><<<grid, kResThreads, smem, stream>>>(ra); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
-hipError_t launch_bwd_resident(const void *dy, const void *x, const void *w, int w_dtype, const void *f_inject,
+hipError_t launch_bwd_resident(const void *dy, const void *x, int x_dtype, const void *w, int w_dtype, const void *f_inject,
                                const float *Hpre, const float *Hpost, const float *M, const float *q,
                                const float *P, const float *r, const float *alpha, const float *b_res,
                                const float *sk_state, BwdCoefOut out, void *dxp, void *df, float *u, int B, int n,
                                int C, int T, float eps, hipStream_t stream) {
     BwdResidentArgs ra{{dy, x, w, f_inject, Hpre, Hpost, M, q, P, r, alpha, b_res, sk_state, out, n,
                         w_dtype == kBF16, B, n, C, T, padded_D(n), eps, nullptr, 1},
-                       static_cast<bf16_t *>(dxp), static_cast<bf16_t *>(df), u};
-#define MHC_RES(NP)                                                                      \
-    return f_inject ? launch_items<NP, kGramInject>(ra, stream)                          \
-                    : (w_dtype == kBF16 ? launch_items<NP, kGramWBf16>(ra, stream)       \
-                                        : launch_items<NP, kGramWF32>(ra, stream))
-    if (n <= 4) MHC_RES(4);
-    MHC_RES(8);
+                       dxp, df, u};
+#define MHC_RES(NP, F32)                                                                      \
+    return f_inject ? launch_items<NP, kGramInject, F32>(ra, stream)                          \
+                    : (w_dtype == kBF16 ? launch_items<NP, kGramWBf16, F32>(ra, stream)       \
+                                        : launch_items<NP, kGramWF32, F32>(ra, stream))
+    if (x_dtype == kF32AsBF16) {
+        if (n <= 4) MHC_RES(4, true);
+        MHC_RES(8, true);
+    }
+    if (n <= 4) MHC_RES(4, false);
+    MHC_RES(8, false);
 #undef MHC_RES
 }
 

@@ -36,8 +36,9 @@ struct Carver {
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool valid_dtype(int d) { return d == MHC_F32 || d == MHC_BF16; }
 inline bool valid_io(int x_dtype, int y_dtype) {
-    // activations in / out: (f32, f32), (bf16, bf16), (bf16 in, f32 out)
-    return (x_dtype == MHC_F32 && y_dtype == MHC_F32) || (x_dtype == MHC_BF16 && valid_dtype(y_dtype));
+    // activations in / out: (f32, f32), (bf16, bf16), (bf16 in, f32 out), (f32 consumed as bf16 in, f32 out)
+    return (x_dtype == MHC_F32 && y_dtype == MHC_F32) || (x_dtype == MHC_BF16 && valid_dtype(y_dtype)) ||
+           (x_dtype == MHC_F32_AS_BF16 && y_dtype == MHC_F32);
 }
 
 int check_shape(int B, int n, int C, int iters) {
@@ -75,6 +76,16 @@ bool bwd_resident_preferred(int B, int n, int C) {
     if (const int hook = tuning_get(kTuneResident)) return hook == 2;
     (void)C;
     return n > 4 || B <= 640;
+}
+
+// Shapes for which the dynamic entry points take fp32 activations that are consumed as bf16
+// (MHC_F32_AS_BF16): the kernels that load fp32 storage directly are the narrow projection, the fused
+// n <= 8 forward and the two launches of the sample-resident backward, where that backward is the
+// path of choice.
+bool f32_as_bf16_accepted(int B, int n, int C, int iters) {
+    return n <= 8 && layer_fwd_fused_supported(n, C, kF32) &&
+           bwd_resident_supported(kF32AsBF16, kF32, kBF16, n, C, iters) && proj_bwd_addx_supported(n) &&
+           bwd_resident_preferred(B, n, C);
 }
 
 int max_ksplit(int B, int n, int C) {
@@ -180,6 +191,10 @@ __attribute__((visibility("default"))) int mhc_tuning_get(int key) {
 
 int mhc_max_sinkhorn_iters(int n) { return (n < 1 || n > MHC_MAX_N) ? 0 : max_layer_sinkhorn_iters(n); }
 
+int mhc_layer_dynamic_accepts_f32_as_bf16(int B, int n, int C, int iters) {
+    return check_shape(B, n, C, iters) == MHC_OK && f32_as_bf16_accepted(B, n, C, iters) ? 1 : 0;
+}
+
 const char *mhc_status_string(int status) {
     switch (status) {
         case MHC_OK: return "ok";
@@ -222,6 +237,8 @@ int mhc_layer_fwd_dynamic(const void *x, int x_dtype, const void *w, int w_dtype
         return MHC_ERR_NULL_POINTER;
     if (!f_inject && !w) return MHC_ERR_NULL_POINTER;
     if (!valid_io(x_dtype, y_dtype) || !valid_dtype(phi_dtype) || (w && !valid_dtype(w_dtype)))
+        return MHC_ERR_BAD_DTYPE;
+    if (x_dtype == MHC_F32_AS_BF16 && (phi_dtype != MHC_BF16 || !f32_as_bf16_accepted(B, n, C, iters)))
         return MHC_ERR_BAD_DTYPE;
     if (!aligned16(x) || !aligned16(y) || !aligned16(phi) || (f_inject && !aligned16(f_inject)))
         return MHC_ERR_MISALIGNED;
@@ -267,6 +284,8 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     if (!f_inject && (!w || !dw)) return MHC_ERR_NULL_POINTER;
     if (!valid_io(x_dtype, y_dtype) || !valid_dtype(phi_dtype) || (w && !valid_dtype(w_dtype)))
         return MHC_ERR_BAD_DTYPE;
+    if (x_dtype == MHC_F32_AS_BF16 && (phi_dtype != MHC_BF16 || !f32_as_bf16_accepted(B, n, C, iters)))
+        return MHC_ERR_BAD_DTYPE;
     if (!aligned16(dy) || !aligned16(x) || !aligned16(dx) || !aligned16(phi) || !aligned16(dphi) ||
         (f_inject && !aligned16(f_inject)) || (df && !aligned16(df)))
         return MHC_ERR_MISALIGNED;
@@ -274,7 +293,7 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int D = n * n + 2 * n, DP = padded_D(n);
-    const bool mfma = proj_bwd_mfma_supported(x_dtype, phi_dtype, C);
+    const bool mfma = proj_bwd_mfma_supported(x_dtype == kF32AsBF16 ? kBF16 : x_dtype, phi_dtype, C);
     BwdCoefOut out{ws.dt, ws.dP, ws.cx, ws.s1, nullptr, mfma ? ws.dPb : nullptr, ws.dPT, ws.BP};
     if (mfma && bwd_resident_supported(x_dtype, y_dtype, phi_dtype, n, C, iters) && proj_bwd_addx_supported(n) &&
         bwd_resident_preferred(B, n, C)) {
@@ -282,17 +301,18 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
         // the channel sums, the coefficient backward and the mixing part of dx; (2) a column-slab
         // kernel over all samples adds dP phi - cx x, finishes dphi without batch-split partial sums
         // and sums dw, dbias and dalpha in a few extra workgroups
-        MHC_LAUNCH(launch_bwd_resident(dy, x, w, w_dtype, f_inject, H_pre, H_post, M, q, P, r, alpha, bias + 2 * n,
+        MHC_LAUNCH(launch_bwd_resident(dy, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, q, P, r, alpha, bias + 2 * n,
                                        sk_state, out, dx, df, ws.u, B, n, C, iters, eps, st));
         const BatchSumArgs sums = make_batch_sums(ws.u, B, C, f_inject ? nullptr : dw, ws.dt, B, D, dbias, dalpha);
         bool tail_taken = false;
-        MHC_LAUNCH(launch_proj_bwd_addx(x, phi, ws.dPb, ws.dPT, ws.BP, ws.cx, dphi, dx, B, n, C,
+        MHC_LAUNCH(launch_proj_bwd_addx(x, x_dtype, phi, ws.dPb, ws.dPT, ws.BP, ws.cx, dphi, dx, B, n, C,
                                         tuning_get(kTuneSeparateFinalize) == 1 ? nullptr : &sums, &tail_taken, st));
         if (!tail_taken)
             MHC_LAUNCH(launch_finalize(ws.u, B, C, f_inject ? nullptr : dw, ws.dt, B, D, dbias, dalpha, nullptr, 1,
                                        0, nullptr, st));
         return MHC_OK;
     }
+    if (x_dtype == kF32AsBF16) return MHC_ERR_BAD_DTYPE;  // not reached: accepted shapes take the path above
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      n, q, P, r, alpha, bias + 2 * n, sk_state, out, ws.raw, B, n, C, iters, eps,
                                      st));

@@ -9,7 +9,9 @@
 
 namespace mhc {
 
-enum DType { kF32 = 0, kBF16 = 1 };
+// kF32AsBF16: stored as fp32, consumed as bf16 - the kernels round the values to bf16 (nearest even) as
+// they load them and compute as for bf16 storage (MHC_F32_AS_BF16 of the C ABI).
+enum DType { kF32 = 0, kBF16 = 1, kF32AsBF16 = 2 };
 
 inline size_t dtype_size(int dt) { return dt == kBF16 ? 2 : 4; }
 
@@ -170,7 +172,7 @@ hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb,
 // outputs of launch_mix_bwd_reduce) and dxp = M^T dy + Hpre (x) da from ONE pass over dy and x, one
 // workgroup per sample; u [B, C] = the samples' summands of dw, df with an injected f.
 bool bwd_resident_supported(int x_dtype, int y_dtype, int phi_dtype, int n, int C, int T);
-hipError_t launch_bwd_resident(const void *dy, const void *x, const void *w, int w_dtype, const void *f_inject,
+hipError_t launch_bwd_resident(const void *dy, const void *x, int x_dtype, const void *w, int w_dtype, const void *f_inject,
                                const float *Hpre, const float *Hpost, const float *M, const float *q,
                                const float *P, const float *r, const float *alpha, const float *b_res,
                                const float *sk_state, BwdCoefOut out, void *dxp, void *df, float *u, int B, int n,
@@ -179,7 +181,7 @@ hipError_t launch_bwd_resident(const void *dy, const void *x, const void *w, int
 // dphi = dP^T x_flat without batch split, dx completed in place (dx = dxp + dP phi - cx x), and `tail`
 // (dw, dbias, dalpha) summed by extra workgroups when the grid has room (*tail_taken).
 bool proj_bwd_addx_supported(int n);
-hipError_t launch_proj_bwd_addx(const void *x, const void *phi, const void *dPb, const void *dPT, int BP,
+hipError_t launch_proj_bwd_addx(const void *x, int x_dtype, const void *phi, const void *dPb, const void *dPT, int BP,
                                 const float *cx, float *dphi, void *dx, int B, int n, int C, const BatchSumArgs *tail,
                                 bool *tail_taken, hipStream_t stream);
 // n <= 18: whether the two products are faster apart (measured: from D > 128 on)

@@ -141,7 +141,21 @@ struct LayerFwdArgs {
     int KS, DP, w_bf16, B, n, C, T;
     float eps;
     float *sk_state;  // dynamic: [B][T + 1][2][NP] Sinkhorn denominators kept for the backward, or nullptr
+    int round_x;      // fp32 x (and f) consumed as bf16: round every value to bf16 as it is unpacked
 };
+
+// The values of a loaded chunk, widened to fp32; fp32 storage that is consumed as bf16 is rounded here
+// (nearest even), so that the mixing sees what the projection and the backward kernels see.
+template <typename T, int V>
+__device__ __forceinline__ void get_act(const RawVec<T, V> &r, float (&v)[V], int round_bf16) {
+    r.get(v);
+    if constexpr (std::is_same<T, float>::value) {
+        if (round_bf16) {
+#pragma unroll
+            for (int i = 0; i < V; i++) v[i] = bf16_to_f32(f32_to_bf16(v[i]));
+        }
+    }
+}
 
 constexpr int kFwdStaggerMinB = 512;  // two or more workgroups per CU
 
@@ -408,7 +422,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             const int c = (ch < nch ? ch : 0) * V;
             float f[V];
             if (inject) {
-                fr[k].get(f);
+                get_act(fr[k], f, a.round_x);
             } else {
                 if (a.w_bf16) load_vec<bf16_t, V>(static_cast<const bf16_t *>(a.w) + c, f);
                 else load_vec<float, V>(static_cast<const float *>(a.w) + c, f);
@@ -480,7 +494,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
             for (int k = 0; k < CPT; k++)
 #pragma unroll
-                for (int i = 0; i < NP; i++) xr[k][i].get(xv[k][i]);  // streams >= n meet zero coefficients
+                for (int i = 0; i < NP; i++) get_act(xr[k][i], xv[k][i], a.round_x);  // streams >= n meet zero coefficients
         }
         float av[LEAN ? 1 : CPT][V];  // LEAN recomputes the aggregate in step 4 instead of keeping it
         float qinv = 1.0f;
@@ -495,7 +509,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
                 for (int i = 0; i < NP; i++) {
                     float t[V];
-                    if constexpr (LEAN) xr[k][i].get(t);
+                    if constexpr (LEAN) get_act(xr[k][i], t, a.round_x);
 #pragma unroll
                     for (int v = 0; v < V; v++) s_a[v] += hpre[i] * (LEAN ? t[v] : xv[LEAN ? 0 : k][i][v]);
                 }
@@ -522,7 +536,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
                 const int c = ch * V;
                 float f[V];
                 if (inject) {
-                    fr[k].get(f);
+                    get_act(fr[k], f, a.round_x);
                 } else {
                     if constexpr (LEAN) {
 #pragma unroll
@@ -530,7 +544,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
                         for (int i = 0; i < NP; i++) {
                             float t[V];
-                            xr[k][i].get(t);
+                            get_act(xr[k][i], t, a.round_x);
 #pragma unroll
                             for (int v = 0; v < V; v++) f[v] += hpre[i] * t[v];
                         }
@@ -550,7 +564,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
                         for (int j = 0; j < NP; j++) {
                             float t[V];
-                            if constexpr (LEAN) xr[k][j].get(t);
+                            if constexpr (LEAN) get_act(xr[k][j], t, a.round_x);
                             const float mij = LEAN ? coef_s[i * NP + j] : Mr[i][j];
 #pragma unroll
                             for (int v = 0; v < V; v++) out[v] += mij * (LEAN ? t[v] : xv[LEAN ? 0 : k][j][v]);
@@ -599,7 +613,8 @@ hipError_t launch_layer_fwd_fused(const void *x, int x_dtype, const void *w, int
                                   float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
                                   float *sk_state, int B, int n, int C, int T, float eps, hipStream_t stream) {
     LayerFwdArgs a{x, w, f_inject, y, Ppart, ssqpart, alpha, b_pre, b_post, b_res, Hpre, Hpost, M, P, r, q,
-                   KS, DP, w_dtype == kBF16, B, n, C, T, eps, sk_state};
+                   KS, DP, w_dtype == kBF16, B, n, C, T, eps, sk_state, x_dtype == kF32AsBF16};
+    if (x_dtype == kF32AsBF16) x_dtype = kF32;  // fp32 storage
     hipError_t err = hipErrorInvalidValue;
     bool ok = false;
 #define MHC_FUSED(TX, TY)                                                        \

@@ -30,13 +30,13 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
 struct ProjAddxArgs {
-    const bf16_t *x;     // [B][nC]
+    const void *x;       // [B][nC], bf16 or (F32) fp32 rounded to bf16 on its way into LDS
     const bf16_t *phi;   // [D][nC]
     const bf16_t *dPb;   // dP, fragment-major (frag_dpb); columns >= D are zero
     const bf16_t *dPT;   // dP^T hi and lo bf16 planes, fragment-major (frag_dpt); rows >= D, columns >= B zero
     const float *cx;     // [B]
     float *dphi;         // [D][nC]
-    bf16_t *dx;          // [B][nC]: in dxp, out dx
+    void *dx;            // [B][nC]: in dxp, out dx; stored like x
     int B, BP, D, DP, nC;
     int tail_row;        // blockIdx.y of the workgroups that compute `tail` (-1: none)
     BatchSumArgs tail;
@@ -51,8 +51,12 @@ constexpr int kAxLDR = 33;         // LDS pitch of the dphi tiles in the final c
 // 4 SPW samples).  PFOP: the dP operands of the next block are requested a block ahead like x and dxp.
 // Measured at B=320, C=1280, n=4 (backward, graphs of ten): SPW 32 without / with PFOP 16.1 / 16.1 us,
 // SPW 64 without PFOP 19.1 us, with PFOP 23.0 us (registers spill).
-template <int NTD, int SPW, bool PFOP>
+// F32: x and dx are stored as fp32 (x is rounded to bf16 for the products and for the -cx x term, as in
+// the bf16 storage case; dxp is read and dx written as fp32).
+template <int NTD, int SPW, bool PFOP, bool F32>
 __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
+    using TS = typename std::conditional<F32, float, bf16_t>::type;
+    constexpr int AW = F32 ? 8 : 4;  // words of an 8-element chunk as stored
     constexpr int SBR = 4 * SPW;   // samples per block
     constexpr int KS = SPW / 16;   // k-steps (16 samples) of a wave per block = its 16-byte chunks of x and of dxp
     constexpr int TT = SPW / 32;   // 32-sample tiles of a wave per block
@@ -81,8 +85,18 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
     const int ech = lane & 3, erow = SPW * wave + (lane >> 2);
     const int kc = k0 + ech * 8;
     const bool kok = kc < nC;  // nC % 8 == 0: a chunk is inside or outside
-    uint32_t xr[2][KS][4], pr[2][KS][4];
+    uint32_t xr[2][KS][AW], pr[2][KS][AW];
     float cxr[2][KS];
+    const TS *xg = static_cast<const TS *>(a.x);
+    TS *dxg = static_cast<TS *>(a.dx);
+    auto load_chunk = [&](const TS *p, uint32_t (&q)[AW], bool ok) {
+        const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(p), ok);
+        q[0] = v.x; q[1] = v.y; q[2] = v.z; q[3] = v.w;
+        if constexpr (F32) {
+            const uint4 v2 = load16_masked(reinterpret_cast<const uint4 *>(p) + 1, ok);
+            q[4] = v2.x; q[5] = v2.y; q[6] = v2.z; q[7] = v2.w;
+        }
+    };
     auto load_block = [&](int sb, auto slot) {
         constexpr int S = decltype(slot)::value;
 #pragma unroll
@@ -90,15 +104,13 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
             const int ch = tid + u * 256;
             const int b = sb + (ch >> 2), k = k0 + (ch & 3) * 8;
             const bool ok = b < B && k < nC;
-            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(a.x + (ok ? (size_t)b * nC + k : 0)), ok);
-            xr[S][u][0] = v.x; xr[S][u][1] = v.y; xr[S][u][2] = v.z; xr[S][u][3] = v.w;
+            load_chunk(xg + (ok ? (size_t)b * nC + k : 0), xr[S][u], ok);
         }
 #pragma unroll
         for (int t = 0; t < KS; t++) {
             const int b = sb + erow + 16 * t;
             const bool ok = b < B && kok;
-            const uint4 v = *reinterpret_cast<const uint4 *>(a.dx + (ok ? (size_t)b * nC + kc : 0));
-            pr[S][t][0] = v.x; pr[S][t][1] = v.y; pr[S][t][2] = v.z; pr[S][t][3] = v.w;
+            load_chunk(dxg + (ok ? (size_t)b * nC + kc : 0), pr[S][t], ok);
             cxr[S][t] = a.cx[b < B ? b : 0];
         }
     };
@@ -172,8 +184,14 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
 #pragma unroll
         for (int u = 0; u < KS; u++) {
             const int ch = tid + u * 256;
-            *reinterpret_cast<uint4 *>(x_s + (size_t)(ch >> 2) * kAxLD + (ch & 3) * 8) =
-                make_uint4(xr[S][u][0], xr[S][u][1], xr[S][u][2], xr[S][u][3]);
+            uint4 xb;
+            if constexpr (F32)
+                xb = make_uint4(pack_bf16x2(__uint_as_float(xr[S][u][0]), __uint_as_float(xr[S][u][1])),
+                                pack_bf16x2(__uint_as_float(xr[S][u][2]), __uint_as_float(xr[S][u][3])),
+                                pack_bf16x2(__uint_as_float(xr[S][u][4]), __uint_as_float(xr[S][u][5])),
+                                pack_bf16x2(__uint_as_float(xr[S][u][6]), __uint_as_float(xr[S][u][7])));
+            else xb = make_uint4(xr[S][u][0], xr[S][u][1], xr[S][u][2], xr[S][u][3]);
+            *reinterpret_cast<uint4 *>(x_s + (size_t)(ch >> 2) * kAxLD + (ch & 3) * 8) = xb;
         }
         __syncthreads();
         // ---- dphi: this wave's samples, every row tile ------------------------------------------------
@@ -217,14 +235,15 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
             const float cxv = cxr[S][t];
             const float ov[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
             const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
-            uint32_t outw[4];
+            float res[8];
 #pragma unroll
             for (int p = 0; p < 4; p++) {
-                const float lo = bf16lo_to_f32(pr[S][t][p]) + ov[2 * p] - cxv * bf16lo_to_f32(xw[p]);
-                const float hi = bf16hi_to_f32(pr[S][t][p]) + ov[2 * p + 1] - cxv * bf16hi_to_f32(xw[p]);
-                outw[p] = pack_bf16x2(lo, hi);
+                const float plo = F32 ? __uint_as_float(pr[S][t][F32 ? 2 * p : p]) : bf16lo_to_f32(pr[S][t][p]);
+                const float phi_ = F32 ? __uint_as_float(pr[S][t][F32 ? 2 * p + 1 : p]) : bf16hi_to_f32(pr[S][t][p]);
+                res[2 * p] = plo + ov[2 * p] - cxv * bf16lo_to_f32(xw[p]);
+                res[2 * p + 1] = phi_ + ov[2 * p + 1] - cxv * bf16hi_to_f32(xw[p]);
             }
-            if (b < B && kok) st16<true>(a.dx + (size_t)b * nC + kc, outw[0], outw[1], outw[2], outw[3]);
+            if (b < B && kok) store_vec<TS, 8, true>(dxg + (size_t)b * nC + kc, res);
         }
         if (sb + 2 * SBR < B) {
             load_block(sb + 2 * SBR, slot);
@@ -255,36 +274,37 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
 
 bool proj_bwd_addx_supported(int n) { return padded_D(n) / 32 <= 3; }
 
-template <int NTD, int SPW, bool PFOP>
+template <int NTD, int SPW, bool PFOP, bool F32>
 static hipError_t launch_addx(const ProjAddxArgs &a, hipStream_t stream) {
     constexpr int SBR = 4 * SPW;
     const size_t tiles = sizeof(bf16_t) * (size_t)kAxLD * (32 * NTD + SBR) + sizeof(float) * SBR * kAxLDO;
     const size_t red = sizeof(float) * 4 * NTD * 32 * kAxLDR;  // the final cross-wave sum reuses the tiles' memory
     const size_t smem = tiles > red ? tiles : red;
-    hipError_t e = allow_dynamic_lds(&proj_bwd_addx_kernel<NTD, SPW, PFOP>, smem);
+    hipError_t e = allow_dynamic_lds(&proj_bwd_addx_kernel<NTD, SPW, PFOP, F32>, smem);
     if (e != hipSuccess) return e;
     const int slabs = (a.nC + kAxKW - 1) / kAxKW;
     dim3 grid(round_up(slabs, 16), 1 + (a.tail_row >= 0 ? 1 : 0));
-    proj_bwd_addx_kernel<NTD, SPW, PFOP><<<grid, 256, smem, stream>>>(a);
+    proj_bwd_addx_kernel<NTD, SPW, PFOP, F32><<<grid, 256, smem, stream>>>(a);
     return hipGetLastError();
 }
 
-hipError_t launch_proj_bwd_addx(const void *x, const void *phi, const void *dPb, const void *dPT, int BP,
+hipError_t launch_proj_bwd_addx(const void *x, int x_dtype, const void *phi, const void *dPb, const void *dPT, int BP,
                                 const float *cx, float *dphi, void *dx, int B, int n, int C, const BatchSumArgs *tail,
                                 bool *tail_taken, hipStream_t stream) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n), NTD = DP / 32;
-    ProjAddxArgs a{static_cast<const bf16_t *>(x), static_cast<const bf16_t *>(phi), static_cast<const bf16_t *>(dPb),
-                   static_cast<const bf16_t *>(dPT), cx, dphi, static_cast<bf16_t *>(dx), B, BP, D, DP, nC, -1, {}};
+    ProjAddxArgs a{x, static_cast<const bf16_t *>(phi), static_cast<const bf16_t *>(dPb),
+                   static_cast<const bf16_t *>(dPT), cx, dphi, dx, B, BP, D, DP, nC, -1, {}};
     if (tail_taken) *tail_taken = false;
     if (tail && tail->nblk <= round_up((nC + kAxKW - 1) / kAxKW, 16)) {
         a.tail = *tail;
         a.tail_row = 1;
         if (tail_taken) *tail_taken = true;
     }
+    const bool f32 = x_dtype == kF32AsBF16;
     switch (NTD) {
-        case 1: return launch_addx<1, 32, false>(a, stream);
-        case 2: return launch_addx<2, 32, false>(a, stream);
-        case 3: return launch_addx<3, 32, false>(a, stream);
+        case 1: return f32 ? launch_addx<1, 32, false, true>(a, stream) : launch_addx<1, 32, false, false>(a, stream);
+        case 2: return f32 ? launch_addx<2, 32, false, true>(a, stream) : launch_addx<2, 32, false, false>(a, stream);
+        case 3: return f32 ? launch_addx<3, 32, false, true>(a, stream) : launch_addx<3, 32, false, false>(a, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -11,6 +11,8 @@
 //                           through a wave-private LDS tile.
 //   proj_fwd_generic_kernel any dtype / any C: fp32 FMA, exact products (the fp32 parity tier).
 #include "launchers.h"
+
+#include <type_traits>
 #include "mhc_common.h"
 #include "phase_profiler.h"
 
@@ -20,7 +22,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
 static inline bool use_mfma(int x_dtype, int phi_dtype, int C) {
-    return x_dtype == kBF16 && phi_dtype == kBF16 && C % 8 == 0;
+    return (x_dtype == kBF16 || x_dtype == kF32AsBF16) && phi_dtype == kBF16 && C % 8 == 0;
 }
 
 // --------------------------------------------------------------------------------------------
@@ -77,14 +79,18 @@ __global__ __launch_bounds__(256) void proj_fwd_generic_kernel(const TX *__restr
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 constexpr int kNarrowPitch = 72;  // LDS row of a 64-element chunk: 128 data bytes + 16 pad (bf16 elements)
 
-template <int NT>
-__global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__restrict__ x,
+// XF32: x is stored as fp32 and rounded to bf16 (nearest even) on its way into the LDS tile; everything
+// behind the tile, the sum of squares included, sees the rounded values.
+template <int NT, bool XF32 = false>
+__global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const void *__restrict__ x_,
                                                             const bf16_t *__restrict__ phi,
                                                             float *__restrict__ Ppart,
                                                             float *__restrict__ ssqpart, int B,
                                                             int D, int DP, int nC, int tiles_s, int KS,
                                                             int sub /* K per wave, multiple of 64 */) {
     extern __shared__ __align__(16) float lds[];  // per wave [(1 + NT) * 32][pitch] bf16; later [4][NT*16 + 1][64] fp32
+    using TXS = typename std::conditional<XF32, float, bf16_t>::type;  // storage type of x
+    const TXS *__restrict__ x = static_cast<const TXS *>(x_);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int set = (blockIdx.x >> 3) / tiles_s;
     const int st = (blockIdx.x >> 3) % tiles_s, ks = (blockIdx.x & 7) + 8 * set;
@@ -106,7 +112,7 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
     // back as fragments; no barrier is involved (a wave's LDS accesses complete in order).
     bf16_t *cb = reinterpret_cast<bf16_t *>(lds) + (size_t)wave * (1 + NT) * 32 * kNarrowPitch;
     const int lr = lane >> 3, seg = lane & 7;
-    const bf16_t *xrow[4];
+    const TXS *xrow[4];
     const bf16_t *prow[NT][4];
     bool xval[4], pval[NT][4];
 #pragma unroll
@@ -121,7 +127,16 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
             prow[t][j] = phi + (size_t)(pval[t][j] ? d : 0) * nC;
         }
     }
-    uint32_t xq[4][4], pq[NT][4][4];  // scalar words: whole-uint4 array elements can end up in scratch
+    constexpr int XW = XF32 ? 8 : 4;  // words of a lane's 8 elements of x as loaded
+    uint32_t xq[4][XW], pq[NT][4][4];  // scalar words: whole-uint4 array elements can end up in scratch
+    auto load_x8 = [&](const TXS *p, uint32_t (&q)[XW], bool ok) {
+        const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(p), ok);
+        q[0] = v.x; q[1] = v.y; q[2] = v.z; q[3] = v.w;
+        if constexpr (XF32) {
+            const uint4 v2 = load16_masked(reinterpret_cast<const uint4 *>(p) + 1, ok);
+            q[4] = v2.x; q[5] = v2.y; q[6] = v2.z; q[7] = v2.w;
+        }
+    };
     // Rows beyond B (x) or D (phi) alias row 0: what they produce is finite and is either not stored
     // (samples >= B) or zeroed at the store (projection rows >= D), so only the K tail of the last
     // slab needs a mask - a uniform test per chunk instead of four selects per load (the kernel is
@@ -131,8 +146,12 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
         if (k0 + 64 <= kend) {
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const uint4 v = *reinterpret_cast<const uint4 *>(xrow[j] + k);
-                xq[j][0] = v.x; xq[j][1] = v.y; xq[j][2] = v.z; xq[j][3] = v.w;
+                if constexpr (XF32) {
+                    load_x8(xrow[j] + k, xq[j], true);
+                } else {
+                    const uint4 v = *reinterpret_cast<const uint4 *>(xrow[j] + k);
+                    xq[j][0] = v.x; xq[j][1] = v.y; xq[j][2] = v.z; xq[j][3] = v.w;
+                }
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
                     const uint4 p = *reinterpret_cast<const uint4 *>(prow[t][j] + k);
@@ -145,8 +164,7 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
         const int off = kv ? k : 0;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint4 v = load16_masked(reinterpret_cast<const uint4 *>(xrow[j] + off), kv);
-            xq[j][0] = v.x; xq[j][1] = v.y; xq[j][2] = v.z; xq[j][3] = v.w;
+            load_x8(xrow[j] + off, xq[j], kv);
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 const uint4 p = load16_masked(reinterpret_cast<const uint4 *>(prow[t][j] + off), kv);
@@ -157,6 +175,13 @@ __global__ __launch_bounds__(256) void proj_fwd_mfma_kernel(const bf16_t *__rest
     auto park = [&]() {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
+            if constexpr (XF32)
+                *reinterpret_cast<uint4 *>(cb + (size_t)(lr + 8 * j) * kNarrowPitch + seg * 8) =
+                    make_uint4(pack_bf16x2(__uint_as_float(xq[j][0]), __uint_as_float(xq[j][1])),
+                               pack_bf16x2(__uint_as_float(xq[j][2]), __uint_as_float(xq[j][3])),
+                               pack_bf16x2(__uint_as_float(xq[j][4]), __uint_as_float(xq[j][5])),
+                               pack_bf16x2(__uint_as_float(xq[j][6]), __uint_as_float(xq[j][7])));
+            else
             *reinterpret_cast<uint4 *>(cb + (size_t)(lr + 8 * j) * kNarrowPitch + seg * 8) =
                 make_uint4(xq[j][0], xq[j][1], xq[j][2], xq[j][3]);
 #pragma unroll
@@ -497,7 +522,7 @@ static hipError_t launch_generic(const void *x, const void *phi, float *Ppart, f
     return hipGetLastError();
 }
 
-template <int NT>
+template <int NT, bool XF32 = false>
 static hipError_t launch_mfma(const void *x, const void *phi, float *Ppart, float *ssqpart, int KS,
                               int B, int D, int DP, int nC, hipStream_t stream) {
     const int tiles_s = (B + 31) / 32;
@@ -507,10 +532,9 @@ static hipError_t launch_mfma(const void *x, const void *phi, float *Ppart, floa
     const size_t smem_chunks = sizeof(bf16_t) * 4 * (1 + NT) * 32 * kNarrowPitch;
     const size_t smem_sum = sizeof(float) * 4 * (NT * 16 + 1) * 64;
     const size_t smem = smem_chunks > smem_sum ? smem_chunks : smem_sum;
-    if (hipError_t e = allow_dynamic_lds(&proj_fwd_mfma_kernel<NT>, smem); e != hipSuccess) return e;
-    proj_fwd_mfma_kernel<NT><<<grid, 256, smem, stream>>>(static_cast<const bf16_t *>(x),
-                                                           static_cast<const bf16_t *>(phi), Ppart,
-                                                           ssqpart, B, D, DP, nC, tiles_s, KS, sub);
+    if (hipError_t e = allow_dynamic_lds(&proj_fwd_mfma_kernel<NT, XF32>, smem); e != hipSuccess) return e;
+    proj_fwd_mfma_kernel<NT, XF32><<<grid, 256, smem, stream>>>(x, static_cast<const bf16_t *>(phi), Ppart,
+                                                                 ssqpart, B, D, DP, nC, tiles_s, KS, sub);
     return hipGetLastError();
 }
 
@@ -518,6 +542,14 @@ hipError_t launch_proj_fwd(const void *x, int x_dtype, const void *phi, int phi_
                            float *ssqpart, int KS, int B, int n, int C, hipStream_t stream) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
     if (use_mfma(x_dtype, phi_dtype, C)) {
+        if (x_dtype == kF32AsBF16) {  // fp32 storage, rounded on load: the narrow kernel only (n <= 8)
+            switch (use_wide(n, C) ? 0 : mfma_nt(n)) {
+                case 1: return launch_mfma<1, true>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
+                case 2: return launch_mfma<2, true>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
+                case 3: return launch_mfma<3, true>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
+                default: return hipErrorInvalidValue;
+            }
+        }
         if (use_wide(n, C)) return launch_wide<1, 2, 4>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);
         switch (mfma_nt(n)) {
             case 1: return launch_mfma<1>(x, phi, Ppart, ssqpart, KS, B, D, DP, nC, stream);

@@ -16,7 +16,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("MHC_HIP_LIBRARY") or os.path.join(_HERE, "libmhc_hip.so")
 
-MHC_F32, MHC_BF16 = 0, 1
+MHC_F32, MHC_BF16, MHC_F32_AS_BF16 = 0, 1, 2
 MHC_MAX_N = 32
 ABI_VERSION = 2
 
@@ -33,6 +33,7 @@ _SIGNATURES = {
     "mhc_abi_version": (c_int, []),
     "mhc_status_string": (c_char_p, [_I]),
     "mhc_max_sinkhorn_iters": (c_int, [_I]),
+    "mhc_layer_dynamic_accepts_f32_as_bf16": (c_int, [_I, _I, _I, _I]),
     "mhc_layer_dynamic_workspace_bytes": (_Z, [_I, _I, _I]),
     "mhc_layer_sinkhorn_state_floats": (_Z, [_I, _I, _I]),
     "mhc_layer_fwd_dynamic": (c_int, [_P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P,

@@ -111,8 +111,11 @@ class MHCLayerDynamicFunction:
 
 def mhc_layer_fused_dynamic(x_expanded, rmsnorm_weight, phi_pre, phi_post, phi_res, alpha_pre,
                             alpha_post, alpha_res, b_pre, b_post, b_res, sinkhorn_iters=20, eps=1e-5,
-                            out_dtype=None, f_inject=None):
+                            out_dtype=None, f_inject=None, compute_bf16=False):
+    """compute_bf16: float32 activations go through the bf16 (matrix-core) kernels, as in the reference's
+    fused path (bindings.cu:421-423); where the kernels load float32 storage themselves no cast pass
+    is launched."""
     return _ext.mhc_layer_dynamic(x_expanded, rmsnorm_weight, phi_pre, phi_post, phi_res,
                                   _as_tensor(alpha_pre, phi_pre), _as_tensor(alpha_post, phi_pre),
                                   _as_tensor(alpha_res, phi_pre), b_pre, b_post, b_res, int(sinkhorn_iters),
-                                  float(eps), out_dtype, f_inject)
+                                  float(eps), out_dtype, f_inject, bool(compute_bf16))

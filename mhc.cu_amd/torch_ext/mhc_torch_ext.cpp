@@ -187,7 +187,7 @@ struct SmallViews {
     }
 };
 
-DynFwdOut dyn_forward(const Tensor &x, const OptTensor &w, const Packed &pk, const OptTensor &f_inject,
+DynFwdOut dyn_forward(const Tensor &x, int x_code, const OptTensor &w, const Packed &pk, const OptTensor &f_inject,
                       at::ScalarType out_dtype, int iters, double eps, bool for_backward) {
     const int B = x.size(0), n = x.size(1), C = x.size(2), D = n * n + 2 * n;
     c10::DeviceGuard guard(x.device());
@@ -203,7 +203,7 @@ DynFwdOut dyn_forward(const Tensor &x, const OptTensor &w, const Packed &pk, con
     const Tensor ft = f_inject.has_value() ? *f_inject : Tensor();
     float *ba = pk.ba.data_ptr<float>();
     check("mhc_layer_fwd_dynamic",
-          mhc_layer_fwd_dynamic(ptr(x), dt(x), ptr(wt), wt.defined() ? dt(wt) : 0, ptr(pk.phi), dt(pk.phi), ba, ba + D,
+          mhc_layer_fwd_dynamic(ptr(x), x_code, ptr(wt), wt.defined() ? dt(wt) : 0, ptr(pk.phi), dt(pk.phi), ba, ba + D,
                                 ptr(ft), ptr(o.y), dt(o.y), v.Hp, v.Ho, v.M, v.P, v.r, v.q, v.sk, B, n, C, iters,
                                 (float)eps, ws.data_ptr(), (size_t)ws.numel(), stream_of(x)));
     return o;
@@ -214,20 +214,34 @@ struct MHCDynamicFn : public torch::autograd::Function<MHCDynamicFn> {
                           const Tensor &phi_post, const Tensor &phi_res, const Tensor &alpha_pre,
                           const Tensor &alpha_post, const Tensor &alpha_res, const Tensor &b_pre, const Tensor &b_post,
                           const Tensor &b_res, int64_t iters, double eps, c10::optional<at::ScalarType> out_dtype,
-                          const OptTensor &f_in, bool grad_mode) {
+                          const OptTensor &f_in, bool grad_mode, bool compute_bf16) {
         TORCH_CHECK(x_in.dim() == 3, "mhc: x must be [B, n, C]");
-        const Tensor x = act(is_act_dtype(x_in) ? x_in : x_in.to(at::kFloat));
-        const int n = x.size(1), C = x.size(2);
+        // compute_bf16 with float32 activations (the reference's default contract: float32 in and out
+        // around a bf16 kernel path): where the library's kernels load fp32 storage themselves, x is
+        // handed over as it is and rounded in registers; elsewhere it is cast here, as the reference
+        // casts it (bindings.cu:421-423)
+        Tensor x = act(is_act_dtype(x_in) ? x_in : x_in.to(at::kFloat));
+        const int B = x.size(0), n = x.size(1), C = x.size(2);
+        int x_code = dt(x);
+        if (compute_bf16 && x.scalar_type() == at::kFloat) {
+            if (out_dtype.value_or(at::kFloat) == at::kFloat && mhc_layer_dynamic_accepts_f32_as_bf16(B, n, C, (int)iters))
+                x_code = MHC_F32_AS_BF16;
+            else {
+                x = x.to(at::kBFloat16);
+                x_code = MHC_BF16;
+            }
+        }
         OptTensor w, f;
         if (w_in.has_value() && w_in->defined()) w = act(is_act_dtype(*w_in) ? *w_in : w_in->to(at::kFloat));
         if (f_in.has_value() && f_in->defined()) f = act(f_in->to(x.scalar_type()));
         const Packed pk = pack_params(phi_pre, phi_post, phi_res, alpha_pre, alpha_post, alpha_res, b_pre, b_post, b_res,
-                                      n, C, x.scalar_type());
-        DynFwdOut o = dyn_forward(x, w, pk, f, out_dtype.value_or(at::kFloat), (int)iters, eps, grad_mode);
+                                      n, C, x_code == MHC_F32 ? at::kFloat : at::kBFloat16);
+        DynFwdOut o = dyn_forward(x, x_code, w, pk, f, out_dtype.value_or(at::kFloat), (int)iters, eps, grad_mode);
         ctx->save_for_backward({x, w.has_value() ? *w : Tensor(), pk.phi, pk.ba, f.has_value() ? *f : Tensor(), o.small});
         ctx->saved_data["iters"] = iters;
         ctx->saved_data["eps"] = eps;
         ctx->saved_data["x_dtype"] = (int64_t)x_in.scalar_type();
+        ctx->saved_data["x_code"] = (int64_t)x_code;
         ctx->saved_data["w_dtype"] = (int64_t)(w_in.has_value() && w_in->defined() ? w_in->scalar_type() : at::kFloat);
         ctx->saved_data["f_dtype"] = (int64_t)(f_in.has_value() && f_in->defined() ? f_in->scalar_type() : at::kFloat);
         ctx->saved_data["phi_dtypes"] = std::vector<int64_t>{(int64_t)phi_pre.scalar_type(), (int64_t)phi_post.scalar_type(),
@@ -258,7 +272,7 @@ struct MHCDynamicFn : public torch::autograd::Function<MHCDynamicFn> {
         Tensor ws = workspace(x, mhc_layer_dynamic_workspace_bytes(B, n, C));
         float *bap = ba.data_ptr<float>();
         check("mhc_layer_bwd_dynamic",
-              mhc_layer_bwd_dynamic(ptr(dy), dt(dy), ptr(x), dt(x), ptr(w), w.defined() ? dt(w) : 0, ptr(phi), dt(phi), bap,
+              mhc_layer_bwd_dynamic(ptr(dy), dt(dy), ptr(x), (int)ctx->saved_data["x_code"].toInt(), ptr(w), w.defined() ? dt(w) : 0, ptr(phi), dt(phi), bap,
                                     bap + D, ptr(f), v.Hp, v.Ho, v.M, v.P, v.r, v.q, v.sk, ptr(dx), ptr(df),
                                     dw.defined() ? dw.data_ptr<float>() : nullptr, dphi.data_ptr<float>(),
                                     dba.data_ptr<float>(), dba.data_ptr<float>() + D, B, n, C, iters, (float)eps,
@@ -271,7 +285,7 @@ struct MHCDynamicFn : public torch::autograd::Function<MHCDynamicFn> {
         const auto ad = ctx->saved_data["alpha_dtypes"].toIntVector();
         const auto bd = ctx->saved_data["b_dtypes"].toIntVector();
         const auto brs = ctx->saved_data["b_res_shape"].toIntVector();
-        variable_list out(16);
+        variable_list out(17);
         out[0] = to(dx, ctx->saved_data["x_dtype"].toInt());
         out[1] = (dw.defined() && w.defined()) ? to(dw, ctx->saved_data["w_dtype"].toInt()) : Tensor();
         out[2] = to(dphi.narrow(0, 0, n), pd[0]);
@@ -471,10 +485,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           [](const Tensor &x, const OptTensor &w, const Tensor &phi_pre, const Tensor &phi_post, const Tensor &phi_res,
              const Tensor &alpha_pre, const Tensor &alpha_post, const Tensor &alpha_res, const Tensor &b_pre,
              const Tensor &b_post, const Tensor &b_res, int64_t iters, double eps, c10::optional<at::ScalarType> out_dtype,
-             const OptTensor &f_inject) {
+             const OptTensor &f_inject, bool compute_bf16) {
               return MHCDynamicFn::apply(x, w, phi_pre, phi_post, phi_res, alpha_pre, alpha_post, alpha_res, b_pre, b_post,
-                                         b_res, iters, eps, out_dtype, f_inject, at::GradMode::is_enabled());
+                                         b_res, iters, eps, out_dtype, f_inject, at::GradMode::is_enabled(), compute_bf16);
           },
+          py::arg("x"), py::arg("w"), py::arg("phi_pre"), py::arg("phi_post"), py::arg("phi_res"), py::arg("alpha_pre"),
+          py::arg("alpha_post"), py::arg("alpha_res"), py::arg("b_pre"), py::arg("b_post"), py::arg("b_res"), py::arg("iters"),
+          py::arg("eps"), py::arg("out_dtype"), py::arg("f_inject"), py::arg("compute_bf16") = false,
           "mhc_layer_fwd_dynamic / mhc_layer_bwd_dynamic with autograd (reference bindings.cu:405-542)");
     m.def("mhc_layer_static",
           [](const Tensor &x, const OptTensor &w, const Tensor &H_pre, const Tensor &H_post, const Tensor &H_res,
