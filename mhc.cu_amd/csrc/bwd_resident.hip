@@ -74,17 +74,24 @@ template <> struct Act8<true> {
 
 // F32: dy, x (and an injected f) are stored as fp32 and rounded to bf16 as they are loaded; dxp and df
 // are written as fp32.  The arithmetic is the same either way.
-template <int NP, int WMODE, int ITEMS, bool F32>
-__global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentArgs ra) {
+// STATIC: shared coefficients ([n] / [n, n] instead of per sample).  There is no projection, so dxp is
+// the complete dx; wave 0 only turns the sums into the sample's row of raw coefficient gradients
+// (dM | dHpre | dHpost), whose batch sum feeds the one Sinkhorn backward of the static layer.
+template <int NP, int WMODE, int ITEMS, bool F32, bool STATIC = false>
+__global__ __launch_bounds__(STATIC ? 64 * kResTileWaves : kResThreads) void bwd_resident_kernel(BwdResidentArgs ra) {
     using TS = typename std::conditional<F32, float, bf16_t>::type;  // storage type of the activations
     static_assert(NP == 4 || NP == 8, "stream groups of four");
     using SK = SkSmall<NP>;
-    using CB = CoefBwdSmall<NP, false, true>;
+    using CB = CoefBwdSmall<NP, false, true, STATIC>;
     constexpr int NB = NP / 4;            // stream groups
     constexpr int K = 3 * NP * NP;
     constexpr int TW = kResTileWaves;
     constexpr bool inject = WMODE == kGramInject;
     const BwdReduceArgs &a = ra.r;
+    const int hs = STATIC ? 0 : a.n;      // sample stride of Hpre / Hpost (M: hs * n)
+    // STATIC has no serial chain to run beside the tile: no coefficient wave, four waves per workgroup
+    // (its few coefficient lanes are the first lanes of tile wave 0), so four workgroups fit a CU
+    constexpr int CW = STATIC ? 0 : 1;    // coefficient waves in front of the tile waves
     __shared__ float slot_s[K * TW * 4];  // one slot per 16-lane row of the tile waves
     __shared__ float tot_s[K + 1];        // the sums, then s1
     extern __shared__ float sc[];         // Sinkhorn denominators, SK::scaling_floats(T), then CB::kXch
@@ -100,24 +107,27 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
     if (tid < SK::kGroup) {
         // everything the coefficient backward needs besides the sums, requested at once
         cb.prefetch(a, b, tid);
-        cb.forward_recompute(a, b, tid, tid, sc);
+        if constexpr (!STATIC) cb.forward_recompute(a, b, tid, tid, sc);
     }
     // the NP^2 threads that will hold the sums of W1 (one DPP row of wave 0 for 4x4, wave 1 for 8x8) ask
     // for their factor of s1 = Hpost^T W1 Hpre now, not behind the barrier
     float hohp = 0.f;
     if (!inject && tid >= NP * NP && tid < 2 * NP * NP) {
         const int e = tid - NP * NP, r = e / NP, c = e % NP;
-        const float ho = a.Hpost[(size_t)b * n + (r < n ? r : 0)], hp = a.Hpre[(size_t)b * n + (c < n ? c : 0)];
+        const float ho = a.Hpost[(size_t)b * hs + (r < n ? r : 0)], hp = a.Hpre[(size_t)b * hs + (c < n ? c : 0)];
         hohp = (r < n && c < n) ? ho * hp : 0.f;
     }
     MHC_PHASE_ADD(kPhaseGramSmall, pwg, 0, pclk);
     const int blk = lane >> 2, i = lane & 3;
-    const int tw = wave - 1;              // tile wave index, -1 for the coefficient wave
+    const int tw = wave - CW;             // tile wave index, -1 for the coefficient wave
     const bool tile = tw >= 0;
 
     // ---- tile waves: every load of the sample up front -----------------------------------------
     uint4 gr[ITEMS][NB], xr[ITEMS][NB], fr[ITEMS];
     Act8<F32> graw[ITEMS][NB], xraw[ITEMS][NB], fraw[ITEMS];
+    // (the RMSNorm weight chunks stay in registers next to the tile: fetching them again where they are
+    // used, one item ahead, to save registers measured slower - B=1280, C=2560 static backward 33.4 -> 34.1 us -
+    // and forcing four workgroups per CU made the compiler spill: 50.1 us)
     RawVec<bf16_t, 8> wb[ITEMS];
     RawVec<float, 8> wf[ITEMS];
     bool in[ITEMS], sv[NB];
@@ -144,7 +154,7 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
             else wf[it].load(static_cast<const float *>(a.w) + cc);
         }
         // this lane's coefficients for step 3 (its own streams j = 4I + i), in flight with the tile
-        const float *Hp = a.Hpre + (size_t)b * n, *Ho = a.Hpost + (size_t)b * n, *Mb = a.M + (size_t)b * n * n;
+        const float *Hp = a.Hpre + (size_t)b * hs, *Ho = a.Hpost + (size_t)b * hs, *Mb = a.M + (size_t)b * hs * n;
 #pragma unroll
         for (int I = 0; I < NB; I++) {
             hpre[I] = Hp[sv[I] ? 4 * I + i : 0];
@@ -234,7 +244,7 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
         }
         // Lane (block, j) holds column j of its block's products, register = row.  Sum over the four
         // blocks of a 16-lane row with DPP, one LDS slot per row.
-        const int slot = (tid - 64) >> 4;
+        const int slot = (tid - 64 * CW) >> 4;
 #pragma unroll
         for (int m = 0; m < 3; m++)
 #pragma unroll
@@ -274,10 +284,10 @@ __global__ __launch_bounds__(kResThreads) void bwd_resident_kernel(BwdResidentAr
     // ---- 2. coefficient backward on the first lanes of wave 0 -----------------------------------------
     if (tid < SK::kGroup) {
         cb.fetch_sums(tot_s, 1);
-        cb.run(a, b, tid, tid, sc, sc + SK::scaling_floats(a.T));
+        cb.run(a, b, tid, tid, sc, sc + (STATIC ? 0 : SK::scaling_floats(a.T)));
     }
     MHC_PHASE_ADD(kPhaseGramSmall, pwg, 3, pclk);
-    if (!tile) return;
+    if (!tile) return;  // the coefficient wave (none with STATIC) is done
 
     // ---- 3. tile waves: dxp, u, df ---------------------------------------------------------------------
     float qinv = 0.f, k2 = 0.f;
@@ -355,19 +365,20 @@ bool bwd_resident_supported(int x_dtype, int y_dtype, int phi_dtype, int n, int 
     return io && phi_dtype == kBF16 && n <= 8 && C % 8 == 0 && C <= 128 * kResTileWaves * kResMaxItems && T <= 32;
 }
 
-template <int NP, int WMODE, bool F32>
+template <int NP, int WMODE, bool F32, bool STATIC = false>
 static hipError_t launch_items(const BwdResidentArgs &ra, hipStream_t stream) {
     using SK = SkSmall<NP>;
-    using CB = CoefBwdSmall<NP, false, true>;
-    const size_t smem = sizeof(float) * (SK::scaling_floats(ra.r.T) + CB::kXch);
+    using CB = CoefBwdSmall<NP, false, true, STATIC>;
+    const size_t smem = sizeof(float) * ((STATIC ? 0 : SK::scaling_floats(ra.r.T)) + CB::kXch);
     const int items = (ra.r.C + 128 * kResTileWaves - 1) / (128 * kResTileWaves);
     const dim3 grid(ra.r.B);
+    const int threads = STATIC ? 64 * kResTileWaves : kResThreads;
     switch (items) {
-        case 1: bwd_resident_kernel<NP, WMODE, 1, F32><<<grid, kResThreads, smem, stream>>>(ra); break;
-        case 2: bwd_resident_kernel<NP, WMODE, 2, F32><<<grid, kResThreads, smem, stream>>>(ra); break;
-        case 3: bwd_resident_kernel<NP, WMODE, 3, F32><<<grid, kResThreads, smem, stream>>>(ra); break;
-        case 4: bwd_resident_kernel<NP, WMODE, 4, F32><<<grid, kResThreads, smem, stream>>>(ra); break;
-        case 5: bwd_resident_kernel<NP, WMODE, 5, F32><<<grid, kResThreads, smem, stream>>>(ra); break;
+        case 1: bwd_resident_kernel<NP, WMODE, 1, F32, STATIC><<<grid, threads, smem, stream>>>(ra); break;
+        case 2: bwd_resident_kernel<NP, WMODE, 2, F32, STATIC><<<grid, threads, smem, stream>>>(ra); break;
+        case 3: bwd_resident_kernel<NP, WMODE, 3, F32, STATIC><<<grid, threads, smem, stream>>>(ra); break;
+        case 4: bwd_resident_kernel<NP, WMODE, 4, F32, STATIC><<<grid, threads, smem, stream>>>(ra); break;
+        case 5: bwd_resident_kernel<NP, WMODE, 5, F32, STATIC><<<grid, threads, smem, stream>>>(ra); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -392,6 +403,24 @@ hipError_t launch_bwd_resident(const void *dy, const void *x, int x_dtype, const
     if (n <= 4) MHC_RES(4, false);
     MHC_RES(8, false);
 #undef MHC_RES
+}
+
+// Static H: the same launch with shared coefficients; dxp is the final dx, out.red [B, D+3] receives the
+// samples' raw coefficient gradients and out.s1 their s1.
+hipError_t launch_bwd_resident_static(const void *dy, const void *x, const void *w, int w_dtype, const void *f_inject,
+                                      const float *Hpre, const float *Hpost, const float *M, const float *q,
+                                      BwdCoefOut out, void *dx, void *df, float *u, int B, int n, int C,
+                                      hipStream_t stream) {
+    BwdResidentArgs ra{{dy, x, w, f_inject, Hpre, Hpost, M, q, nullptr, nullptr, nullptr, nullptr, nullptr, out, 0,
+                        w_dtype == kBF16, B, n, C, 0, padded_D(n), 0.f, nullptr, 1},
+                       dx, df, u};
+#define MHC_RES_STATIC(NP)                                                                        \
+    return f_inject ? launch_items<NP, kGramInject, false, true>(ra, stream)                      \
+                    : (w_dtype == kBF16 ? launch_items<NP, kGramWBf16, false, true>(ra, stream)   \
+                                        : launch_items<NP, kGramWF32, false, true>(ra, stream))
+    if (n <= 4) MHC_RES_STATIC(4);
+    MHC_RES_STATIC(8);
+#undef MHC_RES_STATIC
 }
 
 }  // namespace mhc

@@ -460,6 +460,18 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int D = n * n + 2 * n;
     BwdCoefOut out{nullptr, nullptr, nullptr, ws.s1, ws.red, nullptr, nullptr, 0};
+    if (bwd_resident_supported(x_dtype, y_dtype, kBF16, n, C, 0) && tuning_get(kTuneResident) != 1) {
+        // bf16 activations, n <= 8: with shared coefficients nothing of dx depends on a batch-wide
+        // result, so ONE pass over dy and x (a workgroup keeps its sample's rows in registers) forms
+        // the channel sums, the sample's raw coefficient gradients and the complete dx
+        MHC_LAUNCH(launch_bwd_resident_static(dy, x, w, w_dtype, f_inject, H_pre, H_post, M, q, out, dx, df, ws.u,
+                                              B, n, C, st));
+        MHC_LAUNCH(launch_finalize(ws.u, B, C, f_inject ? nullptr : dw, ws.red, B, D, ws.red_sum, ws.red_sum + D,
+                                   nullptr, 1, 0, nullptr, st));
+        MHC_LAUNCH(launch_coef_bwd_static(ws.red_sum, H_pre, H_post, H_res_logits, dH_pre, dH_post,
+                                          dH_res, n, iters, eps, st));
+        return MHC_OK;
+    }
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      0, q, nullptr, nullptr, nullptr, nullptr, nullptr, out, n > 8 ? ws.raw : nullptr,
                                      B, n, C, iters, eps, st));

@@ -177,6 +177,12 @@ hipError_t launch_bwd_resident(const void *dy, const void *x, int x_dtype, const
                                const float *P, const float *r, const float *alpha, const float *b_res,
                                const float *sk_state, BwdCoefOut out, void *dxp, void *df, float *u, int B, int n,
                                int C, int T, float eps, hipStream_t stream);
+// Static H (bf16 dy and x, bwd_resident_supported with any T): the complete dx from that one pass, u, and
+// per sample out.red [B, D+3] = raw (dM | dHpre | dHpost) and out.s1.
+hipError_t launch_bwd_resident_static(const void *dy, const void *x, const void *w, int w_dtype, const void *f_inject,
+                                      const float *Hpre, const float *Hpost, const float *M, const float *q,
+                                      BwdCoefOut out, void *dx, void *df, float *u, int B, int n, int C,
+                                      hipStream_t stream);
 // Second and last launch of that backward (D <= 96): a column slab for all samples per workgroup;
 // dphi = dP^T x_flat without batch split, dx completed in place (dx = dxp + dP phi - cx x), and `tail`
 // (dw, dbias, dalpha) summed by extra workgroups when the grid has room (*tail_taken).

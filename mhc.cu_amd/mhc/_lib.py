@@ -81,7 +81,7 @@ def tuning_lib():
     this one to compare two launch paths on the same inputs."""
     global _TUNING_LIB
     if _TUNING_LIB is None:
-        path = os.path.join(_HERE, "libmhc_hip_tuning.so")
+        path = os.environ.get("MHC_HIP_TUNING_LIBRARY") or os.path.join(_HERE, "libmhc_hip_tuning.so")
         if not os.path.exists(path):
             raise ImportError(f"{path} not found: python mhc.cu_amd/build.py --tuning")
         handle = _bind(ctypes.CDLL(path))
