@@ -94,6 +94,7 @@ __global__ __launch_bounds__(STATIC ? 64 * kResTileWaves : kResThreads) void bwd
     constexpr int CW = STATIC ? 0 : 1;    // coefficient waves in front of the tile waves
     __shared__ float slot_s[K * TW * 4];  // one slot per 16-lane row of the tile waves
     __shared__ float tot_s[K + 1];        // the sums, then s1
+    __shared__ float park_s[STATIC ? 1 : SkSmall<NP>::kGroup];  // one value per coefficient lane, see below
     extern __shared__ float sc[];         // Sinkhorn denominators, SK::scaling_floats(T), then CB::kXch
     const int b = blockIdx.x, n = a.n, C = a.C;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -107,7 +108,13 @@ __global__ __launch_bounds__(STATIC ? 64 * kResTileWaves : kResThreads) void bwd
     if (tid < SK::kGroup) {
         // everything the coefficient backward needs besides the sums, requested at once
         cb.prefetch(a, b, tid);
-        if constexpr (!STATIC) cb.forward_recompute(a, b, tid, tid, sc);
+        if constexpr (!STATIC) {
+            cb.forward_recompute(a, b, tid, tid, sc);
+            // The coefficient lanes share their register budget with the tile code below; the final
+            // iterate lived across it in scratch memory, and reading it back was a global round trip in
+            // front of the serial Sinkhorn sweep: it is parked in LDS instead.
+            park_s[tid] = cb.m_fin;
+        }
     }
     // the NP^2 threads that will hold the sums of W1 (one DPP row of wave 0 for 4x4, wave 1 for 8x8) ask
     // for their factor of s1 = Hpost^T W1 Hpre now, not behind the barrier
@@ -283,6 +290,9 @@ __global__ __launch_bounds__(STATIC ? 64 * kResTileWaves : kResThreads) void bwd
     MHC_PHASE_ADD_BY(64, kPhaseDxSmall, pwg, 2, tclk);
     // ---- 2. coefficient backward on the first lanes of wave 0 -----------------------------------------
     if (tid < SK::kGroup) {
+        if constexpr (!STATIC) {
+            cb.m_fin = park_s[tid];
+        }
         cb.fetch_sums(tot_s, 1);
         cb.run(a, b, tid, tid, sc, sc + (STATIC ? 0 : SK::scaling_floats(a.T)));
     }

@@ -301,8 +301,10 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
         // the channel sums, the coefficient backward and the mixing part of dx; (2) a column-slab
         // kernel over all samples adds dP phi - cx x, finishes dphi without batch-split partial sums
         // and sums dw, dbias and dalpha in a few extra workgroups
+        BwdCoefOut out2 = out;
+        out2.dP = nullptr;  // the second launch takes dP as matrix-core operands only
         MHC_LAUNCH(launch_bwd_resident(dy, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, q, P, r, alpha, bias + 2 * n,
-                                       sk_state, out, dx, df, ws.u, B, n, C, iters, eps, st));
+                                       sk_state, out2, dx, df, ws.u, B, n, C, iters, eps, st));
         const BatchSumArgs sums = make_batch_sums(ws.u, B, C, f_inject ? nullptr : dw, ws.dt, B, D, dbias, dalpha);
         bool tail_taken = false;
         MHC_LAUNCH(launch_proj_bwd_addx(x, x_dtype, phi, ws.dPb, ws.dPT, ws.BP, ws.cx, dphi, dx, B, n, C,

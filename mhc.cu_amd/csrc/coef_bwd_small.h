@@ -45,7 +45,7 @@ struct DPWriter {
     BwdCoefOut o;
     int b, B, DP;
     __device__ __forceinline__ void put(int d, float v) const {
-        o.dP[(size_t)b * DP + d] = v;
+        if (o.dP) o.dP[(size_t)b * DP + d] = v;  // fp32 copy: only the kernels without matrix-core operands read it
         if (o.dPb) {
             const bf16_t h = f32_to_bf16(v);
             const size_t plane = (size_t)DP * o.BP;
@@ -61,7 +61,7 @@ struct DPWriter {
     }
     __device__ __forceinline__ void pad(int D, int first, int step) const {
         for (int d = D + first; d < DP; d += step) {
-            o.dP[(size_t)b * DP + d] = 0.f;
+            if (o.dP) o.dP[(size_t)b * DP + d] = 0.f;
             if (o.dPb) {
                 const size_t plane = (size_t)DP * o.BP;
                 o.dPb[frag_dpb(b, d, DP)] = 0;
@@ -99,7 +99,7 @@ template <int NP, bool PRECISE, bool GRAM, bool STATIC = false> struct CoefBwdSm
     int r0, c0, gc;
     bool inject, mv;
     float qinv, rinv, inv_c, inv_nc, al0, al1, al2, pres, bres, hp, ho, ppre, ppost, hpre_r, hpost_r;
-    float E, m_fin;  // exp(logit) and the final Sinkhorn iterate of this lane's element (forward_recompute)
+    float m_fin;  // the final Sinkhorn iterate of this lane's element (forward_recompute)
     float dMe, s_a, s_b, s_c, s_d;  // this lane's channel sums (fetch_sums): GRAM w1, w1t, xx | else dHpost, A1, A2, s1
 
     __device__ __forceinline__ void prefetch(const BwdReduceArgs &a, int b, int g) {
@@ -140,10 +140,9 @@ template <int NP, bool PRECISE, bool GRAM, bool STATIC = false> struct CoefBwdSm
             m_fin = a.M[(size_t)b * a.n * a.n + (mv ? r0 * a.n + c0 : 0)];
             SK::load_state(a.sk_state + (size_t)b * SK::state_floats(a.T), g, a.T, sc, lane);
             m_fin = mv ? m_fin : 0.f;
-            E = mv ? (PRECISE ? expf(al2 * pres + bres) : exp_fast(al2 * pres + bres)) : 0.f;
             return;
         }
-        E = mv ? (PRECISE ? expf(al2 * pres + bres) : exp_fast(al2 * pres + bres)) : 0.f;
+        const float E = mv ? (PRECISE ? expf(al2 * pres + bres) : exp_fast(al2 * pres + bres)) : 0.f;
         float m[1] = {E};
         SK::template forward<PRECISE>(m, g, a.n, a.T, a.eps, sc, lane);
         m_fin = m[0];
