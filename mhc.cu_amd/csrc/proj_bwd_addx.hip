@@ -11,7 +11,7 @@
 // workgroups (one more grid row) add up dw, dbias and dalpha (batch_sums.h), so the backward needs no
 // third launch.
 //
-// Samples are walked in blocks of 256 (D <= 32) or 128.  Per block every thread requests its 16-byte
+// Samples are walked in blocks of 128, 256 or 384 (4, 8 or 12 waves of 32 samples).  Per block every thread requests its 16-byte
 // chunks of x and dxp up front (row-contiguous, next block in flight while this one is worked on); x is
 // parked in LDS as [sample][column] and read back transposed as the B operand of
 // v_mfma_f32_32x32x16_bf16 (the contraction of dphi runs over samples, the strided axis).  Wave w owns a
@@ -53,22 +53,24 @@ constexpr int kAxLDR = 33;         // LDS pitch of the dphi tiles in the final c
 // SPW 64 without PFOP 19.1 us, with PFOP 23.0 us (registers spill).
 // F32: x and dx are stored as fp32 (x is rounded to bf16 for the products and for the -cx x term, as in
 // the bf16 storage case; dxp is read and dx written as fp32).
-template <int NTD, int SPW, bool PFOP, bool F32>
-__global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
+// NW: waves per workgroup (a block is NW * SPW samples).
+template <int NTD, int SPW, bool PFOP, bool F32, int NW = 4>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void proj_bwd_addx_kernel(ProjAddxArgs a) {
+    constexpr int NT_ = 64 * NW;  // threads
     using TS = typename std::conditional<F32, float, bf16_t>::type;
     constexpr int AW = F32 ? 8 : 4;  // words of an 8-element chunk as stored
-    constexpr int SBR = 4 * SPW;   // samples per block
+    constexpr int SBR = NW * SPW;  // samples per block
     constexpr int KS = SPW / 16;   // k-steps (16 samples) of a wave per block = its 16-byte chunks of x and of dxp
     constexpr int TT = SPW / 32;   // 32-sample tiles of a wave per block
     extern __shared__ __align__(16) unsigned char ax_smem[];
     bf16_t *phi_s = reinterpret_cast<bf16_t *>(ax_smem);                 // [32 NTD][LD]
     bf16_t *x_s = phi_s + (size_t)32 * NTD * kAxLD;                       // [SBR][LD]
     float *o_s = reinterpret_cast<float *>(x_s + (size_t)SBR * kAxLD);    // [SBR][LDO]
-    float *red_s = reinterpret_cast<float *>(ax_smem);                    // final sum: [4][NTD][32][LDR], over everything
+    float *red_s = reinterpret_cast<float *>(ax_smem);                    // final sum: [NW][NTD][32][LDR], over everything
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if ((int)blockIdx.y == a.tail_row) {
         // the extra row of the grid: its first workgroups do the batch sums, the others have nothing to do
-        if ((int)blockIdx.x < a.tail.nblk) batch_sum_block<4>(a.tail, blockIdx.x, tid, reinterpret_cast<double *>(ax_smem));
+        if ((int)blockIdx.x < a.tail.nblk) batch_sum_block<NW>(a.tail, blockIdx.x, tid, reinterpret_cast<double *>(ax_smem));
         return;
     }
     // Workgroup ids go round robin over the 8 XCDs (each with its own L2, 128-byte lines).  A slab
@@ -85,8 +87,12 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
     const int ech = lane & 3, erow = SPW * wave + (lane >> 2);
     const int kc = k0 + ech * 8;
     const bool kok = kc < nC;  // nC % 8 == 0: a chunk is inside or outside
-    uint32_t xr[2][KS][AW], pr[2][KS][AW];
-    float cxr[2][KS];
+    // dxp of the next block is requested a block ahead like x, except where that costs the registers that
+    // keep two workgroups on a CU (fp32 storage with a wide projection): there it is requested at the top
+    // of its own block and arrives under the matrix-core phase
+    constexpr int PS = (F32 && NTD >= 2) ? 1 : 2;
+    uint32_t xr[2][KS][AW], pr[PS][KS][AW];
+    float cxr[PS][KS];
     const TS *xg = static_cast<const TS *>(a.x);
     TS *dxg = static_cast<TS *>(a.dx);
     auto load_chunk = [&](const TS *p, uint32_t (&q)[AW], bool ok) {
@@ -101,17 +107,28 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
         constexpr int S = decltype(slot)::value;
 #pragma unroll
         for (int u = 0; u < KS; u++) {
-            const int ch = tid + u * 256;
+            const int ch = tid + u * NT_;
             const int b = sb + (ch >> 2), k = k0 + (ch & 3) * 8;
             const bool ok = b < B && k < nC;
             load_chunk(xg + (ok ? (size_t)b * nC + k : 0), xr[S][u], ok);
         }
+        if constexpr (PS == 2) {
+#pragma unroll
+            for (int t = 0; t < KS; t++) {
+                const int b = sb + erow + 16 * t;
+                const bool ok = b < B && kok;
+                load_chunk(dxg + (ok ? (size_t)b * nC + kc : 0), pr[S][t], ok);
+                cxr[S][t] = a.cx[b < B ? b : 0];
+            }
+        }
+    };
+    auto load_prev = [&](int sb) {  // PS == 1: the block's own dxp chunks
 #pragma unroll
         for (int t = 0; t < KS; t++) {
             const int b = sb + erow + 16 * t;
             const bool ok = b < B && kok;
-            load_chunk(dxg + (ok ? (size_t)b * nC + kc : 0), pr[S][t], ok);
-            cxr[S][t] = a.cx[b < B ? b : 0];
+            load_chunk(dxg + (ok ? (size_t)b * nC + kc : 0), pr[0][t], ok);
+            cxr[0][t] = a.cx[b < B ? b : 0];
         }
     };
     // Operands that come straight from global memory in fragment order: dP^T (rounded value and
@@ -147,10 +164,10 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
 
     // ---- every load of the first block (and the next one) is requested before anything is waited for ---
     constexpr int PCH = 32 * NTD * 4;  // 16-byte chunks of the phi slab (rows >= D, columns >= nC read as zero)
-    uint4 phir[(PCH + 255) / 256];
+    uint4 phir[(PCH + NT_ - 1) / NT_];
 #pragma unroll
-    for (int u = 0; u < (PCH + 255) / 256; u++) {
-        const int ch = tid + u * 256;
+    for (int u = 0; u < (PCH + NT_ - 1) / NT_; u++) {
+        const int ch = tid + u * NT_;
         const int d = ch >> 2, k = k0 + (ch & 3) * 8;
         const bool ok = ch < PCH && d < D && k < nC;
         phir[u] = load16_masked(reinterpret_cast<const uint4 *>(a.phi + (ok ? (size_t)d * nC + k : 0)), ok);
@@ -162,8 +179,8 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
         if constexpr (PFOP) load_ops(SBR, ops[1]);
     }
 #pragma unroll
-    for (int u = 0; u < (PCH + 255) / 256; u++) {
-        const int ch = tid + u * 256;
+    for (int u = 0; u < (PCH + NT_ - 1) / NT_; u++) {
+        const int ch = tid + u * NT_;
         if (ch < PCH) *reinterpret_cast<uint4 *>(phi_s + (size_t)(ch >> 2) * kAxLD + (ch & 3) * 8) = phir[u];
     }
 
@@ -176,6 +193,8 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
     auto process_block = [&](int sb, auto slot) {
         constexpr int S = decltype(slot)::value;
         Ops &op = ops[PFOP ? S : 0];
+        constexpr int P = PS == 2 ? S : 0;
+        if constexpr (PS == 1) load_prev(sb);
         if (sb != 0) {
             if constexpr (!PFOP) load_ops(sb, op);
             __syncthreads();  // every wave is done with the previous block's tile
@@ -183,7 +202,7 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
         // ---- x block -> LDS (the first barrier also covers the phi slab) -------------------------------
 #pragma unroll
         for (int u = 0; u < KS; u++) {
-            const int ch = tid + u * 256;
+            const int ch = tid + u * NT_;
             uint4 xb;
             if constexpr (F32)
                 xb = make_uint4(pack_bf16x2(__uint_as_float(xr[S][u][0]), __uint_as_float(xr[S][u][1])),
@@ -232,14 +251,14 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
             const float4 o0 = *reinterpret_cast<const float4 *>(o_s + (size_t)r * kAxLDO + ech * 8);
             const float4 o1 = *reinterpret_cast<const float4 *>(o_s + (size_t)r * kAxLDO + ech * 8 + 4);
             const uint4 xv = *reinterpret_cast<const uint4 *>(x_s + (size_t)r * kAxLD + ech * 8);
-            const float cxv = cxr[S][t];
+            const float cxv = cxr[P][t];
             const float ov[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
             const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
             float res[8];
 #pragma unroll
             for (int p = 0; p < 4; p++) {
-                const float plo = F32 ? __uint_as_float(pr[S][t][F32 ? 2 * p : p]) : bf16lo_to_f32(pr[S][t][p]);
-                const float phi_ = F32 ? __uint_as_float(pr[S][t][F32 ? 2 * p + 1 : p]) : bf16hi_to_f32(pr[S][t][p]);
+                const float plo = F32 ? __uint_as_float(pr[P][t][F32 ? 2 * p : p]) : bf16lo_to_f32(pr[P][t][p]);
+                const float phi_ = F32 ? __uint_as_float(pr[P][t][F32 ? 2 * p + 1 : p]) : bf16hi_to_f32(pr[P][t][p]);
                 res[2 * p] = plo + ov[2 * p] - cxv * bf16lo_to_f32(xw[p]);
                 res[2 * p + 1] = phi_ + ov[2 * p + 1] - cxv * bf16hi_to_f32(xw[p]);
             }
@@ -263,28 +282,28 @@ __global__ __launch_bounds__(256, 2) void proj_bwd_addx_kernel(ProjAddxArgs a) {
         for (int i = 0; i < 16; i++)
             red_s[((size_t)(wave * NTD + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3)) * kAxLDR + row] = acc[m][i];
     __syncthreads();
-    for (int e = tid; e < NTD * 32 * 32; e += 256) {
+    for (int e = tid; e < NTD * 32 * 32; e += NT_) {
         const int d = e >> 5, c = e & 31;
         float s = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; w++) s += red_s[((size_t)w * NTD * 32 + d) * kAxLDR + c];
+        for (int w = 0; w < NW; w++) s += red_s[((size_t)w * NTD * 32 + d) * kAxLDR + c];
         if (d < D && k0 + c < nC) a.dphi[(size_t)d * nC + k0 + c] = s;
     }
 }
 
 bool proj_bwd_addx_supported(int n) { return padded_D(n) / 32 <= 3; }
 
-template <int NTD, int SPW, bool PFOP, bool F32>
+template <int NTD, int SPW, bool PFOP, bool F32, int NW = 4>
 static hipError_t launch_addx(const ProjAddxArgs &a, hipStream_t stream) {
-    constexpr int SBR = 4 * SPW;
+    constexpr int SBR = NW * SPW;
     const size_t tiles = sizeof(bf16_t) * (size_t)kAxLD * (32 * NTD + SBR) + sizeof(float) * SBR * kAxLDO;
-    const size_t red = sizeof(float) * 4 * NTD * 32 * kAxLDR;  // the final cross-wave sum reuses the tiles' memory
+    const size_t red = sizeof(float) * NW * NTD * 32 * kAxLDR;  // the final cross-wave sum reuses the tiles' memory
     const size_t smem = tiles > red ? tiles : red;
-    hipError_t e = allow_dynamic_lds(&proj_bwd_addx_kernel<NTD, SPW, PFOP, F32>, smem);
+    hipError_t e = allow_dynamic_lds(&proj_bwd_addx_kernel<NTD, SPW, PFOP, F32, NW>, smem);
     if (e != hipSuccess) return e;
     const int slabs = (a.nC + kAxKW - 1) / kAxKW;
     dim3 grid(round_up(slabs, 16), 1 + (a.tail_row >= 0 ? 1 : 0));
-    proj_bwd_addx_kernel<NTD, SPW, PFOP, F32><<<grid, 256, smem, stream>>>(a);
+    proj_bwd_addx_kernel<NTD, SPW, PFOP, F32, NW><<<grid, 64 * NW, smem, stream>>>(a);
     return hipGetLastError();
 }
 
@@ -301,8 +320,24 @@ hipError_t launch_proj_bwd_addx(const void *x, int x_dtype, const void *phi, con
         if (tail_taken) *tail_taken = true;
     }
     const bool f32 = x_dtype == kF32AsBF16;
+    // D <= 32: the workgroup is sized so that it walks its samples in as few blocks as possible (4, 8 or
+    // 12 waves of 32 samples; every block costs two barriers and a round of dependent LDS traffic).
+    // Backward at B=320, C=1280, n=4, graphs of ten: 4 waves (three blocks) 16.5 us, 8 waves 16.0, 12 waves
+    // (one block) 14.9; B=128: 9.5 / 9.9 with 4 / 8 waves; B=512: 19.7 / 19.0 / 19.5.  Wider projections
+    // keep four waves: their registers allow two workgroups per CU only that way.
+    int nw = 4;
+    if (NTD == 1) {
+        int best = (B + 127) / 128;
+        if ((B + 255) / 256 < best) { nw = 8; best = (B + 255) / 256; }
+        if ((B + 383) / 384 < best) nw = 12;
+    }
     switch (NTD) {
-        case 1: return f32 ? launch_addx<1, 32, false, true>(a, stream) : launch_addx<1, 32, false, false>(a, stream);
+        case 1:
+            // (fp32 storage needs more registers per wave: eight waves at most)
+            if (nw == 12 && !f32) return launch_addx<1, 32, false, false, 12>(a, stream);
+            if (nw == 12) return launch_addx<1, 32, false, true, 8>(a, stream);
+            if (nw == 8) return f32 ? launch_addx<1, 32, false, true, 8>(a, stream) : launch_addx<1, 32, false, false, 8>(a, stream);
+            return f32 ? launch_addx<1, 32, false, true>(a, stream) : launch_addx<1, 32, false, false>(a, stream);
         case 2: return f32 ? launch_addx<2, 32, false, true>(a, stream) : launch_addx<2, 32, false, false>(a, stream);
         case 3: return f32 ? launch_addx<3, 32, false, true>(a, stream) : launch_addx<3, 32, false, false>(a, stream);
         default: return hipErrorInvalidValue;
