@@ -68,14 +68,15 @@ struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *raw, *dphi_part; unsig
 // is taken where it is supported.  Its second launch walks all samples of a column slab in one
 // workgroup, which stops paying once the batch is large enough to fill the chip with batch splits.
 // Measured, backward in graphs of ten, slab / Gram path -> resident path (us):
-//   n=4 C=1280: B=64 17.1 -> 9.2, 128 17.2 -> 9.7, 320 19.1 -> 16.1, 512 23.6 -> 19.8, 768 25.3 -> 26.0,
-//               1024 29.8 -> 30.5, 2560 46.2 -> 62.5;  n=4 C=2560: B=256 23.9 -> 17.8, 512 32.1 -> 27.7, 1280 42.4 -> 53.9
+//   n=4 C=1280: B=64 17.1 -> 9.2, 128 17.2 -> 9.7, 320 19.1 -> 14.9, 512 23.6 -> 19.0, 768 25.1 -> 24.3,
+//               1024 29.8 -> 29.6, 1536 35.7 -> 39.4, 2560 46.2 -> 62.5;  n=4 C=2048: B=768 33.5 -> 30.3, 1024 35.1 -> 41.2
+//   n=4 C=2560: B=256 23.9 -> 17.8, 512 32.0 -> 26.9, 768 36.3 -> 35.9, 1280 42.4 -> 53.9;  n=2 C=1280: B=1024 23.7 -> 28.8
 //   n=8 C=1280: B=128 25.1 -> 16.9, 256 30.5 -> 22.0, 512 46.1 -> 36.1, 1024 77.3 -> 62.7
 // Experiment hook: 1 = never, 2 = always.
 bool bwd_resident_preferred(int B, int n, int C) {
     if (const int hook = tuning_get(kTuneResident)) return hook == 2;
     (void)C;
-    return n > 4 || B <= 640;
+    return n > 4 || B <= 768;
 }
 
 // Shapes for which the dynamic entry points take fp32 activations that are consumed as bf16

@@ -325,8 +325,10 @@ hipError_t launch_proj_bwd_addx(const void *x, int x_dtype, const void *phi, con
     // Backward at B=320, C=1280, n=4, graphs of ten: 4 waves (three blocks) 16.5 us, 8 waves 16.0, 12 waves
     // (one block) 14.9; B=128: 9.5 / 9.9 with 4 / 8 waves; B=512: 19.7 / 19.0 / 19.5.  Wider projections
     // keep four waves: their registers allow two workgroups per CU only that way.
+    // More than 256 slabs: workgroups of four waves, of which three fit a CU, keep the grid in one round
+    // (B=1280, C=2560, n=4: 24.4 us with 4 waves, 31.7 with 12).
     int nw = 4;
-    if (NTD == 1) {
+    if (NTD == 1 && (nC + kAxKW - 1) / kAxKW <= 256) {
         int best = (B + 127) / 128;
         if ((B + 255) / 256 < best) { nw = 8; best = (B + 255) / 256; }
         if ((B + 383) / 384 < best) nw = 12;

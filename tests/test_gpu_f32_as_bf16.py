@@ -66,7 +66,7 @@ def _run(B, n, C, storage, inject, seed=0):
 
 
 SHAPES = [(5, 4, 64), (1, 4, 128), (3, 2, 40), (7, 1, 136), (33, 4, 1288), (320, 4, 1280), (16, 8, 256),
-          (3, 6, 72), (9, 8, 1288), (257, 8, 136), (640, 3, 64)]
+          (3, 6, 72), (9, 8, 1288), (257, 8, 136), (768, 3, 64)]
 
 
 @pytest.mark.parametrize("B,n,C", SHAPES)

@@ -182,7 +182,7 @@ def test_compute_dtype_bf16_on_float32_activations(B, n, C):
     x = torch.randn(B, n, C, device="cuda")
     dy = torch.randn(B, n, C, device="cuda")
     in_kernel = bool(lib.mhc_layer_dynamic_accepts_f32_as_bf16(B, n, C, T))
-    assert in_kernel == (n <= 8 and (n > 4 or B <= 640))
+    assert in_kernel == (n <= 8 and (n > 4 or B <= 768))
     y, g = _module_grads(layer, x, dy)
     assert y.dtype == torch.float32 and g["x"].dtype == torch.float32
     # the oracle on the rounded activations
