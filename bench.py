@@ -402,6 +402,24 @@ def stream_probe(torch):
                       "empty_kernel_us_per_launch": floor, "ceiling_GBs": {f"{k[0]}_{k[1]}MiB_{k[2]}": round(v["GB/s"], 1) for k, v in sorted(best.items())}}))
 
 
+def vendor_gemm(torch, reps=100):
+    """torch.matmul on P = x phi^T, dxflat = dP phi and dphi = dP^T x (bf16 operands and result) at the shapes of
+    the dynamic configurations; us per call, warm caches, HIP events."""
+    rows = []
+    for name in ("c2", "c3", "c4", "c5"):
+        B, n, C = (CONFIGS[name][k] for k in ("B", "n", "C"))
+        nC, D = n * C, n * n + 2 * n
+        x = torch.randn(B, nC, device="cuda", dtype=torch.bfloat16)
+        phi = torch.randn(D, nC, device="cuda", dtype=torch.bfloat16)
+        dP = torch.randn(B, D, device="cuda", dtype=torch.bfloat16)
+        rows.append({"config": name, "B": B, "n": n, "C": C,
+                     "P=x.phi^T_us": round(event_time_batched(torch, lambda: x @ phi.t(), reps), 1),
+                     "dxflat=dP.phi_us": round(event_time_batched(torch, lambda: dP @ phi, reps), 1),
+                     "dphi=dP^T.x_us": round(event_time_batched(torch, lambda: dP.t() @ x, reps), 1)})
+        print(rows[-1], file=sys.stderr, flush=True)
+    print(json.dumps({"vendor_gemm": True, "library": "torch.matmul (hipBLASLt / rocBLAS)", "dtype": "bf16", "rows": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -417,6 +435,14 @@ def main():
                     help="run the library's plain streaming kernels (read-only, copy, write-only; 16-byte accesses, "
                          "all CUs) over 128 MiB .. 2 GiB and print what this GPU delivers to each, HIP events on the "
                          "launch stream: the measured ceiling that the memory-bound kernels are compared with")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="time torch.matmul (the vendor BLAS) on the three projection products of every configuration: "
+                         "the reference point for the hand-written projection kernels, not part of the layer path")
+    ap.add_argument("--tuning", action="append", default=[], metavar="KEY=VALUE",
+                    help="run the step through the tuning build of the library (libmhc_hip_tuning.so, build.py --tuning) "
+                         "with one of its path-selection hooks set, e.g. 0=1 / 0=2 = two-launch / one-launch forward, "
+                         "7=1 / 7=2 = tiled / two-launch backward for n <= 8 (csrc/tuning.h lists the keys); the line "
+                         "then carries the setting and is not the library's default")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run a plain 64 MiB device copy instead of the layer (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
@@ -445,8 +471,19 @@ def main():
         print(json.dumps({"copy_calibration": True, "bytes_read": nbytes, "bytes_written": nbytes,
                           "copies": max(a.steps, 1)}))
         return
+    if a.vendor_gemm:
+        vendor_gemm(torch)
+        return
     cfg = CONFIGS[a.config]
-    step = Step(cfg, a.view, torch)
+    tuned = None
+    if a.tuning:
+        from mhc import _lib
+        tuned = _lib.tuning_lib()
+        for kv in a.tuning:
+            key, value = (int(t) for t in kv.split("="))
+            if tuned.mhc_tuning_set(key, value) != 0:
+                sys.exit(f"bench.py: the tuning build refused --tuning {kv}")
+    step = Step(cfg, a.view, torch, lib=tuned)
 
     # ---- warm-up, optional graph capture ---------------------------------------------------
     # A HIP graph replay costs ~5 us on top of its kernels (measured: c2 37.1 us per step with one
@@ -557,6 +594,8 @@ def main():
     # the three protocols side by side at top level: `value` above (warm, G steps per graph replay), one
     # step per replay (warm), and cold (one step per replay behind a 512 MiB fill)
     out["single_step_graph_us"] = dev_single
+    if a.tuning:
+        out["config"]["tuning"] = a.tuning
     out["cold_us"] = cold_step
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(step, torch)
