@@ -141,25 +141,23 @@ struct LayerFwdArgs {
     int KS, DP, w_bf16, B, n, C, T;
     float eps;
     float *sk_state;  // dynamic: [B][T + 1][2][NP] Sinkhorn denominators kept for the backward, or nullptr
-    int round_x;      // fp32 x (and f) consumed as bf16: round every value to bf16 as it is unpacked
 };
 
 // The values of a loaded chunk, widened to fp32; fp32 storage that is consumed as bf16 is rounded here
 // (nearest even), so that the mixing sees what the projection and the backward kernels see.
-template <typename T, int V>
-__device__ __forceinline__ void get_act(const RawVec<T, V> &r, float (&v)[V], int round_bf16) {
+template <bool ROUND, typename T, int V>
+__device__ __forceinline__ void get_act(const RawVec<T, V> &r, float (&v)[V]) {
     r.get(v);
-    if constexpr (std::is_same<T, float>::value) {
-        if (round_bf16) {
+    if constexpr (ROUND && std::is_same<T, float>::value) {
 #pragma unroll
-            for (int i = 0; i < V; i++) v[i] = bf16_to_f32(f32_to_bf16(v[i]));
-        }
+        for (int i = 0; i < V; i++) v[i] = bf16_to_f32(f32_to_bf16(v[i]));
     }
 }
 
 constexpr int kFwdStaggerMinB = 512;  // two or more workgroups per CU
 
-template <typename TX, typename TY, int NP, int V, int CPT>
+// RX: fp32 x (and f) consumed as bf16, every value rounded to bf16 as it is unpacked
+template <typename TX, typename TY, int NP, int V, int CPT, bool RX = false>
 __global__ __launch_bounds__(256, (CPT == 2 && NP == 4 && !std::is_same<TX, float>::value) ? 4 : 1)
 void layer_fwd_small_kernel(LayerFwdArgs a) {
     using SK = SkSmall<NP>;
@@ -320,10 +318,11 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             }
             // kept denominators: the fp32 tier divides, so that the backward call can undo the
             // scalings (m * s * rho) without a bias that grows with the iteration count
-            // (the same arithmetic with and without the state: the forward result does not depend on
-            // whether the caller keeps it)
+            // (the same arithmetic with and without the state: the dynamic forward result does not depend
+            // on whether the caller keeps it; static H has no state to undo and takes the reciprocals)
             if (dyn && a.sk_state) SK::template forward_save<!kFast>(m, g, n, a.T, a.eps, a.sk_state + (size_t)b * SK::state_floats(a.T));
-            else SK::template forward<!kFast, false>(m, g, n, a.T, a.eps, nullptr, tid);
+            else if (dyn) SK::template forward<!kFast, false>(m, g, n, a.T, a.eps, nullptr, tid);
+            else SK::template forward<false, false>(m, g, n, a.T, a.eps, nullptr, tid);
             coef_s[r0 * NP + c0] = m[0];
             if (wr && a.M && mv) a.M[ms + r0 * n + c0] = m[0];
         }
@@ -422,7 +421,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
             const int c = (ch < nch ? ch : 0) * V;
             float f[V];
             if (inject) {
-                get_act(fr[k], f, a.round_x);
+                get_act<RX>(fr[k], f);
             } else {
                 if (a.w_bf16) load_vec<bf16_t, V>(static_cast<const bf16_t *>(a.w) + c, f);
                 else load_vec<float, V>(static_cast<const float *>(a.w) + c, f);
@@ -494,7 +493,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
             for (int k = 0; k < CPT; k++)
 #pragma unroll
-                for (int i = 0; i < NP; i++) get_act(xr[k][i], xv[k][i], a.round_x);  // streams >= n meet zero coefficients
+                for (int i = 0; i < NP; i++) get_act<RX>(xr[k][i], xv[k][i]);  // streams >= n meet zero coefficients
         }
         float av[LEAN ? 1 : CPT][V];  // LEAN recomputes the aggregate in step 4 instead of keeping it
         float qinv = 1.0f;
@@ -509,7 +508,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
                 for (int i = 0; i < NP; i++) {
                     float t[V];
-                    if constexpr (LEAN) get_act(xr[k][i], t, a.round_x);
+                    if constexpr (LEAN) get_act<RX>(xr[k][i], t);
 #pragma unroll
                     for (int v = 0; v < V; v++) s_a[v] += hpre[i] * (LEAN ? t[v] : xv[LEAN ? 0 : k][i][v]);
                 }
@@ -536,7 +535,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
                 const int c = ch * V;
                 float f[V];
                 if (inject) {
-                    get_act(fr[k], f, a.round_x);
+                    get_act<RX>(fr[k], f);
                 } else {
                     if constexpr (LEAN) {
 #pragma unroll
@@ -544,7 +543,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
                         for (int i = 0; i < NP; i++) {
                             float t[V];
-                            get_act(xr[k][i], t, a.round_x);
+                            get_act<RX>(xr[k][i], t);
 #pragma unroll
                             for (int v = 0; v < V; v++) f[v] += hpre[i] * t[v];
                         }
@@ -564,7 +563,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 #pragma unroll
                         for (int j = 0; j < NP; j++) {
                             float t[V];
-                            if constexpr (LEAN) get_act(xr[k][j], t, a.round_x);
+                            if constexpr (LEAN) get_act<RX>(xr[k][j], t);
                             const float mij = LEAN ? coef_s[i * NP + j] : Mr[i][j];
 #pragma unroll
                             for (int v = 0; v < V; v++) out[v] += mij * (LEAN ? t[v] : xv[LEAN ? 0 : k][j][v]);
@@ -580,7 +579,7 @@ void layer_fwd_small_kernel(LayerFwdArgs a) {
 
 // Largest CPT instantiated: tiles with more than 4 * 256 vector chunks per stream take the
 // two-kernel path (coefficient kernel + streaming mix kernel).
-template <typename TX, typename TY, int NP>
+template <typename TX, typename TY, int NP, bool RX = false>
 static bool launch_fused_small(const LayerFwdArgs &a, hipStream_t stream, hipError_t *err) {
     constexpr int V = 16 / (int)sizeof(TX);
     if (a.C % V != 0) return false;
@@ -590,9 +589,9 @@ static bool launch_fused_small(const LayerFwdArgs &a, hipStream_t stream, hipErr
     // and the arithmetic on an aliased one (320 chunks on 2 x 256 slots would waste 37 % of both)
     const int per = cpt == 3 ? 4 : cpt;  // chunks per thread of the instantiation that runs
     const int nt = NP == 8 ? 256 : round_up((nch + per - 1) / per, kWave);
-    if (cpt == 1) layer_fwd_small_kernel<TX, TY, NP, V, 1><<<a.B, nt, 0, stream>>>(a);
-    else if (cpt == 2) layer_fwd_small_kernel<TX, TY, NP, V, 2><<<a.B, nt, 0, stream>>>(a);
-    else if (cpt <= 4 && NP == 4) layer_fwd_small_kernel<TX, TY, 4, V, 4><<<a.B, nt, 0, stream>>>(a);
+    if (cpt == 1) layer_fwd_small_kernel<TX, TY, NP, V, 1, RX><<<a.B, nt, 0, stream>>>(a);
+    else if (cpt == 2) layer_fwd_small_kernel<TX, TY, NP, V, 2, RX><<<a.B, nt, 0, stream>>>(a);
+    else if (cpt <= 4 && NP == 4) layer_fwd_small_kernel<TX, TY, 4, V, 4, RX><<<a.B, nt, 0, stream>>>(a);
     else return false;
     *err = hipGetLastError();
     return true;
@@ -613,13 +612,15 @@ hipError_t launch_layer_fwd_fused(const void *x, int x_dtype, const void *w, int
                                   float *Hpre, float *Hpost, float *M, float *P, float *r, float *q,
                                   float *sk_state, int B, int n, int C, int T, float eps, hipStream_t stream) {
     LayerFwdArgs a{x, w, f_inject, y, Ppart, ssqpart, alpha, b_pre, b_post, b_res, Hpre, Hpost, M, P, r, q,
-                   KS, DP, w_dtype == kBF16, B, n, C, T, eps, sk_state, x_dtype == kF32AsBF16};
-    if (x_dtype == kF32AsBF16) x_dtype = kF32;  // fp32 storage
+                   KS, DP, w_dtype == kBF16, B, n, C, T, eps, sk_state};
     hipError_t err = hipErrorInvalidValue;
     bool ok = false;
 #define MHC_FUSED(TX, TY)                                                        \
     ok = n <= 4 ? launch_fused_small<TX, TY, 4>(a, stream, &err) : launch_fused_small<TX, TY, 8>(a, stream, &err)
     if (x_dtype == kF32 && y_dtype == kF32) MHC_FUSED(float, float);
+    else if (x_dtype == kF32AsBF16 && y_dtype == kF32)  // fp32 storage, values rounded to bf16 on the way in
+        ok = n <= 4 ? launch_fused_small<float, float, 4, true>(a, stream, &err)
+                    : launch_fused_small<float, float, 8, true>(a, stream, &err);
     else if (x_dtype == kBF16 && y_dtype == kBF16) MHC_FUSED(bf16_t, bf16_t);
     else if (x_dtype == kBF16 && y_dtype == kF32) MHC_FUSED(bf16_t, float);
 #undef MHC_FUSED

@@ -40,10 +40,18 @@ static float *dev_f32(size_t n, float val) {
     return p;
 }
 
+static bool phase_slot_used(int kernel) {
+    std::vector<unsigned long long> t(8 * 8);
+    if (mhc_phase_read(kernel, t.data(), 8) != 0) return false;
+    return std::any_of(t.begin(), t.end(), [](unsigned long long v) { return v != 0; });
+}
+
 static void summary(const char *title, int kernel, int wgs, const std::vector<const char *> &names, bool stamps) {
     constexpr int M = 8;
     std::vector<unsigned long long> t((size_t)wgs * M);
     if (mhc_phase_read(kernel, t.data(), wgs) != 0) { printf("%s: read failed\n", title); return; }
+    // a kernel that the library did not launch for this shape left no stamps: no table
+    if (std::all_of(t.begin(), t.end(), [](unsigned long long v) { return v == 0; })) return;
     printf("\n%s (first %d workgroups of the grid, shader-clock ticks)\n", title, wgs);
     printf("%-34s %10s %10s %10s %7s\n", "phase", "mean", "p10", "p90", "share");
     const int np = (int)names.size();
@@ -125,13 +133,24 @@ int main(int argc, char **argv) {
                 {"start, first chunk requested", "waits for chunks, parks (all chunks)", "fragments, matrix cores (all chunks)",
                  "cross-wave sum, partial stores"}, false);
     }
-    summary("channel sums + coefficient backward kernel, one workgroup per sample", 4, std::min(B, 4096),
-            {"start: coefficient inputs, Sinkhorn state (wave 0)", "streaming loop (wave 0's steps)",
-             "workgroup sums", "coefficient backward (all of it: the three lines below)",
-             "  channel-sum vectors, dHpre / dHpost", "  Sinkhorn reverse sweep", "  dt / dP stores, alpha sums"}, false);
-    summary("sample-resident backward (--tune 7 2 only), first tile wave of each workgroup", 5, std::min(B, 4096),
-            {"loads requested", "tile arrives, Gram sums, slots written", "two barriers (workgroup sums between them)",
-             "dxp / u computed, stores issued"}, false);
+    // Which backward ran shows in the stamps: the tiled path leaves the slab (n <= 4) or the projection-backward
+    // table, the two-launch path neither.  Both use slots 4 and 5, for different kernels.
+    const bool tiled = phase_slot_used(n > 4 ? 2 : 1);
+    if (tiled) {
+        summary("channel sums + coefficient backward kernel, one workgroup per sample", 4, std::min(B, 4096),
+                {"start: coefficient inputs, Sinkhorn state (wave 0)", "streaming loop (wave 0's steps)",
+                 "workgroup sums", "coefficient backward (all of it: the three lines below)",
+                 "  channel-sum vectors, dHpre / dHpost", "  Sinkhorn reverse sweep", "  dt / dP stores, alpha sums"}, false);
+    } else {
+        summary("sample-resident backward kernel, one workgroup per sample: its coefficient wave (wave 0)", 4, std::min(B, 4096),
+                {"start: coefficient inputs, Sinkhorn state", "waits for the tile waves' Gram sums",
+                 "workgroup sums", "coefficient backward (all of it: the three lines below)",
+                 "  channel-sum vectors, dHpre / dHpost", "  Sinkhorn reverse sweep", "  dt / dP stores, alpha sums"}, false);
+        summary("sample-resident backward kernel: the first tile wave of each workgroup", 5, std::min(B, 4096),
+                {"loads requested", "tile arrives, Gram sums, slots written", "two barriers (workgroup sums between them)",
+                 "dxp / u computed, stores issued"}, false);
+        return 0;
+    }
     if (n > 4) {
         summary("dx kernel (generic, one wave per workgroup)", 5, std::min(B * ((C / 4 + 63) / 64), 4096),
                 {"start: coefficients and all loads requested", "data arrives, df / a / da", "mixing, dx stores issued", "dw / dt partial sums"}, false);
