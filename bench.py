@@ -82,6 +82,20 @@ def algorithmic_bytes(cfg, view):
     return fwd, bwd
 
 
+def kernels_changed_since(commit):
+    """True if the kernel sources differ from the revision a committed profile ran on, False if they do not,
+    None where that cannot be told (no git checkout, as on a box that only holds a copy of the tree)."""
+    import subprocess
+    if not os.path.isdir(os.path.join(ROOT, ".git")):
+        return None
+    try:
+        rc = subprocess.run(["git", "-C", ROOT, "diff", "--quiet", commit, "HEAD", "--", "mhc.cu_amd/csrc"],
+                            stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, timeout=20).returncode
+    except (OSError, subprocess.SubprocessError):
+        return None
+    return {0: False, 1: True}.get(rc)
+
+
 def dominant_kernel(config):
     """roofline.dominant: the step's largest kernel as profiled (not re-timed here: HIP events see whole
     entry points, not the launches inside them); `profiled_at` is the revision the profile ran on."""
@@ -89,6 +103,10 @@ def dominant_kernel(config):
     d["frac"] = d["bytes"] / (d["us"] * 1e-6) / 1e9 / HBM_PEAK_GBS
     d["source"] = f"profiles/layer_step_{config}.txt"
     d["profiled_at"] = PROFILED_AT
+    d["kernels_changed_since"] = kernels_changed_since(PROFILED_AT)
+    if d["kernels_changed_since"]:
+        print(f"bench.py: csrc/ has changed since {PROFILED_AT}, the revision roofline.dominant and roofline.traffic "
+              "were profiled at; regenerate profiles/ and the constants at the top of this file", file=sys.stderr)
     return d
 
 
