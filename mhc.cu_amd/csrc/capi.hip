@@ -62,7 +62,7 @@ int ws_check(void *ws, size_t have, size_t need) {
 
 // ---- dynamic workspace layout ----------------------------------------------------------------
 struct DynFwdWs { float *Ppart, *ssqpart, *agg; size_t bytes; };
-struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *raw, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
+struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *raw, *s1part, *dx_part, *dphi_part; unsigned short *dPb, *dPT; int BP; size_t bytes; };
 
 // Whether the sample-resident backward (bwd_resident.hip + the column-slab kernel without batch split)
 // is taken where it is supported.  Its second launch walks all samples of a column slab in one
@@ -105,6 +105,11 @@ DynFwdWs carve_dyn_fwd(void *ws, int B, int n, int C) {
     return w;
 }
 
+// Wide projections (n > 18) without batch split of dphi: four launches, see mhc_layer_bwd_dynamic.
+bool wide_dx_beside(int B, int n, int C) {
+    return proj_bwd_is_wide(n) && C % 8 == 0 && proj_bwd_batch_splits(B, n, C) == 1;
+}
+
 DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
     Carver c(ws);
     const int D = n * n + 2 * n, nC = n * C;
@@ -116,6 +121,9 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
     w.u = c.floats((size_t)B * C);
     w.dtpart = c.floats((size_t)B * (D + 3));
     w.raw = c.floats(bwd_reduce_raw_floats(B, n, C));
+    w.s1part = c.floats(n > 8 ? (size_t)B * bwd_reduce_parts(B, n, C) : 0);
+    // wide projections: the part of dx that is formed beside the coefficient backward, fp32
+    w.dx_part = c.floats(wide_dx_beside(B, n, C) ? (size_t)B * nC : 0);
     int bs = dphi_batch_splits(B, n, C);
     const int bs2 = proj_bwd_batch_splits(B, n, C);
     if (bs2 > bs) bs = bs2;
@@ -316,6 +324,26 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
         return MHC_OK;
     }
     if (x_dtype == kF32AsBF16) return MHC_ERR_BAD_DTYPE;  // not reached: accepted shapes take the path above
+    if (mfma && x_dtype == kBF16 && y_dtype == kBF16 && wide_dx_beside(B, n, C) && tuning_get(kTuneWideDxBeside) != 1) {
+        // wide projection (n > 18), four launches.  The coefficient backward is one workgroup per sample,
+        // all dependent chains; the part of dx that needs none of its results (M^T dy + Hpre (x) da,
+        // with s1 from the channel sums) runs beside it in the same launch and is handed over in fp32;
+        // the dP phi kernel then completes dx (+ dP phi - cx x, one rounding); dphi comes last and carries
+        // the batch sums.
+        // B=128 n=32 C=1280, backward in graphs of ten: five launches 98.5 us -> four
+        MHC_LAUNCH(launch_mix_bwd_reduce_with_dx(dy, x, w, w_dtype, f_inject, H_pre, H_post, M, n, q, P, r, alpha,
+                                                 bias + 2 * n, sk_state, out, ws.raw, ws.s1part, ws.dx_part, df, ws.u, B, n, C,
+                                                 iters, eps, st));
+        MHC_LAUNCH(launch_dxflat_wide(phi, ws.dPb, ws.BP, dx, x, ws.cx, ws.dx_part, B, n, C, st));
+        const BatchSumArgs sums = make_batch_sums(ws.u, B, C, f_inject ? nullptr : dw, ws.dt, B, D, dbias, dalpha);
+        bool tail_taken = false;
+        MHC_LAUNCH(launch_dphi_large(x, ws.dPT, ws.BP, dphi, 1, B, n, C,
+                                     tuning_get(kTuneSeparateFinalize) != 1 ? &sums : nullptr, &tail_taken, st));
+        if (!tail_taken)
+            MHC_LAUNCH(launch_finalize(ws.u, B, C, f_inject ? nullptr : dw, ws.dt, B, D, dbias, dalpha, nullptr, 1,
+                                       (size_t)D * n * C, dphi, st));
+        return MHC_OK;
+    }
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      n, q, P, r, alpha, bias + 2 * n, sk_state, out, ws.raw, B, n, C, iters, eps,
                                      st));
@@ -347,7 +375,7 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
         const int hook = tuning_get(kTuneProjApart);
         const bool apart = wide || (hook ? hook == 2 : proj_bwd_products_apart(n));
         if (apart) {
-            if (wide) MHC_LAUNCH(launch_dxflat_wide(phi, ws.dPb, ws.BP, dx, B, n, C, st));
+            if (wide) MHC_LAUNCH(launch_dxflat_wide(phi, ws.dPb, ws.BP, dx, nullptr, nullptr, nullptr, B, n, C, st));
             else MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st, kProjPartDx));
         } else {
             MHC_LAUNCH(launch_proj_bwd_mfma(x, phi, ws.dPb, ws.dPT, ws.BP, dphi, ws.dphi_part, dx, B, n, C, st));

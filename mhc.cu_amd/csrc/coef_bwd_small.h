@@ -17,6 +17,7 @@ struct BwdReduceArgs {
     float eps;
     float *raw;   // n <= 8: when set, write the raw channel sums [B][parts][K] and stop
     int parts;    // column parts per sample (gridDim.y)
+    float *s1part = nullptr;  // n > 8: when set, the Gram launch also writes s1 = Hpost^T W1 Hpre of every part, [B][parts]
 };
 
 // Where the weight of the W1 = dy diag(w) x^T Gram matrix comes from: an injected f [B, C] (W1 = dy [f; 0 ..]^T),

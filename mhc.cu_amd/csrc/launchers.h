@@ -120,6 +120,16 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
 // when given, the channel sums and the coefficient backward run as two launches.
 int bwd_reduce_parts(int B, int n, int C);
 size_t bwd_reduce_raw_floats(int B, int n, int C);  // size of `raw` (required for n > 8)
+// n > 16, dynamic H, bf16 dy and x: the same two launches, the second also holding the workgroups of
+// the matrix-core dx kernel in the form that needs no result of the coefficient backward
+// (dxp = M^T dy + Hpre (x) da into `dxp`, fp32 [B][n][C]; df or the dw rows u); they run beside the
+// coefficient workgroups, which are one per sample.  s1part: B * bwd_reduce_parts() floats of scratch.
+hipError_t launch_mix_bwd_reduce_with_dx(const void *dy, const void *x, const void *w, int w_dtype, const void *f_inject,
+                                         const float *Hpre, const float *Hpost, const float *M, int hstride,
+                                         const float *q, const float *P, const float *r, const float *alpha,
+                                         const float *b_res, const float *sk_state, BwdCoefOut out, float *raw,
+                                         float *s1part, float *dxp, void *df, float *u, int B, int n, int C, int T,
+                                         float eps, hipStream_t stream);
 
 // dx = M^T dy + Hpre (x) da - cx * x  [+ dP phi when phi != nullptr] [+ dx_in when != nullptr;
 // may alias dx], df, and u = df * a / q (the per-sample summand of dw).
@@ -195,8 +205,10 @@ bool proj_bwd_products_apart(int n);
 // Wide projections (more than 12 row tiles of 32, n > 18) always run the two products as two GEMM
 // kernels, launched through the two functions below; tail as above.
 bool proj_bwd_is_wide(int n);
-hipError_t launch_dxflat_wide(const void *phi, const void *dPb, int BP, void *dxflat, int B, int n, int C,
-                              hipStream_t stream);
+// x, cx, dx_part: all nullptr, or the inputs of the completion dxflat = dx_part + dP phi - cx x
+// (dx_part: fp32 [B][nC], the part of dx that an earlier launch left), rounded once.
+hipError_t launch_dxflat_wide(const void *phi, const void *dPb, int BP, void *dxflat, const void *x, const float *cx,
+                              const float *dx_part, int B, int n, int C, hipStream_t stream);
 hipError_t launch_dphi_large(const void *x, const void *dPT, int BP, float *dphi_out, int S, int B, int n,
                              int C, const BatchSumArgs *tail, bool *tail_taken, hipStream_t stream);
 

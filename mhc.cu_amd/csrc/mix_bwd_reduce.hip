@@ -15,6 +15,7 @@
 // n > 8 computes three 32x32 Gram matrices per sample on the matrix cores (operands loaded from
 // global memory in MFMA layout) from which all the sums above follow.
 #include "coef_bwd_small.h"
+#include "dx_large.h"
 #include "tuning.h"
 
 namespace mhc {
@@ -430,6 +431,21 @@ __global__ __launch_bounds__(256) void gram_large_kernel(BwdReduceArgs a) {
         const int c = c_begin + cc;
         w_s[cc] = (c < C && !inject) ? load_w_(a.w, a.w_bf16, c) : 0.f;
     }
+    // The part's s1 = Hpost^T W1 Hpre (wave 0, at the end): the coefficients that meet this lane's
+    // accumulator registers are requested now and used behind the streaming loop (aliased beyond n,
+    // masked where they are used).
+    const bool want_s1 = a.s1part != nullptr && !inject && wave == 0;
+    float hp_c = 0.f, ho_r[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) ho_r[i] = 0.f;
+    if (want_s1) {
+        hp_c = a.Hpre[(size_t)b * a.hstride + (row < n ? row : 0)];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int ri = 8 * (i >> 2) + 4 * kh + (i & 3);  // accumulator register i holds row ri
+            ho_r[i] = a.Hpost[(size_t)b * a.hstride + (ri < n ? ri : 0)];
+        }
+    }
     __syncthreads();
 
     // rows >= n alias row 0: they only produce Gram rows / columns that nobody reads
@@ -665,6 +681,7 @@ __global__ __launch_bounds__(256) void gram_large_kernel(BwdReduceArgs a) {
     __syncthreads();
     if (wave == 0) {
         float *out = a.raw + ((size_t)b * a.parts + part) * kGramFloats;
+        float s1 = 0.f;  // Hpost^T W1 Hpre of this part: this lane's column of W1 against Hpost
 #pragma unroll
         for (int m = 0; m < kGramMats; m++)
 #pragma unroll
@@ -673,15 +690,25 @@ __global__ __launch_bounds__(256) void gram_large_kernel(BwdReduceArgs a) {
 #pragma unroll
                 for (int w = 0; w < 3; w++) v += xw[((size_t)w * kGramMats * 16 + m * 16 + i) * 64 + lane];
                 // accumulator layout: column j = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4
-                out[m * 1024 + (8 * (i >> 2) + 4 * kh + (i & 3)) * 32 + row] = v;
+                const int ri = 8 * (i >> 2) + 4 * kh + (i & 3);
+                out[m * 1024 + ri * 32 + row] = v;
+                if (m == 1 && want_s1) s1 += (ri < n ? ho_r[i] : 0.f) * v;
             }
+        if (want_s1) {
+            s1 *= row < n ? hp_c : 0.f;  // rows and columns >= n hold aliased garbage
+            s1 = wave_allreduce_sum(s1);
+            if (lane == 0) a.s1part[(size_t)b * a.parts + part] = s1;
+        }
     }
 }
 
+// One workgroup (256 threads) of the coefficient launch for n > 8: sample b; smem = coef_bwd_large_lds_floats<NP>(T) floats.
+template <int NP>
+static size_t coef_bwd_large_lds_floats(int T) { return 3 * 32 * 33 + 64 + 96 + 4 + SkWg<NP>::lds_floats(T); }
+
 template <int NP, bool PRECISE>
-__global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
+__device__ __forceinline__ void coef_bwd_large_block(const BwdReduceArgs &a, const int b, float *smem) {
     using SK = SkWg<NP>;
-    extern __shared__ __align__(16) float smem[];
     float *W_s = smem;                   // [32][33]  W1 (or dy [f;0]^T)
     float *X_s = W_s + 32 * 33;          // [32][33]  XX
     float *M_s = X_s + 32 * 33;          // [32][33]  dM
@@ -690,7 +717,7 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
     float *vec_s = ho_s + 32;            // [3][32] dHpost | A1 | A2
     float *red_s = vec_s + 96;           // [4]
     float *sk_s = red_s + 4;             // SK::lds_floats(T)
-    const int b = blockIdx.x, n = a.n, C = a.C, tid = threadIdx.x, lane = tid & 63;
+    const int n = a.n, C = a.C, tid = threadIdx.x, lane = tid & 63;
     const bool w0 = tid < 64;
     const bool inject = a.f_inject != nullptr;
     MHC_PHASE(kPhaseCoefBwdWide, b, 0);
@@ -863,6 +890,23 @@ __global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
     MHC_PHASE(kPhaseCoefBwdWide, b, 5);
 }
 
+template <int NP, bool PRECISE>
+__global__ __launch_bounds__(256) void coef_bwd_large_kernel(BwdReduceArgs a) {
+    extern __shared__ __align__(16) float smem[];
+    coef_bwd_large_block<NP, PRECISE>(a, blockIdx.x, smem);
+}
+
+// The same launch with the workgroups of the n > 8 dx kernel behind the B coefficient workgroups.  The
+// coefficient workgroups are one per sample (half of the CUs at B = 128) and spend their time in
+// dependent chains; the dx workgroups given here need nothing that the coefficient workgroups produce
+// (d.s1part, no cx, no projection term) and run in their shadow on the rest of the chip.
+template <int NP, bool PRECISE>
+__global__ __launch_bounds__(256, 4) void coef_bwd_large_dx_kernel(BwdReduceArgs a, BwdDxArgs d) {
+    extern __shared__ __align__(16) float smem[];
+    if ((int)blockIdx.x < a.B) coef_bwd_large_block<NP, PRECISE>(a, blockIdx.x, smem);
+    else dx_large_block(d, blockIdx.x - a.B, reinterpret_cast<unsigned char *>(smem));
+}
+
 // =============================================================================================
 // launch
 // =============================================================================================
@@ -961,7 +1005,7 @@ static hipError_t launch_small_np(const BwdReduceArgs &a, hipStream_t stream) {
 }
 
 template <typename TG, typename TX>
-static hipError_t launch_large(const BwdReduceArgs &a, hipStream_t stream) {
+static hipError_t launch_large(const BwdReduceArgs &a, hipStream_t stream, const BwdDxArgs *shadow = nullptr) {
     constexpr bool kBf16 = std::is_same<TG, bf16_t>::value && std::is_same<TX, bf16_t>::value;
     constexpr int SW = kBf16 ? 16 : 8;
     const int nsteps = (a.C + SW - 1) / SW;
@@ -978,13 +1022,26 @@ static hipError_t launch_large(const BwdReduceArgs &a, hipStream_t stream) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     constexpr bool kPrecise = std::is_same<TX, float>::value;  // fp32 activations: the parity tier
+    if constexpr (kBf16) {
+        if (shadow) {
+            if (a.n <= 16) return hipErrorInvalidValue;
+            size_t smem2 = sizeof(float) * coef_bwd_large_lds_floats<32>(a.T);
+            if (smem2 < dx_large_lds_bytes()) smem2 = dx_large_lds_bytes();
+            e = allow_dynamic_lds(&coef_bwd_large_dx_kernel<32, false>, smem2);
+            if (e != hipSuccess) return e;
+            const unsigned ncb = (unsigned)((a.C + kDxlCB - 1) / kDxlCB);
+            coef_bwd_large_dx_kernel<32, false><<<(unsigned)a.B * (1u + ncb), 256, smem2, stream>>>(a, *shadow);
+            return hipGetLastError();
+        }
+    }
+    if (shadow) return hipErrorInvalidValue;
     if (a.n <= 16) {
-        const size_t smem2 = sizeof(float) * (3 * 32 * 33 + 64 + 96 + 4 + SkWg<16>::lds_floats(a.T));
+        const size_t smem2 = sizeof(float) * coef_bwd_large_lds_floats<16>(a.T);
         e = allow_dynamic_lds(&coef_bwd_large_kernel<16, kPrecise>, smem2);
         if (e != hipSuccess) return e;
         coef_bwd_large_kernel<16, kPrecise><<<a.B, 256, smem2, stream>>>(a);
     } else {
-        const size_t smem2 = sizeof(float) * (3 * 32 * 33 + 64 + 96 + 4 + SkWg<32>::lds_floats(a.T));
+        const size_t smem2 = sizeof(float) * coef_bwd_large_lds_floats<32>(a.T);
         e = allow_dynamic_lds(&coef_bwd_large_kernel<32, kPrecise>, smem2);
         if (e != hipSuccess) return e;
         coef_bwd_large_kernel<32, kPrecise><<<a.B, 256, smem2, stream>>>(a);
@@ -1038,6 +1095,25 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
     if (y_dtype == kBF16 && x_dtype == kBF16) return launch_large<bf16_t, bf16_t>(a, stream);
     if (y_dtype == kF32 && x_dtype == kBF16) return launch_large<float, bf16_t>(a, stream);
     return hipErrorInvalidValue;
+}
+
+// n > 16, dynamic H, bf16 dy and x: the channel sums, then ONE launch that holds the coefficient
+// workgroups and, behind them, the workgroups of the matrix-core dx kernel in the form that needs no
+// result of the coefficient backward: dxp = M^T dy + Hpre (x) da into `dxp` (fp32), df or the dw rows u.
+// s1part: [B][bwd_reduce_parts(B, n, C)] floats of scratch.
+hipError_t launch_mix_bwd_reduce_with_dx(const void *dy, const void *x, const void *w, int w_dtype, const void *f_inject,
+                                         const float *Hpre, const float *Hpost, const float *M, int hstride,
+                                         const float *q, const float *P, const float *r, const float *alpha,
+                                         const float *b_res, const float *sk_state, BwdCoefOut out, float *raw,
+                                         float *s1part, float *dxp, void *df, float *u, int B, int n, int C, int T,
+                                         float eps, hipStream_t stream) {
+    if (n <= 16 || raw == nullptr || s1part == nullptr || hstride == 0 || C % 8 != 0) return hipErrorInvalidValue;
+    const int parts = bwd_reduce_parts(B, n, C);
+    BwdReduceArgs a{dy, x, w, f_inject, Hpre, Hpost, M, q, P, r, alpha, b_res, sk_state, out,
+                    hstride, w_dtype == kBF16, B, n, C, T, padded_D(n), eps, raw, parts, s1part};
+    BwdDxArgs d{dy, x, w, f_inject, nullptr, nullptr, Hpre, Hpost, M, q, nullptr, nullptr, nullptr, nullptr, df, u,
+                nullptr, nullptr, hstride, w_dtype == kBF16, 0, B, n, C, padded_D(n), 1, s1part, parts, dxp};
+    return launch_large<bf16_t, bf16_t>(a, stream, &d);
 }
 
 }  // namespace mhc

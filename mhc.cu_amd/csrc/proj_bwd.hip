@@ -347,7 +347,7 @@ hipError_t launch_proj_bwd_mfma(const void *x, const void *phi, const void *dPb,
                             : part == kProjDx ? launch_what<1, 3, false, kProjDx>(a, 1, stream)
                                               : launch_what<1, 3, false, kProjDphi>(a, S, stream);
     else {
-        e = launch_dxflat_wide(phi, dPb, BP, dxflat, B, n, C, stream);
+        e = launch_dxflat_wide(phi, dPb, BP, dxflat, nullptr, nullptr, nullptr, B, n, C, stream);
         if (e == hipSuccess) e = launch_dphi_large(x, dPT, BP, S > 1 ? dphi_part : dphi, S, B, n, C, nullptr, nullptr, stream);
         (void)part;  // wide shapes: callers that want the products apart use the two launchers themselves
     }

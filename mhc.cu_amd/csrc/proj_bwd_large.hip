@@ -31,6 +31,8 @@ struct ProjBwdLargeArgs {
     int tpw;             // row tiles per workgroup of the single-block dphi kernel
     int tail_row;        // blockIdx.y of the extra row of workgroups that compute `tail` (-1: none)
     BatchSumArgs tail;   // batch sums carried by the dphi launch (see launch_dphi_large)
+    const float *cx = nullptr;     // dxflat kernel: when set, the output is dx = dx_part + dP phi - cx x
+    const float *dx_part = nullptr;  // fp32 [B][nC], the part of dx another launch has left (with cx)
 };
 
 // lane (n = lane & 31, kg = lane >> 5) gets tile[k0 + kg*8 + i][col0 + n], i = 0..7
@@ -197,11 +199,13 @@ __global__ __launch_bounds__(256) void dphi_large_kernel(ProjBwdLargeArgs a) {
 constexpr int kDxfCW = 64;            // columns per workgroup
 constexpr int kDxfLD = kDxfCW + 8;    // LDS row pitch (elements)
 constexpr int kDxfDC = 64;            // phi rows per chunk
+constexpr int kDxfLDF = kDxfCW + 4;   // LDS row pitch of the fp32 output tile of the completing form (elements)
 
 // MT = 32-sample tiles per wave: 2 (four waves) or 1 (eight waves; one wave's MFMAs run under
 // another's LDS reads on the same SIMD: 3 us faster at B=128 n=32 C=1280).
-template <int MT>
-__global__ __launch_bounds__(512 / MT) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
+// FIN: the completing form (a.cx, a.dx_part, a.x set).
+template <int MT, bool FIN>
+__global__ __launch_bounds__(512 / MT) __attribute__((amdgpu_waves_per_eu(6))) void dxflat_wide_kernel(ProjBwdLargeArgs a) {
     constexpr int NTHR = 512 / MT;
     constexpr int PH = 512 / NTHR;       // 16-byte pieces of a phi chunk per thread (64 rows x 8)
     constexpr int PSTEP = NTHR / 8;      // rows covered by one round of the workgroup's loads
@@ -276,6 +280,44 @@ __global__ __launch_bounds__(512 / MT) void dxflat_wide_kernel(ProjBwdLargeArgs 
         }
     };
 
+    // Completing dx (a.cx set): this thread's pieces of the partial dx (fp32, so that dx is rounded
+    // once) and of x are requested behind the loop, in front of the last chunk's products when the
+    // chunk count is odd, and arrive under those products and the accumulators' trip through LDS.  Pieces outside the tensor alias piece 0 and are not stored.
+    constexpr int NP_OUT = 1024 / NTHR;
+    constexpr bool finish = FIN;
+    RawVec<float, 8> din[NP_OUT];
+    RawVec<bf16_t, 8> xin[NP_OUT];
+    float cxv[NP_OUT];
+    // (tid_e: the thread index again, made opaque behind the loop, and everything the epilogue derives
+    // from it: addresses formed there hold no registers across the loop, which runs at the register
+    // count that keeps three workgroups on a CU)
+    int tid_e = 0, prow_e = 0, pseg_e = 0;
+    auto finish_off = [&](int h, bool &ok) {
+        const int bo = sg * 128 + prow_e + PSTEP * h;
+        ok = bo < a.B && k0 + pseg_e * 8 < a.nC;
+        return ok ? (size_t)bo * a.nC + k0 + pseg_e * 8 : (size_t)0;
+    };
+    auto issue_finish_x = [&]() {  // 5 registers per piece: fits beside the last chunk's slot
+        if constexpr (finish) {
+#pragma unroll
+            for (int h = 0; h < NP_OUT; h++) {
+                bool ok;
+                const size_t off = finish_off(h, ok);
+                xin[h].load(a.x + off);
+                cxv[h] = a.cx[ok ? sg * 128 + prow_e + PSTEP * h : 0];
+            }
+        }
+    };
+    auto issue_finish_part = [&]() {  // 8 registers per piece: once the FIFO is empty
+        if constexpr (finish) {
+#pragma unroll
+            for (int h = 0; h < NP_OUT; h++) {
+                bool ok;
+                din[h].load(a.dx_part + finish_off(h, ok));
+            }
+        }
+    };
+
     Slot s0, s1;
     issue(s0, 0);
     issue(s1, min(1, nchunks - 1));
@@ -287,36 +329,74 @@ __global__ __launch_bounds__(512 / MT) void dxflat_wide_kernel(ProjBwdLargeArgs 
         issue(s1, min(c + 3, nchunks - 1));
     }
     if (c < nchunks) compute(s0, 0, c);
+    tid_e = tid;
+    asm volatile("" : "+v"(tid_e) :: "memory");
+    prow_e = tid_e >> 3; pseg_e = tid_e & 7;
+    const int lane_e = tid_e & 63, wave_e = tid_e >> 6;
+    const int row_e = lane_e & 31, kg_e = lane_e >> 5, wm_e = wave_e >> 1, wn_e = wave_e & 1;
+    issue_finish_x();  // the FIFO is empty: its registers take the pieces
+    issue_finish_part();
     __syncthreads();  // all fragment reads done: the buffers become the output tile
 
     // accumulator layout: column = lane & 31, register i -> row 8*(i/4) + 4*(lane/32) + i%4.
+    if constexpr (finish) {
+        // the projection term stays fp32 until the one rounding of dx (the launch sizes the LDS for this tile)
+        float *o_s = reinterpret_cast<float *>(pl_lds);  // [128][kDxfLDF]
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                o_s[(size_t)((wm_e * MT + m) * 32 + 8 * (i >> 2) + 4 * kg_e + (i & 3)) * kDxfLDF + wn_e * 32 + row_e] = o[m][i];
+        __syncthreads();
+#pragma unroll
+        for (int h = 0; h < NP_OUT; h++) {
+            const int r = prow_e + PSTEP * h;
+            const int bo = sg * 128 + r;
+            if (bo < a.B && k0 + pseg_e * 8 < a.nC) {
+                const float4 p0 = *reinterpret_cast<const float4 *>(o_s + (size_t)r * kDxfLDF + pseg_e * 8);
+                const float4 p1 = *reinterpret_cast<const float4 *>(o_s + (size_t)r * kDxfLDF + pseg_e * 8 + 4);
+                float pv[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w}, dv[8], xv[8];
+                din[h].get(dv); xin[h].get(xv);
+#pragma unroll
+                for (int v = 0; v < 8; v++) pv[v] = dv[v] + pv[v] - cxv[h] * xv[v];
+                store_vec<bf16_t, 8, true>(a.dxflat + (size_t)bo * a.nC + k0 + pseg_e * 8, pv);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // one piece after the other: interleaved they need more registers than the loop
+        }
+        return;
+    }
     bf16_t *o_s = pl_lds;  // [128][kDxfLD]
 #pragma unroll
     for (int m = 0; m < MT; m++)
 #pragma unroll
         for (int i = 0; i < 16; i++)
-            o_s[(size_t)((wm * MT + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3)) * kDxfLD + wn * 32 + row] = f32_to_bf16(o[m][i]);
+            o_s[(size_t)((wm_e * MT + m) * 32 + 8 * (i >> 2) + 4 * kg_e + (i & 3)) * kDxfLD + wn_e * 32 + row_e] = f32_to_bf16(o[m][i]);
     __syncthreads();
 #pragma unroll
-    for (int h = 0; h < 1024 / NTHR; h++) {
-        const int r = prow + PSTEP * h;
+    for (int h = 0; h < NP_OUT; h++) {
+        const int r = prow_e + PSTEP * h;
         const int bo = sg * 128 + r;
-        if (bo < a.B && k0 + pseg * 8 < a.nC)
-            *reinterpret_cast<uint4 *>(a.dxflat + (size_t)bo * a.nC + k0 + pseg * 8) =
-                *reinterpret_cast<const uint4 *>(o_s + (size_t)r * kDxfLD + pseg * 8);
+        if (bo < a.B && k0 + pseg_e * 8 < a.nC)
+            *reinterpret_cast<uint4 *>(a.dxflat + (size_t)bo * a.nC + k0 + pseg_e * 8) =
+                *reinterpret_cast<const uint4 *>(o_s + (size_t)r * kDxfLD + pseg_e * 8);
     }
 }
 
 bool proj_bwd_is_wide(int n) { return padded_D(n) / 32 > 12; }
 
-hipError_t launch_dxflat_wide(const void *phi, const void *dPb, int BP, void *dxflat, int B, int n, int C,
-                              hipStream_t stream) {
+// x, cx, dx_part: all nullptr, or the inputs of the completion dxflat = dx_part + dP phi - cx x
+// (dx_part fp32 [B][nC]).
+hipError_t launch_dxflat_wide(const void *phi, const void *dPb, int BP, void *dxflat, const void *x, const float *cx,
+                              const float *dx_part, int B, int n, int C, hipStream_t stream) {
     const int nC = n * C, D = n * n + 2 * n, DP = padded_D(n);
-    ProjBwdLargeArgs a{nullptr, static_cast<const bf16_t *>(phi), static_cast<const bf16_t *>(dPb), nullptr,
-                       nullptr, static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, B, 0, -1, {}};
+    if ((x == nullptr) != (cx == nullptr) || (x == nullptr) != (dx_part == nullptr)) return hipErrorInvalidValue;
+    ProjBwdLargeArgs a{static_cast<const bf16_t *>(x), static_cast<const bf16_t *>(phi), static_cast<const bf16_t *>(dPb), nullptr,
+                       nullptr, static_cast<bf16_t *>(dxflat), B, BP, D, DP, nC, B, 0, -1, {}, cx, dx_part};
     // eight waves: 3 us faster than four at B=128 n=32 C=1280
-    dxflat_wide_kernel<1><<<dim3((nC + kDxfCW - 1) / kDxfCW, (B + 127) / 128), 512,
-                            sizeof(bf16_t) * 128 * kDxfLD, stream>>>(a);
+    const size_t lds = cx ? sizeof(float) * 128 * kDxfLDF : sizeof(bf16_t) * 128 * kDxfLD;
+    const dim3 grid((nC + kDxfCW - 1) / kDxfCW, (B + 127) / 128);
+    if (cx) dxflat_wide_kernel<1, true><<<grid, 512, lds, stream>>>(a);
+    else dxflat_wide_kernel<1, false><<<grid, 512, lds, stream>>>(a);
     return hipGetLastError();
 }
 

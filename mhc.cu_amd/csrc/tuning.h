@@ -16,7 +16,7 @@ enum TuneKey {
     kTuneProjApart = 5,     // n <= 18 projection backward: 1 = both products in one launch, 2 = two launches
     kTuneStaticSpg = 6,     // static backward: samples per workgroup of the dx kernel (n <= 8)
     kTuneResident = 7,      // n <= 8 sample-resident backward: 0 = by heuristic, 1 = never, 2 = whenever the shape allows
-    kTuneSpareA = 8,        // scratch knob for experiments in progress
+    kTuneWideDxBeside = 8,  // wide projections (n > 18): dx workgroups beside the coefficient launch: 1 = never, 2 = always
     kTuneSpareB = 9,
     kTuneCount = 10
 };

@@ -8,6 +8,10 @@ forced on the same inputs):
   tiled     channel sums, then the slab kernel (n <= 4) or projection backward + dx kernel, then the
             batch-sum launch
 
+The same is done for wide projections (n > 18), where the library runs the dx workgroups that need no
+result of the coefficient backward beside it in one launch and lets the dP phi kernel complete dx
+(four launches), against the five-launch order that the tuning build can still force.
+
 Tolerances: the bf16 tier of test_gpu_parity.py against the oracle (fp32 on the bf16-rounded inputs);
 between the paths the parameter gradients (exact bf16 products summed in fp32 on both sides) agree to
 2e-4 of their largest entry, dx to two bf16 roundings.
@@ -20,7 +24,7 @@ from oracle import naive_mhc as nm
 
 pytestmark = pytest.mark.gpu
 
-K_RESIDENT = 7
+K_RESIDENT, K_WIDE_DX_BESIDE = 7, 8
 T_ITERS, EPS = 20, 1e-6
 
 
@@ -58,12 +62,9 @@ SHAPES = [(5, 4, 64), (1, 4, 128), (3, 2, 40), (2, 3, 24), (7, 1, 136), (33, 4, 
           (130, 4, 2560), (16, 8, 256), (3, 6, 72), (9, 8, 1288), (70, 5, 1024), (257, 8, 136), (300, 7, 512)]
 
 
-@pytest.mark.parametrize("B,n,C", SHAPES)
-@pytest.mark.parametrize("inject", [False, True])
-@pytest.mark.parametrize("w_f32", [False, True])
-def test_resident_and_tiled_backward(B, n, C, inject, w_f32):
-    if inject and w_f32:
-        pytest.skip("w is unused with an injected f")
+def _both_paths(key, names, B, n, C, inject, w_f32):
+    """Backward of one step with tuning hook `key` at 1 and at 2 (names = what the two settings are called):
+    each against the oracle, then against each other."""
     st = _step(B, n, C, inject, w_f32)
     lib = st.lib
     h = st.host
@@ -78,15 +79,15 @@ def test_resident_and_tiled_backward(B, n, C, inject, w_f32):
     st.forward()
     got = {}
     try:
-        for mode, name in ((1, "tiled"), (2, "resident")):
-            assert lib.mhc_tuning_set(K_RESIDENT, mode) == 0
+        for mode, name in ((1, names[0]), (2, names[1])):
+            assert lib.mhc_tuning_set(key, mode) == 0
             for t in (st.dx, st.dphi, st.dbias, st.dalpha, st.dw) + ((st.df,) if st.df is not None else ()):
                 t.fill_(float("nan"))
             st.backward()
             torch.cuda.synchronize()
             got[name] = _grads(st)
     finally:
-        lib.mhc_tuning_set(K_RESIDENT, 0)
+        lib.mhc_tuning_set(key, 0)
     for name, g in got.items():
         for k, r in ref.items():
             assert torch.isfinite(g[k]).all(), f"{name}: {k} not finite"
@@ -97,7 +98,28 @@ def test_resident_and_tiled_backward(B, n, C, inject, w_f32):
             bad = (g[k].double() - r.double()).abs() > 2e-2 * r.double().abs() + 1e-2
             assert not bad.any(), f"{name}: {k} {int(bad.sum())} elements outside rtol/atol"
     for k in ("dphi", "dbias", "dalpha") + (() if inject else ("dw",)):
-        e = rel_err(got["resident"][k], got["tiled"][k])
-        assert e <= 2e-4, f"{k} resident vs tiled: {e:.3e}"
-    e = rel_err(got["resident"]["dx"], got["tiled"]["dx"])
-    assert e <= 1.6e-2, f"dx resident vs tiled: {e:.3e}"
+        e = rel_err(got[names[1]][k], got[names[0]][k])
+        assert e <= 2e-4, f"{k} {names[1]} vs {names[0]}: {e:.3e}"
+    e = rel_err(got[names[1]]["dx"], got[names[0]]["dx"])
+    assert e <= 1.6e-2, f"dx {names[1]} vs {names[0]}: {e:.3e}"
+
+
+@pytest.mark.parametrize("B,n,C", SHAPES)
+@pytest.mark.parametrize("inject", [False, True])
+@pytest.mark.parametrize("w_f32", [False, True])
+def test_resident_and_tiled_backward(B, n, C, inject, w_f32):
+    if inject and w_f32:
+        pytest.skip("w is unused with an injected f")
+    _both_paths(K_RESIDENT, ("tiled", "resident"), B, n, C, inject, w_f32)
+
+
+WIDE_SHAPES = [(128, 32, 1280), (5, 32, 64), (1, 19, 128), (130, 20, 136), (33, 27, 264), (260, 32, 8), (64, 24, 2056)]
+
+
+@pytest.mark.parametrize("B,n,C", WIDE_SHAPES)
+@pytest.mark.parametrize("inject", [False, True])
+@pytest.mark.parametrize("w_f32", [False, True])
+def test_wide_backward_dx_beside_the_coefficient_launch(B, n, C, inject, w_f32):
+    if inject and w_f32:
+        pytest.skip("w is unused with an injected f")
+    _both_paths(K_WIDE_DX_BESIDE, ("five launches", "four launches"), B, n, C, inject, w_f32)
