@@ -211,7 +211,6 @@ __global__ __launch_bounds__(512 / MT) __attribute__((amdgpu_waves_per_eu(6))) v
     constexpr int PSTEP = NTHR / 8;      // rows covered by one round of the workgroup's loads
     extern __shared__ bf16_t pl_lds[];  // [2][kDxfDC][kDxfLD]; later the [128][kDxfLD] output tile
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int row = lane & 31, kg = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
     const int k0 = blockIdx.x * kDxfCW;
     const int sg = blockIdx.y;                 // group of 128 samples
