@@ -330,7 +330,7 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
         // with s1 from the channel sums) runs beside it in the same launch and is handed over in fp32;
         // the dP phi kernel then completes dx (+ dP phi - cx x, one rounding); dphi comes last and carries
         // the batch sums.
-        // B=128 n=32 C=1280, backward in graphs of ten: five launches 98.5 us -> four
+        // B=128 n=32 C=1280, backward in graphs of ten, same box: five launches 99.8 us, these four 93.0 us
         MHC_LAUNCH(launch_mix_bwd_reduce_with_dx(dy, x, w, w_dtype, f_inject, H_pre, H_post, M, n, q, P, r, alpha,
                                                  bias + 2 * n, sk_state, out, ws.raw, ws.s1part, ws.dx_part, df, ws.u, B, n, C,
                                                  iters, eps, st));

@@ -15,7 +15,7 @@ namespace mhc {
 
 constexpr int kPhaseMaxWg = 4096;   // workgroups recorded per kernel (the first ones by linear id)
 constexpr int kPhaseMaxMarks = 8;   // stamps per workgroup
-enum PhaseKernel { kPhaseFwdFused = 0, kPhaseBwdSlab = 1, kPhaseProjBwd = 2, kPhaseProjFwd = 3, kPhaseGramSmall = 4, kPhaseDxSmall = 5, kPhaseFwdOnepass = 6, kPhaseCoefFwdWide = 7, kPhaseCoefBwdWide = 8, kPhaseKernels = 9 };
+enum PhaseKernel { kPhaseFwdFused = 0, kPhaseBwdSlab = 1, kPhaseProjBwd = 2, kPhaseProjFwd = 3, kPhaseGramSmall = 4, kPhaseDxSmall = 5, kPhaseFwdOnepass = 6, kPhaseCoefFwdWide = 7, kPhaseCoefBwdWide = 8, kPhaseColSlab = 9, kPhaseKernels = 10 };
 
 #ifdef MHC_PHASE_PROFILE
 extern __device__ unsigned long long g_phase[kPhaseKernels][kPhaseMaxWg][kPhaseMaxMarks];

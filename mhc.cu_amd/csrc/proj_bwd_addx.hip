@@ -23,6 +23,7 @@
 
 #include <type_traits>
 #include "mhc_common.h"
+#include "phase_profiler.h"
 
 namespace mhc {
 
@@ -45,7 +46,7 @@ struct ProjAddxArgs {
 constexpr int kAxKW = 32;          // slab width (columns)
 constexpr int kAxLD = kAxKW + 8;   // LDS pitch of the bf16 tiles (elements): rows stay 16-byte aligned
 constexpr int kAxLDO = kAxKW + 4;  // LDS pitch of the fp32 tile of dP phi
-constexpr int kAxLDR = 33;         // LDS pitch of the dphi tiles in the final cross-wave sum
+constexpr int kAxLDR = 36;         // LDS pitch of the dphi tiles in the final cross-wave sum (rows 16-byte aligned)
 
 // NTD: 32-row tiles of dphi (D <= 32 NTD).  SPW: samples a wave owns per block (32 or 64; a block is
 // 4 SPW samples).  PFOP: the dP operands of the next block are requested a block ahead like x and dxp.
@@ -81,6 +82,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void proj_bwd_addx_kernel
     if (k0 >= a.nC) return;  // ids of the padded grid; the whole workgroup, before any barrier
     const int row = lane & 31, kg = lane >> 5;
     const int D = a.D, nC = a.nC, B = a.B;
+    const int pwg = slab;
+    (void)pwg;
+    MHC_PHASE_ZERO(kPhaseColSlab, pwg);
+    MHC_PHASE_BEGIN(pclk);
 
     // ---- per-block loads: x for the LDS tile (thread -> chunks tid + 256 u) and, for the epilogue,
     // the chunks of dxp this thread completes: sample SPW wave + lane / 4 + 16 t, chunk lane % 4 ------
@@ -189,6 +194,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void proj_bwd_addx_kernel
     for (int m = 0; m < NTD; m++)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[m][i] = 0.f;
+    MHC_PHASE_ADD(kPhaseColSlab, pwg, 0, pclk);
 
     auto process_block = [&](int sb, auto slot) {
         constexpr int S = decltype(slot)::value;
@@ -213,6 +219,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void proj_bwd_addx_kernel
             *reinterpret_cast<uint4 *>(x_s + (size_t)(ch >> 2) * kAxLD + (ch & 3) * 8) = xb;
         }
         __syncthreads();
+        MHC_PHASE_ADD(kPhaseColSlab, pwg, 1, pclk);
         // ---- dphi: this wave's samples, every row tile ------------------------------------------------
         {
             bf16x8_t xf[KS];
@@ -243,6 +250,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void proj_bwd_addx_kernel
             for (int i = 0; i < 16; i++)
                 o_s[(size_t)(SPW * wave + 32 * t + 8 * (i >> 2) + 4 * kg + (i & 3)) * kAxLDO + row] = o[i];
         }
+        MHC_PHASE_ADD(kPhaseColSlab, pwg, 2, pclk);
         // ---- epilogue, row-major: the wave reads back only rows it wrote itself (its LDS accesses
         // complete in order), x from the block's tile ------------------------------------------------------
 #pragma unroll
@@ -268,6 +276,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void proj_bwd_addx_kernel
             load_block(sb + 2 * SBR, slot);
             if constexpr (PFOP) load_ops(sb + 2 * SBR, op);
         }
+        MHC_PHASE_ADD(kPhaseColSlab, pwg, 3, pclk);
     };
     for (int sb = 0; sb < B; sb += 2 * SBR) {
         process_block(sb, Slot0{});
@@ -282,13 +291,18 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void proj_bwd_addx_kernel
         for (int i = 0; i < 16; i++)
             red_s[((size_t)(wave * NTD + m) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3)) * kAxLDR + row] = acc[m][i];
     __syncthreads();
-    for (int e = tid; e < NTD * 32 * 32; e += NT_) {
-        const int d = e >> 5, c = e & 31;
-        float s = 0.f;
+    for (int e = tid; e < NTD * 32 * 8; e += NT_) {  // four columns per thread: 16-byte LDS reads and stores
+        const int d = e >> 3, c = (e & 7) * 4;
+        float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int w = 0; w < NW; w++) s += red_s[((size_t)w * NTD * 32 + d) * kAxLDR + c];
-        if (d < D && k0 + c < nC) a.dphi[(size_t)d * nC + k0 + c] = s;
+        for (int w = 0; w < NW; w++) {
+            const float4 v = *reinterpret_cast<const float4 *>(red_s + ((size_t)w * NTD * 32 + d) * kAxLDR + c);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        // nC % 8 == 0 and k0 % 32 == 0: a quad of columns is inside or outside
+        if (d < D && k0 + c < nC) *reinterpret_cast<float4 *>(a.dphi + (size_t)d * nC + k0 + c) = s;
     }
+    MHC_PHASE_ADD(kPhaseColSlab, pwg, 4, pclk);
 }
 
 bool proj_bwd_addx_supported(int n) { return padded_D(n) / 32 <= 3; }

@@ -149,6 +149,11 @@ int main(int argc, char **argv) {
         summary("sample-resident backward kernel: the first tile wave of each workgroup", 5, std::min(B, 4096),
                 {"loads requested", "tile arrives, Gram sums, slots written", "two barriers (workgroup sums between them)",
                  "dxp / u computed, stores issued"}, false);
+        summary("column-slab kernel, one workgroup per 32 columns of x_flat, all samples (wave 0 of each)", 9,
+                std::min((int)(nC / 32), 4096),
+                {"prologue: phi slab and the first two blocks requested, slab staged",
+                 "operands and x block arrive, block staged, barrier (all blocks)", "matrix cores: dphi and dP phi (all blocks)",
+                 "epilogue: dx completed and stored, next loads requested (all)", "dphi summed over the waves and stored"}, false);
         return 0;
     }
     if (n > 4) {
