@@ -77,15 +77,15 @@ template <> struct Act8<true> {
 // STATIC: shared coefficients ([n] / [n, n] instead of per sample).  There is no projection, so dxp is
 // the complete dx; wave 0 only turns the sums into the sample's row of raw coefficient gradients
 // (dM | dHpre | dHpost), whose batch sum feeds the one Sinkhorn backward of the static layer.
-template <int NP, int WMODE, int ITEMS, bool F32, bool STATIC = false>
-__global__ __launch_bounds__(STATIC ? 64 * kResTileWaves : kResThreads) void bwd_resident_kernel(BwdResidentArgs ra) {
+template <int NP, int WMODE, int ITEMS, bool F32, bool STATIC = false, int TWV = kResTileWaves>
+__global__ __launch_bounds__(64 * (TWV + (STATIC ? 0 : 1))) void bwd_resident_kernel(BwdResidentArgs ra) {
     using TS = typename std::conditional<F32, float, bf16_t>::type;  // storage type of the activations
     static_assert(NP == 4 || NP == 8, "stream groups of four");
     using SK = SkSmall<NP>;
     using CB = CoefBwdSmall<NP, false, true, STATIC>;
     constexpr int NB = NP / 4;            // stream groups
     constexpr int K = 3 * NP * NP;
-    constexpr int TW = kResTileWaves;
+    constexpr int TW = TWV;
     constexpr bool inject = WMODE == kGramInject;
     const BwdReduceArgs &a = ra.r;
     const int hs = STATIC ? 0 : a.n;      // sample stride of Hpre / Hpost (M: hs * n)
@@ -118,11 +118,15 @@ __global__ __launch_bounds__(STATIC ? 64 * kResTileWaves : kResThreads) void bwd
     }
     // the NP^2 threads that will hold the sums of W1 (one DPP row of wave 0 for 4x4, wave 1 for 8x8) ask
     // for their factor of s1 = Hpost^T W1 Hpre now, not behind the barrier
-    float hohp = 0.f;
+    // (the two factors stay as loaded until then: for 8x8 these threads are a tile wave, and a product
+    // here would make it wait for them in front of its tile loads)
+    float ho_l = 0.f, hp_l = 0.f;
+    bool hohp_ok = false;
     if (!inject && tid >= NP * NP && tid < 2 * NP * NP) {
         const int e = tid - NP * NP, r = e / NP, c = e % NP;
-        const float ho = a.Hpost[(size_t)b * hs + (r < n ? r : 0)], hp = a.Hpre[(size_t)b * hs + (c < n ? c : 0)];
-        hohp = (r < n && c < n) ? ho * hp : 0.f;
+        ho_l = a.Hpost[(size_t)b * hs + (r < n ? r : 0)];
+        hp_l = a.Hpre[(size_t)b * hs + (c < n ? c : 0)];
+        hohp_ok = r < n && c < n;
     }
     MHC_PHASE_ADD(kPhaseGramSmall, pwg, 0, pclk);
     const int blk = lane >> 2, i = lane & 3;
@@ -278,7 +282,7 @@ __global__ __launch_bounds__(STATIC ? 64 * kResTileWaves : kResThreads) void bwd
         for (int sl = 0; sl < TW * 4; sl++) v += slot_s[tid * (TW * 4) + sl];
         tot_s[tid] = v;
         if (!inject && tid >= NP * NP && tid < 2 * NP * NP) {
-            float t = hohp * v;
+            float t = hohp_ok ? ho_l * hp_l * v : 0.f;
             if constexpr (NP == 4) t = row16_allreduce(t);
             else t = wave_allreduce_sum(t);
             if (tid == NP * NP) tot_s[K] = t;
@@ -375,23 +379,37 @@ bool bwd_resident_supported(int x_dtype, int y_dtype, int phi_dtype, int n, int 
     return io && phi_dtype == kBF16 && n <= 8 && C % 8 == 0 && C <= 128 * kResTileWaves * kResMaxItems && T <= 32;
 }
 
-template <int NP, int WMODE, bool F32, bool STATIC = false>
-static hipError_t launch_items(const BwdResidentArgs &ra, hipStream_t stream) {
+template <int NP, int WMODE, bool F32, bool STATIC, int TW>
+static hipError_t launch_items_tw(const BwdResidentArgs &ra, hipStream_t stream) {
     using SK = SkSmall<NP>;
     using CB = CoefBwdSmall<NP, false, true, STATIC>;
     const size_t smem = sizeof(float) * ((STATIC ? 0 : SK::scaling_floats(ra.r.T)) + CB::kXch);
-    const int items = (ra.r.C + 128 * kResTileWaves - 1) / (128 * kResTileWaves);
+    const int items = (ra.r.C + 128 * TW - 1) / (128 * TW);
     const dim3 grid(ra.r.B);
-    const int threads = STATIC ? 64 * kResTileWaves : kResThreads;
+    const int threads = 64 * (TW + (STATIC ? 0 : 1));
+    constexpr int kMaxItems = TW == kResTileWaves ? kResMaxItems : 2;  // wider workgroups are for rows they hold in one or two items
     switch (items) {
-        case 1: bwd_resident_kernel<NP, WMODE, 1, F32, STATIC><<<grid, threads, smem, stream>>>(ra); break;
-        case 2: bwd_resident_kernel<NP, WMODE, 2, F32, STATIC><<<grid, threads, smem, stream>>>(ra); break;
-        case 3: bwd_resident_kernel<NP, WMODE, 3, F32, STATIC><<<grid, threads, smem, stream>>>(ra); break;
-        case 4: bwd_resident_kernel<NP, WMODE, 4, F32, STATIC><<<grid, threads, smem, stream>>>(ra); break;
-        case 5: bwd_resident_kernel<NP, WMODE, 5, F32, STATIC><<<grid, threads, smem, stream>>>(ra); break;
+        case 1: bwd_resident_kernel<NP, WMODE, 1, F32, STATIC, TW><<<grid, threads, smem, stream>>>(ra); break;
+        case 2: bwd_resident_kernel<NP, WMODE, 2, F32, STATIC, TW><<<grid, threads, smem, stream>>>(ra); break;
+        case 3: if constexpr (kMaxItems >= 3) { bwd_resident_kernel<NP, WMODE, 3, F32, STATIC, TW><<<grid, threads, smem, stream>>>(ra); break; } return hipErrorInvalidValue;
+        case 4: if constexpr (kMaxItems >= 4) { bwd_resident_kernel<NP, WMODE, 4, F32, STATIC, TW><<<grid, threads, smem, stream>>>(ra); break; } return hipErrorInvalidValue;
+        case 5: if constexpr (kMaxItems >= 5) { bwd_resident_kernel<NP, WMODE, 5, F32, STATIC, TW><<<grid, threads, smem, stream>>>(ra); break; } return hipErrorInvalidValue;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
+}
+
+template <int NP, int WMODE, bool F32, bool STATIC = false>
+static hipError_t launch_items(const BwdResidentArgs &ra, hipStream_t stream) {
+    // Eight streams, rows of at most 1280 channels: ten tile waves hold the row in one item each
+    // instead of four in three - the Gram and mixing products of an 8 x 8 sample are most of such a
+    // workgroup's life, and one wave per SIMD has nobody to overlap them with.  Backward at B=256,
+    // C=1280, n=8, graphs of ten: 4 tile waves 21.3 us, 5 21.8, 8 21.4, 10 20.8 (n=4, B=320: 15.1 / 14.9 /
+    // 15.9 / 15.0: four stay).
+    if constexpr (NP == 8 && !F32 && !STATIC) {
+        if (ra.r.C <= 1280) return launch_items_tw<NP, WMODE, F32, STATIC, 10>(ra, stream);
+    }
+    return launch_items_tw<NP, WMODE, F32, STATIC, kResTileWaves>(ra, stream);
 }
 
 hipError_t launch_bwd_resident(const void *dy, const void *x, int x_dtype, const void *w, int w_dtype, const void *f_inject,
