@@ -58,7 +58,7 @@ def _grads(st):
     return out
 
 
-SHAPES = [(5, 4, 64), (1, 4, 128), (3, 2, 40), (2, 3, 24), (7, 1, 136), (33, 4, 1288), (320, 4, 1280),
+SHAPES = [(5, 4, 64), (1, 4, 128), (3, 2, 40), (2, 3, 24), (7, 1, 136), (33, 4, 1288), (320, 4, 1280), (9, 4, 640),
           (130, 4, 2560), (16, 8, 256), (3, 6, 72), (9, 8, 1288), (70, 5, 1024), (257, 8, 136), (300, 7, 512)]
 
 
