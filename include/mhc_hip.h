@@ -90,9 +90,9 @@ MHC_API int mhc_max_sinkhorn_iters(int n);
 
 /*
  * 1 when the two dynamic-H entry points below take x_dtype = MHC_F32_AS_BF16 for this shape (the
- * kernels that load fp32 storage directly serve n <= 8 and the batch sizes for which the two-launch
- * backward is taken), else 0: the caller then rounds x to bf16 itself, as the reference does
- * (src/python/bindings.cu:421-423).
+ * kernels that load fp32 storage directly serve n <= 8, C % 8 == 0, C <= 2560 and up to 32 Sinkhorn
+ * iterations, at every batch size), else 0: the caller then rounds x to bf16 itself, as the reference
+ * does (src/python/bindings.cu:421-423).
  */
 MHC_API int mhc_layer_dynamic_accepts_f32_as_bf16(int B, int n, int C, int iters);
 

@@ -81,12 +81,13 @@ bool bwd_resident_preferred(int B, int n, int C) {
 
 // Shapes for which the dynamic entry points take fp32 activations that are consumed as bf16
 // (MHC_F32_AS_BF16): the kernels that load fp32 storage directly are the narrow projection, the fused
-// n <= 8 forward and the two launches of the sample-resident backward, where that backward is the
-// path of choice.
+// n <= 8 forward and the two launches of the sample-resident backward.  That backward is taken for fp32
+// storage at every batch size, also where the tiled path is faster on bf16 storage: the alternative is
+// a cast pass over x on top of the tiled path (through the module, fp32 tensors, forward + backward:
+// B=1280 C=2560 n=4 186 -> 184 us, B=2560 C=1280 184 -> 176, B=1024 C=1280 111 -> 100).
 bool f32_as_bf16_accepted(int B, int n, int C, int iters) {
     return n <= 8 && layer_fwd_fused_supported(n, C, kF32) &&
-           bwd_resident_supported(kF32AsBF16, kF32, kBF16, n, C, iters) && proj_bwd_addx_supported(n) &&
-           bwd_resident_preferred(B, n, C);
+           bwd_resident_supported(kF32AsBF16, kF32, kBF16, n, C, iters) && proj_bwd_addx_supported(n);
 }
 
 int max_ksplit(int B, int n, int C) {
@@ -305,7 +306,7 @@ int mhc_layer_bwd_dynamic(const void *dy, int y_dtype, const void *x, int x_dtyp
     const bool mfma = proj_bwd_mfma_supported(x_dtype == kF32AsBF16 ? kBF16 : x_dtype, phi_dtype, C);
     BwdCoefOut out{ws.dt, ws.dP, ws.cx, ws.s1, nullptr, mfma ? ws.dPb : nullptr, ws.dPT, ws.BP};
     if (mfma && bwd_resident_supported(x_dtype, y_dtype, phi_dtype, n, C, iters) && proj_bwd_addx_supported(n) &&
-        bwd_resident_preferred(B, n, C)) {
+        (bwd_resident_preferred(B, n, C) || x_dtype == kF32AsBF16)) {
         // two launches: (1) one workgroup per sample keeps the sample's rows of dy and x in registers for
         // the channel sums, the coefficient backward and the mixing part of dx; (2) a column-slab
         // kernel over all samples adds dP phi - cx x, finishes dphi without batch-split partial sums

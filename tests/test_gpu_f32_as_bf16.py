@@ -1,5 +1,5 @@
 """MHC_F32_AS_BF16 through the C ABI: fp32 activations that the kernels round to bf16 as they load
-them (dynamic H, n <= 8, batch sizes of the two-launch backward), against the oracle on the rounded
+them (dynamic H, n <= 8, rows that the sample-resident backward holds), against the oracle on the rounded
 activations at the bf16 tolerance, and against the same entry points fed bf16 storage.  Shapes the
 library does not take in this form are refused with MHC_ERR_BAD_DTYPE before any launch."""
 import pytest
@@ -66,7 +66,7 @@ def _run(B, n, C, storage, inject, seed=0):
 
 
 SHAPES = [(5, 4, 64), (1, 4, 128), (3, 2, 40), (7, 1, 136), (33, 4, 1288), (320, 4, 1280), (16, 8, 256),
-          (3, 6, 72), (9, 8, 1288), (257, 8, 136), (768, 3, 64)]
+          (3, 6, 72), (9, 8, 1288), (257, 8, 136), (768, 3, 64), (2000, 4, 64), (1100, 4, 1280)]
 
 
 @pytest.mark.parametrize("B,n,C", SHAPES)
@@ -101,7 +101,7 @@ def test_f32_storage_consumed_as_bf16(B, n, C, inject):
         assert rel_err(got[k], ref16[k]) <= 1.6e-2, k
 
 
-@pytest.mark.parametrize("B,n,C", [(2000, 4, 64), (8, 12, 64), (8, 4, 8192), (8, 4, 36)])
+@pytest.mark.parametrize("B,n,C", [(8, 12, 64), (8, 4, 8192), (8, 4, 36)])
 def test_shapes_without_an_fp32_storage_path_are_refused(B, n, C):
     from mhc._lib import lib
 

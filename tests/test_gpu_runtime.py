@@ -162,8 +162,7 @@ def _module_grads(layer, x, dy):
 def test_compute_dtype_bf16_on_float32_activations(B, n, C):
     """MHCLayer(compute_dtype=bfloat16) on float32 activations - the reference's default contract (float32 in
     and out around a bf16 kernel path, ops.py:129,404, bindings.cu:421-423).  Where the kernels load
-    float32 storage themselves (n <= 8, small batch) no cast runs; elsewhere (large batch, n > 8) the
-    operator casts.  Either way the results stay float32 and agree with the oracle on the bf16-rounded
+    float32 storage themselves (n <= 8) no cast runs; elsewhere (n > 8) the operator casts.  Either way the results stay float32 and agree with the oracle on the bf16-rounded
     activations at the bf16 tolerance, and with the same layer fed the bf16-rounded activations."""
     from helpers import rel_err
     from mhc import MHCLayer
@@ -182,7 +181,7 @@ def test_compute_dtype_bf16_on_float32_activations(B, n, C):
     x = torch.randn(B, n, C, device="cuda")
     dy = torch.randn(B, n, C, device="cuda")
     in_kernel = bool(lib.mhc_layer_dynamic_accepts_f32_as_bf16(B, n, C, T))
-    assert in_kernel == (n <= 8 and (n > 4 or B <= 768))
+    assert in_kernel == (n <= 8)
     y, g = _module_grads(layer, x, dy)
     assert y.dtype == torch.float32 and g["x"].dtype == torch.float32
     # the oracle on the rounded activations
