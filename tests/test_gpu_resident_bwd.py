@@ -113,7 +113,8 @@ def test_resident_and_tiled_backward(B, n, C, inject, w_f32):
     _both_paths(K_RESIDENT, ("tiled", "resident"), B, n, C, inject, w_f32)
 
 
-WIDE_SHAPES = [(128, 32, 1280), (5, 32, 64), (1, 19, 128), (130, 20, 136), (33, 27, 264), (260, 32, 8), (64, 24, 2056)]
+WIDE_SHAPES = [(128, 32, 1280), (5, 32, 64), (1, 19, 128), (130, 20, 136), (33, 27, 264), (260, 32, 8), (64, 24, 2056),
+               (3000, 20, 8)]
 
 
 @pytest.mark.parametrize("B,n,C", WIDE_SHAPES)
