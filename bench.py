@@ -445,6 +445,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--shape", default=None, metavar="B,n,C",
+                    help="a dynamic-H bf16 forward+backward step of another shape than the named configurations "
+                         "(for the tables behind the library's path choices); the line then carries no profiled "
+                         "constants (roofline.traffic, roofline.dominant)")
     ap.add_argument("--view", default="L", choices=["L", "K"])
     ap.add_argument("--mode", default="graph", choices=["graph", "eager"])
     ap.add_argument("--graph-steps", type=int, default=10,
@@ -494,6 +498,10 @@ def main():
         vendor_gemm(torch)
         return
     cfg = CONFIGS[a.config]
+    if a.shape:
+        B_, n_, C_ = (int(t) for t in a.shape.split(","))
+        cfg = dict(kind="dynamic", B=B_, n=n_, C=C_, dtype="bf16", bwd=True)
+        a.config = f"shape {a.shape}"
     tuned = None
     if a.tuning:
         from mhc import _lib
@@ -600,7 +608,7 @@ def main():
                      "traffic_profiled_at": MEASURED_TRAFFIC["commit"],
                      # the same step with a 512 MiB fill before every one (nothing served from the caches)
                      "cold_us": cold_step, "cold_frac": alg / (cold_step * 1e-6) / 1e9 / HBM_PEAK_GBS,
-                     "dominant": dominant_kernel(a.config),
+                     "dominant": dominant_kernel(a.config) if a.config in CONFIGS else None,
                      "kernel": "whole step (all launches of one forward+backward)",
                      "algorithmic_bytes": alg, "device_us": dev_step, "single_step_graph_us": dev_single,
                      "fwd": {"algorithmic_bytes": fwd_b, "device_us": dev_fwd,
