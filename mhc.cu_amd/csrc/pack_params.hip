@@ -20,18 +20,20 @@ struct PackArgs {
     size_t total;
 };
 
+// Small parameters (biases, alphas): workgroup 0 of either kernel below.
+__device__ __forceinline__ void pack_small(const PackArgs &a, int t) {
+    if (t < 3) a.alpha[t] = a.alpha_in[t][0];
+    for (int i = t; i < a.bn[0] + a.bn[1] + a.bn[2]; i += 256) {
+        const int g = i < a.bn[0] ? 0 : (i < a.bn[0] + a.bn[1] ? 1 : 2);
+        const int off = g == 0 ? 0 : (g == 1 ? a.bn[0] : a.bn[0] + a.bn[1]);
+        a.bias[i] = a.b[g][i - off];
+    }
+}
+
 template <typename TS, typename TD, int V>
 __global__ __launch_bounds__(256) void pack_params_kernel(PackArgs a) {
     const size_t e0 = ((size_t)blockIdx.x * 256 + threadIdx.x) * V;
-    if (blockIdx.x == 0) {
-        const int t = threadIdx.x;
-        if (t < 3) a.alpha[t] = a.alpha_in[t][0];
-        for (int i = t; i < a.bn[0] + a.bn[1] + a.bn[2]; i += 256) {
-            const int g = i < a.bn[0] ? 0 : (i < a.bn[0] + a.bn[1] ? 1 : 2);
-            const int off = g == 0 ? 0 : (g == 1 ? a.bn[0] : a.bn[0] + a.bn[1]);
-            a.bias[i] = a.b[g][i - off];
-        }
-    }
+    if (blockIdx.x == 0) pack_small(a, threadIdx.x);
     if (e0 >= a.total) return;
     // V > 1 only when every source length is a multiple of V: a chunk never straddles two sources
     const int g = e0 < a.end[0] ? 0 : (e0 < a.end[1] ? 1 : 2);
@@ -41,6 +43,37 @@ __global__ __launch_bounds__(256) void pack_params_kernel(PackArgs a) {
     float v[V];
     load_vec<TS, V>(src, v);
     store_vec<TD, V>(dst, v);
+}
+
+// float32 parameters into a bfloat16 phi, the case of a training step (master weights in fp32, 6 bytes
+// moved per element: 267 MB for n = 32, C = 1280).  A lane takes four elements per chunk (a 16-byte
+// load, an 8-byte store, both contiguous across the wave), a thread keeps kPackU chunks in flight and
+// the grid is a few thousand workgroups that stride over the array; the sources are read once and
+// bypass the caches (nontemporal loads), phi stays cached for the projection kernel that follows.
+constexpr int kPackU = 8;
+__global__ __launch_bounds__(256) void pack_params_stream_kernel(PackArgs a) {
+    if (blockIdx.x == 0) pack_small(a, threadIdx.x);
+    const size_t chunks = a.total / 4;  // every source length is a multiple of 4
+    const size_t per_round = (size_t)gridDim.x * kPackU * 256;
+    for (size_t c0 = (size_t)blockIdx.x * kPackU * 256 + threadIdx.x; c0 < chunks; c0 += per_round) {
+        uint4 v[kPackU];
+#pragma unroll
+        for (int u = 0; u < kPackU; u++) {
+            const size_t c = c0 + (size_t)u * 256;
+            const size_t e = (c < chunks ? c : 0) * 4;
+            const int g = e < a.end[0] ? 0 : (e < a.end[1] ? 1 : 2);
+            const size_t base = g == 0 ? 0 : a.end[g - 1];
+            v[u] = ldg16_stream(reinterpret_cast<const uint4 *>(static_cast<const float *>(a.src[g]) + (e - base)));
+        }
+#pragma unroll
+        for (int u = 0; u < kPackU; u++) {
+            const size_t c = c0 + (size_t)u * 256;
+            if (c < chunks)
+                st8<false>(static_cast<bf16_t *>(a.phi_out) + c * 4,
+                           pack_bf16x2(__uint_as_float(v[u].x), __uint_as_float(v[u].y)),
+                           pack_bf16x2(__uint_as_float(v[u].z), __uint_as_float(v[u].w)));
+        }
+    }
 }
 
 hipError_t launch_pack_params(const void *phi_pre, const void *phi_post, const void *phi_res, int src_dtype,
@@ -58,6 +91,13 @@ hipError_t launch_pack_params(const void *phi_pre, const void *phi_post, const v
     a.alpha_in[0] = alpha_pre; a.alpha_in[1] = alpha_post; a.alpha_in[2] = alpha_res;
     a.phi_out = phi_out; a.bias = bias; a.alpha = alpha; a.total = end;
     auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    // the streaming kernel: fp32 -> bf16, whole 16-byte chunks in every source, enough of them to matter
+    if (src_dtype == kF32 && out_dtype == kBF16 && (n * nC) % 4 == 0 && al16(phi_pre) && al16(phi_post) &&
+        al16(phi_res) && (reinterpret_cast<uintptr_t>(phi_out) & 7u) == 0 && end >= (size_t)1 << 20) {
+        const size_t rounds = (end / 4 + (size_t)kPackU * 256 - 1) / ((size_t)kPackU * 256);
+        pack_params_stream_kernel<<<(unsigned)(rounds < 2048 ? rounds : 2048), 256, 0, stream>>>(a);
+        return hipGetLastError();
+    }
     const bool vec = (n * nC) % 8 == 0 && al16(phi_pre) && al16(phi_post) && al16(phi_res) && al16(phi_out);
     const int V = vec ? 8 : 1;
     const size_t chunks = (end + V - 1) / V;

@@ -187,9 +187,9 @@ def test_compute_dtype_bf16_on_float32_activations(B, n, C):
     # the oracle on the rounded activations
     p = {k: v.detach().float().cpu() for k, v in layer.named_parameters()}
     p["w"] = p.pop("rmsnorm_weight")
-    # (the incoming gradient is an activation too: where the kernels take float32 storage they round it
-    # like x; the cast path hands it to kernels that keep it as it is)
-    dy_seen = dy.bfloat16().float() if in_kernel else dy
+    # (the incoming gradient is an activation too: the kernels that take float32 storage round it like x,
+    # and the cast path rounds it with a cast of its own before the backward call)
+    dy_seen = dy.bfloat16().float()
     y_ref, g_ref = nm.mhc_dynamic_fwd_bwd(x.bfloat16().float().cpu(), p, dy_seen.cpu(), T, eps, dtype=torch.float32)
     g_ref["rmsnorm_weight"] = g_ref.pop("w")
 
@@ -209,3 +209,35 @@ def test_compute_dtype_bf16_on_float32_activations(B, n, C):
     assert rel_err(y, y2) <= 1e-2
     for k in g:
         assert rel_err(g[k], g2[k]) <= 2e-2, k
+
+
+@pytest.mark.parametrize("n,C,src,dst", [
+    (4, 64, torch.float32, torch.bfloat16),      # small: one chunk per thread
+    (3, 20, torch.float32, torch.bfloat16),      # lengths that are no multiple of 8: element-wise kernel
+    (16, 520, torch.float32, torch.bfloat16),    # 2.4 M elements: the streaming kernel, ragged last round
+    (32, 1280, torch.float32, torch.bfloat16),   # the largest benchmark shape (44.6 M elements)
+    (16, 520, torch.float32, torch.float32),
+    (16, 520, torch.bfloat16, torch.bfloat16),
+])
+def test_parameter_gather_is_the_rounded_concatenation(n, C, src, dst):
+    """mhc_pack_dynamic_params: phi is the row concatenation [pre | post | res] converted once (round to
+    nearest even for bfloat16), the biases and alphas are copied; every element, bit for bit."""
+    from mhc import _lib
+
+    g = torch.Generator().manual_seed(5)
+    nC, D = n * C, n * n + 2 * n
+    parts = [torch.randn(r, nC, generator=g).to(src).cuda() for r in (n, n, n * n)]
+    bs = [torch.randn(k, generator=g).cuda() for k in (n, n, n * n)]
+    al = [torch.randn(1, generator=g).cuda() for _ in range(3)]
+    phi = torch.full((D, nC), float("nan"), dtype=dst, device="cuda")
+    bias = torch.empty(D, device="cuda")
+    alpha = torch.empty(3, device="cuda")
+    p = lambda t: t.data_ptr()
+    _lib.check("mhc_pack_dynamic_params", _lib.lib.mhc_pack_dynamic_params(
+        p(parts[0]), p(parts[1]), p(parts[2]), _lib.dtype_code(parts[0]), p(bs[0]), p(bs[1]), p(bs[2]),
+        p(al[0]), p(al[1]), p(al[2]), p(phi), _lib.dtype_code(phi), p(bias), p(alpha), n, C,
+        torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.equal(phi, torch.cat(parts).to(dst))
+    assert torch.equal(bias, torch.cat(bs))
+    assert torch.equal(alpha, torch.cat(al))
