@@ -20,17 +20,19 @@ struct BatchSumArgs {
 
 inline BatchSumArgs make_batch_sums(const float *u, int rows_u, int C, float *dw, const float *dt, int rows_dt,
                                     int D, float *dbias, float *dalpha) {
-    const int ncols = (dw ? C : 0) + D + 3;
+    const int ncols = (dw ? C : 0) + (dt ? D + 3 : 0);  // dt == nullptr: the u columns only
     return BatchSumArgs{u, rows_u, C, dw, dt, rows_dt, D, dbias, dalpha, (ncols + 63) / 64};
 }
 
-// red: RG * 65 doubles of LDS; called by all 64 * RG threads of the workgroup (contains a barrier)
-template <int RG>
+// red: RG * (CW + 1) doubles of LDS; called by all CW * RG threads of the workgroup (contains a barrier).
+// CW = columns per block: 64, or 32 (still whole 128-byte lines per row) where twice the blocks are
+// wanted; a.nblk must count blocks of CW columns.
+template <int RG, int CW = 64>
 __device__ __forceinline__ void batch_sum_block(const BatchSumArgs &a, int blk, int tid, double *red) {
-    const int cl = tid & 63, rg = tid >> 6;
-    const int col = blk * 64 + cl;
+    const int cl = tid % CW, rg = tid / CW;
+    const int col = blk * CW + cl;
     const int ncol_u = a.dw ? a.C : 0;
-    const int ncols = ncol_u + a.D + 3;
+    const int ncols = ncol_u + (a.dt ? a.D + 3 : 0);
     double acc = 0.0;
     if (col < ncols) {
         const bool is_u = col < ncol_u;
@@ -57,12 +59,12 @@ __device__ __forceinline__ void batch_sum_block(const BatchSumArgs &a, int blk, 
         for (; r < rows; r += RG) a0 += (double)src[(size_t)r * ld];
         acc = (a0 + a1) + (a2 + a3);
     }
-    red[rg * 65 + cl] = acc;
+    red[rg * (CW + 1) + cl] = acc;
     __syncthreads();
     if (rg == 0 && col < ncols) {
         double v = 0.0;
 #pragma unroll
-        for (int i = 0; i < RG; i++) v += red[i * 65 + cl];
+        for (int i = 0; i < RG; i++) v += red[i * (CW + 1) + cl];
         if (col < ncol_u) a.dw[col] = (float)v;
         else if (col - ncol_u < a.D) a.dbias[col - ncol_u] = (float)v;
         else a.dalpha[col - ncol_u - a.D] = (float)v;

@@ -490,7 +490,6 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
     const StaBwdWs ws = carve_sta_bwd(workspace, B, n, C);
     if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int D = n * n + 2 * n;
     BwdCoefOut out{nullptr, nullptr, nullptr, ws.s1, ws.red, nullptr, nullptr, 0};
     if (bwd_resident_supported(x_dtype, y_dtype, kBF16, n, C, 0) && tuning_get(kTuneResident) != 1) {
         // bf16 activations, n <= 8: with shared coefficients nothing of dx depends on a batch-wide
@@ -498,10 +497,8 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
         // the channel sums, the sample's raw coefficient gradients and the complete dx
         MHC_LAUNCH(launch_bwd_resident_static(dy, x, w, w_dtype, f_inject, H_pre, H_post, M, q, out, dx, df, ws.u,
                                               B, n, C, st));
-        MHC_LAUNCH(launch_finalize(ws.u, B, C, f_inject ? nullptr : dw, ws.red, B, D, ws.red_sum, ws.red_sum + D,
-                                   nullptr, 1, 0, nullptr, st));
-        MHC_LAUNCH(launch_coef_bwd_static(ws.red_sum, H_pre, H_post, H_res_logits, dH_pre, dH_post,
-                                          dH_res, n, iters, eps, st));
+        MHC_LAUNCH(launch_finalize_static(ws.u, B, C, f_inject ? nullptr : dw, ws.red, B, ws.red_sum, H_pre, H_post,
+                                          H_res_logits, dH_pre, dH_post, dH_res, n, iters, eps, st));
         return MHC_OK;
     }
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
@@ -516,12 +513,10 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
     MHC_LAUNCH(launch_mix_bwd_dx(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M, 0,
                                  q, ws.s1, nullptr, nullptr, 0, nullptr, 0, nullptr, dx, df, ws.u, nullptr,
                                  nullptr, spg, B, n, C, st));
-    // one launch for both batch sums: dw = sum_b u, red_sum = sum_b red (its 3 padding columns land
-    // in red_sum[D..D+2] and are ignored)
-    MHC_LAUNCH(launch_finalize(ws.u, groups, C, f_inject ? nullptr : dw, ws.red, B, D, ws.red_sum, ws.red_sum + D,
-                               nullptr, 1, 0, nullptr, st));
-    MHC_LAUNCH(launch_coef_bwd_static(ws.red_sum, H_pre, H_post, H_res_logits, dH_pre, dH_post,
-                                      dH_res, n, iters, eps, st));
+    // the batch sums (dw = sum_b u, sum_b red) and the coefficient backward on them: one launch for
+    // n <= 8, two beyond
+    MHC_LAUNCH(launch_finalize_static(ws.u, groups, C, f_inject ? nullptr : dw, ws.red, B, ws.red_sum, H_pre, H_post,
+                                      H_res_logits, dH_pre, dH_post, dH_res, n, iters, eps, st));
     return MHC_OK;
 }
 

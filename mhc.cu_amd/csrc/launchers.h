@@ -230,6 +230,10 @@ hipError_t launch_colsum_split(const float *in, int rows, int cols, int ld, floa
 hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const float *Hpost,
                                   const float *H_res_logits, float *dH_pre, float *dH_post,
                                   float *dH_res, int n, int T, float eps, hipStream_t stream);
+hipError_t launch_finalize_static(const float *u, int rows_u, int C, float *dw, const float *red, int rows,
+                                  float *red_sum, const float *Hpre, const float *Hpost,
+                                  const float *H_res_logits, float *dH_pre, float *dH_post, float *dH_res, int n,
+                                  int T, float eps, hipStream_t stream);
 
 // phi [D, nC] (out_dtype) = rows [pre | post | res] of the three parameter matrices (src_dtype),
 // bias [D] and alpha [3] likewise, in one launch.

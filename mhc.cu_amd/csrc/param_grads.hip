@@ -275,4 +275,109 @@ hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const
     return hipGetLastError();
 }
 
+// n <= 8: the batch sums of the static backward and the coefficient backward on them in ONE launch.
+//   blocks [0, nblk_u): dw = column sums of u, 32 columns each (none with an injected f)
+//   last block: the D columns of `red` (per-sample raw gradients dM | dHpre | dHpost, row pitch D + 3)
+//       summed over the batch in float64 by waves 1 .. 15 while wave 0 recomputes the Sinkhorn forward;
+//       wave 0 then runs the sigmoid derivatives and the exact Sinkhorn backward on the sums, which
+//       never leave the workgroup.
+struct FinalizeStaticArgs {
+    BatchSumArgs sums;  // u -> dw only
+    const float *red; int rows, n, T; float eps;
+    const float *Hpre, *Hpost, *H_res_logits;
+    float *dH_pre, *dH_post, *dH_res;
+};
+
+template <int NP>
+__global__ __launch_bounds__(1024) void finalize_static_kernel(FinalizeStaticArgs a) {
+    using SK = SkSmall<NP>;
+    __shared__ double red[32 * 33];
+    __shared__ float sum_s[128];
+    extern __shared__ float sc[];  // SK::scaling_floats(T)
+    const int tid = threadIdx.x;
+    if ((int)blockIdx.x < a.sums.nblk) {
+        batch_sum_block<32, 32>(a.sums, blockIdx.x, tid, red);
+        return;
+    }
+    const int n = a.n, D = n * n + 2 * n, ld = D + 3;
+    // Wave 0 recomputes the Sinkhorn forward (the denominators that its backward needs) from the logits,
+    // which needs none of the sums, while waves 1 .. 15 sum the columns of `red`.
+    const int lane = tid & 63, g = lane % SK::kGroup;
+    const bool first = lane < SK::kGroup;  // a 4 x 4 matrix takes 16 lanes: the other groups compute copies
+    const int r0 = SK::row(g), c0 = SK::col0(g);
+    const bool ok = r0 < n && c0 < n;
+    float m[1] = {0.f};
+    if (tid < 64) {
+        m[0] = ok ? expf(a.H_res_logits[r0 * n + c0]) : 0.f;
+        SK::template forward<true>(m, g, n, a.T, a.eps, sc, lane);
+    } else {
+        // `red` as one flat array: thread t of the 960 takes element t of every pass of RP whole rows, so a
+        // pass is one contiguous piece of memory and a thread stays on its column
+        const int t = tid - 64, RP = 896 / ld;  // ld <= 83: at least 10 rows per pass
+        if (t < RP * ld) {
+            const float *src = a.red + t;
+            const size_t step = (size_t)RP * ld;
+            const int rs = t / ld;
+            double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
+            int r = rs;
+            for (; r + 15 * RP < a.rows; r += 16 * RP, src += 16 * step) {  // sixteen loads in flight
+                float v[16];
+#pragma unroll
+                for (int k = 0; k < 16; k++) v[k] = src[k * step];
+#pragma unroll
+                for (int k = 0; k < 16; k += 4) {
+                    a0 += (double)v[k]; a1 += (double)v[k + 1]; a2 += (double)v[k + 2]; a3 += (double)v[k + 3];
+                }
+            }
+            for (; r < a.rows; r += RP, src += step) a0 += (double)*src;
+            red[t] = (a0 + a1) + (a2 + a3);  // [row slot][column]
+        }
+    }
+    __syncthreads();
+    if (tid >= 64 && tid < 64 + D) {
+        const int RP = 896 / ld;
+        double v = 0.0;
+        for (int i = 0; i < RP; i++) v += red[i * ld + tid - 64];
+        sum_s[tid - 64] = (float)v;
+    }
+    __syncthreads();
+    if (tid >= 64) return;  // the chain below is one wave's (no barrier follows)
+    if (first && g < n) {
+        const float hp = a.Hpre[g], ho = a.Hpost[g];
+        a.dH_pre[g] = sum_s[n * n + g] * hp * (1.0f - hp);
+        a.dH_post[g] = sum_s[n * n + n + g] * ho * (1.0f - 0.5f * ho);
+    }
+    float d[1] = {ok ? sum_s[r0 * n + c0] : 0.f};
+    SK::template backward<true>(d, m, a.T, sc, lane);
+    if (first && ok) a.dH_res[r0 * n + c0] = d[0];  // gradient of the logits
+}
+
+// Batch sums + coefficient backward of the static path.  n <= 8: one launch (above); wider matrices: the
+// finalize launch writes the sums to red_sum [D + 3] and the workgroup-wide Sinkhorn kernel follows.
+hipError_t launch_finalize_static(const float *u, int rows_u, int C, float *dw, const float *red, int rows,
+                                  float *red_sum, const float *Hpre, const float *Hpost,
+                                  const float *H_res_logits, float *dH_pre, float *dH_post, float *dH_res, int n,
+                                  int T, float eps, hipStream_t stream) {
+    const int D = n * n + 2 * n;
+    if (n > 8) {
+        if (hipError_t e = launch_finalize(u, rows_u, C, dw, red, rows, D, red_sum, red_sum + D, nullptr, 1, 0,
+                                           nullptr, stream); e != hipSuccess)
+            return e;
+        return launch_coef_bwd_static(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps, stream);
+    }
+    FinalizeStaticArgs a{make_batch_sums(u, rows_u, C, dw, nullptr, 0, 0, nullptr, nullptr), red, rows, n, T, eps,
+                         Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res};
+    a.sums.nblk = dw ? (C + 31) / 32 : 0;  // blocks of 32 columns
+    if (n <= 4) {
+        const size_t smem = sizeof(float) * SkSmall<4>::scaling_floats(T);
+        if (hipError_t e = allow_dynamic_lds(&finalize_static_kernel<4>, smem); e != hipSuccess) return e;
+        finalize_static_kernel<4><<<a.sums.nblk + 1, 1024, smem, stream>>>(a);
+    } else {
+        const size_t smem = sizeof(float) * SkSmall<8>::scaling_floats(T);
+        if (hipError_t e = allow_dynamic_lds(&finalize_static_kernel<8>, smem); e != hipSuccess) return e;
+        finalize_static_kernel<8><<<a.sums.nblk + 1, 1024, smem, stream>>>(a);
+    }
+    return hipGetLastError();
+}
+
 }  // namespace mhc

@@ -261,11 +261,13 @@ struct MHCDynamicFn : public torch::autograd::Function<MHCDynamicFn> {
         c10::DeviceGuard guard(x.device());
         const int iters = (int)ctx->saved_data["iters"].toInt();
         const double eps = ctx->saved_data["eps"].toDouble();
-        Tensor dy = act(grads[0]);
         // bfloat16 activations with a float32 result hand back a float32 gradient: it is rounded to the
         // activations' format here, so that the backward runs the kernels that take both in 2 bytes (the
-        // mixed pair goes through slower general kernels: 111 against 20 us for dx at B=128 n=32 C=1280)
-        if (x.scalar_type() == at::kBFloat16 && dy.scalar_type() == at::kFloat) dy = dy.to(at::kBFloat16);
+        // mixed pair goes through slower general kernels: 111 against 20 us for dx at B=128 n=32 C=1280).
+        // One pass also when the gradient arrives as a broadcast view (the backward of a sum).
+        const bool round_dy = x.scalar_type() == at::kBFloat16 && grads[0].scalar_type() == at::kFloat;
+        Tensor dy = act(round_dy ? grads[0].to(grads[0].options().dtype(at::kBFloat16), false, false, at::MemoryFormat::Contiguous)
+                                 : grads[0]);
         const auto fo = x.options().dtype(at::kFloat);
         Tensor dx = at::empty_like(x);
         Tensor df = f.defined() ? at::empty_like(f) : Tensor();
@@ -346,11 +348,13 @@ struct MHCStaticFn : public torch::autograd::Function<MHCStaticFn> {
                      &small = saved[6];
         const int B = x.size(0), n = x.size(1), C = x.size(2);
         c10::DeviceGuard guard(x.device());
-        Tensor dy = act(grads[0]);
         // bfloat16 activations with a float32 result hand back a float32 gradient: it is rounded to the
         // activations' format here, so that the backward runs the kernels that take both in 2 bytes (the
-        // mixed pair goes through slower general kernels: 111 against 20 us for dx at B=128 n=32 C=1280)
-        if (x.scalar_type() == at::kBFloat16 && dy.scalar_type() == at::kFloat) dy = dy.to(at::kBFloat16);
+        // mixed pair goes through slower general kernels: 111 against 20 us for dx at B=128 n=32 C=1280).
+        // One pass also when the gradient arrives as a broadcast view (the backward of a sum).
+        const bool round_dy = x.scalar_type() == at::kBFloat16 && grads[0].scalar_type() == at::kFloat;
+        Tensor dy = act(round_dy ? grads[0].to(grads[0].options().dtype(at::kBFloat16), false, false, at::MemoryFormat::Contiguous)
+                                 : grads[0]);
         const auto fo = x.options().dtype(at::kFloat);
         Tensor dx = at::empty_like(x);
         Tensor df = f.defined() ? at::empty_like(f) : Tensor();
