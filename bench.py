@@ -345,6 +345,43 @@ def cpu_baseline(step, torch, budget_s=20.0):
                       f"fp32 naive PyTorch layer, median"}
 
 
+def box_rates(torch):
+    """What this box's memory does for plain hand-written kernels (libmhc_probe.so): one 256 MiB buffer read
+    and one written, cold, median of 5.  Boxes of the pool differ by 10-20 % in the write rate, which
+    moves the write-bound kernels (the 178 MB of dphi at n = 32) by as much; the figures let two bench
+    lines from different boxes be compared.  None when the probe library is not built."""
+    path = os.path.join(ROOT, "mhc.cu_amd", "mhc", "libmhc_probe.so")
+    if not os.path.exists(path):
+        return None
+    fn = ctypes.CDLL(path).mhc_stream_probe
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
+                   ctypes.c_void_p]
+    nbytes = 256 * 1024 * 1024
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    flush = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda")
+    src = torch.empty(nbytes // 4, dtype=torch.int32, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+    for mode, name in ((0, "read_GBs"), (2, "write_GBs")):
+        times = []
+        for it in range(7):
+            flush.fill_(1.0)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            if fn(mode, src.data_ptr(), dst.data_ptr(), nbytes, 16384, sink.data_ptr(), stream) != 0:
+                return None
+            e1.record()
+            e1.synchronize()
+            if it >= 2:
+                times.append(e0.elapsed_time(e1) * 1e-3)
+        times.sort()
+        out[name] = round(nbytes / times[len(times) // 2] / 1e9, 1)
+    out["protocol"] = "256 MiB, 16-byte nontemporal accesses, 16384 workgroups, cold (512 MiB fill before each), median of 5"
+    return out
+
+
 def stream_probe(torch):
     """Read-only / copy / write-only streaming rates of hand-written kernels and the cost of an empty launch
     (csrc/stream_probe.hip, built into its own libmhc_probe.so)."""
@@ -624,6 +661,7 @@ def main():
     if a.tuning:
         out["config"]["tuning"] = a.tuning
     out["cold_us"] = cold_step
+    out["box"] = box_rates(torch)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(step, torch)
     print(json.dumps(out))

@@ -84,3 +84,5 @@ def test_bench_prints_one_json_line_with_the_agreed_keys():
     for k in ("value", "unit", "cores", "kind", "sample"):
         assert k in cb, k
     assert cb["kind"] == "port" and cb["cores"] >= 1
+    # the box's own read and write rates, for comparing lines from different boxes (None without the probe library)
+    assert d["box"] is None or (1000 < d["box"]["write_GBs"] < 8000 and 1000 < d["box"]["read_GBs"] < 8000)
