@@ -318,6 +318,13 @@ def test_configs_2_to_5_bf16_full_size(B, n, C, inject):
     _check(y, y_ref, "bf16", "y")
     for k, ref in g_ref.items():
         _check(g[k], ref, "bf16", "d" + k)
+    # The float32 gradients of this tier are float32 sums of products of the rounded inputs (the
+    # coefficient gradients enter the matrix cores as bf16 value + remainder): they sit at a few 1e-6 of
+    # the oracle, far inside the tier's tolerance, and a dropped low-order term would show here.
+    for k in ("phi_pre", "phi_post", "phi_res", "b_pre", "b_post", "b_res"):
+        if k in g_ref:
+            e = rel_err(torch.as_tensor(g[k]).double(), torch.as_tensor(g_ref[k]).double())
+            assert e <= 1e-4, f"d{k}: rel err {e:.3e} > 1e-4"
 
 
 def test_config2_fp32_full_size():
