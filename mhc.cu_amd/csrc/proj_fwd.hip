@@ -15,6 +15,7 @@
 #include <type_traits>
 #include "mhc_common.h"
 #include "phase_profiler.h"
+#include "tuning.h"
 
 namespace mhc {
 
@@ -483,16 +484,26 @@ int proj_fwd_ksplit(int x_dtype, int phi_dtype, int B, int n, int C) {
     if (!use_mfma(x_dtype, phi_dtype, C)) return 1;
     const int nC = n * C, DP = padded_D(n);
     if (use_wide(n, C)) {
-        // ~1.6 workgroups per CU; a slab is at least 8 chunks; the partial sums (written here, read
-        // by the coefficient kernel) stay below ~0.3 of the bytes streamed
+        // Workgroups = (64-row groups) x (128-sample tiles) x splits.  The chip has 256 CUs and a workgroup
+        // (8 waves) loads one: the count that fills every CU once, or twice where that still keeps the
+        // splits within the 24 that the coefficient kernel sums in one round of loads, beats the counts in
+        // between, which leave some CUs with twice the work of others
+        // (forward us, B n C: 128 32 1280  15 splits 41.8 | 24: 43.0 | 30: 44.2 | 16: 48.7;
+        //  256 32 1280  15: 62.1 | 12: 66.2 | 7: 67.5;  512 12 512  16: 28.1 | 3: 35.8).
         const int wgs = ((DP + 63) / 64) * ((B + 127) / 128);
-        int ks = (410 + wgs / 2) / wgs;
-        const int cap_chunks = nC / 64 / 8;
-        const int cap_bytes = (int)(0.28 * (2.0 * B * nC + 2.0 * DP * nC) / (8.0 * B * DP));
+        int ks = 512 / wgs <= 24 ? 512 / wgs : 256 / wgs;
+        if (ks > 24) ks = 24;
+        const int cap_chunks = nC / 64 / 8;  // a slab is at least 8 chunks
         if (ks > cap_chunks) ks = cap_chunks;
-        if (ks > cap_bytes) ks = cap_bytes;
-        if (ks > 64) ks = 64;
+        // the partial sums (written here, read by the coefficient kernel) stay below the bytes streamed,
+        // unless that would leave half the CUs without a workgroup
+        const int cap_bytes = (int)((2.0 * B * nC + 2.0 * DP * nC) / (8.0 * B * DP));
+        if (ks > cap_bytes) {
+            const int half_chip = (128 + wgs - 1) / wgs;
+            ks = cap_bytes > (ks < half_chip ? ks : half_chip) ? cap_bytes : (ks < half_chip ? ks : half_chip);
+        }
         if (ks < 1) ks = 1;
+        if (const int forced = tuning_get(kTuneSpareB); forced > 0) ks = forced;  // experiment hook
         return ks;
     }
     const int tiles_s = (B + 31) / 32;
