@@ -1052,11 +1052,14 @@ static hipError_t launch_large(const BwdReduceArgs &a, hipStream_t stream, const
 // Column parts per sample when the channel sums are a launch of their own.
 int bwd_reduce_parts(int B, int n, int C) {
     if (n > 8) {
-        // ~512 workgroups, at least ~128 columns per part
+        // ~512 workgroups, at least ~128 columns per part, at most four parts: the coefficient launch
+        // sums the parts of a sample at the head of its chain, and more of them cost it more than the
+        // channel-sum kernel gains (backward us, n=32 C=1280: B=64  4 parts 86.3 | 8: 88.6;
+        // B=128  4: 92.3 | 6: 99.9; B=32  4: 83.6 | 10: 84.3)
         int parts = (512 + B - 1) / B;
         const int cap = C / 128 > 0 ? C / 128 : 1;
         if (parts > cap) parts = cap;
-        if (parts > 16) parts = 16;
+        if (parts > 4) parts = 4;
         if (parts < 1) parts = 1;
         return parts;
     }
