@@ -521,6 +521,7 @@ int proj_fwd_ksplit(int x_dtype, int phi_dtype, int B, int n, int C) {
     if (n <= 8 && ks > fused_cap) ks = fused_cap;
     if (ks > 64) ks = 64;
     if (ks < 1) ks = 1;
+    if (const int forced = tuning_get(kTuneSpareB); forced > 0) ks = forced;  // experiment hook
     // a wave's share is whole 64-element chunks (launch_mfma): with that share fixed, only as many
     // splits as have work (B=1280 n=4 C=2560: 16 splits of 4 x 192 elements would leave the last two
     // and a half empty; 14 do the same work and the forward sums two partial rows fewer per sample)

@@ -17,7 +17,7 @@ enum TuneKey {
     kTuneStaticSpg = 6,     // static backward: samples per workgroup of the dx kernel (n <= 8)
     kTuneResident = 7,      // n <= 8 sample-resident backward: 0 = by heuristic, 1 = never, 2 = whenever the shape allows
     kTuneWideDxBeside = 8,  // wide projections (n > 18): dx workgroups beside the coefficient launch: 1 = never, 2 = always
-    kTuneSpareB = 9,        // wide projection forward (n >= 11): K splits, 0 = by heuristic
+    kTuneSpareB = 9,        // projection forward (matrix-core kernels): K splits, 0 = by heuristic
     kTuneCount = 10
 };
 
