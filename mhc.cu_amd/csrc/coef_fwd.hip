@@ -4,6 +4,7 @@
 // Replaces, in one launch: the split-K reduction of the projection, fused_h_activations
 // (reference src/csrc/include/utils.cuh:50-126) and sinkhorn_knopp_forward_batched /
 // sinkhorn_knopp_forward_fused_exp (src/csrc/kernels/sinkhorn_knopp.cuh:986-1046, :461-519).
+#include <type_traits>
 #include "launchers.h"
 #include "phase_profiler.h"
 #include "sinkhorn_device.h"
@@ -139,30 +140,36 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     if (dyn) {
         const float4 *pb = reinterpret_cast<const float4 *>(a.Ppart + (size_t)b * a.DP);
         const int q4 = a.DP / 4;
-        constexpr int KB = 24;  // splits per round: at most 48 loads in flight per thread
         int cm[M4];
 #pragma unroll
         for (int m = 0; m < M4; m++) cm[m] = tid + 256 * m < q4 ? tid + 256 * m : 0;
-        for (int k0 = 0; k0 < a.KS; k0 += KB) {
-            float4 tv[M4][KB];
+        // splits per round: 16 or 24 (at most 48 loads in flight per thread); the split counts that the
+        // projection picks for a full chip are 15 and 24 at the benchmark shapes
+        auto sum_splits = [&](auto kb_tag) {
+            constexpr int KB = decltype(kb_tag)::value;
+            for (int k0 = 0; k0 < a.KS; k0 += KB) {
+                float4 tv[M4][KB];
 #pragma unroll
-            for (int m = 0; m < M4; m++) {
-                if (256 * m + 64 * wave_u >= q4) continue;
+                for (int m = 0; m < M4; m++) {
+                    if (256 * m + 64 * wave_u >= q4) continue;
 #pragma unroll
-                for (int q = 0; q < KB; q++)
-                    tv[m][q] = pb[(size_t)(k0 + q < a.KS ? k0 + q : 0) * (pstride / 4) + cm[m]];
-            }
+                    for (int q = 0; q < KB; q++)
+                        tv[m][q] = pb[(size_t)(k0 + q < a.KS ? k0 + q : 0) * (pstride / 4) + cm[m]];
+                }
 #pragma unroll
-            for (int m = 0; m < M4; m++) {
-                if (256 * m + 64 * wave_u >= q4) continue;
+                for (int m = 0; m < M4; m++) {
+                    if (256 * m + 64 * wave_u >= q4) continue;
 #pragma unroll
-                for (int q = 0; q < KB; q++) {
-                    const bool ok = k0 + q < a.KS;
-                    psum[m][0] += ok ? tv[m][q].x : 0.f; psum[m][1] += ok ? tv[m][q].y : 0.f;
-                    psum[m][2] += ok ? tv[m][q].z : 0.f; psum[m][3] += ok ? tv[m][q].w : 0.f;
+                    for (int q = 0; q < KB; q++) {
+                        const bool ok = k0 + q < a.KS;
+                        psum[m][0] += ok ? tv[m][q].x : 0.f; psum[m][1] += ok ? tv[m][q].y : 0.f;
+                        psum[m][2] += ok ? tv[m][q].z : 0.f; psum[m][3] += ok ? tv[m][q].w : 0.f;
+                    }
                 }
             }
-        }
+        };
+        if (a.KS <= 16) sum_splits(std::integral_constant<int, 16>{});
+        else sum_splits(std::integral_constant<int, 24>{});
     }
     // AGG: this thread's chunk of every stream is requested now and consumed behind the Sinkhorn
     // chain (whose barriers also publish hp_s); streams >= n alias stream 0 and meet Hpre = 0
