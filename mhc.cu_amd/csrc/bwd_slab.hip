@@ -494,12 +494,12 @@ int bwd_slab_batch_splits(int B, int n, int C) {
     }
     int S = (512 + slabs - 1) / slabs;  // two workgroups per CU
     if (S > tiles) S = tiles;
-    // the dphi partial copies (written here, read once by the finalize launch) stay below 12 MB or
+    // the dphi partial copies (written here, read once by the finalize launch) stay below 16 MB or
     // ~1/4 of the activation bytes this kernel moves, whichever is larger
     const int D = n * n + 2 * n;
     const double part = 2.0 * 4.0 * D * n * C;  // bytes written + read per split
     double budget = 0.25 * (3.0 * 2.0 * B * n * C);
-    if (budget < 12e6) budget = 12e6;
+    if (budget < 16e6) budget = 16e6;
     if (S > (int)(budget / part)) S = (int)(budget / part);
     if (S < 1) S = 1;
     // splits are whole 32-sample tiles: drop the splits that would get none
