@@ -72,11 +72,16 @@ struct DynBwdWs { float *dt, *dP, *cx, *s1, *u, *dtpart, *raw, *s1part, *dx_part
 //               1024 29.8 -> 29.6, 1536 35.7 -> 39.4, 2560 46.2 -> 62.5;  n=4 C=2048: B=768 33.5 -> 30.3, 1024 35.1 -> 41.2
 //   n=4 C=2560: B=256 23.9 -> 17.8, 512 32.0 -> 26.9, 768 36.3 -> 35.9, 1280 42.4 -> 53.9;  n=2 C=1280: B=1024 23.7 -> 28.8
 //   n=8 C=1280: B=128 25.1 -> 16.9, 256 30.5 -> 22.0, 512 46.1 -> 36.1, 1024 77.3 -> 62.7
+// n = 5 .. 8 with short rows and a large batch: a workgroup per sample then has too little to do, and the
+// tiled path (several samples per workgroup) wins:
+//   n=8 C=256: B=512 30.9 -> 23.8, 1024 39.9 -> 41.3, 2048 59.8 -> 73.4, 4096 94.0 -> 137.7;  C=128: B=8192 139.7 -> 261.4
+//   n=8 C=512: B=1024 43.7 -> 45.7, 2048 74.0 -> 83.1, 4096 124.2 -> 157.7;  C=1024: 1024 61.1 -> 51.6, 4096 182.2 -> 179.3
+//   n=6 C=512: B=1024 40.1 -> 43.5, 4096 113.0 -> 149.8;  n=5 C=384: B=3000 85.2 -> 97.8
 // Experiment hook: 1 = never, 2 = always.
 bool bwd_resident_preferred(int B, int n, int C) {
     if (const int hook = tuning_get(kTuneResident)) return hook == 2;
-    (void)C;
-    return n > 4 || B <= 768;
+    if (n > 4) return !(B >= 1024 && C <= 512);
+    return B <= 768;
 }
 
 // Shapes for which the dynamic entry points take fp32 activations that are consumed as bf16
@@ -107,8 +112,13 @@ DynFwdWs carve_dyn_fwd(void *ws, int B, int n, int C) {
 }
 
 // Wide projections (n > 18) without batch split of dphi: four launches, see mhc_layer_bwd_dynamic.
+// Up to 16 M activation elements: the fp32 hand-over costs 4 more bytes per element than completing dx
+// in place, which the shorter chain repays only while the coefficient launch leaves CUs idle
+// (backward us, four launches | five: B=128 n=32 C=1280 92 | 100, 384 n=32 C=1280 214 | 215,
+//  512 n=32 C=1280 283 | 269, 256 n=32 C=2560 338 | 312).
 bool wide_dx_beside(int B, int n, int C) {
-    return proj_bwd_is_wide(n) && C % 8 == 0 && proj_bwd_batch_splits(B, n, C) == 1;
+    return proj_bwd_is_wide(n) && C % 8 == 0 && proj_bwd_batch_splits(B, n, C) == 1 &&
+           (long long)B * n * C <= (16ll << 20);
 }
 
 DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {

@@ -59,7 +59,8 @@ def _grads(st):
 
 
 SHAPES = [(5, 4, 64), (1, 4, 128), (3, 2, 40), (2, 3, 24), (7, 1, 136), (33, 4, 1288), (320, 4, 1280), (9, 4, 640),
-          (130, 4, 2560), (16, 8, 256), (3, 6, 72), (9, 8, 1288), (70, 5, 1024), (257, 8, 136), (300, 7, 512)]
+          (130, 4, 2560), (16, 8, 256), (3, 6, 72), (9, 8, 1288), (70, 5, 1024), (257, 8, 136), (300, 7, 512),
+          (1100, 8, 128), (1030, 5, 264)]   # short rows, large batch: where the default takes the tiled path for n > 4
 
 
 def _both_paths(key, names, B, n, C, inject, w_f32):
