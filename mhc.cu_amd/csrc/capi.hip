@@ -150,7 +150,7 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
 
 // ---- static workspace layout -----------------------------------------------------------------
 struct StaFwdWs { float *Hpre, *Hpost, *M, *q, *agg; size_t bytes; };
-struct StaBwdWs { float *red, *s1, *u, *red_sum, *raw; size_t bytes; };
+struct StaBwdWs { float *red, *s1, *u, *red_sum, *raw, *sk; size_t bytes; };
 
 StaFwdWs carve_sta_fwd(void *ws, int B, int n, int C) {
     Carver c(ws);
@@ -170,6 +170,7 @@ StaBwdWs carve_sta_bwd(void *ws, int B, int n, int C) {
     w.u = c.floats((size_t)B * C);
     w.red_sum = c.floats(D + 3);
     w.raw = c.floats(n > 8 ? bwd_reduce_raw_floats(B, n, C) : 0);
+    w.sk = c.floats(n > 8 ? (size_t)(2 * max_layer_sinkhorn_iters(n) + 2) * 32 : 0);  // Sinkhorn denominators of the shared logits
     w.bytes = c.off;
     return w;
 }
@@ -474,11 +475,16 @@ int mhc_layer_fwd(const void *x, int x_dtype, const void *w, int w_dtype,
         if (int s = ws_check(workspace, workspace_bytes, ws.bytes)) return s;
     float *hp = H_pre ? H_pre : ws.Hpre, *ho = H_post ? H_post : ws.Hpost;
     float *m = M ? M : ws.M, *qq = q ? q : ws.q;
+    // n > 8, up to two samples per CU: the coefficient launch runs once per sample, each workgroup with
+    // the shared Sinkhorn chain and its sample's aggregate and RMS under it, instead of one workgroup
+    // followed by an aggregate launch (forward, cold, B=128 n=32 C=1280: 26 -> 20 us)
+    const bool agg = !f_inject && n > 8 && B <= 512 && coef_fwd_aggregates(n, C, x_dtype);
     MHC_LAUNCH(launch_coef_fwd(nullptr, nullptr, 0, 0, nullptr, H_pre_logits, H_post_logits,
-                               H_res_logits, hp, ho, m, nullptr, nullptr, 1, n, n * C, iters, eps,
-                               x_dtype == kF32, nullptr, nullptr, nullptr, nullptr, st));
+                               H_res_logits, hp, ho, m, nullptr, nullptr, agg ? B : 1, n, n * C, iters, eps,
+                               x_dtype == kF32, agg ? x : nullptr, agg ? ws.agg : nullptr, agg ? qq : nullptr,
+                               nullptr, st));
     MHC_LAUNCH(launch_mix_fwd(x, x_dtype, w, w_dtype, f_inject, y, y_dtype, hp, ho, m, 0, qq,
-                              n > 8 ? ws.agg : nullptr, B, n, C, eps, false, st));
+                              n > 8 ? ws.agg : nullptr, B, n, C, eps, agg, st));
     return MHC_OK;
 }
 
@@ -513,7 +519,7 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
     }
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,
                                      0, q, nullptr, nullptr, nullptr, nullptr, nullptr, out, n > 8 ? ws.raw : nullptr,
-                                     B, n, C, iters, eps, st));
+                                     B, n, C, iters, eps, st, H_res_logits, n > 8 ? ws.sk : nullptr));
     // samples per workgroup of the dx kernel: with a large batch a workgroup adds up the dw terms of a
     // few samples itself, so that the batch-sum launch reads fewer rows
     const int hook = tuning_get(kTuneStaticSpg);
@@ -526,7 +532,7 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
     // the batch sums (dw = sum_b u, sum_b red) and the coefficient backward on them: one launch for
     // n <= 8, two beyond
     MHC_LAUNCH(launch_finalize_static(ws.u, groups, C, f_inject ? nullptr : dw, ws.red, B, ws.red_sum, H_pre, H_post,
-                                      H_res_logits, dH_pre, dH_post, dH_res, n, iters, eps, st));
+                                      H_res_logits, dH_pre, dH_post, dH_res, n, iters, eps, st, n > 8 ? ws.sk : nullptr));
     return MHC_OK;
 }
 

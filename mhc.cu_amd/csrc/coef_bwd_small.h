@@ -18,6 +18,11 @@ struct BwdReduceArgs {
     float *raw;   // n <= 8: when set, write the raw channel sums [B][parts][K] and stop
     int parts;    // column parts per sample (gridDim.y)
     float *s1part = nullptr;  // n > 8: when set, the Gram launch also writes s1 = Hpost^T W1 Hpre of every part, [B][parts]
+    // static H, n > 8: the channel-sum launch carries one more workgroup that recomputes the Sinkhorn forward
+    // of the shared logits (IEEE divisions) and leaves its denominators here for the static coefficient
+    // backward, which then has half its chain left (SkWg::save_state layout, (2 T + 2) * NP floats)
+    const float *static_logits = nullptr;
+    float *static_state = nullptr;
 };
 
 // Where the weight of the W1 = dy diag(w) x^T Gram matrix comes from: an injected f [B, C] (W1 = dy [f; 0 ..]^T),

@@ -209,8 +209,12 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     __syncthreads();
     if (tid < n) {
         const float hp = PRECISE ? sigmoidf_acc(lg[tid]) : sigmoid_fast(lg[tid]);
-        a.Hpre[b * n + tid] = hp;
-        a.Hpost[b * n + tid] = 2.0f * (PRECISE ? sigmoidf_acc(lg[n + tid]) : sigmoid_fast(lg[n + tid]));
+        // static H with the aggregate: every sample's workgroup derives the shared coefficients (for its
+        // aggregate), the first one stores them
+        if (dyn || b == 0) {
+            a.Hpre[(dyn ? b * n : 0) + tid] = hp;
+            a.Hpost[(dyn ? b * n : 0) + tid] = 2.0f * (PRECISE ? sigmoidf_acc(lg[n + tid]) : sigmoid_fast(lg[n + tid]));
+        }
         if constexpr (AGG) hp_s[tid] = hp;
     } else if (AGG && tid < 32) {
         hp_s[tid] = 0.f;
@@ -225,7 +229,7 @@ __global__ __launch_bounds__(256) void coef_fwd_lds_kernel(CoefArgs a) {
     MHC_PHASE(kPhaseCoefFwdWide, b, 3);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
-        if (r0 < n && c0 + e < n) a.M[(size_t)b * n * n + r0 * n + c0 + e] = u * E[e] * v[e];
+        if (r0 < n && c0 + e < n && (dyn || b == 0)) a.M[(dyn ? (size_t)b * n * n : 0) + r0 * n + c0 + e] = u * E[e] * v[e];
     if (a.sk_state) SK::save_state(sk_s, a.T, a.sk_state + (size_t)b * SK::state_floats(a.T), tid, u, v);
     MHC_PHASE(kPhaseCoefFwdWide, b, 4);
     if constexpr (AGG) {
@@ -290,8 +294,9 @@ hipError_t launch_coef_fwd(const float *Ppart, const float *ssqpart, int KS, int
     return hipGetLastError();
 }
 
-// Whether launch_coef_fwd can also produce the stream aggregate and its RMS for this shape (dynamic
-// H, n > 8, bf16 x, one 16-byte chunk per thread and stream).
+// Whether launch_coef_fwd can also produce the stream aggregate and its RMS for this shape (n > 8,
+// bf16 x, one 16-byte chunk per thread and stream).  With static H every sample's workgroup then
+// repeats the shared Sinkhorn chain (they run side by side: worth it while they fit the chip together).
 bool coef_fwd_aggregates(int n, int C, int x_dtype) {
     return n > 8 && x_dtype == kBF16 && C % 8 == 0 && C / 8 <= 256;
 }

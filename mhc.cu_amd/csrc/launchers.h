@@ -115,7 +115,11 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
                                  const float *Hpre, const float *Hpost, const float *M, int hstride,
                                  const float *q, const float *P, const float *r, const float *alpha,
                                  const float *b_res, const float *sk_state, BwdCoefOut out, float *raw, int B,
-                                 int n, int C, int T, float eps, hipStream_t stream);
+                                 int n, int C, int T, float eps, hipStream_t stream,
+                                 const float *static_logits = nullptr, float *static_state = nullptr);
+// static_logits / static_state (optional, static H, n > 8): the channel-sum launch also recomputes the
+// Sinkhorn forward of the shared logits and leaves its denominators in static_state ((2 T + 2) * 32 floats)
+// for launch_finalize_static.
 // raw (optional, dynamic H, n <= 8): scratch of B * bwd_reduce_parts() * (NP*NP + 3*NP + 1) floats;
 // when given, the channel sums and the coefficient backward run as two launches.
 int bwd_reduce_parts(int B, int n, int C);
@@ -229,11 +233,11 @@ hipError_t launch_colsum_split(const float *in, int rows, int cols, int ld, floa
 // Static H: coefficient backward on the sample-summed raw gradients.
 hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const float *Hpost,
                                   const float *H_res_logits, float *dH_pre, float *dH_post,
-                                  float *dH_res, int n, int T, float eps, hipStream_t stream);
+                                  float *dH_res, int n, int T, float eps, hipStream_t stream, const float *state = nullptr);
 hipError_t launch_finalize_static(const float *u, int rows_u, int C, float *dw, const float *red, int rows,
                                   float *red_sum, const float *Hpre, const float *Hpost,
                                   const float *H_res_logits, float *dH_pre, float *dH_post, float *dH_res, int n,
-                                  int T, float eps, hipStream_t stream);
+                                  int T, float eps, hipStream_t stream, const float *static_state = nullptr);
 
 // phi [D, nC] (out_dtype) = rows [pre | post | res] of the three parameter matrices (src_dtype),
 // bias [D] and alpha [3] likewise, in one launch.

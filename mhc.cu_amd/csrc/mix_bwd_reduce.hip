@@ -411,13 +411,37 @@ __global__ __launch_bounds__(256, NP == 4 ? 4 : 1) void gram_small_kernel(BwdRed
 constexpr int kGramMats = 3;
 constexpr int kGramFloats = kGramMats * 1024;  // per (sample, part), row-major [m][i][j], 32 x 32
 
+// Static H: one workgroup behind the samples' (blockIdx.x == B) recomputes the Sinkhorn forward of the shared
+// logits with IEEE divisions and leaves the denominators of its iterations in a.static_state for the
+// static coefficient backward, the last launch of the call, which then has only the reverse sweep left.
+// The chain (about 6 us for 20 iterations of a 32 x 32 matrix) runs in the shadow of the channel sums.
+template <int NP>
+__device__ __forceinline__ void static_sinkhorn_forward_block(const BwdReduceArgs &a, float *smem) {
+    using SK = SkWg<NP>;
+    const int tid = threadIdx.x, n = a.n;
+    const int r0 = SK::row(tid), c0 = SK::col0(tid);
+    float E[SK::EPL], u, v[SK::EPL];
+#pragma unroll
+    for (int e = 0; e < SK::EPL; e++)
+        E[e] = (r0 < n && c0 + e < n) ? expf(a.static_logits[r0 * n + c0 + e]) : 0.f;
+    SK::template forward<true>(E, u, v, n, a.T, a.eps, smem, tid);
+    SK::save_state(smem, a.T, a.static_state, tid, u, v);
+}
+
 template <typename TG, typename TX>
 __global__ __launch_bounds__(256) void gram_large_kernel(BwdReduceArgs a) {
     constexpr bool kBf16 = std::is_same<TG, bf16_t>::value && std::is_same<TX, bf16_t>::value;
     constexpr int VL = kBf16 ? 8 : 4;  // columns per lane and k-step
     constexpr int SW = 2 * VL;         // columns per k-step (two lane halves)
     constexpr int U = 4;               // k-steps in flight per wave
-    extern __shared__ float smem[];
+    extern __shared__ __align__(16) float smem[];
+    if ((int)blockIdx.x >= a.B) {  // only launched with a.static_state set
+        if (blockIdx.y == 0) {
+            if (a.n <= 16) static_sinkhorn_forward_block<16>(a, smem);
+            else static_sinkhorn_forward_block<32>(a, smem);
+        }
+        return;
+    }
     float *w_s = smem;  // [cols of this part] fp32 weights (zero beyond C)
     const int b = blockIdx.x, part = blockIdx.y, n = a.n, C = a.C, tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6, row = lane & 31, kh = lane >> 5;
@@ -1012,13 +1036,17 @@ static hipError_t launch_large(const BwdReduceArgs &a, hipStream_t stream, const
     const int spp = (nsteps + a.parts - 1) / a.parts;
     // weights of the part | cross-wave scratch, which first holds the four waves' chunk tiles (bf16 path)
     const size_t scratch = sizeof(float) * 3 * kGramMats * 16 * 64, tiles = sizeof(bf16_t) * 4 * (2 * 32 + 1) * 72;
-    const size_t smem1 = sizeof(float) * (size_t)spp * SW + (kBf16 && tiles > scratch ? tiles : scratch);
+    size_t smem1 = sizeof(float) * (size_t)spp * SW + (kBf16 && tiles > scratch ? tiles : scratch);
+    if (a.static_state) {
+        const size_t sk = sizeof(float) * (a.n <= 16 ? SkWg<16>::lds_floats(a.T) : SkWg<32>::lds_floats(a.T));
+        if (smem1 < sk) smem1 = sk;
+    }
     if (smem1 > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gram_large_kernel<TG, TX>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1);
         if (e != hipSuccess) return e;
     }
-    gram_large_kernel<TG, TX><<<dim3(a.B, a.parts), 256, smem1, stream>>>(a);
+    gram_large_kernel<TG, TX><<<dim3(a.B + (a.static_state ? 1 : 0), a.parts), 256, smem1, stream>>>(a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     constexpr bool kPrecise = std::is_same<TX, float>::value;  // fp32 activations: the parity tier
@@ -1077,7 +1105,8 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
                                  const float *Hpre, const float *Hpost, const float *M, int hstride,
                                  const float *q, const float *P, const float *r, const float *alpha,
                                  const float *b_res, const float *sk_state, BwdCoefOut out, float *raw, int B,
-                                 int n, int C, int T, float eps, hipStream_t stream) {
+                                 int n, int C, int T, float eps, hipStream_t stream, const float *static_logits,
+                                 float *static_state) {
     // n <= 8, dynamic H: channel sums per (sample, column part), coefficient backward as a second
     // small launch (static H: everything in the per-sample workgroup).  n > 8: always two launches.
     if (n > 8 && raw == nullptr) return hipErrorInvalidValue;
@@ -1085,6 +1114,10 @@ hipError_t launch_mix_bwd_reduce(const void *dy, int y_dtype, const void *x, int
     BwdReduceArgs a{dy, x, w, f_inject, Hpre, Hpost, M, q, P, r, alpha, b_res, sk_state, out,
                     hstride, w_dtype == kBF16, B, n, C, T, padded_D(n), eps,
                     split ? raw : nullptr, split ? bwd_reduce_parts(B, n, C) : 1};
+    if (n > 8 && hstride == 0 && static_logits && static_state) {
+        a.static_logits = static_logits;
+        a.static_state = static_state;
+    }
     if (n <= 8) {
 #define MHC_SMALL(TG, TX)                                                   \
     return n <= 4 ? launch_small_np<TG, TX, 4>(a, stream) : launch_small_np<TG, TX, 8>(a, stream)

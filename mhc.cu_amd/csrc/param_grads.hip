@@ -195,9 +195,11 @@ __global__ __launch_bounds__(256) void coef_bwd_static_kernel(const float *__res
                                                               float *__restrict__ dH_pre,
                                                               float *__restrict__ dH_post,
                                                               float *__restrict__ dH_res, int n, int T,
-                                                              float eps) {
+                                                              float eps, const float *__restrict__ state) {
     // one workgroup, the matrix spread over the registers of its 256 threads (IEEE divisions: this
-    // kernel serves both precision tiers and runs once per backward call)
+    // kernel serves both precision tiers and runs once per backward call).  state: the denominators of
+    // the forward iterations as an earlier launch of the same backward call left them (SkWg::save_state);
+    // without it the forward is recomputed here
     using SK = SkWg<NP>;
     extern __shared__ __align__(16) float lds[];  // SK::lds_floats(T)
     const int tid = threadIdx.x;
@@ -214,7 +216,8 @@ __global__ __launch_bounds__(256) void coef_bwd_static_kernel(const float *__res
         E[e] = ok ? expf(H_res_logits[r0 * n + c0 + e]) : 0.f;
         d[e] = ok ? red_sum[r0 * n + c0 + e] : 0.f;
     }
-    SK::template forward<true>(E, u, v, n, T, eps, lds, tid);
+    if (state) SK::load_state(state, u, v, T, lds, tid);
+    else SK::template forward<true>(E, u, v, n, T, eps, lds, tid);
     SK::template backward<true>(E, d, u, v, T, lds, tid);
 #pragma unroll
     for (int e = 0; e < SK::EPL; e++)
@@ -252,7 +255,7 @@ __global__ __launch_bounds__(64) void coef_bwd_static_small_kernel(const float *
 
 hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const float *Hpost,
                                   const float *H_res_logits, float *dH_pre, float *dH_post,
-                                  float *dH_res, int n, int T, float eps, hipStream_t stream) {
+                                  float *dH_res, int n, int T, float eps, hipStream_t stream, const float *state) {
     if (n <= 8) {
         if (n <= 4) {
             const size_t smem = sizeof(float) * SkSmall<4>::scaling_floats(T);
@@ -266,11 +269,11 @@ hipError_t launch_coef_bwd_static(const float *red_sum, const float *Hpre, const
     } else if (n <= 16) {
         const size_t smem = sizeof(float) * SkWg<16>::lds_floats(T);
         if (hipError_t e = allow_dynamic_lds(&coef_bwd_static_kernel<16>, smem); e != hipSuccess) return e;
-        coef_bwd_static_kernel<16><<<1, 256, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
+        coef_bwd_static_kernel<16><<<1, 256, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps, state);
     } else {
         const size_t smem = sizeof(float) * SkWg<32>::lds_floats(T);
         if (hipError_t e = allow_dynamic_lds(&coef_bwd_static_kernel<32>, smem); e != hipSuccess) return e;
-        coef_bwd_static_kernel<32><<<1, 256, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps);
+        coef_bwd_static_kernel<32><<<1, 256, smem, stream>>>(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps, state);
     }
     return hipGetLastError();
 }
@@ -357,13 +360,14 @@ __global__ __launch_bounds__(1024) void finalize_static_kernel(FinalizeStaticArg
 hipError_t launch_finalize_static(const float *u, int rows_u, int C, float *dw, const float *red, int rows,
                                   float *red_sum, const float *Hpre, const float *Hpost,
                                   const float *H_res_logits, float *dH_pre, float *dH_post, float *dH_res, int n,
-                                  int T, float eps, hipStream_t stream) {
+                                  int T, float eps, hipStream_t stream, const float *static_state) {
     const int D = n * n + 2 * n;
     if (n > 8) {
         if (hipError_t e = launch_finalize(u, rows_u, C, dw, red, rows, D, red_sum, red_sum + D, nullptr, 1, 0,
                                            nullptr, stream); e != hipSuccess)
             return e;
-        return launch_coef_bwd_static(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps, stream);
+        return launch_coef_bwd_static(red_sum, Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res, n, T, eps, stream,
+                                      static_state);
     }
     FinalizeStaticArgs a{make_batch_sums(u, rows_u, C, dw, nullptr, 0, 0, nullptr, nullptr), red, rows, n, T, eps,
                          Hpre, Hpost, H_res_logits, dH_pre, dH_post, dH_res};
