@@ -150,7 +150,7 @@ DynBwdWs carve_dyn_bwd(void *ws, int B, int n, int C) {
 
 // ---- static workspace layout -----------------------------------------------------------------
 struct StaFwdWs { float *Hpre, *Hpost, *M, *q, *agg; size_t bytes; };
-struct StaBwdWs { float *red, *s1, *u, *red_sum, *raw, *sk; size_t bytes; };
+struct StaBwdWs { float *red, *s1, *u, *red_sum, *raw, *sk, *s1part; size_t bytes; };
 
 StaFwdWs carve_sta_fwd(void *ws, int B, int n, int C) {
     Carver c(ws);
@@ -170,7 +170,8 @@ StaBwdWs carve_sta_bwd(void *ws, int B, int n, int C) {
     w.u = c.floats((size_t)B * C);
     w.red_sum = c.floats(D + 3);
     w.raw = c.floats(n > 8 ? bwd_reduce_raw_floats(B, n, C) : 0);
-    w.sk = c.floats(n > 8 ? (size_t)(2 * max_layer_sinkhorn_iters(n) + 2) * 32 : 0);  // Sinkhorn denominators of the shared logits
+    w.sk = c.floats(n > 8 ? (size_t)(2 * max_layer_sinkhorn_iters(n) + 2) * 32 : 0);
+    w.s1part = c.floats(n > 16 ? (size_t)B * bwd_reduce_parts(B, n, C) : 0);  // Sinkhorn denominators of the shared logits
     w.bytes = c.off;
     return w;
 }
@@ -515,6 +516,17 @@ int mhc_layer_bwd(const void *dy, int y_dtype, const void *x, int x_dtype, const
                                               B, n, C, st));
         MHC_LAUNCH(launch_finalize_static(ws.u, B, C, f_inject ? nullptr : dw, ws.red, B, ws.red_sum, H_pre, H_post,
                                           H_res_logits, dH_pre, dH_post, dH_res, n, iters, eps, st));
+        return MHC_OK;
+    }
+    if (n > 16 && x_dtype == kBF16 && y_dtype == kBF16 && C % 8 == 0) {
+        // three launches: channel sums (+ the Sinkhorn forward recompute), the per-sample coefficient sums
+        // with the complete dx beside them, batch sums + coefficient backward
+        // (cold, B=128 n=32 C=1280: 44.7 us -> see profiles/native_bench_all_configs.txt)
+        MHC_LAUNCH(launch_mix_bwd_reduce_with_dx_static(dy, x, w, w_dtype, f_inject, H_pre, H_post, M, q, out, ws.raw,
+                                                        ws.s1part, dx, df, ws.u, B, n, C, iters, eps, st, H_res_logits,
+                                                        ws.sk));
+        MHC_LAUNCH(launch_finalize_static(ws.u, B, C, f_inject ? nullptr : dw, ws.red, B, ws.red_sum, H_pre, H_post,
+                                          H_res_logits, dH_pre, dH_post, dH_res, n, iters, eps, st, ws.sk));
         return MHC_OK;
     }
     MHC_LAUNCH(launch_mix_bwd_reduce(dy, y_dtype, x, x_dtype, w, w_dtype, f_inject, H_pre, H_post, M,

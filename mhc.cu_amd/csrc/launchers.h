@@ -134,6 +134,13 @@ hipError_t launch_mix_bwd_reduce_with_dx(const void *dy, const void *x, const vo
                                          const float *b_res, const float *sk_state, BwdCoefOut out, float *raw,
                                          float *s1part, float *dxp, void *df, float *u, int B, int n, int C, int T,
                                          float eps, hipStream_t stream);
+// Static H, n > 16, bf16: the dx workgroups beside the coefficient launch write the final dx.
+hipError_t launch_mix_bwd_reduce_with_dx_static(const void *dy, const void *x, const void *w, int w_dtype,
+                                                const void *f_inject, const float *Hpre, const float *Hpost,
+                                                const float *M, const float *q, BwdCoefOut out, float *raw,
+                                                float *s1part, void *dx, void *df, float *u, int B, int n, int C,
+                                                int T, float eps, hipStream_t stream, const float *static_logits,
+                                                float *static_state);
 
 // dx = M^T dy + Hpre (x) da - cx * x  [+ dP phi when phi != nullptr] [+ dx_in when != nullptr;
 // may alias dx], df, and u = df * a / q (the per-sample summand of dw).

@@ -1152,4 +1152,26 @@ hipError_t launch_mix_bwd_reduce_with_dx(const void *dy, const void *x, const vo
     return launch_large<bf16_t, bf16_t>(a, stream, &d);
 }
 
+// The same for static H (n > 16, bf16 dy and x): with shared coefficients nothing of dx waits for another
+// launch, so the dx workgroups beside the coefficient workgroups write the final dx (bf16) themselves.
+// static_logits / static_state as in launch_mix_bwd_reduce.
+hipError_t launch_mix_bwd_reduce_with_dx_static(const void *dy, const void *x, const void *w, int w_dtype,
+                                                const void *f_inject, const float *Hpre, const float *Hpost,
+                                                const float *M, const float *q, BwdCoefOut out, float *raw,
+                                                float *s1part, void *dx, void *df, float *u, int B, int n, int C,
+                                                int T, float eps, hipStream_t stream, const float *static_logits,
+                                                float *static_state) {
+    if (n <= 16 || raw == nullptr || s1part == nullptr || dx == nullptr || C % 8 != 0) return hipErrorInvalidValue;
+    const int parts = bwd_reduce_parts(B, n, C);
+    BwdReduceArgs a{dy, x, w, f_inject, Hpre, Hpost, M, q, nullptr, nullptr, nullptr, nullptr, nullptr, out,
+                    0, w_dtype == kBF16, B, n, C, T, padded_D(n), eps, raw, parts, s1part};
+    if (static_logits && static_state) {
+        a.static_logits = static_logits;
+        a.static_state = static_state;
+    }
+    BwdDxArgs d{dy, x, w, f_inject, nullptr, nullptr, Hpre, Hpost, M, q, nullptr, nullptr, nullptr, dx, df, u,
+                nullptr, nullptr, 0, w_dtype == kBF16, 0, B, n, C, padded_D(n), 1, s1part, parts, nullptr};
+    return launch_large<bf16_t, bf16_t>(a, stream, &d);
+}
+
 }  // namespace mhc
