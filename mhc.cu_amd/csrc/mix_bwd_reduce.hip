@@ -945,6 +945,10 @@ static int gram_small_parts(int B, int C) { return C >= 1024 && B < 1024 ? 2 : 1
 // too small to do without column parts.
 static bool gram_small_fused(const BwdReduceArgs &a) {
     if (const int hook = tuning_get(kTuneGramFused); hook && a.T <= 32) return hook == 2;  // experiment hook
+    // very short rows in a very large batch: the tail of a workgroup (one wave, 2.6 us) outweighs its
+    // streaming, and a separate launch packs the chains of four samples into a wave
+    // (backward us, one launch | two: B=8192 n=4 C=128 50.3 | 45.2, 6000 C=256 46.7 | 45.4, 4096 C=512 42.4 | 45.5)
+    if (a.B >= 6000 && a.C <= 256) return false;
     return a.T <= 32 && (a.B >= 128 || a.C <= 2048);
 }
 

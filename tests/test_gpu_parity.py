@@ -372,6 +372,8 @@ _KEPT_CASES += [(3, 4, 32768, 20, True, True, False), (2, 32, 32768, 20, True, T
 # 11 <= n <= 18 with a large batch: the two projection-backward products as launches of their own, with batch
 # splits (the finalize launch sums the dphi copies) and, in the second case, without dw
 _KEPT_CASES += [(2000, 12, 32, 20, True, True, False), (3000, 16, 32, 20, True, True, True)]
+# very large batches of short rows: the channel sums and the coefficient backward as two launches (n <= 4)
+_KEPT_CASES += [(6100, 4, 128, 20, True, True, False), (6500, 3, 256, 20, True, True, True)]
 
 
 @pytest.mark.parametrize("B,n,C,T,dyn,bf16,inject", _random_cases(40, seed=2024) + _KEPT_CASES)
