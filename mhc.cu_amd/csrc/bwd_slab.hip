@@ -48,7 +48,7 @@ struct BwdSlabArgs {
     float *dphi_part;        // [S][D][nC]
     float *dw_part;          // [S][C]
     float *dt_part;          // [S][D+3]
-    int w_bf16, B, BP, n, C, b_per_split;
+    int w_bf16, B, BP, n, C, tiles;  // tiles = 32-sample tiles of the batch; split y takes tiles [y T / S, (y + 1) T / S)
 };
 
 __device__ __forceinline__ bf16x8_t slab_frag_t(const bf16_t *tile, int k0, int col0, int lane) {
@@ -95,8 +95,12 @@ __global__ __launch_bounds__(256, 2) void bwd_slab_kernel(BwdSlabArgs a) {
     MHC_PHASE_ZERO(kPhaseBwdSlab, pwg);
     MHC_PHASE_BEGIN(pclk);
     const int c0 = blockIdx.x * kSlabCW;
-    const int b_begin = blockIdx.y * a.b_per_split;
-    const int b_end = min(a.B, b_begin + a.b_per_split);
+    // whole tiles per split, the counts of two splits differing by at most one: any split count up to the
+    // tile count can be used, so the grid can be sized to the chip instead of to a divisor of the batch
+    const unsigned nsplit = gridDim.y;
+    // (tiles <= 2^26 and at most 512 splits: the products fit 32 bits)
+    const int b_begin = (int)(blockIdx.y * (unsigned)a.tiles / nsplit) * 32;
+    const int b_end = min(a.B, (int)((blockIdx.y + 1) * (unsigned)a.tiles / nsplit) * 32);
     const bool inject = a.f_inject != nullptr;
     const int row = lane & 31, kg = lane >> 5;
     // VALU ownership: sample bl of the tile, channels c0 + ch*8 .. +8 of every stream
@@ -489,22 +493,26 @@ int bwd_slab_batch_splits(int B, int n, int C) {
     const int slabs = (C + kSlabCW - 1) / kSlabCW;
     const int tiles = (B + 31) / 32;
     if (const int forced = tuning_get(kTuneSlabSplits); forced > 0) {  // experiment hook
-        const int tps = (tiles + (forced < tiles ? forced : tiles) - 1) / (forced < tiles ? forced : tiles);
-        return (tiles + tps - 1) / tps;
+        return forced < tiles ? forced : tiles;
     }
-    int S = (512 + slabs - 1) / slabs;  // two workgroups per CU
+    // Two workgroups per CU, all resident at once (one split more than that costs a second round:
+    // B=1280 C=2560, 12 splits 42.5 us, 13 splits 48.5).
+    int S = 512 / slabs;
     if (S > tiles) S = tiles;
     // the dphi partial copies (written here, read once by the finalize launch) stay below 16 MB or
-    // ~1/4 of the activation bytes this kernel moves, whichever is larger
+    // 0.4 of the activation bytes this kernel moves, whichever is larger
     const int D = n * n + 2 * n;
     const double part = 2.0 * 4.0 * D * n * C;  // bytes written + read per split
-    double budget = 0.25 * (3.0 * 2.0 * B * n * C);
+    double budget = 0.4 * (3.0 * 2.0 * B * n * C);
     if (budget < 16e6) budget = 16e6;
     if (S > (int)(budget / part)) S = (int)(budget / part);
     if (S < 1) S = 1;
-    // splits are whole 32-sample tiles: drop the splits that would get none
+    // the longest split decides: the fewest splits that keep its tile count
+    // (backward us: B=1024 C=2560  11 splits of 3 tiles 37 | 8 of 4: 40.0;  B=1536 C=1920  16 of 3: 39.4 | 12 of 4: 41.7;
+    //  B=800 C=1280  13 of 2: 25.5 | 12 of 2 or 3: 28.8)
     const int tps = (tiles + S - 1) / S;
-    return (tiles + tps - 1) / tps;
+    S = (tiles + tps - 1) / tps;
+    return S;  // <= tiles: every split has at least one tile
 }
 
 hipError_t launch_bwd_slab(const void *dy, int y_dtype, const void *x, const void *w, int w_dtype,
@@ -514,11 +522,11 @@ hipError_t launch_bwd_slab(const void *dy, int y_dtype, const void *x, const voi
                            void *dx, void *df, float *dphi_part, float *dw_part, float *dt_part, int S,
                            int B, int n, int C, hipStream_t stream) {
     const int tiles = (B + 31) / 32;
-    const int bps = (tiles + S - 1) / S * 32;
+    if (S < 1 || S > tiles) return hipErrorInvalidValue;
     BwdSlabArgs a{dy, static_cast<const bf16_t *>(x), w, f_inject, static_cast<const bf16_t *>(phi),
                   Hpre, Hpost, M, q, s1, cx, static_cast<const bf16_t *>(dPb),
                   static_cast<const bf16_t *>(dPT), dt, static_cast<bf16_t *>(dx),
-                  static_cast<bf16_t *>(df), dphi_part, dw_part, dt_part, w_dtype == kBF16, B, BP, n, C, bps};
+                  static_cast<bf16_t *>(df), dphi_part, dw_part, dt_part, w_dtype == kBF16, B, BP, n, C, tiles};
     const size_t smem = sizeof(float) * 32 * kSlabLDF + sizeof(bf16_t) * 32 * kSlabLDX;
     dim3 grid((C + kSlabCW - 1) / kSlabCW, S);
     if (y_dtype == kBF16) bwd_slab_kernel<bf16_t><<<grid, 256, smem, stream>>>(a);
