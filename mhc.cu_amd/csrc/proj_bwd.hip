@@ -16,6 +16,7 @@
 #include <type_traits>
 #include "mhc_common.h"
 #include "phase_profiler.h"
+#include "tuning.h"
 
 namespace mhc {
 
@@ -295,6 +296,7 @@ int proj_bwd_batch_splits(int B, int n, int C) {
     const double cap = 0.25 * (2.0 * 2.0 * B * nC) / (4.0 * D * nC);
     if (S > (int)cap) S = (int)cap;
     if (S < 1) S = 1;
+    if (const int forced = tuning_get(kTuneSlabSplits); forced > 0) S = forced < nblocks ? forced : nblocks;  // experiment hook
     return S;
 }
 

@@ -11,7 +11,7 @@ enum TuneKey {
     kTuneOnepassOff = 0,    // one-launch forward: 0 = by cost model, 1 = never, 2 = whenever the shape allows
     kTuneOnepassG = 1,      // samples per workgroup of the one-launch forward
     kTuneGramFused = 2,     // n <= 8 channel sums and coefficient backward: 1 = two launches, 2 = one launch
-    kTuneSlabSplits = 3,    // batch splits of the slab backward
+    kTuneSlabSplits = 3,    // batch splits of the slab backward (n <= 4) and of the projection backward (n = 5 .. 18)
     kTuneSeparateFinalize = 4,  // 1 = batch sums always as a launch of their own, never inside the dphi launch
     kTuneProjApart = 5,     // n <= 18 projection backward: 1 = both products in one launch, 2 = two launches
     kTuneStaticSpg = 6,     // static backward: samples per workgroup of the dx kernel (n <= 8)
