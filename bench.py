@@ -36,22 +36,22 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # `--copy-calibration` (a 64 MiB copy).  Filled from the committed counter summary
 # (profiles/hbm_traffic_counters.txt); `commit` is the revision of the kernels the counters ran on.
 MEASURED_TRAFFIC = {
-    "commit": "bd92725",
-    "bytes": {"c1": 13281066, "c2": 37946869, "c3": 246954926, "c4": 64736211, "c5": 577712964},
+    "commit": "44e4d8b",
+    "bytes": {"c1": 13281066, "c2": 37946871, "c3": 246954758, "c4": 64736245, "c5": 577687318},
 }
 
 # The kernel with the largest share of a step's device time, from the committed kernel-trace summaries
 # (profiles/layer_step_<config>.txt): average duration per dispatch and the HBM bytes the algorithm
 # needs that kernel to move (its own inputs and outputs once; for the split projections the partial
 # sums are not counted).
-PROFILED_AT = "bd92725"
+PROFILED_AT = "44e4d8b"
 PROFILED_DOMINANT = {
-    "c1": dict(kernel="layer_fwd_small_kernel<float,float,4,4,2>", us=6.61, bytes=2 * 4 * 320 * 4 * 1280),
+    "c1": dict(kernel="layer_fwd_small_kernel<float,float,4,4,2>", us=6.60, bytes=2 * 4 * 320 * 4 * 1280),
     # sample-resident backward kernel: reads dy and x, writes the partial dx and the fp32 rows the batch sums are made of
-    "c2": dict(kernel="bwd_resident_kernel<4,bf16 w,3 items>", us=10.06, bytes=3 * 2 * 320 * 4 * 1280 + 4 * 320 * 1280),
-    "c3": dict(kernel="bwd_slab_kernel<bf16>", us=24.29, bytes=3 * 2 * 1280 * 4 * 2560 + 2 * 24 * 10240 + 4 * 24 * 10240),
+    "c2": dict(kernel="bwd_resident_kernel<4,bf16 w,3 items>", us=10.07, bytes=3 * 2 * 320 * 4 * 1280 + 4 * 320 * 1280),
+    "c3": dict(kernel="bwd_slab_kernel<bf16>", us=24.35, bytes=3 * 2 * 1280 * 4 * 2560 + 2 * 24 * 10240 + 4 * 24 * 10240),
     "c4": dict(kernel="bwd_resident_kernel<8,bf16 w,3 items>", us=11.94, bytes=3 * 2 * 256 * 8 * 1280 + 4 * 256 * 1280),
-    "c5": dict(kernel="dphi_large_kernel<9,true>", us=35.40, bytes=2 * 128 * 40960 + 4 * 1088 * 40960),
+    "c5": dict(kernel="dphi_large_kernel<9,true>", us=35.90, bytes=2 * 128 * 40960 + 4 * 1088 * 40960),
 }
 
 CONFIGS = {
