@@ -48,9 +48,9 @@ PROFILED_AT = "44e4d8b"
 PROFILED_DOMINANT = {
     "c1": dict(kernel="layer_fwd_small_kernel<float,float,4,4,2>", us=6.60, bytes=2 * 4 * 320 * 4 * 1280),
     # sample-resident backward kernel: reads dy and x, writes the partial dx and the fp32 rows the batch sums are made of
-    "c2": dict(kernel="bwd_resident_kernel<4,bf16 w,3 items>", us=10.07, bytes=3 * 2 * 320 * 4 * 1280 + 4 * 320 * 1280),
+    "c2": dict(kernel="bwd_resident_kernel<4,bf16 w,2 items,5 tile waves>", us=10.07, bytes=3 * 2 * 320 * 4 * 1280 + 4 * 320 * 1280),
     "c3": dict(kernel="bwd_slab_kernel<bf16>", us=24.35, bytes=3 * 2 * 1280 * 4 * 2560 + 2 * 24 * 10240 + 4 * 24 * 10240),
-    "c4": dict(kernel="bwd_resident_kernel<8,bf16 w,3 items>", us=11.94, bytes=3 * 2 * 256 * 8 * 1280 + 4 * 256 * 1280),
+    "c4": dict(kernel="bwd_resident_kernel<8,bf16 w,1 item,10 tile waves>", us=11.94, bytes=3 * 2 * 256 * 8 * 1280 + 4 * 256 * 1280),
     "c5": dict(kernel="dphi_large_kernel<9,true>", us=35.90, bytes=2 * 128 * 40960 + 4 * 1088 * 40960),
 }
 
